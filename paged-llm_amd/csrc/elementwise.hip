@@ -1,0 +1,191 @@
+// Row-wise and element-wise kernels of the decoder: embedding gather, RMS norm (with the
+// residual sum fused in), SiLU-gated product, rotary position encoding fused with the write of
+// K and V into their pages, page copies.  All arithmetic is done in float; the element type T
+// (float or bfloat16) is only the storage type.
+#include "common.h"
+
+using namespace pllm;
+
+// ---------------------------------------------------------------------------------------------
+// Embedding: out[t, :] = table[ids[t], :]
+template <typename T>
+__global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                    T* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range; never fault
+  const T* src = table + (size_t)id * hidden;
+  T* dst = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+}
+
+PLLM_API int pllm_embed_gather(int dtype, const int* ids, const void* table, void* out, int num_tokens,
+                               int hidden, int vocab, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(embed_gather_kernel<float>, grid, block, 0, stream, ids, (const float*)table, (float*)out, hidden, vocab);
+  else
+    hipLaunchKernelGGL(embed_gather_kernel<bf16>, grid, block, 0, stream, ids, (const bf16*)table, (bf16*)out, hidden, vocab);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// RMS norm of one row per workgroup, optionally after adding `delta` to the residual stream:
+//   s = x[src] + delta[src]   (sum in float, rounded to T: that rounded value is the new residual)
+//   out[r] = T( (s * rsqrt(mean(s^2) + eps)) * w )
+// `row_index` (optional) picks the source rows, so the last norm runs only on rows whose logits
+// are wanted.  `x_out` (optional) receives the new residual rows (may alias x).
+template <typename T>
+__global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const int* __restrict__ row_index,
+                               const float* __restrict__ w, float eps, T* __restrict__ out, T* x_out, int hidden) {
+  extern __shared__ float lds[];
+  float* row = lds;             // [hidden]
+  float* scratch = lds + hidden;  // [16]
+  const int r = blockIdx.x;
+  const size_t src = row_index ? (size_t)row_index[r] : (size_t)r;
+  const T* xr = x + src * hidden;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = to_f32(xr[i]);
+    if (delta) {
+      v = to_f32(from_f32<T>(v + to_f32(delta[src * hidden + i])));
+      if (x_out) x_out[src * hidden + i] = from_f32<T>(v);
+    }
+    row[i] = v;
+    acc += v * v;
+  }
+  const float total = block_sum(acc, scratch);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  T* o = out + (size_t)r * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_f32<T>((row[i] * inv) * w[i]);
+}
+
+PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int* row_index, const float* w, float eps,
+                          void* out, void* x_out, int rows, int hidden, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  const size_t lds = ((size_t)hidden + 16) * sizeof(float);
+  if (lds > 64 * 1024) return -2;  // row does not fit the staging buffer
+  dim3 grid(rows), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, lds, stream, (const float*)x, (const float*)delta, row_index, w, eps,
+                       (float*)out, (float*)x_out, hidden);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16>, grid, block, lds, stream, (const bf16*)x, (const bf16*)delta, row_index, w, eps,
+                       (bf16*)out, (bf16*)x_out, hidden);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Gated activation: out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z / (1 + exp(-z)).
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / inter;
+  const int i = (int)(idx - t * inter);
+  const float g = to_f32(gu[t * 2 * inter + i]);
+  const float u = to_f32(gu[t * 2 * inter + inter + i]);
+  out[idx] = from_f32<T>((g / (1.f + expf(-g))) * u);
+}
+
+PLLM_API int pllm_silu_mul(int dtype, const void* gate_up, void* out, int num_tokens, int inter, hipStream_t stream) {
+  const size_t total = (size_t)num_tokens * inter;
+  if (total == 0) return 0;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total);
+  else
+    hipLaunchKernelGGL(silu_mul_kernel<bf16>, grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rotary encoding of q and k (half-split pairing: element i turns with element i + d/2 by the
+// angle pos * inv_freq[i]; cos/sin come from float tables [positions, d/2]) fused with the cache
+// write.  q is rotated in place inside the fused projection buffer
+//   qkv[t] = [ q heads | k heads | v heads ],  row stride `row_stride` elements.
+// Rotated k goes to k_pages [page, kv_head, offset, d]; v goes, transposed, to
+// v_pages [page, kv_head, d, offset].  slot = page * block_size + offset; slot < 0 skips the write.
+// With write_kv == 0 only q is rotated (a layer that reads another layer's cache).
+template <typename T>
+__global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
+                                    const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                    const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                    int num_heads, int num_kv_heads, int head_dim, int block_size, int write_kv) {
+  const int t = blockIdx.x;
+  const int half = head_dim >> 1;
+  const int pos = positions[t];
+  const float* cs = cos_table ? cos_table + (size_t)pos * half : nullptr;  // no tables: no rotation
+  const float* sn = sin_table ? sin_table + (size_t)pos * half : nullptr;
+  T* row = qkv + (size_t)t * row_stride;
+  const int slot = write_kv ? slot_mapping[t] : -1;
+  const int page = slot >= 0 ? slot / block_size : 0;
+  const int off = slot >= 0 ? slot - page * block_size : 0;
+
+  const int rot_heads = write_kv ? num_heads + num_kv_heads : num_heads;
+  for (int w = threadIdx.x; w < rot_heads * half; w += blockDim.x) {
+    const int head = w / half, i = w - head * half;
+    T* h = row + (size_t)head * head_dim;
+    const float lo = to_f32(h[i]), hi = to_f32(h[i + half]);
+    const float c = cs ? cs[i] : 1.f, s = sn ? sn[i] : 0.f;
+    const T out_lo = from_f32<T>(lo * c - hi * s);
+    const T out_hi = from_f32<T>(hi * c + lo * s);
+    if (head < num_heads) {
+      h[i] = out_lo;
+      h[i + half] = out_hi;
+    } else if (slot >= 0) {
+      const int kvh = head - num_heads;
+      T* dst = k_pages + (((size_t)page * num_kv_heads + kvh) * block_size + off) * head_dim;
+      dst[i] = out_lo;
+      dst[i + half] = out_hi;
+    }
+  }
+  if (slot >= 0) {
+    const T* v = row + (size_t)(num_heads + num_kv_heads) * head_dim;
+    for (int w = threadIdx.x; w < num_kv_heads * head_dim; w += blockDim.x) {
+      const int kvh = w / head_dim, i = w - kvh * head_dim;
+      v_pages[(((size_t)page * num_kv_heads + kvh) * head_dim + i) * block_size + off] = v[w];
+    }
+  }
+}
+
+PLLM_API int pllm_rope_scatter(int dtype, void* qkv, int row_stride, const int* positions, const float* cos_table,
+                               const float* sin_table, const int* slot_mapping, void* k_pages, void* v_pages,
+                               int num_tokens, int num_heads, int num_kv_heads, int head_dim, int block_size,
+                               int write_kv, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  dim3 grid(num_tokens), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(rope_scatter_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, positions, cos_table,
+                       sin_table, slot_mapping, (float*)k_pages, (float*)v_pages, num_heads, num_kv_heads, head_dim,
+                       block_size, write_kv);
+  else
+    hipLaunchKernelGGL(rope_scatter_kernel<bf16>, grid, block, 0, stream, (bf16*)qkv, row_stride, positions, cos_table,
+                       sin_table, slot_mapping, (bf16*)k_pages, (bf16*)v_pages, num_heads, num_kv_heads, head_dim,
+                       block_size, write_kv);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Page copies (copy-on-write): pages[dst[i]] = pages[src[i]], `page_elems` elements each.
+template <typename T>
+__global__ void copy_pages_kernel(T* __restrict__ pages, const int* __restrict__ src, const int* __restrict__ dst,
+                                  size_t page_elems) {
+  const T* s = pages + (size_t)src[blockIdx.x] * page_elems;
+  T* d = pages + (size_t)dst[blockIdx.x] * page_elems;
+  for (size_t i = (size_t)blockIdx.y * blockDim.x + threadIdx.x; i < page_elems; i += (size_t)gridDim.y * blockDim.x) d[i] = s[i];
+}
+
+PLLM_API int pllm_copy_pages(int dtype, void* pages, const int* src, const int* dst, int num_copies, long page_elems,
+                             hipStream_t stream) {
+  if (num_copies <= 0 || page_elems <= 0) return 0;
+  unsigned gy = (unsigned)((page_elems + 255) / 256);
+  if (gy > 64) gy = 64;
+  dim3 grid(num_copies, gy), block(256);
+  if (dtype == PLLM_F32)
+    hipLaunchKernelGGL(copy_pages_kernel<float>, grid, block, 0, stream, (float*)pages, src, dst, (size_t)page_elems);
+  else
+    hipLaunchKernelGGL(copy_pages_kernel<bf16>, grid, block, 0, stream, (bf16*)pages, src, dst, (size_t)page_elems);
+  PLLM_RETURN_LAST_ERROR();
+}

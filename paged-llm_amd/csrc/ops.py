@@ -1,0 +1,290 @@
+"""Python faces of the HIP kernels.
+
+Every function checks on the host that shapes, element types, strides and devices are what the
+kernel and its launch grid assume, and only then passes raw device pointers and the current HIP
+stream through ctypes.  A kernel that cannot take a size says so here with a clear error; there
+is no CPU fallback, and a missing or unbuildable library raises at the first call.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_longlong, c_ulonglong, c_void_p
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+MAX_HEAD_DIM_GENERIC = 256
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: torch.Tensor | None) -> c_void_p:
+    return c_void_p(0) if t is None else c_void_p(t.data_ptr())
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        raise KernelError(f"{what}: kernel launch failed with code {code}")
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _on_gpu(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operands must live on the GPU (there is no CPU path)")
+
+
+_SIGNATURES = {
+    "pllm_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "pllm_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "pllm_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "pllm_rope_scatter": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "pllm_copy_pages": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p],
+    "pllm_gemm_nt": [c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "pllm_paged_attention_generic": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                     c_void_p],
+    "pllm_sample": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_ulonglong, c_void_p,
+                    c_void_p],
+    "pllm_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p],
+}
+_FUNCS: dict = {}
+
+
+def _fn(source: str, name: str, defines: dict | None = None, signature: list | None = None):
+    key = (source, name, tuple(sorted((defines or {}).items())))
+    f = _FUNCS.get(key)
+    if f is None:
+        lib = build.load_library(source, defines)
+        f = getattr(lib, name)
+        f.argtypes = signature or _SIGNATURES[name]
+        f.restype = c_int
+        _FUNCS[key] = f
+    return f
+
+
+# ------------------------------------------------------------------------------------------- rows
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = table[ids[t]]; ids int32 [T] (range already checked by the caller)."""
+    _on_gpu(ids, table)
+    _need(ids.dtype == torch.int32 and ids.dim() == 1 and ids.is_contiguous(), "ids must be contiguous int32 [T]")
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, hidden]")
+    T, (V, H) = ids.numel(), table.shape
+    if out is None:
+        out = torch.empty((T, H), dtype=table.dtype, device=table.device)
+    _need(out.shape == (T, H) and out.dtype == table.dtype and out.is_contiguous(), "bad output for embed_gather")
+    _check(_fn("elementwise.hip", "pllm_embed_gather")(dtype_code(table.dtype), _ptr(ids), _ptr(table), _ptr(out),
+                                                        T, H, V, _stream()), "embed_gather")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, delta: torch.Tensor | None = None,
+            row_index: torch.Tensor | None = None, write_residual: bool = True) -> torch.Tensor:
+    """RMS norm of the rows of x (after adding delta, when given).
+
+    With ``delta`` the sum ``x + delta`` (float add, rounded to the element type) is the new
+    residual; it is written back into ``x`` unless ``write_residual`` is False.  ``row_index``
+    (int32) selects which rows are normed; the output then has one row per index.
+    """
+    _on_gpu(x, weight, delta, row_index)
+    _need(x.dim() == 2 and x.is_contiguous(), "x must be contiguous [rows, hidden]")
+    H = x.shape[1]
+    _need(weight.dtype == torch.float32 and weight.shape == (H,) and weight.is_contiguous(),
+          f"norm weight must be float32 [{H}], got {weight.dtype} {tuple(weight.shape)}")
+    _need(H + 16 <= 16384, f"rmsnorm kernel stages one row in LDS: hidden size {H} is above its limit of 16368")
+    if delta is not None:
+        _need(delta.shape == x.shape and delta.dtype == x.dtype and delta.is_contiguous(), "delta must match x")
+    if row_index is not None:
+        _need(row_index.dtype == torch.int32 and row_index.dim() == 1 and row_index.is_contiguous(),
+              "row_index must be contiguous int32")
+        rows = row_index.numel()
+    else:
+        rows = x.shape[0]
+    out = torch.empty((rows, H), dtype=x.dtype, device=x.device)
+    x_out = x if (delta is not None and write_residual) else None
+    _check(_fn("elementwise.hip", "pllm_rmsnorm")(dtype_code(x.dtype), _ptr(x), _ptr(delta), _ptr(row_index), _ptr(weight),
+                                                   c_float(eps), _ptr(out), _ptr(x_out), rows, H, _stream()), "rmsnorm")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """[T, 2I] -> silu(first half) * second half, [T, I]."""
+    _on_gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gate_up must be contiguous [T, 2I]")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    _check(_fn("elementwise.hip", "pllm_silu_mul")(dtype_code(gate_up.dtype), _ptr(gate_up), _ptr(out), T, I, _stream()),
+           "silu_mul")
+    return out
+
+
+def rope_scatter(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                 num_heads: int, num_kv_heads: int, head_dim: int, slot_mapping: torch.Tensor | None,
+                 k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, block_size: int) -> None:
+    """Rotate q (in place) and k by the tables' angles at ``positions``; write k and v into pages.
+
+    qkv: [T, >= (num_heads + 2 kv_heads) * d] rows (only q columns are needed when nothing is
+    written).  k_pages [P, kv, bs, d], v_pages [P, kv, d, bs].  The caller guarantees
+    positions < cos.shape[0] and slots < P * bs (checked on the host where the batch is built).
+    """
+    write_kv = k_pages is not None
+    _on_gpu(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages)
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be [T, width] with unit inner stride")
+    need_cols = (num_heads + (2 * num_kv_heads if write_kv else 0)) * head_dim
+    _need(qkv.shape[1] >= need_cols, f"qkv rows hold {qkv.shape[1]} values, need {need_cols}")
+    _need(head_dim % 2 == 0, "rotary pairing needs an even head size")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(), "positions: int32 [T]")
+    half = head_dim // 2
+    _need((cos is None) == (sin is None), "cos and sin tables come together")
+    for t in (cos, sin):
+        if t is None:
+            continue
+        _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == half and t.is_contiguous(),
+              f"rotary tables must be float32 [positions, {half}]")
+    if write_kv:
+        _need(slot_mapping is not None and slot_mapping.dtype == torch.int32 and slot_mapping.shape == (T,)
+              and slot_mapping.is_contiguous(), "slot_mapping: int32 [T]")
+        P = k_pages.shape[0]
+        _need(tuple(k_pages.shape) == (P, num_kv_heads, block_size, head_dim) and k_pages.is_contiguous()
+              and k_pages.dtype == qkv.dtype, "k_pages must be contiguous [pages, kv_heads, block_size, head_dim]")
+        _need(tuple(v_pages.shape) == (P, num_kv_heads, head_dim, block_size) and v_pages.is_contiguous()
+              and v_pages.dtype == qkv.dtype, "v_pages must be contiguous [pages, kv_heads, head_dim, block_size]")
+    _check(_fn("elementwise.hip", "pllm_rope_scatter")(
+        dtype_code(qkv.dtype), _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
+        _ptr(k_pages), _ptr(v_pages), T, num_heads, num_kv_heads, head_dim, block_size, 1 if write_kv else 0, _stream()),
+        "rope_scatter")
+
+
+def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
+    """pages[dst[i]] = pages[src[i]] (whole pages of one layer's K or V)."""
+    _on_gpu(pages, src, dst)
+    _need(pages.is_contiguous() and pages.dim() >= 2, "pages must be contiguous [pages, ...]")
+    _need(src.dtype == torch.int32 and dst.dtype == torch.int32 and src.shape == dst.shape and src.dim() == 1,
+          "src and dst must be int32 vectors of one length")
+    page_elems = pages[0].numel()
+    _check(_fn("elementwise.hip", "pllm_copy_pages")(dtype_code(pages.dtype), _ptr(pages), _ptr(src), _ptr(dst),
+                                                      src.numel(), page_elems, _stream()), "copy_pages")
+
+
+# ------------------------------------------------------------------------------------------- products
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """a [M, K] times w [N, K] transposed, float accumulation in ascending k, any sizes."""
+    _on_gpu(a, w)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], f"gemm shapes {tuple(a.shape)} x {tuple(w.shape)}^T")
+    _need(a.stride(1) == 1 and w.stride(1) == 1, "gemm operands need unit inner stride")
+    _need(a.dtype == w.dtype, "gemm operands must share their element type")
+    out_dtype = out_dtype or a.dtype
+    M, K = a.shape
+    N = w.shape[0]
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    _check(_fn("gemm_generic.hip", "pllm_gemm_nt")(dtype_code(a.dtype), dtype_code(out_dtype), _ptr(a), a.stride(0),
+                                                    _ptr(w), w.stride(0), _ptr(out), N, M, N, K, _stream()), "gemm_generic")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- attention
+def _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim):
+    _on_gpu(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k)
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= num_heads * head_dim, "q must be [T, >= heads * d]")
+    P, kvh, bs, d = k_pages.shape
+    _need(kvh == num_kv_heads and d == head_dim and k_pages.is_contiguous(), "k_pages: contiguous [pages, kv_heads, bs, d]")
+    _need(tuple(v_pages.shape) == (P, kvh, d, bs) and v_pages.is_contiguous(), "v_pages: contiguous [pages, kv_heads, d, bs]")
+    _need(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype, "q, k_pages and v_pages must share their element type")
+    _need(num_heads % num_kv_heads == 0, "heads must be a multiple of kv heads")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1, "block_tables: int32 [S, B]")
+    S = block_tables.shape[0]
+    _need(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.numel() >= S + 1 and cu_seqlens_q.is_contiguous(), "cu_seqlens_q: int32 [S+1]")
+    _need(seq_lens_k.dtype == torch.int32 and seq_lens_k.numel() >= S and seq_lens_k.is_contiguous(), "seq_lens_k: int32 [S]")
+    return S, bs
+
+
+def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
+                            cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
+                            head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Causal attention over paged keys and values; one wavefront per (token, head), all in float.
+
+    The caller guarantees (and the step function checks on the host) that every table entry
+    below ceil(seq_len / block_size) is a valid page and that cu_seqlens_q ends at q.shape[0].
+    """
+    S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
+    _need(0 < head_dim <= MAX_HEAD_DIM_GENERIC, f"attention kernel takes head sizes up to {MAX_HEAD_DIM_GENERIC}, got {head_dim}")
+    _need(num_heads <= 65535, "too many heads for one launch")
+    T = q.shape[0]
+    if out is None:
+        out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
+    _need(out.shape == (T, num_heads * head_dim) and out.stride(1) == 1 and out.dtype == q.dtype, "bad attention output")
+    _check(_fn("attention_generic.hip", "pllm_paged_attention_generic")(
+        dtype_code(q.dtype), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0),
+        _ptr(block_tables), block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, num_heads, num_kv_heads,
+        head_dim, bs, c_float(scale), int(window or 0), _stream()), "paged_attention_generic")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- sampling
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    _on_gpu(logits)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "logits: contiguous float32 [n, vocab]")
+    n, V = logits.shape
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _check(_fn("sampling.hip", "pllm_argmax")(_ptr(logits), n, V, _ptr(out), _stream()), "argmax")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           request_key: torch.Tensor, step: torch.Tensor, seed: int) -> torch.Tensor:
+    """One token per row: greedy where temperature < 1e-5, else a draw under top-k / top-p."""
+    _on_gpu(logits, temperature, top_k, top_p, request_key, step)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "logits: contiguous float32 [n, vocab]")
+    n, V = logits.shape
+    for t, dt, nm in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"), (top_p, torch.float32, "top_p"),
+                      (request_key, torch.int64, "request_key"), (step, torch.int32, "step")):
+        _need(t.dtype == dt and t.shape == (n,) and t.is_contiguous(), f"{nm}: {dt} [{n}]")
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _check(_fn("sampling.hip", "pllm_sample")(_ptr(logits), n, V, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                               _ptr(request_key), _ptr(step), c_ulonglong(seed & (2**64 - 1)), _ptr(out),
+                                               _stream()), "sample")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- choices
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """The fast bfloat16 products; None when neither takes the shape (the caller falls back to
+    the plain kernel).  The choice looks at the number of rows only."""
+    return None
+
+
+def gate_up_silu(h: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(h Wg^T) * (h Wu^T) with Wg, Wu stacked in w_gate_up [2I, K]."""
+    from ..parts.linear import linear
+    return silu_mul(linear(h, w_gate_up))
+
+
+def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
+                    scale, window, ctx) -> torch.Tensor:
+    """Attention of one step's queries over the paged cache: the MFMA kernel for bfloat16 where it
+    takes the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions."""
+    return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
+                                   num_kv_heads, head_dim, scale, window)

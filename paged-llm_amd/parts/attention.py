@@ -1,0 +1,87 @@
+"""Causal attention over the paged cache with grouped heads.
+
+q/k/v projections without bias -> rotary encoding of q and k -> k and v written to their slots ->
+attention over all keys of the request through the block table -> output projection
+(pagedllm/model/llama.py:131-160).  Sizes, the score scale, an optional window and the position
+encoding come in as parameters.  The three input projections are fused into one matrix when the
+weights arrive, so one product serves them.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..csrc import ops
+from .base import CacheSpec, Mixer
+from .linear import linear
+from .registry import BuildEnv, register_mixer
+from .spec import PartSpec, WeightSpec
+
+
+class PagedAttention(Mixer):
+    def __init__(self, params: dict, env: BuildEnv):
+        self.hidden = env.hidden_size
+        self.num_heads = int(params["num_heads"])
+        self.num_kv_heads = int(params.get("num_kv_heads", self.num_heads))
+        self.head_dim = int(params["head_dim"])
+        self.scale = float(params.get("scale", self.head_dim ** -0.5))
+        self.window = int(params.get("window") or 0)
+        # False for a layer that always reads another layer's cache: it then has no k/v weights.
+        self.kv_proj = bool(params.get("kv_proj", True))
+        if self.num_heads % self.num_kv_heads:
+            raise ValueError(f"{self.num_heads} heads are no multiple of {self.num_kv_heads} kv heads")
+        if self.head_dim % 16 or not 16 <= self.head_dim <= 256:
+            raise ValueError(f"attention kernels take head sizes 16..256 in steps of 16, got {self.head_dim}")
+        pos = params.get("position")
+        self.position = env.position_encoding(PartSpec(**pos) if isinstance(pos, dict) else pos) if pos else None
+        self.dtype, self.device = env.dtype, env.device
+        self._w: dict[str, torch.Tensor] = {}
+        self.w_qkv: torch.Tensor | None = None
+        self.w_o: torch.Tensor | None = None
+
+    # ---- weights
+    def weight_specs(self):
+        q, kv = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        specs = {"q_proj.weight": WeightSpec((q, self.hidden)), "o_proj.weight": WeightSpec((self.hidden, q))}
+        if self.kv_proj:
+            specs["k_proj.weight"] = WeightSpec((kv, self.hidden))
+            specs["v_proj.weight"] = WeightSpec((kv, self.hidden))
+        return specs
+
+    def assign(self, name, tensor):
+        if name not in self.weight_specs():
+            raise KeyError(name)
+        self._w[name] = tensor.to(device=self.device, dtype=self.dtype)
+
+    def finalize(self):
+        names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.kv_proj else [])
+        self.w_qkv = torch.cat([self._w[n] for n in names], dim=0).contiguous()
+        self.w_o = self._w["o_proj.weight"].contiguous()
+        self._w.clear()
+
+    # ---- what it keeps
+    def cache_spec(self):
+        kind = "window" if self.window > 0 else "full"
+        return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
+
+    # ---- compute
+    def forward(self, h, ctx, cache, state):
+        nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        view = ctx.groups[cache.group]
+        write = cache.writable
+        if write and not self.kv_proj:
+            raise RuntimeError("this attention layer has no k/v projections and must read another layer's cache")
+        w_in = self.w_qkv if write or not self.kv_proj else self.w_qkv[: nh * d]
+        qkv = linear(h, w_in)
+        cos = sin = None
+        if self.position is not None:
+            cos, sin = self.position.cos, self.position.sin
+        ops.rope_scatter(qkv, ctx.positions, cos, sin, nh, nkv, d,
+                         view.slot_mapping if write else None,
+                         cache.k_pages if write else None, cache.v_pages if write else None, cache.block_size)
+        o = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
+                                nh, nkv, d, self.scale, self.window, ctx)
+        return linear(o, self.w_o)
+
+
+register_mixer("paged_attention", PagedAttention)

@@ -1,0 +1,102 @@
+"""Interfaces of the parts a decoder layer is put together from.
+
+A part gets every size and constant through its constructor, declares the tensors it wants by
+name (relative to its own prefix), receives them from the loader, and computes on the rows the
+step function hands it.  No part knows which model it is in, which layer it is, or how the
+batch was cut.
+
+* ``Norm``            rows -> rows; ``add_norm`` fuses the residual sum in front of it.
+* ``PositionEncoding``  owns its tables; a mixer asks it to encode q/k (rotary) in place.
+* ``Mixer``           mixes information between the tokens of a request.  It may keep a growing
+                      cache (it then names a ``CacheSpec``: pages of keys and values) and/or a
+                      state of fixed size per request (``StateSpec``: a slot in a state tensor).
+* ``FeedForward``     rows -> rows, no mixing between tokens.
+* ``Block``           the arrangement of two norms, a mixer and a feed-forward around the
+                      residual stream.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .spec import WeightSpec
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """What a mixer keeps per token.  Layers with equal specs share a group of pages."""
+    kind: str                 # "full": all keys;  "window": only the last `window` positions
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0           # > 0 for kind "window"
+
+    def group_name(self) -> str:
+        base = f"{self.kind}{self.window if self.kind == 'window' else ''}"
+        return f"{base}_kv{self.num_kv_heads}x{self.head_dim}"
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state per request: one slot of shape ``shape`` in a [slots, *shape] tensor."""
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    """Common ground: declared weights, assignment, and a hook once all weights are there."""
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {}
+
+    def assign(self, name: str, tensor: torch.Tensor) -> None:
+        raise KeyError(name)
+
+    def finalize(self) -> None:
+        pass
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, row_index: torch.Tensor | None = None) -> torch.Tensor:
+        raise NotImplementedError
+
+    def add_norm(self, x: torch.Tensor, delta: torch.Tensor, row_index: torch.Tensor | None = None,
+                 write_residual: bool = True) -> torch.Tensor:
+        """x += delta (the residual sum, in float, rounded once), then the norm of the new x."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, max_positions: int) -> None:
+        """Make tables for positions below ``max_positions``."""
+
+
+class Mixer(Part):
+    def cache_spec(self) -> CacheSpec | None:
+        return None
+
+    def state_spec(self) -> StateSpec | None:
+        return None
+
+    def forward(self, h: torch.Tensor, ctx, cache, state) -> torch.Tensor:
+        """h: normed rows [T, hidden].  ctx: the step's StepContext.  cache: LayerCache of the
+        layer this mixer reads (with ``writable`` False when it belongs to another layer), or
+        None.  state: [slots, *shape] tensor, or None."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of the parts around the residual stream.
+
+    The stream is handed on as a pair (x, delta): delta is the last branch output that has not
+    been added yet, so that the next norm can add it in the same kernel.
+    """
+
+    def forward(self, x: torch.Tensor, delta: torch.Tensor | None, ctx, cache, state):
+        raise NotImplementedError

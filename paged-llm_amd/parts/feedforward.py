@@ -1,0 +1,48 @@
+"""Gated feed-forward: down(act(gate(x)) * up(x)) without bias, act = SiLU
+(pagedllm/model/llama.py:163-171).  gate and up are fused into one matrix [2I, H] when the
+weights arrive; the activation and the product run in float in one kernel."""
+
+from __future__ import annotations
+
+import torch
+
+from ..csrc import ops
+from .base import FeedForward
+from .linear import linear
+from .registry import BuildEnv, register_feed_forward
+from .spec import WeightSpec
+
+
+class GatedMLP(FeedForward):
+    def __init__(self, params: dict, env: BuildEnv):
+        self.hidden = env.hidden_size
+        self.inter = int(params["intermediate_size"])
+        act = params.get("activation", "silu")
+        if act != "silu":
+            raise NotImplementedError(f"gated feed-forward activation {act!r} (silu only)")
+        self.dtype, self.device = env.dtype, env.device
+        self._w: dict[str, torch.Tensor] = {}
+        self.w_gate_up: torch.Tensor | None = None
+        self.w_down: torch.Tensor | None = None
+
+    def weight_specs(self):
+        return {"gate_proj.weight": WeightSpec((self.inter, self.hidden)),
+                "up_proj.weight": WeightSpec((self.inter, self.hidden)),
+                "down_proj.weight": WeightSpec((self.hidden, self.inter))}
+
+    def assign(self, name, tensor):
+        if name not in self.weight_specs():
+            raise KeyError(name)
+        self._w[name] = tensor.to(device=self.device, dtype=self.dtype)
+
+    def finalize(self):
+        self.w_gate_up = torch.cat([self._w["gate_proj.weight"], self._w["up_proj.weight"]], dim=0).contiguous()
+        self.w_down = self._w["down_proj.weight"].contiguous()
+        self._w.clear()
+
+    def forward(self, h, ctx):
+        act = ops.gate_up_silu(h, self.w_gate_up)
+        return linear(act, self.w_down)
+
+
+register_feed_forward("gated_mlp", GatedMLP)

@@ -1,0 +1,287 @@
+"""Each HIP kernel alone against a plain float reference, at sizes other than the tiny models'."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from tests.plain import llama_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1.6e-2}
+
+
+def ops():
+    from paged_llm_amd.csrc import ops as _ops
+    return _ops
+
+
+def rel_err(got, want):
+    got, want = got.float().cpu(), want.float().cpu()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ----------------------------------------------------------------------------------- rows
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_gather(dtype):
+    table = rnd(301, 72, dtype=dtype).cuda()
+    ids = torch.tensor([0, 300, 7, 7, 150], dtype=torch.int32).cuda()
+    out = ops().embed_gather(ids, table)
+    assert torch.equal(out.cpu(), table.cpu()[ids.cpu().long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [48, 200, 2048, 5000])
+def test_rmsnorm(dtype, hidden):
+    x = rnd(9, hidden, seed=1, dtype=dtype, scale=3.0)
+    w = 1 + 0.3 * rnd(hidden, seed=2)
+    eps = 1e-3
+    out = ops().rmsnorm(x.cuda(), w.cuda(), eps)
+    want = plain.rms_norm(x.float(), w, eps)
+    assert rel_err(out, want) <= TOL[dtype]
+    # the library routine the formula reduces to
+    lib = torch.nn.functional.rms_norm(x.float(), (hidden,), w, eps)
+    assert rel_err(want, lib) <= 1e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_with_residual_sum_and_row_choice(dtype):
+    hidden = 136
+    x = rnd(12, hidden, seed=3, dtype=dtype)
+    d = rnd(12, hidden, seed=4, dtype=dtype)
+    w = 1 + 0.3 * rnd(hidden, seed=5)
+    xg = x.cuda().clone()
+    out = ops().rmsnorm(xg, w.cuda(), 1e-5, delta=d.cuda())
+    summed = (x.float() + d.float()).to(dtype)                 # the residual is rounded once
+    assert torch.equal(xg.cpu(), summed)
+    assert rel_err(out, plain.rms_norm(summed.float(), w, 1e-5)) <= TOL[dtype]
+    # chosen rows, residual left alone
+    idx = torch.tensor([11, 0, 5], dtype=torch.int32)
+    xg = x.cuda().clone()
+    out = ops().rmsnorm(xg, w.cuda(), 1e-5, delta=d.cuda(), row_index=idx.cuda(), write_residual=False)
+    assert torch.equal(xg.cpu(), x)
+    assert rel_err(out, plain.rms_norm(summed.float()[idx.long()], w, 1e-5)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    inter = 150
+    gu = rnd(7, 2 * inter, seed=6, dtype=dtype, scale=2.0)
+    out = ops().silu_mul(gu.cuda())
+    want = torch.nn.functional.silu(gu.float()[:, :inter]) * gu.float()[:, inter:]
+    assert rel_err(out, want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 16, 16), (3, 1, 48, 8), (8, 8, 128, 32)])
+def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs):
+    from paged_llm_amd.parts.registry import BuildEnv
+    from paged_llm_amd.parts.rope import RotaryEncoding
+    T, pages = 23, 9
+    rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, dtype, torch.device("cuda"), 512, {}))
+    rope.prepare(512)
+    width = (heads + 2 * kv_heads) * d
+    qkv = rnd(T, width, seed=7, dtype=dtype)
+    positions = torch.tensor([(5 * t + 3) % 500 for t in range(T)], dtype=torch.int32)
+    perm = torch.randperm(pages * bs, generator=torch.Generator().manual_seed(8))[:T].to(torch.int32)
+    k_pages = torch.zeros(pages, kv_heads, bs, d, dtype=dtype).cuda()
+    v_pages = torch.zeros(pages, kv_heads, d, bs, dtype=dtype).cuda()
+    g = qkv.cuda().clone()
+    ops().rope_scatter(g, positions.cuda(), rope.cos, rope.sin, heads, kv_heads, d, perm.cuda(), k_pages, v_pages, bs)
+
+    inv = plain.inverse_frequencies(d, 10000.0, None)
+    ang = plain.rotary_angles(positions, inv)
+    q = plain.apply_rotary(qkv.float()[:, :heads * d].view(T, heads, d), ang)
+    k = plain.apply_rotary(qkv.float()[:, heads * d:(heads + kv_heads) * d].view(T, kv_heads, d), ang)
+    v = qkv.float()[:, (heads + kv_heads) * d:].view(T, kv_heads, d)
+    assert rel_err(g[:, :heads * d].view(T, heads, d), q) <= TOL[dtype]
+    kp, vp = k_pages.float().cpu(), v_pages.float().cpu()
+    for t in range(T):
+        page, off = int(perm[t]) // bs, int(perm[t]) % bs
+        assert rel_err(kp[page, :, off, :], k[t]) <= TOL[dtype]
+        assert torch.equal(vp[page, :, :, off], v[t].to(dtype).float())
+    # untouched slots stay zero
+    written = torch.zeros(pages * bs, dtype=torch.bool)
+    written[perm.long()] = True
+    assert kp.permute(0, 2, 1, 3).reshape(pages * bs, -1)[~written].abs().max() == 0
+
+
+def test_copy_pages():
+    pages = rnd(6, 2, 8, 16, seed=9).cuda()
+    before = pages.cpu().clone()
+    ops().copy_pages(pages, torch.tensor([0, 3], dtype=torch.int32).cuda(), torch.tensor([5, 1], dtype=torch.int32).cuda())
+    after = pages.cpu()
+    assert torch.equal(after[5], before[0]) and torch.equal(after[1], before[3])
+    assert torch.equal(after[[0, 2, 3, 4]], before[[0, 2, 3, 4]])
+
+
+# ----------------------------------------------------------------------------------- products
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 64), (65, 64, 33), (200, 96, 176), (17, 517, 96)])
+def test_gemm_generic(dtype, m, n, k):
+    a, w = rnd(m, k, seed=10, dtype=dtype), rnd(n, k, seed=11, dtype=dtype)
+    want = a.double() @ w.double().T
+    out = ops().gemm_generic(a.cuda(), w.cuda())
+    assert rel_err(out, want) <= TOL[dtype]
+    out32 = ops().gemm_generic(a.cuda(), w.cuda(), out_dtype=torch.float32)
+    assert out32.dtype == torch.float32 and rel_err(out32, want) <= 1e-5
+
+
+def test_gemm_generic_rows_do_not_depend_on_the_batch():
+    a, w = rnd(70, 200, seed=12), rnd(90, 200, seed=13)
+    whole = ops().gemm_generic(a.cuda(), w.cuda()).cpu()
+    for lo, hi in [(0, 1), (5, 7), (63, 70)]:
+        part = ops().gemm_generic(a[lo:hi].cuda(), w.cuda()).cpu()
+        assert torch.equal(part, whole[lo:hi])
+
+
+# ----------------------------------------------------------------------------------- attention
+def paged_case(seq_lens_k, num_q, heads, kv_heads, d, bs, dtype, seed=0, spare=3):
+    """Keys and values in shuffled pages (test vectors of the reference's
+    tests/test_attention_reference.py:10-28, in this engine's page layout)."""
+    g = torch.Generator().manual_seed(seed)
+    nblocks = [(L + bs - 1) // bs for L in seq_lens_k]
+    total = sum(nblocks) + spare
+    perm = torch.randperm(total, generator=g)
+    tables = torch.zeros(len(seq_lens_k), max(nblocks), dtype=torch.int32)
+    p = 0
+    for s, nb in enumerate(nblocks):
+        tables[s, :nb] = perm[p:p + nb]
+        p += nb
+    k_pages = torch.randn(total, kv_heads, bs, d, generator=g).to(dtype)
+    v_pages = torch.randn(total, kv_heads, d, bs, generator=g).to(dtype)
+    q = torch.randn(sum(num_q), heads * d, generator=g).to(dtype)
+    cu = torch.tensor([0] + list(np.cumsum(num_q)), dtype=torch.int32)
+    return q, k_pages, v_pages, tables, cu, torch.tensor(seq_lens_k, dtype=torch.int32)
+
+
+def dense_attention(q, k_pages, v_pages, tables, cu, lens, heads, kv_heads, d, scale, window=None):
+    bs = k_pages.shape[2]
+    out = torch.empty(q.shape[0], heads * d)
+    for s in range(len(lens)):
+        L, lo, hi = int(lens[s]), int(cu[s]), int(cu[s + 1])
+        idx = torch.arange(L)
+        page, off = tables[s][idx // bs].long(), idx % bs
+        k = k_pages.float()[page, :, off, :]                       # [L, kv, d]
+        v = v_pages.float()[page, :, :, off]                       # [L, kv, d]
+        q_full = torch.zeros(L, heads, d)
+        q_full[L - (hi - lo):] = q[lo:hi].float().view(-1, heads, d)
+        o = plain.causal_attention(q_full, k, v, scale, window)
+        out[lo:hi] = o[L - (hi - lo):].reshape(hi - lo, heads * d)
+    return out
+
+
+CASES = [([5], [5]), ([33, 8, 17], [33, 8, 17]), ([40, 9, 64], [1, 1, 1]), ([40, 9, 64], [8, 1, 3]),
+         ([7], [7]), ([129, 300, 17], [129, 300, 17]), ([1000, 33, 2048, 5], [1, 1, 1, 1]), ([500, 64, 77], [37, 1, 12]),
+         ([1], [1])]
+SHAPES = [(4, 2, 32, 8), (8, 8, 64, 16), (32, 4, 64, 16), (3, 1, 48, 32), (5, 5, 16, 4), (6, 2, 128, 16), (2, 1, 256, 16)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,d,bs", SHAPES)
+@pytest.mark.parametrize("lens,num_q", CASES)
+def test_paged_attention_generic(dtype, heads, kv_heads, d, bs, lens, num_q):
+    if sum(lens) * heads * d > 3_000_000 and (heads, d) not in ((32, 64),):
+        pytest.skip("long case kept for one shape")
+    q, kp, vp, tables, cu, sl = paged_case(lens, num_q, heads, kv_heads, d, bs, dtype, seed=1)
+    scale = 1 / math.sqrt(d)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, scale)
+    got = ops().paged_attention_generic(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
+                                        d, scale)
+    assert rel_err(got, want) <= (2e-5 if dtype == torch.float32 else 1.6e-2)
+
+
+@pytest.mark.parametrize("window", [1, 5, 64, 100])
+def test_paged_attention_generic_window(window):
+    heads, kv_heads, d, bs = 4, 2, 32, 16
+    q, kp, vp, tables, cu, sl = paged_case([150, 70, 9], [30, 1, 9], heads, kv_heads, d, bs, torch.float32, seed=2)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, 0.2, window)
+    got = ops().paged_attention_generic(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
+                                        d, 0.2, window)
+    assert rel_err(got, want) <= 2e-5
+
+
+def test_attention_ignores_table_padding_and_stale_slots():
+    """Garbage in table entries past the context and in slots past it must not change anything
+    (tests/test_triton_kernel.py:37-44 of the reference)."""
+    heads, kv_heads, d, bs = 4, 2, 32, 16
+    q, kp, vp, tables, cu, sl = paged_case([20, 5], [1, 1], heads, kv_heads, d, bs, torch.float32, seed=3)
+    args = (heads, kv_heads, d, 0.3)
+    a = ops().paged_attention_generic(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), *args)
+    t2 = tables.clone()
+    t2[1, 1:] = 999_999
+    kp2, vp2 = kp.clone(), vp.clone()
+    kp2[tables[1, 0], :, 5:, :] = float("nan")            # slots behind the 5 tokens of request 1
+    vp2[tables[1, 0], :, :, 5:] = float("nan")
+    b = ops().paged_attention_generic(q.cuda(), kp2.cuda(), vp2.cuda(), t2.cuda(), cu.cuda(), sl.cuda(), *args)
+    assert torch.equal(a.cpu(), b.cpu())
+
+
+def test_attention_one_far_key_stands_out():
+    """One key among 700 is made to dominate: the output must be that key's value row."""
+    heads, kv_heads, d, bs = 2, 1, 32, 16
+    q, kp, vp, tables, cu, sl = paged_case([700], [1], heads, kv_heads, d, bs, torch.float32, seed=4)
+    far = 3
+    page, off = int(tables[0, far // bs]), far % bs
+    kp[page, 0, off, :] = q[0, :d] * 50
+    got = ops().paged_attention_generic(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
+                                        d, 1.0).cpu()
+    assert torch.allclose(got[0, :d], vp[page, 0, :, off], atol=1e-5)
+
+
+# ----------------------------------------------------------------------------------- sampling
+def test_argmax_takes_the_first_maximum():
+    z = rnd(5, 1000, seed=14)
+    z[1, 17] = z[1, 900] = 50.0
+    z[2, :] = 0.0
+    got = ops().argmax(z.cuda()).cpu()
+    assert got.tolist() == z.argmax(-1).tolist()[:1] + [17, 0] + z.argmax(-1).tolist()[3:]
+
+
+def sample_rows(z, temperature, top_k, top_p, draws, seed=0):
+    n = z.shape[0]
+    out = []
+    zg = z.cuda()
+    t = torch.full((n,), temperature, dtype=torch.float32).cuda()
+    k = torch.full((n,), top_k, dtype=torch.int32).cuda()
+    p = torch.full((n,), top_p, dtype=torch.float32).cuda()
+    keys = torch.arange(n, dtype=torch.int64).cuda()
+    for step in range(draws):
+        s = torch.full((n,), step, dtype=torch.int32).cuda()
+        out.append(ops().sample(zg, t, k, p, keys, s, seed).cpu())
+    return torch.stack(out)            # [draws, n]
+
+
+def test_sampling_reduces_to_argmax():
+    z = rnd(4, 333, seed=15)
+    assert sample_rows(z, 0.0, -1, 1.0, 1)[0].tolist() == z.argmax(-1).tolist()
+    assert sample_rows(z, 1.0, 1, 1.0, 3).tolist() == [z.argmax(-1).tolist()] * 3
+    assert sample_rows(z, 1.0, -1, 1e-6, 3).tolist() == [z.argmax(-1).tolist()] * 3
+
+
+def test_sampling_same_seed_same_tokens_other_seed_other_tokens():
+    z = rnd(6, 97, seed=16)
+    a, b, c = sample_rows(z, 1.0, -1, 1.0, 20, seed=1), sample_rows(z, 1.0, -1, 1.0, 20, seed=1), sample_rows(z, 1.0, -1, 1.0, 20, seed=2)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+
+
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, -1, 1.0), (0.7, -1, 1.0), (1.3, 5, 1.0), (1.0, -1, 0.6), (0.9, 8, 0.8)])
+def test_sampling_frequencies_follow_the_filtered_distribution(temperature, top_k, top_p):
+    vocab, draws = 24, 4000
+    z = rnd(1, vocab, seed=17, scale=1.5)
+    probs = plain.filtered_probabilities(z[0], temperature, top_k, top_p).numpy()
+    got = sample_rows(z, temperature, top_k, top_p, draws)[:, 0].numpy()
+    counts = np.bincount(got, minlength=vocab)
+    assert counts[probs == 0].sum() == 0, "a filtered token was drawn"
+    keep = probs > 0
+    chi2 = float(((counts[keep] - draws * probs[keep]) ** 2 / (draws * probs[keep])).sum())
+    dof = int(keep.sum()) - 1
+    assert chi2 < dof + 5 * math.sqrt(2 * max(dof, 1)) + 5, f"chi-square {chi2:.1f} for {dof} degrees of freedom"

@@ -1,0 +1,149 @@
+"""The engine's logits against the plain implementation under every way of cutting the work:
+whole prompts, the last 32 tokens one by one, portions of changing size down to two tokens, and up
+to four live requests mixed in one batch with so few pages that they are used again; in true
+32-bit and in bfloat16.  The engine is driven through the replay session (the model, step
+function, cache manager and kernels that generation uses)."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers
+from tests.helpers import TraceBuilder
+from tests.tiny_configs import TINY_A, TINY_B, TINY_C
+
+pytestmark = pytest.mark.gpu
+
+# Largest difference allowed, relative to the largest logit of the request.
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+LENGTHS = {"A": [5, 17, 33, 40, 150], "B": [1, 9, 60, 100, 127], "C": [3, 64, 65, 200]}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, cfg in CONFIGS.items():
+        for stored in ("float32", "bfloat16"):
+            out[name, stored] = helpers.make_folder(tmp_path_factory.mktemp(f"{name}_{stored}"), cfg, seed=11, stored=stored)
+    return out
+
+
+def session_for(folder, dtype, max_tokens):
+    from paged_llm_amd.engine.replay import ReplaySession
+    return ReplaySession(folder, dtype, max_tokens, None)
+
+
+def requests_for(name):
+    vocab = CONFIGS[name]["vocab_size"]
+    return {f"r{i}": helpers.random_tokens(n, vocab, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
+
+
+def check(got: dict, folder: str, reqs: dict, dtype: str):
+    assert got, "nothing was compared"
+    by_req = {}
+    for (rid, pos), row in got.items():
+        by_req.setdefault(rid, {})[pos] = row
+    for rid, rows in by_req.items():
+        want = helpers.plain_logits(folder, reqs[rid])
+        for pos, row in rows.items():
+            err = helpers.worst(row, want[pos])
+            assert err <= TOL[dtype], f"request {rid} position {pos}: relative error {err:.3g} > {TOL[dtype]}"
+
+
+def rounded(n, m=64):
+    return (n + m - 1) // m * m
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_each_request_whole(folders, name, dtype):
+    folder = folders[name, "float32" if dtype == "float32" else "bfloat16"]
+    reqs = requests_for(name)
+    session = session_for(folder, dtype, rounded(max(len(t) for t in reqs.values())))
+    trace = TraceBuilder()
+    for rid, toks in reqs.items():
+        trace.step([(rid, toks, "all")], end=[rid])
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_32_tokens_one_by_one(folders, name, dtype):
+    folder = folders[name, "float32" if dtype == "float32" else "bfloat16"]
+    reqs = {rid: t for rid, t in requests_for(name).items() if len(t) > 34}
+    session = session_for(folder, dtype, rounded(max(len(t) for t in reqs.values())))
+    trace = TraceBuilder()
+    for rid, toks in reqs.items():
+        cut = len(toks) - 32
+        trace.step([(rid, toks[:cut], "last")])
+        for i in range(cut, len(toks)):
+            trace.step([(rid, toks[i:i + 1], "all")], end=[rid] if i == len(toks) - 1 else [])
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(folders, name, dtype):
+    folder = folders[name, "float32" if dtype == "float32" else "bfloat16"]
+    reqs = requests_for(name)
+    session = session_for(folder, dtype, rounded(max(len(t) for t in reqs.values())))
+    trace = TraceBuilder()
+    sizes = itertools.cycle([7, 2, 13, 3, 2, 21, 16, 5, 1, 32, 2])
+    for rid, toks in reqs.items():
+        at = 0
+        while at < len(toks):
+            n = min(next(sizes), len(toks) - at)
+            trace.step([(rid, toks[at:at + n], "all")], end=[rid] if at + n == len(toks) else [])
+            at += n
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+
+
+def mixed_trace(reqs: dict, max_live: int, seed: int):
+    """Portions of some requests beside decoded tokens of others, up to ``max_live`` at a time.
+    Returns the trace and the largest number of tokens (rounded up per request to 64) live at once."""
+    rng = np.random.default_rng(seed)
+    waiting = list(reqs.items())
+    live: dict = {}
+    trace, peak = TraceBuilder(), 0
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, toks = waiting.pop(0)
+            live[rid] = [toks, 0, max(1, len(toks) - int(rng.integers(0, 12)))]   # tokens, sent, prompt part
+        entries, ended = [], []
+        for rid, st in list(live.items()):
+            toks, sent, prompt = st
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                                   # left out of this step, goes on later
+            n = 1 if sent >= prompt else int(min(prompt - sent, rng.choice([2, 3, 5, 8, 19, 40])))
+            entries.append((rid, toks[sent:sent + n], "all"))
+            st[1] = sent + n
+            if st[1] == len(toks):
+                ended.append(rid)
+        peak = max(peak, sum(rounded(len(st[0])) for st in live.values()))
+        if entries:
+            trace.step(entries, end=ended)
+        for rid in ended:
+            del live[rid]
+    return trace, peak
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_pages_used_again(folders, name, dtype):
+    folder = folders[name, "float32" if dtype == "float32" else "bfloat16"]
+    base = requests_for(name)
+    vocab = CONFIGS[name]["vocab_size"]
+    # Each request twice (other tokens the second time), so that freed pages hold stale keys.
+    reqs = dict(base)
+    for i, (rid, toks) in enumerate(base.items()):
+        reqs[rid + "x"] = helpers.random_tokens(len(toks), vocab, seed=900 + i)
+    trace, peak = mixed_trace(reqs, max_live=4, seed=5)
+    session = session_for(folder, dtype, peak)
+    got = helpers.replay_in_process(session, trace)
+    assert len(got) == sum(len(t) for t in reqs.values())
+    check(got, folder, reqs, dtype)
+    session.manager.check_invariants()
+    assert session.manager.num_free_pages() == session.manager.num_pages()
