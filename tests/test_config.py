@@ -1,0 +1,100 @@
+import json
+
+import pytest
+import torch
+
+from paged_llm_amd import EngineConfig, SamplingParams
+from paged_llm_amd.config import LlamaConfig, lookup_architecture, read_config_json, resolve_dtype
+from tests.tiny_configs import TINY_A, TINY_B, TINY_C
+
+MINIMAL = {"architectures": ["LlamaForCausalLM"], "vocab_size": 10, "hidden_size": 32, "intermediate_size": 8,
+           "num_hidden_layers": 1, "num_attention_heads": 4}
+
+
+def test_defaults_follow_the_reference():
+    c = LlamaConfig.from_hf(MINIMAL)
+    assert (c.num_key_value_heads, c.head_dim, c.rms_norm_eps, c.rope_theta) == (4, 8, 1e-5, 10000.0)
+    assert c.rope_scaling is None and c.max_position_embeddings == 4096 and c.tie_word_embeddings is False
+    assert c.torch_dtype == "float16"
+    assert LlamaConfig.from_hf({**MINIMAL, "head_dim": None}).head_dim == 8
+    assert LlamaConfig.from_hf({**MINIMAL, "dtype": "bfloat16"}).torch_dtype == "bfloat16"
+
+
+def test_both_spellings_of_the_rotary_keys():
+    new = LlamaConfig.from_hf({**MINIMAL, "rope_parameters": {"rope_theta": 5e5, "rope_type": "llama3", "factor": 8.0}})
+    old = LlamaConfig.from_hf({**MINIMAL, "rope_theta": 5e5, "rope_scaling": {"type": "llama3", "factor": 8.0}})
+    assert new.rope_theta == old.rope_theta == 5e5
+    assert new.rope_scaling["factor"] == old.rope_scaling["factor"] == 8.0
+    d = LlamaConfig.from_hf({**MINIMAL, "rope_parameters": {"rope_theta": 7.0, "rope_type": "default"}})
+    assert d.rope_theta == 7.0 and d.rope_scaling is None
+
+
+@pytest.mark.parametrize("bad,msg", [
+    ({"num_key_value_heads": 3}, "multiple"),
+    ({"head_dim": 7}, "even"),
+    ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "not supported"),
+    ({"rope_scaling": {"rope_type": "llama3"}}, "factor"),
+    ({"vocab_size": 0}, "positive"),
+])
+def test_bad_values_are_refused(bad, msg):
+    with pytest.raises(ValueError, match=msg):
+        LlamaConfig.from_hf({**MINIMAL, **bad})
+
+
+def test_missing_size_is_a_key_error():
+    raw = dict(MINIMAL)
+    del raw["intermediate_size"]
+    with pytest.raises(KeyError):
+        LlamaConfig.from_hf(raw)
+
+
+def test_round_trip_through_config_json(tmp_path):
+    for cfg in (TINY_A, TINY_B, TINY_C):
+        c = LlamaConfig.from_hf(cfg)
+        (tmp_path / "config.json").write_text(json.dumps(c.to_hf()))
+        assert LlamaConfig.from_hf(read_config_json(str(tmp_path))) == c
+
+
+def test_registry_chooses_by_architecture_name():
+    arch = lookup_architecture(TINY_A)
+    assert arch.name == "LlamaForCausalLM"
+    spec = arch.build_spec(arch.read_config(TINY_B))
+    assert len(spec.layers) == 3 and [s.layer for s in spec.schedule] == [0, 1, 2]
+    assert spec.layers[0].mixer.params["num_kv_heads"] == 1 and spec.head.params["tied"] is True
+    with pytest.raises(ValueError, match="unsupported architecture"):
+        lookup_architecture({"architectures": ["GPT2LMHeadModel"]})
+    with pytest.raises(ValueError):
+        lookup_architecture({})
+
+
+def test_no_size_of_the_config_is_a_constant_in_the_spec():
+    arch = lookup_architecture(TINY_C)
+    spec = arch.build_spec(arch.read_config(TINY_C))
+    m = spec.layers[0].mixer.params
+    assert (m["num_heads"], m["num_kv_heads"], m["head_dim"]) == (5, 1, 48) and abs(m["scale"] - 48 ** -0.5) < 1e-12
+    assert spec.layers[0].feed_forward.params["intermediate_size"] == 100
+    assert spec.layers[0].mixer_norm.params["eps"] == 1e-4 and spec.vocab_size == 131 and spec.hidden_size == 80
+    assert m["position"]["params"]["theta"] == 1000.0
+
+
+def test_engine_config_validation():
+    assert EngineConfig().block_size == 16 and EngineConfig().max_num_batched_tokens == 2048
+    with pytest.raises(ValueError, match="power of two"):
+        EngineConfig(block_size=12)
+    with pytest.raises(ValueError, match="max_num_batched_tokens"):
+        EngineConfig(block_size=16, max_num_batched_tokens=8)
+
+
+def test_dtype_resolution():
+    assert resolve_dtype("auto", "bfloat16") is torch.bfloat16
+    assert resolve_dtype("auto", "float32") is torch.float32
+    assert resolve_dtype("auto", "float16") is torch.bfloat16
+    assert resolve_dtype("float32", "bfloat16") is torch.float32
+    with pytest.raises(KeyError):
+        resolve_dtype("int8", "bfloat16")
+
+
+def test_sampling_params():
+    sp = SamplingParams()
+    assert (sp.temperature, sp.top_p, sp.top_k, sp.max_tokens, sp.ignore_eos, sp.stop_token_ids) == (1.0, 1.0, -1, 128, False, ())
+    assert SamplingParams(temperature=0.0).greedy and not sp.greedy
