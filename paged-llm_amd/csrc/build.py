@@ -86,15 +86,13 @@ def compile_library(source: str, defines: dict | None = None, force: bool = Fals
     for d in _build_dirs():
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".w{os.getpid()}")
-            with open(probe, "w"):
+            with tempfile.NamedTemporaryFile(dir=d, prefix=".probe"):
                 pass
-            os.remove(probe)
         except OSError as e:
             last_err = e
             continue
         out = os.path.join(d, name)
-        tmp = out + f".tmp{os.getpid()}"
+        tmp = out + f".tmp{os.getpid()}_{threading.get_ident()}"
         cmd = [_hipcc(), *FLAGS, *[f"-D{k}={v}" for k, v in sorted(defines.items())],
                os.path.join(CSRC, source), "-o", tmp]
         if not quiet:
@@ -116,6 +114,14 @@ def compile_library(source: str, defines: dict | None = None, force: bool = Fals
                 os.remove(tmp)
             raise BuildError(f"hipcc failed on {source} (exit {proc.returncode}):\n{log.decode(errors='replace')}")
         os.replace(tmp, out)
+        # Older builds of the same target (other digests) are stale now.
+        prefix = name[: name.rfind("_") + 1]
+        for old in os.listdir(d):
+            if old.startswith(prefix) and old.endswith(".so") and old != name and len(old) == len(name):
+                try:
+                    os.remove(os.path.join(d, old))
+                except OSError:
+                    pass
         if not quiet:
             print(f"[paged-llm_amd] built {name} in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
         return out

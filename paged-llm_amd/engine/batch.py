@@ -46,6 +46,7 @@ class StepContext:
     # Host copies for launch decisions (never for results).
     q_lens: list
     k_lens: list
+    state_slot_list: list          # host copy of state_slots
     max_q_len: int
     max_k_len: int
     dtype: torch.dtype

@@ -125,7 +125,7 @@ class ModelRunner:
         return StepContext(
             num_tokens=T, num_seqs=S, input_ids=piece(0), positions=piece(1), cu_seqlens_q=piece(2), seq_lens_k=piece(3),
             state_slots=piece(4), seq_starts=piece(5), logits_index=piece(6), groups=groups, q_lens=q_lens, k_lens=k_lens,
-            max_q_len=max(q_lens), max_k_len=max(k_lens), dtype=self.model.dtype, device=self.device)
+            state_slot_list=slots_state.tolist(), max_q_len=max(q_lens), max_k_len=max(k_lens), dtype=self.model.dtype, device=self.device)
 
     # ------------------------------------------------------------------ run
     @torch.no_grad()

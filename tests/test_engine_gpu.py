@@ -1,0 +1,186 @@
+"""Generation through the entry point: greedy tokens equal the plain implementation's (also under
+preemption, prefix reuse and copy-on-write), sampling is reproducible and independent of the
+batch, and the command line and the replay program run as a user would run them."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers
+from tests.plain import llama_plain
+from tests.tiny_configs import TINY_A, TINY_B
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folder_a(tmp_path_factory):
+    return helpers.make_folder(tmp_path_factory.mktemp("A"), TINY_A, seed=21, stored="float32")
+
+
+@pytest.fixture(scope="module")
+def folder_b(tmp_path_factory):
+    return helpers.make_folder(tmp_path_factory.mktemp("B"), TINY_B, seed=22, stored="float32")
+
+
+def engine_for(folder, **kw):
+    from paged_llm_amd import EngineConfig
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    base = dict(dtype="float32", num_gpu_blocks=64, block_size=16, max_num_batched_tokens=24, max_model_len=128)
+    base.update(kw)
+    return LLMEngine(folder, EngineConfig(**base))
+
+
+def plain_greedy(folder, prompt, n):
+    return llama_plain.greedy(llama_plain.read_config(folder), llama_plain.load_weights(folder), prompt, n)
+
+
+def test_greedy_generation_matches_the_plain_implementation(folder_a):
+    from paged_llm_amd import SamplingParams
+    prompts = [helpers.random_tokens(n, 256, seed=n) for n in (5, 17, 33, 40)]
+    engine = engine_for(folder_a)
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == plain_greedy(folder_a, p, 12) and o.finish_reason == "length"
+        assert o.prompt_token_ids == p
+    assert engine.cache_manager.num_free_pages() == 64 and engine.stats.num_preemptions == 0
+    assert engine.stats.num_prefill_tokens == 95 and engine.stats.num_decode_tokens == 4 * 11
+    engine.cache_manager.check_invariants()
+
+
+def test_tiny_b_small_pages_and_mixed_steps(folder_b):
+    from paged_llm_amd import SamplingParams
+    prompts = [helpers.random_tokens(n, 512, seed=40 + n) for n in (1, 9, 60, 23, 37, 2)]
+    engine = engine_for(folder_b, block_size=8, max_num_batched_tokens=16, num_gpu_blocks=80, max_model_len=100)
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == plain_greedy(folder_b, p, 10)
+    assert engine.cache_manager.num_free_pages() == 80
+
+
+def test_preemption_under_memory_pressure_is_lossless(folder_a):
+    from paged_llm_amd import SamplingParams
+    prompts = [helpers.random_tokens(n, 256, seed=60 + n) for n in (20, 22, 18, 25)]
+    # 14 pages of 8 for four requests that grow to about 40 tokens each
+    engine = engine_for(folder_a, block_size=8, num_gpu_blocks=14, enable_prefix_caching=False)
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
+    assert engine.stats.num_preemptions > 0 and sum(o.num_preemptions for o in outs) > 0
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == plain_greedy(folder_a, p, 16)
+    assert engine.cache_manager.num_free_pages() == 14
+
+
+def test_prefix_reuse_gives_the_same_tokens_and_counts_hits(folder_a):
+    from paged_llm_amd import SamplingParams
+    shared = helpers.random_tokens(40, 256, seed=70)
+    prompts = [shared + [3, 4], shared + [5, 6, 7, 8]]
+    engine = engine_for(folder_a, max_num_batched_tokens=1000)
+    sp = SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)
+    first = engine.generate(prompts[:1], sp)[0]
+    second = engine.generate(prompts[1:], sp)[0]
+    assert first.num_cached_tokens == 0 and second.num_cached_tokens == 32
+    assert engine.cache_manager.num_cache_hits == 1
+    assert first.token_ids == plain_greedy(folder_a, prompts[0], 8)
+    assert second.token_ids == plain_greedy(folder_a, prompts[1], 8)
+
+
+def test_fork_and_copy_on_write_are_applied(folder_a):
+    """Two children forked from a parent that owns a partial page diverge correctly
+    (tests/test_engine_cpu.py:96-127 of the reference)."""
+    from paged_llm_amd.engine import StepEntry
+    engine = engine_for(folder_a, enable_prefix_caching=False)
+    cm, runner, g = engine.cache_manager, engine.runner, engine.groups[0]
+    base = helpers.random_tokens(21, 256, seed=80)                 # one full page and five slots of the next
+    assert cm.allocate("root", 0, len(base))
+    runner.step([StepEntry("root", base, 0, {g: cm.block_table("root", g)}, None, [])])
+    want = {}
+    for child, token in (("c1", 50), ("c2", 60)):
+        cm.fork("root", child)
+        want[child] = helpers.plain_logits(folder_a, base + [token])[-1]
+    cm.free("root")
+    for child, token in (("c1", 50), ("c2", 60)):
+        assert cm.allocate(child, len(base), 1)
+    copies = cm.take_pending_copies()
+    assert len(copies[g]) == 1                                     # the second child is alone on the page by then
+    entries = [StepEntry(c, [t], len(base), {g: cm.block_table(c, g)}, None, [0]) for c, t in (("c1", 50), ("c2", 60))]
+    logits = runner.step(entries, copies).cpu().numpy()
+    for row, child in zip(logits, ("c1", "c2")):
+        assert helpers.worst(row, want[child]) <= 2e-5
+    cm.free("c1")
+    cm.free("c2")
+    assert cm.num_free_pages() == 64
+
+
+def test_sampling_is_reproducible_and_independent_of_the_batch(folder_a):
+    from paged_llm_amd import SamplingParams
+    prompts = [helpers.random_tokens(n, 256, seed=90 + n) for n in (7, 12, 9)]
+    sp = SamplingParams(temperature=0.9, top_k=40, top_p=0.95, max_tokens=10, ignore_eos=True)
+    def run(seed, subset, reset_ids=True):
+        import itertools
+
+        import paged_llm_amd.engine.request as rq
+        if reset_ids:
+            rq._ids = itertools.count(1000)                         # the draw is keyed by the request id
+        return [o.token_ids for o in engine_for(folder_a, seed=seed).generate([prompts[i] for i in subset], sp)]
+    a, b = run(5, [0, 1, 2]), run(5, [0, 1, 2])
+    assert a == b
+    assert run(6, [0, 1, 2]) != a
+    alone = run(5, [0])
+    assert alone[0] == a[0]                                         # same request id, same tokens, whatever runs beside it
+    greedy = engine_for(folder_a).generate(prompts[:1], SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))[0]
+    assert greedy.token_ids != a[0]
+
+
+def test_step_api_and_abort(folder_a):
+    from paged_llm_amd import SamplingParams
+    engine = engine_for(folder_a)
+    a = engine.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=50))
+    b = engine.add_request([4, 5], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))
+    outs = engine.step()
+    assert [o.seq_id for o in outs] == [a, b] and all(o.new_token is not None and not o.finished for o in outs)
+    engine.abort_request(a)
+    outs = engine.step()
+    assert [o.seq_id for o in outs] == [b] and outs[0].finished
+    assert not engine.has_unfinished_requests and engine.cache_manager.num_free_pages() == 64
+    with pytest.raises(ValueError, match="token id"):
+        engine.add_request([999])
+    with pytest.raises(ValueError, match="tokenizer"):
+        engine.add_request("text")
+
+
+def test_command_line(folder_a):
+    cmd = [sys.executable, os.path.join(ROOT, "examples", "generate.py"), "--model", folder_a, "--max-tokens", "6",
+           "--dtype", "float32", "--num-gpu-blocks", "32", "--max-model-len", "128", "--ignore-eos",
+           "--prompt-ids", "5,17,3", "--prompt-ids", "9,8,7,6"]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [l for l in out.stdout.splitlines() if l and not l.startswith("---") and not l.startswith("steps=")]
+    got = [[int(t) for t in l.split()] for l in lines[-2:]]
+    assert got == [plain_greedy(folder_a, [5, 17, 3], 6), plain_greedy(folder_a, [9, 8, 7, 6], 6)]
+    assert "steps=" in out.stdout and "prefill_tokens=7" in out.stdout
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folder_a, tmp_path, dtype):
+    toks = {"a": helpers.random_tokens(70, 256, seed=1), "b": helpers.random_tokens(45, 256, seed=2)}
+    trace = helpers.TraceBuilder()
+    trace.step([("a", toks["a"][:50], [0, 49])])
+    trace.step([("a", toks["a"][50:52], "all"), ("b", toks["b"][:30], [])])
+    trace.step([("b", toks["b"][30:], "last"), ("a", toks["a"][52:53], "all")], end=["b"])
+    trace.step([("a", toks["a"][53:], "all")], end=["a"])
+    out_dir = tmp_path / "out"
+    proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder_a, "--dtype", dtype, "--out", str(out_dir),
+                           "--max-tokens", "192"], input=trace.jsonl(), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"]
+    got = helpers.read_replay_output(str(out_dir), trace, 256)
+    assert len(got) == 2 + 2 + 1 + 1 + 17
+    tol = 2e-5 if dtype == "float32" else 4e-2
+    for (rid, pos), row in got.items():
+        assert helpers.worst(row, helpers.plain_logits(folder_a, toks[rid])[pos]) <= tol

@@ -147,3 +147,26 @@ def test_mixed_batches_with_pages_used_again(folders, name, dtype):
     check(got, folder, reqs, dtype)
     session.manager.check_invariants()
     assert session.manager.num_free_pages() == session.manager.num_pages()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(folders, dtype):
+    folder = folders["A", "float32" if dtype == "float32" else "bfloat16"]
+    reqs = {f"s{n}": helpers.random_tokens(n, 256, seed=300 + n) for n in (1, 2, 3)}
+    session = session_for(folder, dtype, 64 * 3)
+    trace = TraceBuilder()
+    trace.step([(rid, toks[:1], "all") for rid, toks in reqs.items()])                  # three first tokens in one batch
+    trace.step([(rid, toks[1:], "all") for rid, toks in reqs.items() if len(toks) > 1], end=list(reqs))
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    folder = folders["C", "float32" if dtype == "float32" else "bfloat16"]
+    toks = helpers.random_tokens(290, 131, seed=400)
+    session = session_for(folder, dtype, 320)
+    trace = TraceBuilder()
+    trace.step([("long", toks[:6], "all")])
+    for i in range(6, len(toks)):
+        trace.step([("long", toks[i:i + 1], "all")])
+    check(helpers.replay_in_process(session, trace), folder, {"long": toks}, dtype)

@@ -1,0 +1,165 @@
+"""The framework's generality, shown with toy parts that are defined here and registered without a
+change to the framework's files: a mixer with per-request state of fixed size, a layer that runs
+twice, a layer that reads another layer's cache, and a windowed attention layer with pages of its
+own.  The toy model is replayed whole, in portions and mixed, and compared with a plain
+implementation written here."""
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers
+from tests.helpers import TraceBuilder
+from tests.plain import llama_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+TOY = {"architectures": ["ToyHybridForCausalLM"], "vocab_size": 120, "hidden_size": 48, "intermediate_size": 72,
+       "heads": 3, "kv_heads": 1, "head_dim": 16, "decay": 0.8, "window": 7, "eps": 1e-5, "theta": 100.0,
+       "max_position_embeddings": 256}
+# step -> (layer, cache_from): layer 1 (the stateful mixer) runs twice, step 2 reads the cache of step 0
+SCHEDULE = [(0, None), (1, None), (2, 0), (3, None), (1, None)]
+
+
+def register_toy():
+    from paged_llm_amd.config.registry import ARCHITECTURES, Architecture, register_architecture
+    from paged_llm_amd.parts import (LayerSpec, Mixer, ModelSpec, PartSpec, ScheduleStep, StateSpec, WeightSpec,
+                                     register_mixer)
+    from paged_llm_amd.parts.linear import linear
+    if "ToyHybridForCausalLM" in ARCHITECTURES:
+        return
+
+    class DecayMixer(Mixer):
+        """s_t = decay * s_{t-1} + W x_t, output s_t; the state is one float vector per request."""
+
+        def __init__(self, params, env):
+            self.hidden, self.decay = env.hidden_size, float(params["decay"])
+            self.dtype, self.device, self.w = env.dtype, env.device, None
+
+        def weight_specs(self):
+            return {"in_proj.weight": WeightSpec((self.hidden, self.hidden))}
+
+        def assign(self, name, tensor):
+            assert name == "in_proj.weight"
+            self.w = tensor.to(device=self.device, dtype=self.dtype).contiguous()
+
+        def state_spec(self):
+            return StateSpec((self.hidden,), torch.float32)
+
+        def forward(self, h, ctx, cache, state):
+            u = linear(h, self.w).float()
+            out = torch.empty_like(u)
+            at = 0
+            for n, k_len, slot in zip(ctx.q_lens, ctx.k_lens, ctx.state_slot_list):
+                s0 = state[slot] if k_len - n > 0 else torch.zeros_like(state[slot])     # a fresh request starts at zero
+                i = torch.arange(n, device=u.device, dtype=torch.float32)
+                powers = torch.tril(self.decay ** (i[:, None] - i[None, :]).clamp_min(0))
+                seg = powers @ u[at:at + n] + (self.decay ** (i + 1))[:, None] * s0
+                out[at:at + n] = seg
+                state[slot] = seg[-1]
+                at += n
+            return out.to(h.dtype)
+
+    register_mixer("toy_decay", DecayMixer)
+
+    def build_spec(c):
+        norm = PartSpec("rmsnorm", {"eps": c["eps"]})
+        rotary = {"kind": "rotary", "params": {"head_dim": c["head_dim"], "theta": c["theta"], "scaling": None}}
+        def attention(**extra):
+            return PartSpec("paged_attention", {"num_heads": c["heads"], "num_kv_heads": c["kv_heads"], "head_dim": c["head_dim"],
+                                                "position": rotary, **extra})
+        ffn = PartSpec("gated_mlp", {"intermediate_size": c["intermediate_size"]})
+        block = PartSpec("prenorm", {"mixer_norm": "norm1", "mixer": "mixer", "feed_forward_norm": "norm2", "feed_forward": "ffn"})
+        mixers = [attention(), PartSpec("toy_decay", {"decay": c["decay"]}), attention(kv_proj=False), attention(window=c["window"])]
+        layers = [LayerSpec(f"layers.{i}", block, m, ffn, norm, norm) for i, m in enumerate(mixers)]
+        return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"],
+                         embedding=PartSpec("token_embedding", {"vocab_size": c["vocab_size"]}), layers=layers, final_norm=norm,
+                         head=PartSpec("lm_head", {"vocab_size": c["vocab_size"], "tied": False}),
+                         schedule=[ScheduleStep(l, cf) for l, cf in SCHEDULE], embedding_name="embed", final_norm_name="norm",
+                         head_name="head", max_positions=c["max_position_embeddings"], stored_dtype="float32")
+
+    register_architecture(Architecture("ToyHybridForCausalLM", lambda raw: dict(raw), build_spec))
+
+
+def plain_toy(folder, tokens):
+    c, w = TOY, {k: v.float() for k, v in plain.load_weights(folder).items()}
+    T, nh, nkv, d = len(tokens), c["heads"], c["kv_heads"], c["head_dim"]
+    ang = plain.rotary_angles(torch.arange(T), plain.inverse_frequencies(d, c["theta"], None))
+    x = w["embed.weight"][torch.tensor(tokens)]
+    kept = {}
+    for step, (layer, cache_from) in enumerate(SCHEDULE):
+        p = f"layers.{layer}."
+        h = plain.rms_norm(x, w[p + "norm1.weight"], c["eps"])
+        if layer == 1:
+            u, s, rows = h @ w[p + "mixer.in_proj.weight"].T, torch.zeros(c["hidden_size"]), []
+            for t in range(T):
+                s = c["decay"] * s + u[t]
+                rows.append(s)
+            a = torch.stack(rows)
+        else:
+            q = plain.apply_rotary((h @ w[p + "mixer.q_proj.weight"].T).view(T, nh, d), ang)
+            if cache_from is None:
+                k = plain.apply_rotary((h @ w[p + "mixer.k_proj.weight"].T).view(T, nkv, d), ang)
+                v = (h @ w[p + "mixer.v_proj.weight"].T).view(T, nkv, d)
+                kept[step] = (k, v)
+            else:
+                k, v = kept[cache_from]
+            o = plain.causal_attention(q, k, v, d ** -0.5, c["window"] if layer == 3 else None)
+            a = o.reshape(T, nh * d) @ w[p + "mixer.o_proj.weight"].T
+        x = x + a
+        h = plain.rms_norm(x, w[p + "norm2.weight"], c["eps"])
+        x = x + plain.swiglu(h, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+    return (plain.rms_norm(x, w["norm.weight"], c["eps"]) @ w["head.weight"].T).numpy()
+
+
+@pytest.fixture(scope="module")
+def toy_folder(tmp_path_factory):
+    register_toy()
+    return helpers.make_folder(tmp_path_factory.mktemp("toy"), TOY, seed=31, stored="float32")
+
+
+def test_toy_model_is_built_from_registered_parts(toy_folder):
+    from paged_llm_amd.engine.replay import ReplaySession
+    s = ReplaySession(toy_folder, "float32", 256, None)
+    groups = s.model.cache_groups()
+    assert sorted(groups) == ["full_kv1x16", "window7_kv1x16"]
+    assert groups["full_kv1x16"].owners == [0] and groups["window7_kv1x16"].owners == [3]      # step 2 owns no pages
+    assert sorted(s.model.state_specs()) == [1, 4]                                             # one state per step, not per layer
+    assert "layers.2.mixer.k_proj.weight" not in s.model.weight_specs()
+    assert s.manager.uses_state and set(s.runner.states) == {1, 4}
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 5e-2)])
+def test_toy_model_whole_in_portions_and_mixed(toy_folder, dtype, tol):
+    from paged_llm_amd.engine.replay import ReplaySession
+    reqs = {f"t{i}": helpers.random_tokens(n, TOY["vocab_size"], seed=200 + i) for i, n in enumerate([3, 41, 90, 64, 17])}
+    want = {rid: plain_toy(toy_folder, toks) for rid, toks in reqs.items()}
+
+    def compare(got):
+        assert len(got) == sum(len(t) for t in reqs.values())
+        for (rid, pos), row in got.items():
+            err = helpers.worst(row, want[rid][pos])
+            assert err <= tol, f"{rid} position {pos}: {err:.3g}"
+
+    whole = TraceBuilder()
+    for rid, toks in reqs.items():
+        whole.step([(rid, toks, "all")], end=[rid])
+    compare(helpers.replay_in_process(ReplaySession(toy_folder, dtype, 128, None), whole))
+
+    portions = TraceBuilder()
+    for rid, toks in reqs.items():
+        at, sizes = 0, iter([2, 5, 1, 9, 3] * 40)
+        while at < len(toks):
+            n = min(next(sizes), len(toks) - at)
+            portions.step([(rid, toks[at:at + n], "all")], end=[rid] if at + n == len(toks) else [])
+            at += n
+    compare(helpers.replay_in_process(ReplaySession(toy_folder, dtype, 128, None), portions))
+
+    from tests.test_replay_gpu import mixed_trace
+    trace, peak = mixed_trace(reqs, max_live=3, seed=9)
+    session = ReplaySession(toy_folder, dtype, peak, None)
+    compare(helpers.replay_in_process(session, trace))
+    session.manager.check_invariants()
+    assert session.manager.slots.num_free == session.manager.slots.num_slots
+    # the windowed group gave pages back while requests were still running
+    assert all(session.manager.num_free_pages(g) == session.manager.num_pages(g) for g in session.manager.groups)
