@@ -1,0 +1,175 @@
+"""Decode and prefill throughput of the engine on one MI355X, with roofline fractions.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers N]
+
+The model has the layer sizes of TinyLlama-1.1B (22 layers, hidden 2048, 32 heads, 4 KV heads,
+head size 64, intermediate 5632, vocabulary 32000) with seeded random weights in bfloat16; prompts
+are seeded random token ids, sampling is greedy and end-of-sequence is ignored, as in the
+reference's benchmarks/bench.py:27-45.  A step is one decode step of the whole engine: scheduling,
+the forward pass over the paged cache, and sampling.  One JSON line goes to stdout.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+TINYLLAMA = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 22, "hidden_size": 2048,
+    "num_attention_heads": 32, "num_key_value_heads": 4, "head_dim": 64, "intermediate_size": 5632, "vocab_size": 32000,
+    "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 4096,
+    "torch_dtype": "bfloat16",
+}
+# Published peaks of the MI355X: HBM3E bandwidth and dense MFMA rates.
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+PREFILL_TOKENS = 2048
+
+
+def model_numbers(cfg: dict, dtype_bytes: int) -> dict:
+    L, H, I, V = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    per_layer = H * (nh + 2 * nkv) * d + nh * d * H + 3 * H * I
+    return {
+        "matrix_params": L * per_layer, "head_params": V * H,
+        "weight_bytes": (L * per_layer + V * H) * dtype_bytes + (2 * L + 1) * H * 4,
+        "kv_bytes_per_token": 2 * L * nkv * d * dtype_bytes,
+        "attn_flops_per_pair": 4 * nh * d * L,
+    }
+
+
+def prefill_flops(cfg: dict, tokens: int, rows_with_logits: int) -> float:
+    m = model_numbers(cfg, 2)
+    causal_pairs = tokens * (tokens + 1) / 2
+    return 2.0 * tokens * m["matrix_params"] + 2.0 * rows_with_logits * m["head_params"] + m["attn_flops_per_pair"] * causal_pairs
+
+
+def make_engine(cfg: dict, folder: str, dtype: str, max_seqs: int, context: int):
+    from paged_llm_amd import EngineConfig
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    block = 16
+    pages = max_seqs * ((context + 128 + block - 1) // block) + 64
+    return LLMEngine(folder, EngineConfig(
+        block_size=block, num_gpu_blocks=pages, max_num_seqs=max_seqs, max_num_batched_tokens=8192,
+        max_model_len=context + 128, dtype=dtype, seed=0, enable_prefix_caching=True), random_weights=0)
+
+
+def random_prompts(n: int, length: int, vocab: int, seed: int):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(100, vocab, (length,), generator=g).tolist() for _ in range(n)]
+
+
+def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int) -> float:
+    """Seconds per decode step at `batch` requests whose contexts end at `context` tokens."""
+    import torch
+    from paged_llm_amd import SamplingParams
+    prompt_len = context - (steps + warmup)
+    assert prompt_len >= 1, "context too short for this many steps"
+    sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 40, ignore_eos=True)
+    for p in random_prompts(batch, prompt_len, engine.model.spec.vocab_size, seed):
+        engine.add_request(p, sp)
+    while any(not r.is_prefill_done for r in engine.scheduler.running) or engine.scheduler.waiting:
+        engine.step()
+    assert len(engine.scheduler.running) == batch
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = engine.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert len(out) == batch
+    for r in list(engine.scheduler.running):
+        engine.abort_request(r.request_id)
+    return elapsed / steps
+
+
+def time_prefill(engine, tokens: int, seed: int, repeats: int = 3) -> float:
+    """Seconds of one step that computes a whole prompt of `tokens` tokens (best of a few)."""
+    import torch
+    from paged_llm_amd import SamplingParams
+    best = float("inf")
+    for r in range(repeats + 1):                     # the first run warms up
+        prompt = random_prompts(1, tokens, engine.model.spec.vocab_size, seed + r)[0]
+        rid = engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert not engine.has_unfinished_requests, rid
+        if r > 0:
+            best = min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (reported as such)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    cfg = dict(TINYLLAMA)
+    model_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    cfg["torch_dtype"] = args.dtype
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    nbytes = 2 if short == "bf16" else 4
+    numbers = model_numbers(cfg, nbytes)
+
+    with tempfile.TemporaryDirectory() as folder:
+        engine = make_engine(cfg, folder, args.dtype, max(64, args.batch), args.context)
+        sec = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
+        value = args.batch / sec
+        decode_bytes = numbers["weight_bytes"] + args.batch * args.context * numbers["kv_bytes_per_token"]
+        achieved = decode_bytes / sec / 1e9
+        record = {
+            "metric": "decode tokens/s (TinyLlama-1.1B shapes, random weights)", "value": round(value, 1), "unit": "tokens/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
+            "config": {"model": "TinyLlama-1.1B shapes", "layers": cfg["num_hidden_layers"], "layers_of_model": model_layers,
+                       "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+                       "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+                       "global_batch": args.batch, "seq_len": args.context, "block_size": 16, "weights": "random seed 0",
+                       "parallelism": "single GPU"},
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        }
+        if not args.no_points:
+            points = {}
+            for b in (1, 64):
+                s = time_decode(engine, b, args.context, max(16, args.steps // 2), max(4, args.warmup // 2), seed=10 + b)
+                points[f"decode_b{b}"] = round(b / s, 1)
+            record["points"] = points
+            psec = time_prefill(engine, PREFILL_TOKENS, seed=100)
+            flops = prefill_flops(cfg, PREFILL_TOKENS, 1)
+            record["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3),
+                                 "frac": round(flops / psec / PEAK_FLOPS[short], 4)}
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
