@@ -270,14 +270,93 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
 
 
 # ------------------------------------------------------------------------------------------- choices
+SKINNY_MAX_ROWS = 64
+_SKINNY_SIG = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p,
+               c_void_p, c_void_p]
+_skinny_scratch: dict = {}
+
+
+def _skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    K = a.shape[1]
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and a.stride(1) == 1 and w.stride(1) == 1
+            and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def _skinny_split(n_out_tiles: int, K: int) -> int:
+    """How many workgroups share the K range of one tile: enough to put work on every CU, while
+    every wavefront still gets at least one slab of 128."""
+    split = 1
+    while n_out_tiles * split < 512 and split * 2 * 4 * 128 <= K and split < 8:
+        split *= 2
+    return split
+
+
+def _skinny_buffers(device, floats: int, counters: int):
+    """Workspace for split-K partials and the arrival counters (zero once; kernels reset them)."""
+    key = str(device)
+    ws, cnt = _skinny_scratch.get(key, (None, None))
+    if ws is None or ws.numel() < floats:
+        ws = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=device)
+    if cnt is None or cnt.numel() < counters:
+        cnt = torch.zeros(max(counters, 4096), dtype=torch.int32, device=device)
+    _skinny_scratch[key] = (ws, cnt)
+    return ws, cnt
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None, gated: bool = False,
+                ksplit: int | None = None) -> torch.Tensor:
+    """a [M <= 64, K] times w [N, K]^T (gated: w is [gate; up], result silu(a Wg^T) * (a Wu^T))."""
+    _on_gpu(a, w)
+    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], f"gemm shapes {tuple(a.shape)} x {tuple(w.shape)}^T")
+    _need(_skinny_ok(a, w), "gemm_skinny needs bfloat16 operands with K, row strides and addresses in multiples of 8 elements")
+    M, K = a.shape
+    _need(0 < M <= SKINNY_MAX_ROWS, f"gemm_skinny takes 1..{SKINNY_MAX_ROWS} rows, got {M}")
+    N = w.shape[0]
+    if gated:
+        _need(N % 2 == 0, "gated product needs [gate; up] rows")
+        N //= 2
+    out_dtype = out_dtype or torch.bfloat16
+    _need(out_dtype in (torch.bfloat16, torch.float32), "output is bfloat16 or float32")
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    tiles_out = 1 if (gated or M <= 32) else 2
+    blocks = (N + tiles_out * 16 - 1) // (tiles_out * 16)
+    if ksplit is None:
+        ksplit = _skinny_split(blocks, K)
+    ws = cnt = None
+    if ksplit > 1:
+        floats = _fn("gemm_skinny.hip", "pllm_gemm_skinny_workspace_floats", signature=[c_int, c_int, c_int])(M, N, ksplit)
+        ws, cnt = _skinny_buffers(a.device, floats, blocks)
+    _check(_fn("gemm_skinny.hip", "pllm_gemm_skinny", signature=_SKINNY_SIG)(
+        _ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), M, N, K, 1 if out_dtype == torch.float32 else 0,
+        1 if gated else 0, ksplit, _ptr(ws), _ptr(cnt), _stream()), "gemm_skinny")
+    return out
+
+
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
     """The fast bfloat16 products; None when neither takes the shape (the caller falls back to
     the plain kernel).  The choice looks at the number of rows only."""
-    return None
+    if not _skinny_ok(a, w):
+        return None
+    M = a.shape[0]
+    out_dtype = out_dtype or torch.bfloat16
+    if M <= SKINNY_MAX_ROWS:
+        return gemm_skinny(a, w, out_dtype)
+    if out_dtype == torch.float32:
+        # Float results for many rows (logits of a whole prompt): the same kernel, 64 rows at a time.
+        return torch.cat([gemm_skinny(a[i:i + SKINNY_MAX_ROWS], w, out_dtype) for i in range(0, M, SKINNY_MAX_ROWS)], dim=0)
+    return gemm_large_bf16(a, w)
+
+
+def gemm_large_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """Many rows (prompt portions): the vendor's matrix-product library, as the reference's engine
+    uses a library for its products (nn.Linear, pagedllm/model/llama.py:141-144)."""
+    return torch.mm(a, w.t())
 
 
 def gate_up_silu(h: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     """silu(h Wg^T) * (h Wu^T) with Wg, Wu stacked in w_gate_up [2I, K]."""
+    if h.shape[0] <= SKINNY_MAX_ROWS and _skinny_ok(h, w_gate_up):
+        return gemm_skinny(h, w_gate_up, gated=True)
     from ..parts.linear import linear
     return silu_mul(linear(h, w_gate_up))
 

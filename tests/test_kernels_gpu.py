@@ -285,3 +285,54 @@ def test_sampling_frequencies_follow_the_filtered_distribution(temperature, top_
     chi2 = float(((counts[keep] - draws * probs[keep]) ** 2 / (draws * probs[keep])).sum())
     dof = int(keep.sum()) - 1
     assert chi2 < dof + 5 * math.sqrt(2 * max(dof, 1)) + 5, f"chi-square {chi2:.1f} for {dof} degrees of freedom"
+
+
+# ----------------------------------------------------------------------------------- bfloat16 products for few rows
+@pytest.mark.parametrize("m", [1, 5, 8, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("n,k", [(16, 64), (100, 96), (517, 176), (2048, 2048), (2048, 5632), (96, 1000)])
+def test_gemm_skinny(m, n, k):
+    a, w = rnd(m, k, seed=20, dtype=torch.bfloat16), rnd(n, k, seed=21, dtype=torch.bfloat16)
+    want = a.double() @ w.double().T
+    for split in (None, 1, 2, 4):
+        if split and split > 1 and split * 512 > max(k, 512):
+            continue
+        out = ops().gemm_skinny(a.cuda(), w.cuda(), torch.float32, ksplit=split)
+        assert rel_err(out, want) <= 2e-5, f"split {split}"
+    out16 = ops().gemm_skinny(a.cuda(), w.cuda())
+    assert out16.dtype == torch.bfloat16 and rel_err(out16, want) <= 1e-2
+
+
+def test_gemm_skinny_repeated_split_calls_leave_counters_clean():
+    a, w = rnd(8, 2048, seed=22, dtype=torch.bfloat16).cuda(), rnd(2048, 2048, seed=23, dtype=torch.bfloat16).cuda()
+    first = ops().gemm_skinny(a, w, torch.float32, ksplit=4).cpu()
+    for _ in range(5):
+        assert torch.equal(ops().gemm_skinny(a, w, torch.float32, ksplit=4).cpu(), first)
+
+
+def test_gemm_skinny_strided_rows():
+    big = rnd(9, 300, seed=24, dtype=torch.bfloat16).cuda()
+    a = big[:, 40:40 + 176]                                       # row stride 300: not a multiple of 8
+    assert ops().gemm_bf16(a, rnd(64, 176, seed=25, dtype=torch.bfloat16).cuda()) is None
+    big = rnd(9, 304, seed=24, dtype=torch.bfloat16).cuda()
+    a, w = big[:, 40:40 + 176], rnd(64, 176, seed=25, dtype=torch.bfloat16).cuda()
+    assert rel_err(ops().gemm_skinny(a, w, torch.float32), a.double().cpu() @ w.double().cpu().T) <= 2e-5
+
+
+@pytest.mark.parametrize("m", [1, 8, 24, 64])
+@pytest.mark.parametrize("inter,k", [(176, 64), (250, 96), (5632, 2048)])
+def test_gated_product(m, inter, k):
+    x = rnd(m, k, seed=26, dtype=torch.bfloat16)
+    w = rnd(2 * inter, k, seed=27, dtype=torch.bfloat16, scale=k ** -0.5)
+    g, u = x.double() @ w[:inter].double().T, x.double() @ w[inter:].double().T
+    want = torch.nn.functional.silu(g) * u
+    got = ops().gemm_skinny(x.cuda(), w.cuda(), torch.float32, gated=True)
+    assert rel_err(got, want) <= 3e-5
+    assert rel_err(ops().gate_up_silu(x.cuda(), w.cuda()), want) <= 1e-2
+
+
+def test_large_bf16_product_and_float_rows():
+    a, w = rnd(200, 256, seed=28, dtype=torch.bfloat16), rnd(130, 256, seed=29, dtype=torch.bfloat16)
+    want = a.double() @ w.double().T
+    assert rel_err(ops().gemm_bf16(a.cuda(), w.cuda()), want) <= 1e-2
+    out = ops().gemm_bf16(a.cuda(), w.cuda(), torch.float32)
+    assert out.dtype == torch.float32 and rel_err(out, want) <= 2e-5
