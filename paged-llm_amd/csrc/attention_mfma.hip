@@ -1,0 +1,336 @@
+// Paged causal attention in bfloat16 on the matrix cores, for prompt portions and for decoding.
+// Compiled once per head size (-DHEAD_DIM=16..256 in steps of 16).
+//
+// Work item = (sequence, kv head, tile of columns, partition of keys), one wavefront each.
+// A *column* is a (query token, query head of the kv head's group) pair, numbered
+// c = token * G + head_in_group, so the G heads that share a kv head sit side by side and every
+// loaded key/value tile serves all of them: a decode step has G columns, a prompt portion
+// num_q * G.  A wavefront owns 16 * NCB columns.
+//
+// Scores are computed transposed, S^T = K Q^T, with v_mfma_f32_16x16x32_bf16: the A operand is a
+// tile of 16 keys (each lane loads 16 contiguous bytes of one key row straight from the page),
+// the B operand is Q^T, held in registers for the whole kernel.  The result leaves every lane
+// with 4 keys of ONE column, so the softmax statistics of a column live in one lane (and its
+// three mirror lanes), and the probabilities are already in B-operand layout for O^T = V^T P^T.
+// V pages are stored transposed ([d, block_size]), so the A operand of that product (16 channels
+// x 32 keys) is two 8-byte loads per lane.  Nothing goes through LDS.
+//
+// Keys are walked in blocks of 64 aligned to absolute positions; partitions (split-K for
+// decoding) are aligned multiples of 64 as well, and are merged by a second kernel.  Softmax
+// statistics, the running output and the merge are float; probabilities are rounded to bfloat16
+// for the second product, as the reference's kernel does (pagedllm/attention/triton_kernel.py:88).
+// Page-table entries past the context are never read; values of keys that no column of the tile
+// may see are zeroed, so stale or non-finite data in reused pages cannot leak (0 * NaN).
+#include "common.h"
+
+using namespace pllm;
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<16..256, multiple of 16>"
+#endif
+static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size must be 16..256 in steps of 16");
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+
+constexpr int D = HEAD_DIM;
+constexpr int KSTEPS = (D + 31) / 32;   // MFMA steps over the head dimension for Q K^T
+constexpr int DBLOCKS = D / 16;          // 16-channel blocks of the output
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+// v_exp_f32: 2^x, with 2^-inf = 0 and tiny results flushed to zero (harmless in a softmax).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float group_max(float v) {      // over the 4 lanes that mirror a column
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+__device__ __forceinline__ float group_sum(float v) {
+  v += __shfl_xor(v, 16, 64);
+  return v + __shfl_xor(v, 32, 64);
+}
+
+// Partials of one (token, head, partition): [m (log2 units), l, acc[D]].
+constexpr int kPartialFloats = D + 2;
+
+template <int NCB>
+__global__ __launch_bounds__(64) void paged_attention_mfma_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
+    int block_size, float scale, int window, int partition_size, int num_partitions, float* __restrict__ partials) {
+  const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+  const int seq = blockIdx.z;
+  const int kvh = blockIdx.y / num_partitions, part = blockIdx.y - kvh * num_partitions;
+  const int G = num_heads / num_kv_heads;
+  const int q_begin = cu_seqlens_q[seq], num_q = cu_seqlens_q[seq + 1] - q_begin;
+  const int len_k = seq_lens_k[seq];
+  const int num_cols = num_q * G;
+  const int col0 = blockIdx.x * 16 * NCB;
+  if (col0 >= num_cols) return;
+  const int last_col = min(col0 + 16 * NCB, num_cols) - 1;
+  const int pos0 = len_k - num_q;                               // position of the sequence's first query
+  const int qpos_min = pos0 + col0 / G, qpos_max = pos0 + last_col / G;
+  // Keys any column of this tile may see: [vis_lo, vis_hi)
+  const int vis_hi = qpos_max + 1;
+  const int vis_lo = (window > 0 && qpos_min - window + 1 > 0) ? qpos_min - window + 1 : 0;
+  int k_lo = vis_lo & ~63, k_hi = vis_hi;
+  if (partition_size > 0) {
+    k_lo = max(k_lo, part * partition_size);
+    k_hi = min(k_hi, (part + 1) * partition_size);
+  }
+  if (k_lo >= k_hi) return;                                     // nothing of this partition is visible
+
+  // ---- this lane's column in each column block, and Q^T in B-operand layout
+  int my_qpos[NCB], my_first[NCB];
+  bool my_valid[NCB];
+  size_t my_out[NCB];
+  bf16x8 qreg[NCB][KSTEPS];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int c = col0 + cb * 16 + r;
+    my_valid[cb] = c < num_cols;
+    const int tok = my_valid[cb] ? c / G : 0, hg = my_valid[cb] ? c - tok * G : 0;
+    my_qpos[cb] = my_valid[cb] ? pos0 + tok : -1;               // -1: sees nothing
+    my_first[cb] = (window > 0 && my_qpos[cb] - window + 1 > 0) ? my_qpos[cb] - window + 1 : 0;
+    const size_t row = (size_t)(q_begin + tok) * q_stride + (size_t)(kvh * G + hg) * D;
+    my_out[cb] = (size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int dd = s * 32 + g * 8;
+      qreg[cb][s] = (my_valid[cb] && dd < D) ? *reinterpret_cast<const bf16x8*>(q + row + dd) : zero8();
+    }
+  }
+
+  floatx4 acc[NCB][DBLOCKS];
+  float m_run[NCB], l_run[NCB];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    m_run[cb] = -INFINITY;
+    l_run[cb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) acc[cb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float sl2 = scale * kLog2e;
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  const size_t page_elems = (size_t)block_size * D;             // one kv head's part of a page
+  const size_t page_stride = page_elems * num_kv_heads;
+
+  for (int n0 = k_lo; n0 < k_hi; n0 += 64) {
+    // Every key of the block visible to every column?  Then no masking is needed.
+    const bool interior = (n0 + 63 <= qpos_min) && (n0 >= (window > 0 ? max(qpos_max - window + 1, 0) : 0)) && (n0 + 64 <= k_hi) &&
+                          (col0 + 16 * NCB <= num_cols);
+    floatx4 s_t[4][NCB];
+    const bf16* vbase[4];
+    bool tile_on[4];
+    // ---- S^T = K Q^T for four tiles of 16 keys
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      const int nk = n0 + kt * 16;
+      tile_on[kt] = nk < k_hi;                                  // uniform: tiles past the range are skipped, their table entries unread
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
+      vbase[kt] = v_pages;
+      if (!tile_on[kt]) continue;
+      const int page = bt[nk / block_size];
+      const int off = nk & (block_size - 1);
+      const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
+      vbase[kt] = v_pages + base + off;                         // + channel * block_size + key
+      const bf16* krow = k_pages + base + (size_t)(off + r) * D;
+      bf16x8 kreg[KSTEPS];
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        const int dd = s * 32 + g * 8;
+        kreg[s] = (dd < D) ? *reinterpret_cast<const bf16x8*>(krow + dd) : zero8();
+      }
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+          s_t[kt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[s], qreg[cb][s], s_t[kt][cb], 0, 0, 0);
+    }
+
+    // ---- online softmax per column; lane holds keys n0 + kt*16 + g*4 + i of its column
+    bf16x8 p_op[2][NCB];                                        // B operands of the second product
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      float sc[4][4];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = s_t[kt][cb][i] * sl2;
+          if (!interior) {
+            const int n = n0 + kt * 16 + g * 4 + i;
+            const bool vis = tile_on[kt] && n <= my_qpos[cb] && n >= my_first[cb];
+            v = vis ? v : -INFINITY;
+          }
+          sc[kt][i] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = group_max(mx);
+      const float m_new = fmaxf(m_run[cb], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen nothing yet
+      const float alpha = fast_exp2(m_run[cb] - m_safe);
+      m_run[cb] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = fast_exp2(sc[kt][i] - m_safe);
+          psum += p;
+          p_op[kt >> 1][cb][(kt & 1) * 4 + i] = (__bf16)p;
+        }
+      l_run[cb] = l_run[cb] * alpha + psum;                     // per lane; mirrored lanes are added at the end
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) acc[cb][db] *= alpha;
+    }
+
+    // ---- O^T += V^T P^T : A operand = 16 channels x 32 keys (k slots 0-3: tile 2a, 4-7: tile 2a+1)
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      if (!tile_on[2 * a]) continue;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) {
+        bf16x8 vreg;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int kt = 2 * a + h;
+          bf16x4 v4;
+          if (tile_on[kt]) {
+            v4 = *reinterpret_cast<const bf16x4*>(vbase[kt] + (size_t)(db * 16 + r) * block_size + g * 4);
+            if (!interior) {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const int n = n0 + kt * 16 + g * 4 + i;
+                if (n >= vis_hi || n < vis_lo) v4[i] = (__bf16)0.0f;
+              }
+            }
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v4[i] = (__bf16)0.0f;
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vreg[h * 4 + i] = v4[i];
+        }
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+          acc[cb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg, p_op[a][cb], acc[cb][db], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- write: lane holds channels db*16 + g*4 + i of its column
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    if (!my_valid[cb]) continue;
+    const float l_tot = group_sum(l_run[cb]);
+    if (partition_size > 0) {
+      const int c = col0 + cb * 16 + r;
+      const int tok = c / G, hg = c - tok * G;
+      float* dst = partials + (((size_t)(q_begin + tok) * num_heads + (kvh * G + hg)) * num_partitions + part) * kPartialFloats;
+      if (g == 0) { dst[0] = m_run[cb]; dst[1] = l_tot; }
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[2 + db * 16 + g * 4 + i] = acc[cb][db][i];
+    } else {
+      const float inv = 1.f / l_tot;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) {
+        bf16x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = (__bf16)(acc[cb][db][i] * inv);
+        *reinterpret_cast<bf16x4*>(out + my_out[cb] + db * 16 + g * 4) = o;
+      }
+    }
+  }
+}
+
+// Merge of the partitions of one (token, head): out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p,
+// over the partitions that hold a visible key, in partition order.
+__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ partials, bf16* __restrict__ out, int out_stride,
+                                                            const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k,
+                                                            int num_seqs, int num_heads, int window, int partition_size,
+                                                            int num_partitions) {
+  const int tok = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  int lo = 0, hi = num_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu_seqlens_q[mid] <= tok) lo = mid; else hi = mid - 1;
+  }
+  const int q_begin = cu_seqlens_q[lo], num_q = cu_seqlens_q[lo + 1] - q_begin;
+  const int qpos = seq_lens_k[lo] - num_q + (tok - q_begin);
+  const int first_key = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  const int p_lo = first_key / partition_size, p_hi = min(qpos / partition_size, num_partitions - 1);
+  const float* base = partials + ((size_t)tok * num_heads + head) * num_partitions * kPartialFloats;
+  float M = -INFINITY;
+  for (int p = p_lo; p <= p_hi; ++p) M = fmaxf(M, base[(size_t)p * kPartialFloats]);
+  float l = 0.f;
+  float o[(D + 63) / 64];
+#pragma unroll
+  for (int j = 0; j < (D + 63) / 64; ++j) o[j] = 0.f;
+  for (int p = p_lo; p <= p_hi; ++p) {
+    const float* pp = base + (size_t)p * kPartialFloats;
+    const float w = fast_exp2(pp[0] - M);
+    l += w * pp[1];
+#pragma unroll
+    for (int j = 0; j < (D + 63) / 64; ++j) {
+      const int i = lane + j * 64;
+      if (i < D) o[j] += w * pp[2 + i];
+    }
+  }
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int j = 0; j < (D + 63) / 64; ++j) {
+    const int i = lane + j * 64;
+    if (i < D) out[(size_t)tok * out_stride + (size_t)head * D + i] = __float2bfloat16(o[j] * inv);
+  }
+}
+
+PLLM_API int pllm_attention_mfma_head_dim() { return D; }
+
+// partition_size == 0: every work item walks its whole key range and writes the result.
+// partition_size > 0 (a multiple of 64): num_partitions = ceil(max context / partition_size) work
+// items per tile write partials into `partials` (total_q * heads * num_partitions * (D + 2) floats).
+PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
+                                       int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
+                                       const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
+                                       int num_kv_heads, int block_size, float scale, int window, int partition_size,
+                                       int num_partitions, float* partials, hipStream_t stream) {
+  if (total_q <= 0 || num_seqs <= 0) return 0;
+  if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
+  const int G = num_heads / num_kv_heads;
+  if (G > 64 || block_size < 16 || (block_size & (block_size - 1))) return -2;
+  if (partition_size < 0 || (partition_size & 63) || (partition_size > 0 && (!partials || num_partitions < 1))) return -2;
+  if (partition_size == 0) num_partitions = 1;
+  const int max_cols = max_q_len * G;
+  const int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
+  const int tiles = (max_cols + 16 * ncb - 1) / (16 * ncb);
+  if (num_kv_heads * num_partitions > 65535 || num_seqs > 65535) return -2;
+  dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64);
+#define PLLM_LAUNCH(NCB_)                                                                                                       \
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<NCB_>), grid, block, 0, stream, (const bf16*)q, q_stride, (const bf16*)k_pages, \
+                     (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_heads,  \
+                     num_kv_heads, block_size, scale, window, partition_size, num_partitions, partials)
+  if (ncb == 1) PLLM_LAUNCH(1); else if (ncb == 2) PLLM_LAUNCH(2); else PLLM_LAUNCH(4);
+#undef PLLM_LAUNCH
+  int err = (int)hipGetLastError();
+  if (err) return err;
+  if (partition_size > 0) {
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_q, num_heads), dim3(64), 0, stream, partials, (bf16*)out, out_stride,
+                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, window, partition_size, num_partitions);
+    err = (int)hipGetLastError();
+  }
+  return err;
+}

@@ -361,9 +361,74 @@ def gate_up_silu(h: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     return silu_mul(linear(h, w_gate_up))
 
 
+_ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p]
+_attn_scratch: dict = {}
+
+
+def mfma_attention_takes(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int, block_size: int) -> bool:
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size >= 16
+            and block_size & (block_size - 1) == 0 and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 64)
+
+
+def attention_partition(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: int, group: int) -> tuple[int, int]:
+    """(partition_size, num_partitions) for a step: keys are split between work items when the
+    queries alone give too few of them to fill the GPU (decoding).  (0, 1) = no split."""
+    cols = max_q_len * group
+    tiles = (cols + 63) // 64
+    items = num_seqs * num_kv_heads * tiles
+    if items >= 512 or max_k_len <= 128:
+        return 0, 1
+    want = max(1, 1024 // items)
+    size = 64
+    while (max_k_len + size - 1) // size > want:
+        size *= 2
+    parts = (max_k_len + size - 1) // size
+    return (size, parts) if parts > 1 else (0, 1)
+
+
+def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
+                         cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
+                         head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
+                         num_partitions: int = 1, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
+    the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
+    work item into aligned partitions that a second kernel merges."""
+    S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
+    _need(mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs),
+          f"MFMA attention takes bfloat16, head sizes 16..256 in steps of 16, pages of >= 16 positions and groups of <= 64 "
+          f"heads; got {q.dtype}, head size {head_dim}, page {bs}, {num_heads}/{num_kv_heads} heads")
+    _need(q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0, "q rows must start on 16-byte boundaries")
+    T = q.shape[0]
+    if out is None:
+        out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
+    _need(out.shape == (T, num_heads * head_dim) and out.stride(1) == 1 and out.dtype == q.dtype and out.stride(0) % 4 == 0,
+          "bad attention output")
+    _need(max_q_len >= 1 and partition_size % 64 == 0, "bad launch parameters")
+    ws = None
+    if partition_size > 0:
+        floats = T * num_heads * num_partitions * (head_dim + 2)
+        key = str(q.device)
+        ws = _attn_scratch.get(key)
+        if ws is None or ws.numel() < floats:
+            ws = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=q.device)
+            _attn_scratch[key] = ws
+    f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
+    _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
+             block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
+             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), _stream()),
+           "paged_attention_mfma")
+    return out
+
+
 def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
                     scale, window, ctx) -> torch.Tensor:
     """Attention of one step's queries over the paged cache: the MFMA kernel for bfloat16 where it
     takes the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions."""
+    bs = k_pages.shape[2]
+    if mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
+        size, parts = attention_partition(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, num_heads // num_kv_heads)
+        return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
+                                    head_dim, scale, window, ctx.max_q_len, size, parts)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window)

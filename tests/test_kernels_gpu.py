@@ -336,3 +336,71 @@ def test_large_bf16_product_and_float_rows():
     assert rel_err(ops().gemm_bf16(a.cuda(), w.cuda()), want) <= 1e-2
     out = ops().gemm_bf16(a.cuda(), w.cuda(), torch.float32)
     assert out.dtype == torch.float32 and rel_err(out, want) <= 2e-5
+
+
+# ----------------------------------------------------------------------------------- attention on the matrix cores
+MFMA_SHAPES = [(4, 2, 32, 16), (8, 8, 64, 16), (32, 4, 64, 16), (3, 1, 48, 32), (5, 5, 16, 16), (6, 2, 128, 64), (2, 1, 256, 16),
+               (16, 1, 80, 16), (40, 1, 64, 16)]
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,bs", MFMA_SHAPES)
+@pytest.mark.parametrize("lens,num_q", CASES)
+def test_paged_attention_mfma(heads, kv_heads, d, bs, lens, num_q):
+    if sum(lens) * heads * d > 3_000_000 and (heads, d) not in ((32, 64),):
+        pytest.skip("long case kept for one shape")
+    q, kp, vp, tables, cu, sl = paged_case(lens, num_q, heads, kv_heads, d, bs, torch.bfloat16, seed=1)
+    scale = 1 / math.sqrt(d)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, scale)
+    args = (q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, scale, 0, max(num_q))
+    assert rel_err(ops().paged_attention_mfma(*args), want) <= 1.6e-2
+    for size in (64, 256):
+        parts = (max(lens) + size - 1) // size
+        assert rel_err(ops().paged_attention_mfma(*args, size, parts), want) <= 1.6e-2, f"partition {size}"
+
+
+@pytest.mark.parametrize("window", [1, 5, 64, 100])
+def test_paged_attention_mfma_window(window):
+    heads, kv_heads, d, bs = 4, 2, 32, 16
+    q, kp, vp, tables, cu, sl = paged_case([150, 70, 9, 300], [30, 1, 9, 1], heads, kv_heads, d, bs, torch.bfloat16, seed=2)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, 0.2, window)
+    args = (q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, 0.2, window, 30)
+    assert rel_err(ops().paged_attention_mfma(*args), want) <= 1.6e-2
+    assert rel_err(ops().paged_attention_mfma(*args, 64, 5), want) <= 1.6e-2
+
+
+def test_mfma_attention_ignores_table_padding_and_stale_slots():
+    heads, kv_heads, d, bs = 4, 2, 32, 16
+    q, kp, vp, tables, cu, sl = paged_case([20, 5, 70], [1, 1, 3], heads, kv_heads, d, bs, torch.bfloat16, seed=3)
+    def run(kp, vp, tables, *split):
+        return ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
+                                          d, 0.3, 0, 3, *split).cpu()
+    t2 = tables.clone()
+    t2[0, 2:] = 999_999
+    t2[1, 1:] = 999_999
+    kp2, vp2 = kp.clone(), vp.clone()
+    kp2[tables[1, 0], :, 5:, :] = float("nan")
+    vp2[tables[1, 0], :, :, 5:] = float("nan")
+    kp2[tables[0, 1], :, 4:, :] = float("inf")
+    vp2[tables[0, 1], :, :, 4:] = float("nan")
+    for split in ((), (64, 2)):
+        assert torch.equal(run(kp, vp, tables, *split), run(kp2, vp2, t2, *split))
+
+
+@pytest.mark.parametrize("far", [3, 64, 200, 699])
+def test_mfma_attention_one_far_key_stands_out(far):
+    heads, kv_heads, d, bs = 8, 1, 64, 16
+    q, kp, vp, tables, cu, sl = paged_case([700], [1], heads, kv_heads, d, bs, torch.bfloat16, seed=4)
+    page, off = int(tables[0, far // bs]), far % bs
+    kp[page, 0, off, :] = (q[0, 5 * d:6 * d].float() * 40).to(torch.bfloat16)       # head 5 looks at that key only
+    for split in ((), (128, 6)):
+        got = ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
+                                         d, 1.0, 0, 1, *split).cpu().float()
+        assert torch.allclose(got[0, 5 * d:6 * d], vp[page, 0, :, off].float(), atol=2e-2)
+
+
+def test_attention_partition_choice():
+    part = ops().attention_partition
+    assert part(8, 4, 1, 2048, 8) == (64, 32)          # decoding: keys are split to fill the GPU
+    assert part(64, 4, 1, 2048, 8) == (512, 4)
+    assert part(1, 4, 2048, 2048, 8) == (0, 1)         # a long prompt portion fills it alone
+    assert part(2, 4, 1, 100, 8) == (0, 1)
