@@ -285,10 +285,9 @@ def _skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 def _skinny_split(n_out_tiles: int, K: int) -> int:
     """How many workgroups share the K range of one tile: enough to put work on every CU, while
     every wavefront still gets at least one slab of 128."""
-    split = 1
-    while n_out_tiles * split < 512 and split * 2 * 4 * 128 <= K and split < 8:
-        split *= 2
-    return split
+    # Measured on MI355X: the cross-workgroup fix-up (device-scope fences) costs tens of
+    # microseconds, far more than the under-filled GPU it was meant to cure.  One split.
+    return 1
 
 
 def _skinny_buffers(device, floats: int, counters: int):

@@ -80,7 +80,8 @@ class LLMEngine:
 
         num_pages = cfg.num_gpu_blocks or self._profile_num_pages()
         self.cache_manager, self.kv_cache, self.runner = build_runtime(
-            self.model, cfg.block_size, num_pages, cfg.max_num_seqs, cfg.enable_prefix_caching)
+            self.model, cfg.block_size, num_pages, cfg.max_num_seqs, cfg.enable_prefix_caching,
+            use_graphs=cfg.enable_hip_graphs)
         self.groups = list(self.cache_manager.groups)
         eos = self.model.spec.eos_token_id
         self.scheduler = Scheduler(cfg, self.cache_manager, eos)

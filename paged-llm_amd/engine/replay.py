@@ -28,7 +28,7 @@ class ReplaySession:
         bs = REPLAY_BLOCK_SIZE
         num_pages = max(1, (max_tokens + bs - 1) // bs)
         self.manager, self.storage, self.runner = build_runtime(
-            self.model, bs, num_pages, MAX_LIVE_REQUESTS, enable_prefix_caching=False)
+            self.model, bs, num_pages, MAX_LIVE_REQUESTS, enable_prefix_caching=False, use_graphs=True)
         self.groups = list(self.manager.groups)
         self.computed: dict = {}
         self.out_dir = out_dir

@@ -22,8 +22,14 @@ class StepError(ValueError):
 
 
 class ModelRunner:
-    def __init__(self, model, kv_storage: KVCacheStorage, num_state_slots: int = 0):
+    def __init__(self, model, kv_storage: KVCacheStorage, num_state_slots: int = 0, use_graphs: bool = False,
+                 max_graph_batch: int = 256):
         self.model = model
+        # Graph replay needs every part of the model to do nothing but launch kernels on the
+        # current stream; parts say so with ``graph_capturable``.
+        self.use_graphs = bool(use_graphs) and model.graph_capturable()
+        self.max_graph_batch = max_graph_batch
+        self._graphs: dict = {}
         self.kv = kv_storage
         self.device = model.device
         self.block_size = kv_storage.block_size
@@ -33,7 +39,14 @@ class ModelRunner:
                        for pos, ss in model.state_specs().items()}
 
     # ------------------------------------------------------------------ batch -> device tensors
-    def build_context(self, entries: list) -> StepContext:
+    def _stage(self, entries: list, fixed_blocks: int | None = None):
+        """Checks the batch and lays all its integer arrays out in one host buffer.
+
+        Returns (buffer, offsets, sizes, host) where piece i is buffer[offsets[i]: offsets[i] + sizes[i]]
+        in the order: ids, positions, cu_seqlens_q, seq_lens_k, state slots, starts, logits rows, then
+        per cache group its block tables and slots.  ``fixed_blocks`` pads every block table to that
+        many entries, so that the layout depends on the counts only (needed to replay a graph).
+        """
         if not entries:
             raise StepError("a step needs at least one entry")
         bs = self.block_size
@@ -72,6 +85,9 @@ class ModelRunner:
         for name, cs in self.group_specs.items():
             num_pages = self.kv.num_pages[name]
             max_blocks = max((k + bs - 1) // bs for k in k_lens)
+            if fixed_blocks is not None:
+                assert fixed_blocks >= max_blocks
+                max_blocks = fixed_blocks
             tables = np.zeros((S, max_blocks), dtype=np.int32)
             slots = []
             for s, e in enumerate(entries):
@@ -97,12 +113,13 @@ class ModelRunner:
         if self.states and (slots_state < 0).any():
             raise StepError("this model keeps per-request state: every entry needs a state slot")
 
-        # One staging buffer, one copy to the device.
         pieces = [np.concatenate(ids_parts).astype(np.int32), positions.astype(np.int32),
                   np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32), np.asarray(k_lens, dtype=np.int32),
                   slots_state, np.asarray(starts, dtype=np.int32), np.asarray(logits_idx, dtype=np.int32)]
+        table_shapes = {}
         for name in self.group_specs:
             tables, slots = group_arrays[name]
+            table_shapes[name] = tables.shape
             pieces += [tables.reshape(-1), slots]
         # Each piece starts on a 16-byte boundary (kernels may read them with vector loads).
         padded, offsets, cursor = [], [], 0
@@ -113,19 +130,75 @@ class ModelRunner:
             if pad:
                 padded.append(np.zeros(pad, dtype=np.int32))
             cursor += p.size + pad
-        staged = torch.from_numpy(np.concatenate(padded)).to(self.device, non_blocking=False)
+        host = dict(T=T, S=S, q_lens=q_lens, k_lens=k_lens, slots_state=slots_state.tolist(), table_shapes=table_shapes)
+        return np.concatenate(padded), offsets, [p.size for p in pieces], host
 
+    def _context(self, staged: torch.Tensor, offsets: list, sizes: list, host: dict, max_k_len: int | None = None,
+                 capturing: bool = False) -> StepContext:
         def piece(i):
-            return staged[offsets[i]: offsets[i] + pieces[i].size]
+            return staged[offsets[i]: offsets[i] + sizes[i]]
 
         groups = {}
         for gi, name in enumerate(self.group_specs):
-            tables, _ = group_arrays[name]
-            groups[name] = GroupView(piece(7 + 2 * gi).view(S, tables.shape[1]), piece(8 + 2 * gi), bs)
+            groups[name] = GroupView(piece(7 + 2 * gi).view(*host["table_shapes"][name]), piece(8 + 2 * gi), self.block_size)
         return StepContext(
-            num_tokens=T, num_seqs=S, input_ids=piece(0), positions=piece(1), cu_seqlens_q=piece(2), seq_lens_k=piece(3),
-            state_slots=piece(4), seq_starts=piece(5), logits_index=piece(6), groups=groups, q_lens=q_lens, k_lens=k_lens,
-            state_slot_list=slots_state.tolist(), max_q_len=max(q_lens), max_k_len=max(k_lens), dtype=self.model.dtype, device=self.device)
+            num_tokens=host["T"], num_seqs=host["S"], input_ids=piece(0), positions=piece(1), cu_seqlens_q=piece(2),
+            seq_lens_k=piece(3), state_slots=piece(4), seq_starts=piece(5), logits_index=piece(6), groups=groups,
+            q_lens=host["q_lens"], k_lens=host["k_lens"], state_slot_list=host["slots_state"], max_q_len=max(host["q_lens"]),
+            max_k_len=max_k_len or max(host["k_lens"]), dtype=self.model.dtype, device=self.device, capturing=capturing)
+
+    def build_context(self, entries: list) -> StepContext:
+        buf, offsets, sizes, host = self._stage(entries)
+        staged = torch.from_numpy(buf).to(self.device, non_blocking=False)
+        return self._context(staged, offsets, sizes, host)
+
+    # ------------------------------------------------------------------ decode steps as HIP graphs
+    def _graph_key(self, entries: list):
+        """Decode-only steps (one token per request) of a model whose parts launch kernels only can
+        be replayed from a captured graph.  The key holds everything launch shapes depend on: the
+        number of requests, of wanted rows, and a bound on the context length."""
+        if not self.use_graphs or len(entries) > self.max_graph_batch:
+            return None
+        if any(len(e.tokens) != 1 for e in entries):
+            return None
+        longest = max(e.start + 1 for e in entries)
+        bound = ((longest + 511) // 512) * 512 if longest <= 8192 else 1 << (longest - 1).bit_length()
+        bound = min(bound, max(self.model.max_positions, longest))
+        return (len(entries), sum(len(e.want) for e in entries), bound)
+
+    def _capture(self, key, buf, offsets, sizes, host):
+        S, n_want, bound = key
+        pinned = torch.empty(buf.size, dtype=torch.int32, pin_memory=True)
+        pinned.numpy()[:] = buf
+        static = torch.empty(buf.size, dtype=torch.int32, device=self.device)
+        static.copy_(pinned)
+        ctx = self._context(static, offsets, sizes, host, max_k_len=bound, capturing=True)
+        stream = torch.cuda.Stream(device=self.device)
+        stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(stream):
+            self.model.forward(ctx, self.kv, self.states)          # warm-up: loads libraries, sizes workspaces
+        torch.cuda.current_stream(self.device).wait_stream(stream)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            logits = self.model.forward(ctx, self.kv, self.states)
+        entry = dict(graph=graph, pinned=pinned, static=static, logits=logits, ctx=ctx, offsets=offsets, sizes=sizes)
+        if len(self._graphs) >= 48:
+            self._graphs.pop(next(iter(self._graphs)))
+        self._graphs[key] = entry
+        return entry
+
+    def _graph_step(self, key, entries: list) -> torch.Tensor:
+        S, n_want, bound = key
+        buf, offsets, sizes, host = self._stage(entries, fixed_blocks=(bound + self.block_size - 1) // self.block_size)
+        entry = self._graphs.get(key)
+        if entry is None:
+            entry = self._capture(key, buf, offsets, sizes, host)
+        assert entry["offsets"] == offsets and entry["sizes"] == sizes
+        entry["pinned"].numpy()[:] = buf
+        entry["static"].copy_(entry["pinned"], non_blocking=True)
+        entry["graph"].replay()
+        return entry["logits"].clone()
 
     # ------------------------------------------------------------------ run
     @torch.no_grad()
@@ -133,5 +206,8 @@ class ModelRunner:
         """Float logits [wanted rows, vocab], in the order of the entries and of their ``want``."""
         if copies:
             self.kv.apply_copies(copies)
+        key = self._graph_key(entries)
+        if key is not None:
+            return self._graph_step(key, entries)
         ctx = self.build_context(entries)
         return self.model.forward(ctx, self.kv, self.states)

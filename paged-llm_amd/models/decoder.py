@@ -91,6 +91,12 @@ class DecoderModel:
                 out[pos] = ss
         return out
 
+    def graph_capturable(self) -> bool:
+        """True when every mixer and feed-forward only launches kernels (no host reads of device
+        data, no Python-side state): a decode step can then be captured into a HIP graph."""
+        return all(getattr(b.mixer, "graph_capturable", False) and getattr(b.parts["feed_forward"], "graph_capturable", False)
+                   for b in self.blocks)
+
     # ------------------------------------------------------------------ compute
     def forward(self, ctx, kv_storage, states: dict) -> torch.Tensor:
         """Float logits [n, vocab] at ctx.logits_index (empty tensor when nothing is wanted;

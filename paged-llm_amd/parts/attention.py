@@ -19,6 +19,8 @@ from .spec import PartSpec, WeightSpec
 
 
 class PagedAttention(Mixer):
+    graph_capturable = True
+
     def __init__(self, params: dict, env: BuildEnv):
         self.hidden = env.hidden_size
         self.num_heads = int(params["num_heads"])

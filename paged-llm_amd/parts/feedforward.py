@@ -14,6 +14,8 @@ from .spec import WeightSpec
 
 
 class GatedMLP(FeedForward):
+    graph_capturable = True
+
     def __init__(self, params: dict, env: BuildEnv):
         self.hidden = env.hidden_size
         self.inter = int(params["intermediate_size"])

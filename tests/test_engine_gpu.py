@@ -184,3 +184,40 @@ def test_trace_run_program(folder_a, tmp_path, dtype):
     tol = 2e-5 if dtype == "float32" else 4e-2
     for (rid, pos), row in got.items():
         assert helpers.worst(row, helpers.plain_logits(folder_a, toks[rid])[pos]) <= tol
+
+
+def test_decode_steps_replayed_from_graphs_equal_eager_steps(folder_a):
+    """Decode steps captured into HIP graphs are replayed many times, with eager prefill steps of
+    other requests in between; every replay must give what the eager step function gives."""
+    from paged_llm_amd.engine.replay import ReplaySession
+    import paged_llm_amd.engine.loading as loading
+    toks = {f"g{i}": helpers.random_tokens(60 + 7 * i, 256, seed=500 + i) for i in range(3)}
+
+    def run(use_graphs):
+        real = loading.build_runtime
+        def patched(*a, **kw):
+            kw["use_graphs"] = use_graphs
+            return real(*a, **kw)
+        import paged_llm_amd.engine.replay as replay
+        replay.build_runtime = patched
+        try:
+            session = ReplaySession(folder_a, "bfloat16", 64 * 2 * 3, None)
+        finally:
+            replay.build_runtime = real
+        assert session.runner.use_graphs == use_graphs
+        trace = helpers.TraceBuilder()
+        trace.step([(r, t[:20], "last") for r, t in toks.items()])
+        for i in range(20, 60):
+            live = [(r, t[i:i + 1], "all") for r, t in toks.items()]
+            trace.step(live if i % 7 else live[:2])                      # batch size changes: other graphs
+            if i == 40:
+                trace.step([("late", toks["g0"][:33], "last")], end=["late"])   # an eager step between replays
+        out = helpers.replay_in_process(session, trace)
+        return out, session
+
+    eager, _ = run(False)
+    graphed, session = run(True)
+    assert len(session.runner._graphs) >= 2
+    assert eager.keys() == graphed.keys()
+    for key in eager:
+        assert helpers.worst(graphed[key], eager[key]) <= 1e-6, key
