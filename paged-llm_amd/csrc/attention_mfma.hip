@@ -61,13 +61,13 @@ __device__ __forceinline__ float group_sum(float v) {
 // Partials of one (token, head, partition): [m (log2 units), l, acc[D]].
 constexpr int kPartialFloats = D + 2;
 
-template <int NCB>
-__global__ __launch_bounds__(64) void paged_attention_mfma_kernel(
+template <int NCB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
     int block_size, float scale, int window, int partition_size, int num_partitions, float* __restrict__ partials) {
-  const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int seq = blockIdx.z;
   const int kvh = blockIdx.y / num_partitions, part = blockIdx.y - kvh * num_partitions;
   const int G = num_heads / num_kv_heads;
@@ -124,7 +124,9 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(
   const size_t page_elems = (size_t)block_size * D;             // one kv head's part of a page
   const size_t page_stride = page_elems * num_kv_heads;
 
-  for (int n0 = k_lo; n0 < k_hi; n0 += 64) {
+  // With several wavefronts per work item the blocks of 64 keys are dealt round-robin; their
+  // partial results are merged through LDS below.
+  for (int n0 = k_lo + wave * 64; n0 < k_hi; n0 += WAVES * 64) {
     // Every key of the block visible to every column?  Then no masking is needed.
     const bool interior = (n0 + 63 <= qpos_min) && (n0 >= (window > 0 ? max(qpos_max - window + 1, 0) : 0)) && (n0 + 64 <= k_hi) &&
                           (col0 + 16 * NCB <= num_cols);
@@ -230,6 +232,45 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(
     }
   }
 
+  if (WAVES > 1) {
+    // ---- merge the wavefronts: common maximum per column, rescale, add in wave order
+    extern __shared__ float lds[];
+    float* m_s = lds;                                            // [WAVES][NCB * 16]
+    float* l_s = lds + WAVES * NCB * 16;                         // [WAVES][NCB * 16]
+    float* acc_s = lds + 2 * WAVES * NCB * 16;                   // [WAVES][NCB * DBLOCKS * 4][64]
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+      if (g == 0) m_s[(wave * NCB + cb) * 16 + r] = m_run[cb];
+    __syncthreads();
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      float mx = -INFINITY;
+      for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, m_s[(w * NCB + cb) * 16 + r]);
+      const float f = (m_run[cb] == -INFINITY) ? 0.f : fast_exp2(m_run[cb] - mx);
+      const float l_tot = group_sum(l_run[cb]) * f;
+      if (g == 0) l_s[(wave * NCB + cb) * 16 + r] = l_tot;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc_s[((size_t)(wave * NCB + cb) * DBLOCKS * 4 + db * 4 + i) * 64 + lane] = acc[cb][db][i] * f;
+    }
+    __syncthreads();
+    // entry e = (cb, db, i); thread (e, lane) owns column cb*16 + r, channel db*16 + g*4 + i
+    for (int e = wave; e < NCB * DBLOCKS * 4; e += WAVES) {
+      const int cb = e / (DBLOCKS * 4), rest = e - cb * DBLOCKS * 4, db = rest >> 2, i = rest & 3;
+      const int c = col0 + cb * 16 + r;
+      if (c >= num_cols) continue;
+      float o = 0.f, l_tot = 0.f;
+      for (int w = 0; w < WAVES; ++w) {
+        o += acc_s[((size_t)(w * NCB + cb) * DBLOCKS * 4 + rest) * 64 + lane];
+        l_tot += l_s[(w * NCB + cb) * 16 + r];
+      }
+      const int tok = c / G, hg = c - tok * G;
+      out[(size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D + db * 16 + g * 4 + i] = __float2bfloat16(o / l_tot);
+    }
+    return;
+  }
+
   // ---- write: lane holds channels db*16 + g*4 + i of its column
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb) {
@@ -300,14 +341,19 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
 
 PLLM_API int pllm_attention_mfma_head_dim() { return D; }
 
-// partition_size == 0: every work item walks its whole key range and writes the result.
-// partition_size > 0 (a multiple of 64): num_partitions = ceil(max context / partition_size) work
-// items per tile write partials into `partials` (total_q * heads * num_partitions * (D + 2) floats).
+// LDS floats of the several-wavefront variant.
+static size_t merge_lds_bytes(int ncb, int waves) { return (size_t)(2 * waves * ncb * 16 + waves * ncb * DBLOCKS * 4 * 64) * sizeof(float); }
+
+// partition_size == 0, waves == 1: every work item (one wavefront) walks its whole key range.
+// partition_size == 0, waves in {4, 8, 16}: one work item per (sequence, kv head) whose wavefronts
+//   share the key range and merge through LDS; needs max_q_len * G <= 64 (decoding, tiny portions).
+// partition_size > 0 (a multiple of 64), waves == 1: num_partitions work items per tile write partials
+//   into `partials` (total_q * heads * num_partitions * (D + 2) floats) and a second kernel merges them.
 PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
                                        int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                        const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                                        int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                       int num_partitions, float* partials, hipStream_t stream) {
+                                       int num_partitions, float* partials, int waves, hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
   const int G = num_heads / num_kv_heads;
@@ -318,12 +364,27 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   const int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
   const int tiles = (max_cols + 16 * ncb - 1) / (16 * ncb);
   if (num_kv_heads * num_partitions > 65535 || num_seqs > 65535) return -2;
-  dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64);
-#define PLLM_LAUNCH(NCB_)                                                                                                       \
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<NCB_>), grid, block, 0, stream, (const bf16*)q, q_stride, (const bf16*)k_pages, \
-                     (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_heads,  \
-                     num_kv_heads, block_size, scale, window, partition_size, num_partitions, partials)
-  if (ncb == 1) PLLM_LAUNCH(1); else if (ncb == 2) PLLM_LAUNCH(2); else PLLM_LAUNCH(4);
+  if (waves != 1 && (partition_size > 0 || tiles != 1 || (waves != 4 && waves != 8 && waves != 16))) return -2;
+  dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64 * waves);
+  const size_t lds = waves > 1 ? merge_lds_bytes(ncb, waves) : 0;
+#define PLLM_LAUNCH(NCB_, WAVES_)                                                                                                    \
+  do {                                                                                                                               \
+    auto kern = paged_attention_mfma_kernel<NCB_, WAVES_>;                                                                           \
+    if (lds > 48 * 1024) {                                                                                                           \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return (int)e;                                                                                            \
+    }                                                                                                                                \
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages,         \
+                       (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,           \
+                       block_size, scale, window, partition_size, num_partitions, partials);                                         \
+  } while (0)
+#define PLLM_BY_WAVES(NCB_)                                                                          \
+  do {                                                                                               \
+    if (waves == 1) PLLM_LAUNCH(NCB_, 1); else if (waves == 4) PLLM_LAUNCH(NCB_, 4);                 \
+    else if (waves == 8) PLLM_LAUNCH(NCB_, 8); else PLLM_LAUNCH(NCB_, 16);                           \
+  } while (0)
+  if (ncb == 1) PLLM_BY_WAVES(1); else if (ncb == 2) PLLM_BY_WAVES(2); else PLLM_BY_WAVES(4);
+#undef PLLM_BY_WAVES
 #undef PLLM_LAUNCH
   int err = (int)hipGetLastError();
   if (err) return err;
@@ -333,4 +394,12 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     err = (int)hipGetLastError();
   }
   return err;
+}
+
+// Largest number of wavefronts per work item whose merge buffers fit `lds_limit` bytes (0: none).
+PLLM_API int pllm_attention_mfma_max_waves(int max_cols, long lds_limit) {
+  const int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
+  for (int w = 16; w >= 4; w /= 2)
+    if ((long)merge_lds_bytes(ncb, w) <= lds_limit) return w;
+  return 0;
 }

@@ -79,7 +79,7 @@ def _fn(source: str, name: str, defines: dict | None = None, signature: list | N
     if f is None:
         lib = build.load_library(source, defines)
         f = getattr(lib, name)
-        f.argtypes = signature or _SIGNATURES[name]
+        f.argtypes = signature if signature is not None else _SIGNATURES[name]
         f.restype = c_int
         _FUNCS[key] = f
     return f
@@ -269,6 +269,93 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     return out
 
 
+# ------------------------------------------------------------------------------------------- fused decode products
+EPI_BF16, EPI_F32, EPI_GATED, EPI_ROPE_KV = 0, 1, 2, 3
+DECODE_MAX_ROWS = 16
+_DECODE_SIG = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
+               c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+               c_void_p]
+_lds_limit: dict = {}
+
+
+def _max_lds_bytes(device) -> int:
+    key = str(device)
+    if key not in _lds_limit:
+        f = _fn("decode_linear.hip", "pllm_max_lds_bytes", signature=[])
+        f.restype = c_long
+        with torch.cuda.device(device):
+            _lds_limit[key] = int(f())
+    return _lds_limit[key]
+
+
+def decode_linear_takes(rows: int, K: int, x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the fused decode product takes these operands (else the caller runs the parts apart)."""
+    if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < rows <= DECODE_MAX_ROWS and K % 8 == 0):
+        return False
+    if not (x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        return False
+    waves = 16 if K >= 4096 else 8
+    need = max(rows * (K + 8) * 2, waves * 2 * 256 * 4)
+    return need <= _max_lds_bytes(x.device)
+
+
+def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: torch.Tensor | None = None,
+                  norm_weight: torch.Tensor | None = None, eps: float = 0.0, x_out: torch.Tensor | None = None,
+                  row_index: torch.Tensor | None = None, rope: dict | None = None) -> torch.Tensor:
+    """rows = x[row_index] (+ delta) -> optional RMS norm -> rows W^T -> epilogue, in one kernel.
+
+    epi EPI_BF16 / EPI_F32: [M, N] out.  EPI_GATED: w = [gate; up], out = silu(gate) * up [M, N/2].
+    EPI_ROPE_KV: w = [q; k; v] rows; q is rotated and returned [M, heads * d]; k (rotated) and v go
+    into the cache pages; ``rope`` = dict(positions, cos, sin, slots, k_pages, v_pages, num_heads,
+    num_kv_heads, head_dim, block_size).  ``x_out`` receives x + delta (the new residual).
+    """
+    _on_gpu(x, w, delta, norm_weight, x_out, row_index)
+    M = row_index.numel() if row_index is not None else x.shape[0]
+    K = x.shape[1]
+    _need(x.dim() == 2 and w.dim() == 2 and w.shape[1] == K, f"decode_linear shapes {tuple(x.shape)} x {tuple(w.shape)}^T")
+    _need(decode_linear_takes(M, K, x, w), "decode_linear takes bfloat16, 1..16 rows, K a multiple of 8, rows that fit LDS")
+    if delta is not None:
+        _need(delta.shape == x.shape and delta.dtype == x.dtype and delta.stride(1) == 1 and delta.stride(0) % 8 == 0
+              and delta.data_ptr() % 16 == 0, "delta must match x")
+    if x_out is not None:
+        _need(delta is not None and x_out.shape == x.shape and x_out.dtype == x.dtype and x_out.stride(1) == 1
+              and x_out.stride(0) % 8 == 0 and x_out.data_ptr() != x.data_ptr(), "x_out must be a separate buffer like x")
+    if norm_weight is not None:
+        _need(norm_weight.dtype == torch.float32 and norm_weight.shape == (K,) and norm_weight.is_contiguous(), "norm weight: float32 [K]")
+    if row_index is not None:
+        _need(row_index.dtype == torch.int32 and row_index.dim() == 1 and row_index.is_contiguous(), "row_index: int32")
+    N = w.shape[0]
+    r = rope or {}
+    if epi == EPI_GATED:
+        _need(N % 2 == 0, "gated product needs [gate; up] rows")
+        N //= 2
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    elif epi == EPI_ROPE_KV:
+        nh, nkv, d, bs = r["num_heads"], r["num_kv_heads"], r["head_dim"], r["block_size"]
+        _need(d % 32 == 0 and N == (nh + 2 * nkv) * d, "fused rotary epilogue needs head sizes in multiples of 32 and [q; k; v] rows")
+        kp, vp = r["k_pages"], r["v_pages"]
+        P = kp.shape[0]
+        _need(tuple(kp.shape) == (P, nkv, bs, d) and tuple(vp.shape) == (P, nkv, d, bs) and kp.is_contiguous() and vp.is_contiguous()
+              and kp.dtype == torch.bfloat16 and vp.dtype == torch.bfloat16, "bad cache pages")
+        for name in ("positions", "slots"):
+            t = r[name]
+            _need(t.dtype == torch.int32 and t.shape == (M,) and t.is_contiguous(), f"{name}: int32 [{M}]")
+        if r.get("cos") is not None:
+            for t in (r["cos"], r["sin"]):
+                _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == d // 2 and t.is_contiguous(), "rotary tables")
+        out = torch.empty((M, nh * d), dtype=torch.bfloat16, device=x.device)
+    else:
+        out = torch.empty((M, N), dtype=torch.float32 if epi == EPI_F32 else torch.bfloat16, device=x.device)
+    f = _fn("decode_linear.hip", "pllm_decode_linear", signature=_DECODE_SIG)
+    _check(f(epi, _ptr(x), x.stride(0), _ptr(delta), delta.stride(0) if delta is not None else 0, _ptr(norm_weight), c_float(eps),
+             _ptr(x_out), x_out.stride(0) if x_out is not None else 0, _ptr(row_index), _ptr(w), w.stride(0), _ptr(out),
+             out.stride(0), M, N, K, _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")),
+             _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)),
+             int(r.get("head_dim", 0)), int(r.get("block_size", 0)), _stream()), "decode_linear")
+    return out
+
+
 # ------------------------------------------------------------------------------------------- choices
 SKINNY_MAX_ROWS = 64
 _SKINNY_SIG = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p,
@@ -338,8 +425,6 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = 
         return None
     M = a.shape[0]
     out_dtype = out_dtype or torch.bfloat16
-    if M <= SKINNY_MAX_ROWS:
-        return gemm_skinny(a, w, out_dtype)
     if out_dtype == torch.float32:
         # Float results for many rows (logits of a whole prompt): the same kernel, 64 rows at a time.
         return torch.cat([gemm_skinny(a[i:i + SKINNY_MAX_ROWS], w, out_dtype) for i in range(0, M, SKINNY_MAX_ROWS)], dim=0)
@@ -352,16 +437,8 @@ def gemm_large_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return torch.mm(a, w.t())
 
 
-def gate_up_silu(h: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(h Wg^T) * (h Wu^T) with Wg, Wu stacked in w_gate_up [2I, K]."""
-    if h.shape[0] <= SKINNY_MAX_ROWS and _skinny_ok(h, w_gate_up):
-        return gemm_skinny(h, w_gate_up, gated=True)
-    from ..parts.linear import linear
-    return silu_mul(linear(h, w_gate_up))
-
-
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p]
+             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
 _attn_scratch: dict = {}
 
 
@@ -370,29 +447,45 @@ def mfma_attention_takes(dtype: torch.dtype, num_heads: int, num_kv_heads: int, 
             and block_size & (block_size - 1) == 0 and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 64)
 
 
-def attention_partition(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: int, group: int) -> tuple[int, int]:
-    """(partition_size, num_partitions) for a step: keys are split between work items when the
-    queries alone give too few of them to fill the GPU (decoding).  (0, 1) = no split."""
+def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: int, group: int, head_dim: int,
+                   lds_limit: int) -> tuple[int, int, int]:
+    """(wavefronts per work item, partition_size, num_partitions) for a step.
+
+    Prompt portions have many query tiles: one wavefront per tile walks all its keys (1, 0, 1).
+    Decoding has one tile per (sequence, kv head): its keys are shared between the wavefronts of a
+    workgroup, which merge in LDS (w, 0, 1); only when the sequences are few and very long are the
+    keys also split between workgroups, merged by a second kernel (1, size, parts)."""
     cols = max_q_len * group
-    tiles = (cols + 63) // 64
-    items = num_seqs * num_kv_heads * tiles
-    if items >= 512 or max_k_len <= 128:
-        return 0, 1
-    want = max(1, 1024 // items)
-    size = 64
-    while (max_k_len + size - 1) // size > want:
-        size *= 2
-    parts = (max_k_len + size - 1) // size
-    return (size, parts) if parts > 1 else (0, 1)
+    if cols > 64:
+        return 1, 0, 1
+    items = num_seqs * num_kv_heads
+    if items < 64 and max_k_len > 16384:
+        want = max(1, 512 // items)
+        size = 64
+        while (max_k_len + size - 1) // size > want:
+            size *= 2
+        parts = (max_k_len + size - 1) // size
+        if parts > 1:
+            return 1, size, parts
+    ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
+    waves = 16
+    while waves >= 4 and (2 * waves * ncb * 16 + waves * ncb * (head_dim // 16) * 4 * 64) * 4 > lds_limit:
+        waves //= 2
+    if waves < 4 or max_k_len <= 64:
+        return 1, 0, 1
+    while waves > 4 and (waves // 2) * 64 >= max_k_len:
+        waves //= 2
+    return waves, 0, 1
 
 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
                          cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
                          head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
-                         num_partitions: int = 1, out: torch.Tensor | None = None) -> torch.Tensor:
+                         num_partitions: int = 1, waves: int = 1, out: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
-    work item into aligned partitions that a second kernel merges."""
+    work item into aligned partitions that a second kernel merges; ``waves`` > 1 shares the keys
+    of a work item between the wavefronts of one workgroup (few queries per sequence only)."""
     S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
     _need(mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs),
           f"MFMA attention takes bfloat16, head sizes 16..256 in steps of 16, pages of >= 16 positions and groups of <= 64 "
@@ -403,7 +496,9 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
         out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
     _need(out.shape == (T, num_heads * head_dim) and out.stride(1) == 1 and out.dtype == q.dtype and out.stride(0) % 4 == 0,
           "bad attention output")
-    _need(max_q_len >= 1 and partition_size % 64 == 0, "bad launch parameters")
+    _need(max_q_len >= 1 and partition_size % 64 == 0 and waves in (1, 4, 8, 16), "bad launch parameters")
+    _need(waves == 1 or (partition_size == 0 and max_q_len * (num_heads // num_kv_heads) <= 64),
+          "several wavefronts per work item need at most 64 (query, head) columns per kv head and no partitions")
     ws = None
     if partition_size > 0:
         floats = T * num_heads * num_partitions * (head_dim + 2)
@@ -415,7 +510,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
     _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
              block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
-             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), _stream()),
+             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), _stream()),
            "paged_attention_mfma")
     return out
 
@@ -426,8 +521,9 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
     takes the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions."""
     bs = k_pages.shape[2]
     if mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
-        size, parts = attention_partition(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, num_heads // num_kv_heads)
+        waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, num_heads // num_kv_heads,
+                                            head_dim, _max_lds_bytes(q.device))
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
-                                    head_dim, scale, window, ctx.max_q_len, size, parts)
+                                    head_dim, scale, window, ctx.max_q_len, size, parts, waves)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window)

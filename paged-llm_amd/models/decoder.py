@@ -114,8 +114,5 @@ class DecoderModel:
         n = ctx.logits_index.numel()
         if n == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        if delta is None:
-            h = self.final_norm.forward(x, ctx.logits_index)
-        else:
-            h = self.final_norm.add_norm(x, delta, ctx.logits_index, write_residual=False)
+        h = self.final_norm.pending(x, delta, ctx.logits_index, write_residual=False)
         return self.head.forward(h)

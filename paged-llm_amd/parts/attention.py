@@ -13,7 +13,7 @@ import torch
 
 from ..csrc import ops
 from .base import CacheSpec, Mixer
-from .linear import linear
+from .linear import linear, qkv_rotary_cache
 from .registry import BuildEnv, register_mixer
 from .spec import PartSpec, WeightSpec
 
@@ -74,13 +74,11 @@ class PagedAttention(Mixer):
         if write and not self.kv_proj:
             raise RuntimeError("this attention layer has no k/v projections and must read another layer's cache")
         w_in = self.w_qkv if write or not self.kv_proj else self.w_qkv[: nh * d]
-        qkv = linear(h, w_in)
         cos = sin = None
         if self.position is not None:
             cos, sin = self.position.cos, self.position.sin
-        ops.rope_scatter(qkv, ctx.positions, cos, sin, nh, nkv, d,
-                         view.slot_mapping if write else None,
-                         cache.k_pages if write else None, cache.v_pages if write else None, cache.block_size)
+        qkv = qkv_rotary_cache(h, w_in, ctx.positions, cos, sin, nh, nkv, d, view.slot_mapping if write else None,
+                               cache.k_pages if write else None, cache.v_pages if write else None, cache.block_size)
         o = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
                                 nh, nkv, d, self.scale, self.window, ctx)
         return linear(o, self.w_o)

@@ -66,6 +66,29 @@ class Norm(Part):
         """x += delta (the residual sum, in float, rounded once), then the norm of the new x."""
         raise NotImplementedError
 
+    def pending(self, x: torch.Tensor, delta: torch.Tensor | None = None, row_index: torch.Tensor | None = None,
+                write_residual: bool = True):
+        """The normed rows as an object with ``rows()`` (a tensor), ``residual()`` (x after the sum)
+        and shape/dtype/device.  A norm whose kernel cannot be folded into a consumer computes at
+        once; see ``norm.PendingNorm`` for the lazy form."""
+        rows = self.forward(x, row_index) if delta is None else self.add_norm(x, delta, row_index, write_residual)
+        return _ComputedNorm(rows, x)
+
+
+class _ComputedNorm:
+    def __init__(self, rows: torch.Tensor, x: torch.Tensor):
+        self._rows, self._x = rows, x
+        self.shape, self.dtype, self.device = tuple(rows.shape), rows.dtype, rows.device
+
+    def rows(self) -> torch.Tensor:
+        return self._rows
+
+    def fusable(self) -> bool:
+        return False
+
+    def residual(self) -> torch.Tensor:
+        return self._x
+
 
 class PositionEncoding(Part):
     def prepare(self, max_positions: int) -> None:
@@ -79,8 +102,9 @@ class Mixer(Part):
     def state_spec(self) -> StateSpec | None:
         return None
 
-    def forward(self, h: torch.Tensor, ctx, cache, state) -> torch.Tensor:
-        """h: normed rows [T, hidden].  ctx: the step's StepContext.  cache: LayerCache of the
+    def forward(self, h, ctx, cache, state) -> torch.Tensor:
+        """h: normed rows [T, hidden], as a tensor or as a pending norm (``parts.linear.linear`` and
+        its relatives take both; ``parts.norm.rows_of(h)`` gives the tensor).  ctx: the step's StepContext.  cache: LayerCache of the
         layer this mixer reads (with ``writable`` False when it belongs to another layer), or
         None.  state: [slots, *shape] tensor, or None."""
         raise NotImplementedError

@@ -54,11 +54,12 @@ class PreNormBlock(Block):
 
     def forward(self, x, delta, ctx, cache, state):
         p = self.parts
-        h = p["mixer_norm"].forward(x) if delta is None else p["mixer_norm"].add_norm(x, delta)
+        h = p["mixer_norm"].pending(x, delta)             # summed and normed by whoever consumes it first
         a = p["mixer"].forward(h, ctx, cache, state)
-        h = p["feed_forward_norm"].add_norm(x, a)
+        x = h.residual()
+        h = p["feed_forward_norm"].pending(x, a)
         m = p["feed_forward"].forward(h, ctx)
-        return x, m
+        return h.residual(), m
 
 
 register_block("prenorm", PreNormBlock)

@@ -50,7 +50,7 @@ class LMHead(Part):
     def tie(self, table: torch.Tensor) -> None:
         self.weight = table
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h) -> torch.Tensor:
         return linear(h, self.weight, out_dtype=torch.float32)
 
 

@@ -8,7 +8,7 @@ import torch
 
 from ..csrc import ops
 from .base import FeedForward
-from .linear import linear
+from .linear import gated_linear, linear
 from .registry import BuildEnv, register_feed_forward
 from .spec import WeightSpec
 
@@ -43,7 +43,7 @@ class GatedMLP(FeedForward):
         self._w.clear()
 
     def forward(self, h, ctx):
-        act = ops.gate_up_silu(h, self.w_gate_up)
+        act = gated_linear(h, self.w_gate_up)
         return linear(act, self.w_down)
 
 

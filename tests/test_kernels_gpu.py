@@ -327,7 +327,6 @@ def test_gated_product(m, inter, k):
     want = torch.nn.functional.silu(g) * u
     got = ops().gemm_skinny(x.cuda(), w.cuda(), torch.float32, gated=True)
     assert rel_err(got, want) <= 3e-5
-    assert rel_err(ops().gate_up_silu(x.cuda(), w.cuda()), want) <= 1e-2
 
 
 def test_large_bf16_product_and_float_rows():
@@ -356,6 +355,10 @@ def test_paged_attention_mfma(heads, kv_heads, d, bs, lens, num_q):
     for size in (64, 256):
         parts = (max(lens) + size - 1) // size
         assert rel_err(ops().paged_attention_mfma(*args, size, parts), want) <= 1.6e-2, f"partition {size}"
+    if max(num_q) * (heads // kv_heads) <= 64:
+        for waves in (4, 8, 16):
+            if ops().attention_plan(1, 1, max(num_q), 10 ** 5, heads // kv_heads, d, 160 * 1024)[0] >= waves:
+                assert rel_err(ops().paged_attention_mfma(*args, 0, 1, waves), want) <= 1.6e-2, f"{waves} wavefronts"
 
 
 @pytest.mark.parametrize("window", [1, 5, 64, 100])
@@ -366,6 +369,13 @@ def test_paged_attention_mfma_window(window):
     args = (q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, 0.2, window, 30)
     assert rel_err(ops().paged_attention_mfma(*args), want) <= 1.6e-2
     assert rel_err(ops().paged_attention_mfma(*args, 64, 5), want) <= 1.6e-2
+    args = args[:-1] + (2,)
+    q2 = torch.cat([q[28:30], q[30:31], q[38:40], q[40:41]])          # at most two queries per sequence: 16 columns
+    cu2 = torch.tensor([0, 2, 3, 5, 6], dtype=torch.int32)
+    want2 = torch.cat([want[28:30], want[30:31], want[38:40], want[40:41]])
+    got = ops().paged_attention_mfma(q2.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu2.cuda(), sl.cuda(), heads, kv_heads, d, 0.2,
+                                     window, 2, 0, 1, 8)
+    assert rel_err(got, want2) <= 1.6e-2
 
 
 def test_mfma_attention_ignores_table_padding_and_stale_slots():
@@ -382,7 +392,7 @@ def test_mfma_attention_ignores_table_padding_and_stale_slots():
     vp2[tables[1, 0], :, :, 5:] = float("nan")
     kp2[tables[0, 1], :, 4:, :] = float("inf")
     vp2[tables[0, 1], :, :, 4:] = float("nan")
-    for split in ((), (64, 2)):
+    for split in ((), (64, 2), (0, 1, 4)):
         assert torch.equal(run(kp, vp, tables, *split), run(kp2, vp2, t2, *split))
 
 
@@ -392,15 +402,96 @@ def test_mfma_attention_one_far_key_stands_out(far):
     q, kp, vp, tables, cu, sl = paged_case([700], [1], heads, kv_heads, d, bs, torch.bfloat16, seed=4)
     page, off = int(tables[0, far // bs]), far % bs
     kp[page, 0, off, :] = (q[0, 5 * d:6 * d].float() * 40).to(torch.bfloat16)       # head 5 looks at that key only
-    for split in ((), (128, 6)):
+    for split in ((), (128, 6), (0, 1, 16)):
         got = ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
                                          d, 1.0, 0, 1, *split).cpu().float()
         assert torch.allclose(got[0, 5 * d:6 * d], vp[page, 0, :, off].float(), atol=2e-2)
 
 
-def test_attention_partition_choice():
-    part = ops().attention_partition
-    assert part(8, 4, 1, 2048, 8) == (64, 32)          # decoding: keys are split to fill the GPU
-    assert part(64, 4, 1, 2048, 8) == (512, 4)
-    assert part(1, 4, 2048, 2048, 8) == (0, 1)         # a long prompt portion fills it alone
-    assert part(2, 4, 1, 100, 8) == (0, 1)
+def test_attention_plan():
+    plan = ops().attention_plan
+    lds = 160 * 1024
+    assert plan(8, 4, 1, 2048, 8, 64, lds) == (16, 0, 1)        # decoding: the wavefronts of a workgroup share the keys
+    assert plan(8, 4, 1, 200, 8, 64, lds) == (4, 0, 1)
+    assert plan(1, 4, 2048, 2048, 8, 64, lds) == (1, 0, 1)      # a long prompt portion: one wavefront per query tile
+    assert plan(2, 4, 1, 50, 8, 64, lds) == (1, 0, 1)
+    assert plan(1, 8, 1, 100000, 4, 128, lds) == (1, 2048, 49)  # one very long sequence: keys split between workgroups too
+    assert plan(8, 1, 1, 4096, 8, 256, lds) == (8, 0, 1)        # wide heads: fewer wavefronts fit LDS
+
+
+# ----------------------------------------------------------------------------------- fused decode products
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("n,k", [(16, 64), (100, 96), (517, 176), (2560, 2048), (2048, 5632), (96, 1000)])
+def test_decode_linear_plain(m, n, k):
+    o = ops()
+    x, w = rnd(m, k, seed=30, dtype=torch.bfloat16), rnd(n, k, seed=31, dtype=torch.bfloat16)
+    if not o.decode_linear_takes(m, k, x.cuda(), w.cuda()):
+        pytest.skip("rows do not fit LDS")
+    want = x.double() @ w.double().T
+    assert rel_err(o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32), want) <= 2e-5
+    assert rel_err(o.decode_linear(x.cuda(), w.cuda(), o.EPI_BF16), want) <= 1e-2
+
+
+@pytest.mark.parametrize("m", [1, 8, 13])
+@pytest.mark.parametrize("k", [96, 2048])
+def test_decode_linear_with_residual_sum_norm_and_row_choice(m, k):
+    o = ops()
+    x, d = rnd(m, k, seed=32, dtype=torch.bfloat16), rnd(m, k, seed=33, dtype=torch.bfloat16)
+    nw, w = 1 + 0.3 * rnd(k, seed=34), rnd(130, k, seed=35, dtype=torch.bfloat16, scale=k ** -0.5)
+    summed = (x.float() + d.float()).to(torch.bfloat16)
+    h = plain.rms_norm(summed.float(), nw, 1e-4).to(torch.bfloat16)
+    want = h.double() @ w.double().T
+    x_out = torch.zeros(m, k, dtype=torch.bfloat16).cuda()
+    got = o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32, delta=d.cuda(), norm_weight=nw.cuda(), eps=1e-4, x_out=x_out)
+    assert torch.equal(x_out.cpu(), summed)
+    assert rel_err(got, want) <= 1e-2                      # h differs from the plain one by its bfloat16 rounding at most
+    # no delta, chosen rows
+    idx = torch.tensor(list(range(m - 1, -1, -2)), dtype=torch.int32)
+    h2 = plain.rms_norm(x.float()[idx.long()], nw, 1e-4).to(torch.bfloat16)
+    got = o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32, norm_weight=nw.cuda(), eps=1e-4, row_index=idx.cuda())
+    assert rel_err(got, h2.double() @ w.double().T) <= 1e-2
+    # the fused norm against the norm kernel followed by the plain product
+    sep = o.decode_linear(o.rmsnorm(x.cuda(), nw.cuda(), 1e-4), w.cuda(), o.EPI_F32)
+    fused = o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32, norm_weight=nw.cuda(), eps=1e-4)
+    assert rel_err(fused, sep) <= 2e-3
+
+
+@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("inter,k", [(176, 64), (250, 96), (5632, 2048)])
+def test_decode_linear_gated(m, inter, k):
+    o = ops()
+    x = rnd(m, k, seed=36, dtype=torch.bfloat16)
+    w = rnd(2 * inter, k, seed=37, dtype=torch.bfloat16, scale=k ** -0.5)
+    want = torch.nn.functional.silu(x.double() @ w[:inter].double().T) * (x.double() @ w[inter:].double().T)
+    assert rel_err(o.decode_linear(x.cuda(), w.cuda(), o.EPI_GATED), want) <= 1e-2
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 32, 16), (32, 4, 64, 16), (3, 1, 96, 32), (8, 8, 128, 16)])
+@pytest.mark.parametrize("m", [1, 7, 16])
+def test_decode_linear_rotary_and_cache_write(heads, kv_heads, d, bs, m):
+    from paged_llm_amd.parts.registry import BuildEnv
+    from paged_llm_amd.parts.rope import RotaryEncoding
+    o = ops()
+    k_in, pages = 256, 12
+    rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, torch.bfloat16, torch.device("cuda"), 512, {}))
+    rope.prepare(512)
+    width = (heads + 2 * kv_heads) * d
+    x = rnd(m, k_in, seed=38, dtype=torch.bfloat16)
+    w = rnd(width, k_in, seed=39, dtype=torch.bfloat16, scale=k_in ** -0.5)
+    positions = torch.tensor([(37 * t + 11) % 500 for t in range(m)], dtype=torch.int32)
+    slots = torch.randperm(pages * bs, generator=torch.Generator().manual_seed(40))[:m].to(torch.int32)
+    def run_fused():
+        kp = torch.zeros(pages, kv_heads, bs, d, dtype=torch.bfloat16).cuda()
+        vp = torch.zeros(pages, kv_heads, d, bs, dtype=torch.bfloat16).cuda()
+        q = o.decode_linear(x.cuda(), w.cuda(), o.EPI_ROPE_KV, rope=dict(
+            positions=positions.cuda(), cos=rope.cos, sin=rope.sin, slots=slots.cuda(), k_pages=kp, v_pages=vp, num_heads=heads,
+            num_kv_heads=kv_heads, head_dim=d, block_size=bs))
+        return q, kp, vp
+    def run_apart():
+        kp = torch.zeros(pages, kv_heads, bs, d, dtype=torch.bfloat16).cuda()
+        vp = torch.zeros(pages, kv_heads, d, bs, dtype=torch.bfloat16).cuda()
+        qkv = o.decode_linear(x.cuda(), w.cuda(), o.EPI_BF16)
+        o.rope_scatter(qkv, positions.cuda(), rope.cos, rope.sin, heads, kv_heads, d, slots.cuda(), kp, vp, bs)
+        return qkv[:, :heads * d], kp, vp
+    for a, b in zip(run_fused(), run_apart()):
+        assert torch.equal(a.cpu(), b.cpu())
