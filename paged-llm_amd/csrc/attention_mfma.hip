@@ -124,40 +124,51 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   const size_t page_elems = (size_t)block_size * D;             // one kv head's part of a page
   const size_t page_stride = page_elems * num_kv_heads;
 
-  // With several wavefronts per work item the blocks of 64 keys are dealt round-robin; their
-  // partial results are merged through LDS below.
-  for (int n0 = k_lo + wave * 64; n0 < k_hi; n0 += WAVES * 64) {
-    // Every key of the block visible to every column?  Then no masking is needed.
-    const bool interior = (n0 + 63 <= qpos_min) && (n0 >= (window > 0 ? max(qpos_max - window + 1, 0) : 0)) && (n0 + 64 <= k_hi) &&
-                          (col0 + 16 * NCB <= num_cols);
-    floatx4 s_t[4][NCB];
-    const bf16* vbase[4];
-    bool tile_on[4];
-    // ---- S^T = K Q^T for four tiles of 16 keys
+  // One block = 64 keys = four tiles of 16.  All of a block's keys and values are requested
+  // together, and (when the wavefronts of a workgroup share the keys) the next block is
+  // requested before the current one is used, so that a wavefront waits for memory once, not once
+  // per dependent step.
+  struct KVBlock {
+    bf16x8 k[4][KSTEPS];
+    bf16x4 v[4][DBLOCKS];
+    bool on[4];
+  };
+  auto load_block = [&](KVBlock& blk, int n0) {
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
       const int nk = n0 + kt * 16;
-      tile_on[kt] = nk < k_hi;                                  // uniform: tiles past the range are skipped, their table entries unread
-#pragma unroll
-      for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
-      vbase[kt] = v_pages;
-      if (!tile_on[kt]) continue;
+      blk.on[kt] = nk < k_hi;                                   // uniform; tiles past the range: table entries stay unread
+      if (!blk.on[kt]) continue;
       const int page = bt[nk / block_size];
       const int off = nk & (block_size - 1);
       const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
-      vbase[kt] = v_pages + base + off;                         // + channel * block_size + key
       const bf16* krow = k_pages + base + (size_t)(off + r) * D;
-      bf16x8 kreg[KSTEPS];
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
         const int dd = s * 32 + g * 8;
-        kreg[s] = (dd < D) ? *reinterpret_cast<const bf16x8*>(krow + dd) : zero8();
+        blk.k[kt][s] = (dd < D) ? *reinterpret_cast<const bf16x8*>(krow + dd) : zero8();
       }
+      const bf16* vrow = v_pages + base + off + g * 4;          // + channel * block_size
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) blk.v[kt][db] = *reinterpret_cast<const bf16x4*>(vrow + (size_t)(db * 16 + r) * block_size);
+    }
+  };
+  auto compute_block = [&](KVBlock& blk, int n0) {
+    // Every key of the block visible to every column?  Then no masking is needed.
+    const bool interior = (n0 + 63 <= qpos_min) && (n0 >= (window > 0 ? max(qpos_max - window + 1, 0) : 0)) && (n0 + 64 <= k_hi) &&
+                          (col0 + 16 * NCB <= num_cols);
+    // ---- S^T = K Q^T for four tiles of 16 keys
+    floatx4 s_t[4][NCB];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
+      if (!blk.on[kt]) continue;
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s)
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb)
-          s_t[kt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[s], qreg[cb][s], s_t[kt][cb], 0, 0, 0);
+          s_t[kt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[kt][s], qreg[cb][s], s_t[kt][cb], 0, 0, 0);
     }
 
     // ---- online softmax per column; lane holds keys n0 + kt*16 + g*4 + i of its column
@@ -173,7 +184,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
           float v = s_t[kt][cb][i] * sl2;
           if (!interior) {
             const int n = n0 + kt * 16 + g * 4 + i;
-            const bool vis = tile_on[kt] && n <= my_qpos[cb] && n >= my_first[cb];
+            const bool vis = blk.on[kt] && n <= my_qpos[cb] && n >= my_first[cb];
             v = vis ? v : -INFINITY;
           }
           sc[kt][i] = v;
@@ -201,7 +212,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     // ---- O^T += V^T P^T : A operand = 16 channels x 32 keys (k slots 0-3: tile 2a, 4-7: tile 2a+1)
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
-      if (!tile_on[2 * a]) continue;
+      if (!blk.on[2 * a]) continue;
 #pragma unroll
       for (int db = 0; db < DBLOCKS; ++db) {
         bf16x8 vreg;
@@ -209,8 +220,8 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
         for (int h = 0; h < 2; ++h) {
           const int kt = 2 * a + h;
           bf16x4 v4;
-          if (tile_on[kt]) {
-            v4 = *reinterpret_cast<const bf16x4*>(vbase[kt] + (size_t)(db * 16 + r) * block_size + g * 4);
+          if (blk.on[kt]) {
+            v4 = blk.v[kt][db];
             if (!interior) {
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
@@ -229,6 +240,36 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
         for (int cb = 0; cb < NCB; ++cb)
           acc[cb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg, p_op[a][cb], acc[cb][db], 0, 0, 0);
       }
+    }
+  };
+
+  // With several wavefronts per work item the blocks are dealt round-robin; their partial
+  // results are merged through LDS below.
+  constexpr int kStride = WAVES * 64;
+  if (WAVES > 1) {
+    KVBlock blk_a, blk_b;
+    int n0 = k_lo + wave * 64;
+    if (n0 < k_hi) {
+      load_block(blk_a, n0);
+      while (true) {
+        const int n1 = n0 + kStride;
+        const bool has1 = n1 < k_hi;
+        if (has1) load_block(blk_b, n1);
+        compute_block(blk_a, n0);
+        if (!has1) break;
+        const int n2 = n1 + kStride;
+        const bool has2 = n2 < k_hi;
+        if (has2) load_block(blk_a, n2);
+        compute_block(blk_b, n1);
+        if (!has2) break;
+        n0 = n2;
+      }
+    }
+  } else {
+    KVBlock blk;
+    for (int n0 = k_lo; n0 < k_hi; n0 += 64) {
+      load_block(blk, n0);
+      compute_block(blk, n0);
     }
   }
 
@@ -266,7 +307,19 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
         l_tot += l_s[(w * NCB + cb) * 16 + r];
       }
       const int tok = c / G, hg = c - tok * G;
-      out[(size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D + db * 16 + g * 4 + i] = __float2bfloat16(o / l_tot);
+      if (partition_size > 0) {
+        // this workgroup's partition: unnormalised sum, its maximum and its weight, for the merge kernel
+        float* dst = partials + (((size_t)(q_begin + tok) * num_heads + (kvh * G + hg)) * num_partitions + part) * kPartialFloats;
+        if (rest == 0 && g == 0) {
+          float mx = -INFINITY;
+          for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, m_s[(w * NCB + cb) * 16 + r]);
+          dst[0] = mx;
+          dst[1] = l_tot;
+        }
+        dst[2 + db * 16 + g * 4 + i] = o;
+      } else {
+        out[(size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D + db * 16 + g * 4 + i] = __float2bfloat16(o / l_tot);
+      }
     }
     return;
   }
@@ -298,13 +351,18 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   }
 }
 
-// Merge of the partitions of one (token, head): out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p,
-// over the partitions that hold a visible key, in partition order.
-__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ partials, bf16* __restrict__ out, int out_stride,
-                                                            const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k,
-                                                            int num_seqs, int num_heads, int window, int partition_size,
-                                                            int num_partitions) {
-  const int tok = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+// Merge of the partitions of one (token, head), one wavefront each:
+//   out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p   over the partitions that hold a visible key,
+// added in partition order.  The maxima are fetched by different lanes at once, then every lane
+// walks the partitions for its channels with independent loads.
+__global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ partials, bf16* __restrict__ out, int out_stride,
+                                                             const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k,
+                                                             int num_seqs, int total_q, int num_heads, int window, int partition_size,
+                                                             int num_partitions) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= total_q * num_heads) return;
+  const int tok = item / num_heads, head = item - tok * num_heads;
   int lo = 0, hi = num_seqs - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
@@ -314,13 +372,15 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
   const int qpos = seq_lens_k[lo] - num_q + (tok - q_begin);
   const int first_key = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
   const int p_lo = first_key / partition_size, p_hi = min(qpos / partition_size, num_partitions - 1);
-  const float* base = partials + ((size_t)tok * num_heads + head) * num_partitions * kPartialFloats;
+  const float* base = partials + (size_t)item * num_partitions * kPartialFloats;
   float M = -INFINITY;
-  for (int p = p_lo; p <= p_hi; ++p) M = fmaxf(M, base[(size_t)p * kPartialFloats]);
+  for (int p = p_lo + lane; p <= p_hi; p += 64) M = fmaxf(M, base[(size_t)p * kPartialFloats]);
+  M = wave_max(M);
   float l = 0.f;
   float o[(D + 63) / 64];
 #pragma unroll
   for (int j = 0; j < (D + 63) / 64; ++j) o[j] = 0.f;
+#pragma unroll 4
   for (int p = p_lo; p <= p_hi; ++p) {
     const float* pp = base + (size_t)p * kPartialFloats;
     const float w = fast_exp2(pp[0] - M);
@@ -344,11 +404,13 @@ PLLM_API int pllm_attention_mfma_head_dim() { return D; }
 // LDS floats of the several-wavefront variant.
 static size_t merge_lds_bytes(int ncb, int waves) { return (size_t)(2 * waves * ncb * 16 + waves * ncb * DBLOCKS * 4 * 64) * sizeof(float); }
 
-// partition_size == 0, waves == 1: every work item (one wavefront) walks its whole key range.
-// partition_size == 0, waves in {4, 8, 16}: one work item per (sequence, kv head) whose wavefronts
-//   share the key range and merge through LDS; needs max_q_len * G <= 64 (decoding, tiny portions).
-// partition_size > 0 (a multiple of 64), waves == 1: num_partitions work items per tile write partials
-//   into `partials` (total_q * heads * num_partitions * (D + 2) floats) and a second kernel merges them.
+// waves == 1: every work item is one wavefront that walks its key range.
+// waves in {4, 8, 16}: the wavefronts of a workgroup share the key range of one work item and merge
+//   through LDS; needs max_q_len * G <= 64 (decoding, tiny portions).
+// partition_size == 0: a work item's key range is everything its queries may see; it writes the result.
+// partition_size > 0 (a multiple of 64): num_partitions work items per tile each take one aligned
+//   partition of the keys and write partials into `partials` (total_q * heads * num_partitions *
+//   (D + 2) floats); a second kernel merges them.
 PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
                                        int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                        const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
@@ -364,7 +426,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   const int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
   const int tiles = (max_cols + 16 * ncb - 1) / (16 * ncb);
   if (num_kv_heads * num_partitions > 65535 || num_seqs > 65535) return -2;
-  if (waves != 1 && (partition_size > 0 || tiles != 1 || (waves != 4 && waves != 8 && waves != 16))) return -2;
+  if (waves != 1 && (tiles != 1 || (waves != 4 && waves != 8 && waves != 16))) return -2;
   dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64 * waves);
   const size_t lds = waves > 1 ? merge_lds_bytes(ncb, waves) : 0;
 #define PLLM_LAUNCH(NCB_, WAVES_)                                                                                                    \
@@ -389,8 +451,8 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   int err = (int)hipGetLastError();
   if (err) return err;
   if (partition_size > 0) {
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_q, num_heads), dim3(64), 0, stream, partials, (bf16*)out, out_stride,
-                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, window, partition_size, num_partitions);
+    hipLaunchKernelGGL(attention_merge_kernel, dim3((total_q * num_heads + 3) / 4), dim3(256), 0, stream, partials, (bf16*)out,
+                       out_stride, cu_seqlens_q, seq_lens_k, num_seqs, total_q, num_heads, window, partition_size, num_partitions);
     err = (int)hipGetLastError();
   }
   return err;

@@ -7,9 +7,10 @@
 //   epilogue              plain (bfloat16 or float out) | silu(gate) * up | rotary encoding of q and
 //                         k and the write of k, v into their cache pages
 //
-// One workgroup owns NT tiles of 16 weight rows and all of K.  Its wavefronts deal the K slabs of
-// 128 round-robin; each lane fetches 64 contiguous bytes of a weight row per slab (four 16-byte
-// loads) as the A operand of v_mfma_f32_16x16x32_bf16.  The first slab's weights are requested
+// One workgroup owns units of 16 weight rows over all of K.  Its wavefronts deal the K slabs of
+// 128 round-robin; per slab a lane issues four 16-byte loads of one weight row, laid out so that the
+// four lanes that share a row read 64 contiguous bytes in each load instruction; the loaded pieces
+// are the A operands of v_mfma_f32_16x16x32_bf16 (the rows use the same k assignment).  The first slab's weights are requested
 // before the prologue runs, so the prologue hides behind HBM latency.  The rows (after the norm)
 // sit in LDS and are the B operand of every wavefront.  Partial sums of the wavefronts are added
 // through LDS in wave order: every output is summed in one fixed order.
@@ -38,6 +39,9 @@ struct DecodeLinearParams {
   const int* positions; const float* cos_t; const float* sin_t; const int* slots;
   bf16* k_pages; bf16* v_pages;
   int num_heads, num_kv_heads, head_dim, block_size;
+#ifdef PLLM_TRACE
+  long long* trace;
+#endif
 };
 
 __device__ __forceinline__ bf16x8 zero8() {
@@ -47,51 +51,66 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-template <int NT, int EPI, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p) {
+// One unit of work = 16 weight rows (one MFMA tile) over all of K:
+//   plain        rows 16u .. 16u+15
+//   gated        rows 0-7: gate rows 8u .. 8u+7, rows 8-15: the up rows of the same outputs
+//   rotary/cache rows 0-7: columns j*8 .. j*8+7 of the lower half of a head, rows 8-15: their partners
+//                in the upper half (element i turns with element i + d/2)
+// so that both members of a pair are in one tile and the epilogue finds them in LDS.
+template <int EPI>
+__device__ __forceinline__ int unit_row(const DecodeLinearParams& p, int unit, int r) {
+  if (EPI == EPI_GATED) {
+    const int n = min(unit * 8 + (r & 7), p.N - 1);
+    return r < 8 ? n : n + p.N;                                 // up rows follow the gate rows
+  }
+  if (EPI == EPI_ROPE_KV) {
+    const int half = p.head_dim >> 1, per_head = half >> 3;
+    const int head = unit / per_head, j = unit - head * per_head;
+    return head * p.head_dim + j * 8 + (r & 7) + (r < 8 ? 0 : half);
+  }
+  return min(unit * 16 + r, p.N - 1);
+}
+
+#ifdef PLLM_TRACE
+#define PLLM_STAMP(i) do { if (p.trace && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1)) p.trace[(blockIdx.x ? 16 : 0) + (i)] = wall_clock64(); } while (0)
+#else
+#define PLLM_STAMP(i) do { } while (0)
+#endif
+
+template <int EPI, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p, int num_units) {
+  PLLM_STAMP(0);
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  bf16* xs = reinterpret_cast<bf16*>(lds_raw);                 // [M][K + kPad]
-  float* part = reinterpret_cast<float*>(lds_raw);             // [WAVES][NT * 256], reuses the space after the product
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int r = lane & 15, g = lane >> 4;
   const int M = p.M, N = p.N, K = p.K;
   const int row_len = K + kPad;
+  bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                       // [M][K + kPad]
+  float* part = reinterpret_cast<float*>(lds_raw + (((size_t)M * row_len * 2 + 15) & ~(size_t)15));   // [WAVES][256]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
 
-  // ---- rows of W for this workgroup's tiles
-  const bf16* wrow[NT];
-  int tile_col[NT];                                            // first output column of each tile
-  if (EPI == EPI_GATED) {
-    const int n = min(blockIdx.x * 16 + r, N - 1);
-    wrow[0] = p.W + (size_t)n * p.ldw;
-    wrow[NT - 1] = p.W + (size_t)(n + N) * p.ldw;              // up rows follow the gate rows
-    tile_col[0] = tile_col[NT - 1] = blockIdx.x * 16;
-  } else if (EPI == EPI_ROPE_KV) {
-    const int half = p.head_dim >> 1, per_head = half >> 4;
-    const int head = blockIdx.x / per_head, j = blockIdx.x - head * per_head;
-    tile_col[0] = head * p.head_dim + j * 16;
-    tile_col[NT - 1] = tile_col[0] + half;
-    wrow[0] = p.W + (size_t)(tile_col[0] + r) * p.ldw;
-    wrow[NT - 1] = p.W + (size_t)(tile_col[NT - 1] + r) * p.ldw;
-  } else {
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      tile_col[t] = (blockIdx.x * NT + t) * 16;
-      wrow[t] = p.W + (size_t)min(tile_col[t] + r, N - 1) * p.ldw;
-    }
-  }
-
-  // ---- request the first slab of weights, then build the rows in LDS while it travels
+  // ---- request this wavefront's slabs of the first unit, then build the rows in LDS while they travel
   const int num_slabs = (K + kSlab - 1) / kSlab;
-  bf16x8 wreg[NT][4];
-  auto load_w = [&](int slab, bf16x8 (&dst)[NT][4]) {
+  const int my_slabs = wave < num_slabs ? (num_slabs - wave + WAVES - 1) / WAVES : 0;
+  constexpr int PRE = 3;                                        // slabs in flight per wavefront (registers)
+  bf16x8 wbuf[PRE][4];
+  const bf16* wrow = p.W;
+  auto load_w = [&](int nth, bf16x8 (&dst)[4]) {                // nth slab of this wavefront, from wrow
+    const int slab = wave + nth * WAVES;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kk = slab * kSlab + g * 32 + j * 8;
-#pragma unroll
-      for (int t = 0; t < NT; ++t) dst[t][j] = (kk < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + kk) : zero8();
+      const int kk = slab * kSlab + j * 32 + g * 8;
+      dst[j] = (kk < K) ? *reinterpret_cast<const bf16x8*>(wrow + kk) : zero8();
     }
   };
-  if (wave < num_slabs) load_w(wave, wreg);
+  auto request_unit = [&](int unit) {
+    wrow = p.W + (size_t)unit_row<EPI>(p, unit, r) * p.ldw;
+#pragma unroll
+    for (int s = 0; s < PRE; ++s)
+      if (s < my_slabs) load_w(s, wbuf[s]);
+  };
+  int unit = blockIdx.x;
+  if (unit < num_units) request_unit(unit);
+  PLLM_STAMP(1);
 
   for (int m = wave; m < M; m += WAVES) {
     const size_t src = p.row_index ? (size_t)p.row_index[m] : (size_t)m;
@@ -125,112 +144,113 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
     }
   }
   __syncthreads();
+  PLLM_STAMP(2);
 
-  // ---- product: this wavefront's slabs
-  floatx4 acc[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int slab = wave; slab < num_slabs; slab += WAVES) {
-    bf16x8 wnext[NT][4];
-    const bool more = slab + WAVES < num_slabs;
-    if (more) load_w(slab + WAVES, wnext);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int kk = slab * kSlab + g * 32 + j * 8;
-      const bf16x8 xb = (r < M && kk < K) ? *reinterpret_cast<const bf16x8*>(xs + (size_t)r * row_len + kk) : zero8();
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wreg[t][j], xb, acc[t], 0, 0, 0);
-    }
-    if (more) {
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) wreg[t][j] = wnext[t][j];
-    }
-  }
-  __syncthreads();                                              // everyone is done with the rows: reuse LDS
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) part[(size_t)wave * (NT * 256) + (t * 4 + i) * 64 + lane] = acc[t][i];
-  __syncthreads();
-
-  // ---- epilogue: work item (i, lane) holds output row m = r and tile column g * 4 + i
-  if (tid >= 256) return;
-  const int i = tid >> 6;                                       // lane is tid & 63 again
-  auto total = [&](int t) {
-    float s = 0.f;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) s += part[(size_t)w * (NT * 256) + (t * 4 + i) * 64 + lane];
-    return s;
+  auto x_operand = [&](int nth, int j) {
+    const int kk = (wave + nth * WAVES) * kSlab + j * 32 + g * 8;
+    return (r < M && kk < K) ? *reinterpret_cast<const bf16x8*>(xs + (size_t)r * row_len + kk) : zero8();
   };
-  const int m = r, c = g * 4 + i;
-  if (m >= M) return;
-  if (EPI == EPI_BF16 || EPI == EPI_F32) {
+
+  // ---- units of this workgroup, one after the other; the next unit's weights are requested as
+  //      soon as the current unit's have been consumed, and travel during the reduction
+  for (; unit < num_units; unit += gridDim.x) {
+    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int base = 0; base < my_slabs; base += PRE) {
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int n = tile_col[t] + c;
-      if (n < N) {
-        const float v = total(t);
-        if (EPI == EPI_F32) ((float*)p.out)[(size_t)m * p.ldo + n] = v;
-        else ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(v);
+      for (int s = 0; s < PRE; ++s) {
+        const int nth = base + s;
+        if (nth >= my_slabs) break;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[s][j], x_operand(nth, j), acc, 0, 0, 0);
+        if (nth + PRE < my_slabs) load_w(nth + PRE, wbuf[s]);   // keep PRE slabs in flight
       }
     }
-  } else if (EPI == EPI_GATED) {
-    const int n = tile_col[0] + c;
-    if (n < N) {
-      const float gate = total(0), up = total(NT - 1);
-      ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16((gate / (1.f + expf(-gate))) * up);
-    }
-  } else {  // EPI_ROPE_KV
-    const int d = p.head_dim, half = d >> 1;
-    const int head = tile_col[0] / d, ri = tile_col[0] - head * d + c;          // rotation index in [0, half)
-    float lo = total(0), hi = total(NT - 1);
-    const int nh = p.num_heads, nkv = p.num_kv_heads;
-    if (head < nh + nkv) {
-      // q and k are rounded to bfloat16 by the projection before they are rotated
-      lo = __bfloat162float(__float2bfloat16(lo));
-      hi = __bfloat162float(__float2bfloat16(hi));
-      float cs = 1.f, sn = 0.f;
-      if (p.cos_t) {
-        const int pos = p.positions[m];
-        cs = p.cos_t[(size_t)pos * half + ri];
-        sn = p.sin_t[(size_t)pos * half + ri];
-      }
-      const bf16 out_lo = __float2bfloat16(lo * cs - hi * sn), out_hi = __float2bfloat16(hi * cs + lo * sn);
-      if (head < nh) {
-        bf16* q = (bf16*)p.out + (size_t)m * p.ldo + (size_t)head * d;
-        q[ri] = out_lo;
-        q[ri + half] = out_hi;
-      } else {
-        const int slot = p.slots[m];
-        if (slot >= 0) {
-          const int page = slot / p.block_size, off = slot - page * p.block_size;
-          bf16* k = p.k_pages + (((size_t)page * nkv + (head - nh)) * p.block_size + off) * d;
-          k[ri] = out_lo;
-          k[ri + half] = out_hi;
+    PLLM_STAMP(3);
+    const int next = unit + gridDim.x;
+    if (next < num_units) request_unit(next);
+
+    // acc[i] = element (tile row g*4 + i, input row r); add the wavefronts in wave order
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave * 256 + i * 64 + lane] = acc[i];
+    __syncthreads();
+    if (tid < 256) {
+      const int i = tid >> 6;                                   // lane is tid & 63 again
+      auto total = [&](int ln) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) s += part[w * 256 + i * 64 + ln];
+        return s;
+      };
+      const int m = r, row = g * 4 + i;                         // row of the tile
+      if (m < M) {
+        if (EPI == EPI_BF16 || EPI == EPI_F32) {
+          const int n = unit * 16 + row;
+          if (n < N) {
+            const float v = total(lane);
+            if (EPI == EPI_F32) ((float*)p.out)[(size_t)m * p.ldo + n] = v;
+            else ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(v);
+          }
+        } else if (EPI == EPI_GATED) {
+          const int n = unit * 8 + row;
+          if (row < 8 && n < N) {
+            const float gate = total(lane), up = total(lane + 32);    // same outputs, 8 tile rows further
+            ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16((gate / (1.f + expf(-gate))) * up);
+          }
+        } else if (row < 8) {  // EPI_ROPE_KV
+          const int d = p.head_dim, half = d >> 1, per_head = half >> 3;
+          const int head = unit / per_head, ri = (unit - head * per_head) * 8 + row;   // rotation index in [0, half)
+          float lo = total(lane), hi = total(lane + 32);
+          const int nh = p.num_heads, nkv = p.num_kv_heads;
+          if (head < nh + nkv) {
+            // q and k are rounded to bfloat16 by the projection before they are rotated
+            lo = __bfloat162float(__float2bfloat16(lo));
+            hi = __bfloat162float(__float2bfloat16(hi));
+            float cs = 1.f, sn = 0.f;
+            if (p.cos_t) {
+              const int pos = p.positions[m];
+              cs = p.cos_t[(size_t)pos * half + ri];
+              sn = p.sin_t[(size_t)pos * half + ri];
+            }
+            const bf16 out_lo = __float2bfloat16(lo * cs - hi * sn), out_hi = __float2bfloat16(hi * cs + lo * sn);
+            if (head < nh) {
+              bf16* q = (bf16*)p.out + (size_t)m * p.ldo + (size_t)head * d;
+              q[ri] = out_lo;
+              q[ri + half] = out_hi;
+            } else {
+              const int slot = p.slots[m];
+              if (slot >= 0) {
+                const int page = slot / p.block_size, off = slot - page * p.block_size;
+                bf16* k = p.k_pages + (((size_t)page * nkv + (head - nh)) * p.block_size + off) * d;
+                k[ri] = out_lo;
+                k[ri + half] = out_hi;
+              }
+            }
+          } else {
+            const int slot = p.slots[m];
+            if (slot >= 0) {
+              const int page = slot / p.block_size, off = slot - page * p.block_size;
+              bf16* v = p.v_pages + ((size_t)page * nkv + (head - nh - nkv)) * d * p.block_size + off;
+              v[(size_t)ri * p.block_size] = __float2bfloat16(lo);
+              v[(size_t)(ri + half) * p.block_size] = __float2bfloat16(hi);
+            }
+          }
         }
       }
-    } else {
-      const int slot = p.slots[m];
-      if (slot >= 0) {
-        const int page = slot / p.block_size, off = slot - page * p.block_size;
-        bf16* v = p.v_pages + ((size_t)page * nkv + (head - nh - nkv)) * d * p.block_size + off;
-        v[(size_t)ri * p.block_size] = __float2bfloat16(lo);
-        v[(size_t)(ri + half) * p.block_size] = __float2bfloat16(hi);
-      }
     }
+    __syncthreads();                                            // the partial sums are read: the buffer may be reused
+    PLLM_STAMP(4);
   }
 }
 
-template <int NT, int EPI, int WAVES>
-static int launch(const DecodeLinearParams& p, int blocks, size_t lds, hipStream_t stream) {
-  auto kernel = decode_linear_kernel<NT, EPI, WAVES>;
+template <int EPI, int WAVES>
+static int launch(const DecodeLinearParams& p, int units, int blocks, size_t lds, hipStream_t stream) {
+  auto kernel = decode_linear_kernel<EPI, WAVES>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WAVES * 64), lds, stream, p);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(WAVES * 64), lds, stream, p, units);
   return (int)hipGetLastError();
 }
 
@@ -244,9 +264,24 @@ PLLM_API long pllm_max_lds_bytes() {
 
 // Bytes of LDS a call needs; the caller checks them against the device's limit.
 PLLM_API long pllm_decode_linear_lds_bytes(int M, int K, int waves) {
-  const long rows = (long)M * (K + kPad) * 2;
-  const long reduce = (long)waves * 2 * 256 * 4;
-  return rows > reduce ? rows : reduce;
+  const long rows = (((long)M * (K + kPad) * 2) + 15) & ~15L;
+  return rows + (long)waves * 256 * 4;
+}
+
+#ifdef PLLM_TRACE
+static long long* pllm_trace_buffer = nullptr;
+PLLM_API void pllm_set_trace(long long* buf) { pllm_trace_buffer = buf; }
+#endif
+
+static int num_compute_units() {
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
 }
 
 PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* delta, int ldd, const float* norm_w, float eps,
@@ -262,19 +297,32 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   p.M = M; p.N = N; p.K = K; p.positions = positions; p.cos_t = cos_t; p.sin_t = sin_t; p.slots = slots;
   p.k_pages = (bf16*)k_pages; p.v_pages = (bf16*)v_pages; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads;
   p.head_dim = head_dim; p.block_size = block_size;
+#ifdef PLLM_TRACE
+  p.trace = pllm_trace_buffer;
+#endif
   const int waves = (K >= 4096) ? 16 : 8;
   const size_t lds = (size_t)pllm_decode_linear_lds_bytes(M, K, waves);
-  const int tiles = (N + 15) / 16;
-#define GO(NT_, EPI_, BLOCKS_)                                                        \
-  return waves == 16 ? launch<NT_, EPI_, 16>(p, BLOCKS_, lds, stream) : launch<NT_, EPI_, 8>(p, BLOCKS_, lds, stream)
+  int units;
   switch (epi) {
-    case EPI_BF16: GO(1, EPI_BF16, tiles);
-    case EPI_F32: GO(1, EPI_F32, tiles);
-    case EPI_GATED: GO(2, EPI_GATED, tiles);
-    case EPI_ROPE_KV: {
-      if (head_dim % 32 || (!slots) || !k_pages || !v_pages || N != (num_heads + 2 * num_kv_heads) * head_dim) return -2;
-      GO(2, EPI_ROPE_KV, (num_heads + 2 * num_kv_heads) * (head_dim / 32));
-    }
+    case EPI_BF16: case EPI_F32: units = (N + 15) / 16; break;
+    case EPI_GATED: units = (N + 7) / 8; break;
+    case EPI_ROPE_KV:
+      if (head_dim % 16 || !slots || !k_pages || !v_pages || N != (num_heads + 2 * num_kv_heads) * head_dim) return -2;
+      units = (num_heads + 2 * num_kv_heads) * (head_dim / 16);
+      break;
+    default: return -3;
+  }
+  // Up to two workgroups per compute unit stay resident; more units than that are dealt evenly
+  // to that many workgroups, which walk them with the next unit's weights already on their way.
+  const int resident = 2 * num_compute_units();
+  const int per_block = (units + resident - 1) / resident;
+  const int blocks = (units + per_block - 1) / per_block;
+#define GO(EPI_) return waves == 16 ? launch<EPI_, 16>(p, units, blocks, lds, stream) : launch<EPI_, 8>(p, units, blocks, lds, stream)
+  switch (epi) {
+    case EPI_BF16: GO(EPI_BF16);
+    case EPI_F32: GO(EPI_F32);
+    case EPI_GATED: GO(EPI_GATED);
+    case EPI_ROPE_KV: GO(EPI_ROPE_KV);
   }
 #undef GO
   return -3;

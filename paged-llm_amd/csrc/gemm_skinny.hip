@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
     bf16x8 wreg[NT][4], xreg[MT][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kk = ks + g * 32 + j * 8;
+      const int kk = ks + j * 32 + g * 8;
       const bool in_k = kk < K;                               // K is a multiple of 8: whole chunks only
 #pragma unroll
       for (int t = 0; t < NT; ++t) wreg[t][j] = in_k ? load8(wrow[t] + kk) : zero8();

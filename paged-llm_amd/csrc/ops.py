@@ -296,7 +296,7 @@ def decode_linear_takes(rows: int, K: int, x: torch.Tensor, w: torch.Tensor) -> 
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return False
     waves = 16 if K >= 4096 else 8
-    need = max(rows * (K + 8) * 2, waves * 2 * 256 * 4)
+    need = ((rows * (K + 8) * 2 + 15) // 16) * 16 + waves * 256 * 4
     return need <= _max_lds_bytes(x.device)
 
 
@@ -333,7 +333,7 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
         out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     elif epi == EPI_ROPE_KV:
         nh, nkv, d, bs = r["num_heads"], r["num_kv_heads"], r["head_dim"], r["block_size"]
-        _need(d % 32 == 0 and N == (nh + 2 * nkv) * d, "fused rotary epilogue needs head sizes in multiples of 32 and [q; k; v] rows")
+        _need(d % 16 == 0 and N == (nh + 2 * nkv) * d, "fused rotary epilogue needs head sizes in multiples of 16 and [q; k; v] rows")
         kp, vp = r["k_pages"], r["v_pages"]
         P = kp.shape[0]
         _need(tuple(kp.shape) == (P, nkv, bs, d) and tuple(vp.shape) == (P, nkv, d, bs) and kp.is_contiguous() and vp.is_contiguous()
@@ -452,30 +452,28 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
     """(wavefronts per work item, partition_size, num_partitions) for a step.
 
     Prompt portions have many query tiles: one wavefront per tile walks all its keys (1, 0, 1).
-    Decoding has one tile per (sequence, kv head): its keys are shared between the wavefronts of a
-    workgroup, which merge in LDS (w, 0, 1); only when the sequences are few and very long are the
-    keys also split between workgroups, merged by a second kernel (1, size, parts)."""
+    Decoding has one tile per (sequence, kv head), far too few to fill the GPU: the keys are cut
+    into aligned partitions, one workgroup each (merged by a second kernel), and inside a
+    workgroup the wavefronts share the partition's blocks of 64 keys (merged in LDS)."""
     cols = max_q_len * group
-    if cols > 64:
+    if cols > 64 or max_k_len <= 64:
+        return 1, 0, 1
+    ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
+    max_waves = 8
+    while max_waves >= 4 and (2 * max_waves * ncb * 16 + max_waves * ncb * (head_dim // 16) * 4 * 64) * 4 > lds_limit:
+        max_waves //= 2
+    if max_waves < 4:
         return 1, 0, 1
     items = num_seqs * num_kv_heads
-    if items < 64 and max_k_len > 16384:
-        want = max(1, 512 // items)
-        size = 64
-        while (max_k_len + size - 1) // size > want:
-            size *= 2
-        parts = (max_k_len + size - 1) // size
-        if parts > 1:
-            return 1, size, parts
-    ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
-    waves = 16
-    while waves >= 4 and (2 * waves * ncb * 16 + waves * ncb * (head_dim // 16) * 4 * 64) * 4 > lds_limit:
+    want_parts = max(1, 384 // items)
+    size = 256                                        # at least four blocks of 64 keys per workgroup
+    while (max_k_len + size - 1) // size > want_parts:
+        size *= 2
+    parts = (max_k_len + size - 1) // size
+    waves = max_waves
+    while waves > 4 and (waves // 2) * 64 >= min(size, max_k_len):
         waves //= 2
-    if waves < 4 or max_k_len <= 64:
-        return 1, 0, 1
-    while waves > 4 and (waves // 2) * 64 >= max_k_len:
-        waves //= 2
-    return waves, 0, 1
+    return (waves, size, parts) if parts > 1 else (waves, 0, 1)
 
 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
@@ -497,8 +495,8 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     _need(out.shape == (T, num_heads * head_dim) and out.stride(1) == 1 and out.dtype == q.dtype and out.stride(0) % 4 == 0,
           "bad attention output")
     _need(max_q_len >= 1 and partition_size % 64 == 0 and waves in (1, 4, 8, 16), "bad launch parameters")
-    _need(waves == 1 or (partition_size == 0 and max_q_len * (num_heads // num_kv_heads) <= 64),
-          "several wavefronts per work item need at most 64 (query, head) columns per kv head and no partitions")
+    _need(waves == 1 or max_q_len * (num_heads // num_kv_heads) <= 64,
+          "several wavefronts per work item need at most 64 (query, head) columns per kv head")
     ws = None
     if partition_size > 0:
         floats = T * num_heads * num_partitions * (head_dim + 2)

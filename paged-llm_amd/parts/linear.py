@@ -62,7 +62,7 @@ def qkv_rotary_cache(x, w_qkv: torch.Tensor, positions: torch.Tensor, cos, sin, 
     Returns q as rows of a matrix whose first num_heads * head_dim columns hold the rotated heads
     (the row stride may be larger).  With k_pages None only q is projected and rotated."""
     write = k_pages is not None
-    if write and w_qkv.dtype == torch.bfloat16 and head_dim % 32 == 0:
+    if write and w_qkv.dtype == torch.bfloat16 and head_dim % 16 == 0:
         rope = dict(positions=positions, cos=cos, sin=sin, slots=slot_mapping, k_pages=k_pages, v_pages=v_pages,
                     num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size)
         q = _fused(x, w_qkv, ops.EPI_ROPE_KV, rope)

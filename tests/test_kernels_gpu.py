@@ -356,9 +356,13 @@ def test_paged_attention_mfma(heads, kv_heads, d, bs, lens, num_q):
         parts = (max(lens) + size - 1) // size
         assert rel_err(ops().paged_attention_mfma(*args, size, parts), want) <= 1.6e-2, f"partition {size}"
     if max(num_q) * (heads // kv_heads) <= 64:
+        cols = max(num_q) * (heads // kv_heads)
+        ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
         for waves in (4, 8, 16):
-            if ops().attention_plan(1, 1, max(num_q), 10 ** 5, heads // kv_heads, d, 160 * 1024)[0] >= waves:
+            if (2 * waves * ncb * 16 + waves * ncb * (d // 16) * 4 * 64) * 4 <= 160 * 1024:
                 assert rel_err(ops().paged_attention_mfma(*args, 0, 1, waves), want) <= 1.6e-2, f"{waves} wavefronts"
+                parts = (max(lens) + 255) // 256
+                assert rel_err(ops().paged_attention_mfma(*args, 256, parts, waves), want) <= 1.6e-2, f"{waves} wavefronts, partitions"
 
 
 @pytest.mark.parametrize("window", [1, 5, 64, 100])
@@ -392,7 +396,7 @@ def test_mfma_attention_ignores_table_padding_and_stale_slots():
     vp2[tables[1, 0], :, :, 5:] = float("nan")
     kp2[tables[0, 1], :, 4:, :] = float("inf")
     vp2[tables[0, 1], :, :, 4:] = float("nan")
-    for split in ((), (64, 2), (0, 1, 4)):
+    for split in ((), (64, 2), (0, 1, 4), (64, 2, 4)):
         assert torch.equal(run(kp, vp, tables, *split), run(kp2, vp2, t2, *split))
 
 
@@ -402,7 +406,7 @@ def test_mfma_attention_one_far_key_stands_out(far):
     q, kp, vp, tables, cu, sl = paged_case([700], [1], heads, kv_heads, d, bs, torch.bfloat16, seed=4)
     page, off = int(tables[0, far // bs]), far % bs
     kp[page, 0, off, :] = (q[0, 5 * d:6 * d].float() * 40).to(torch.bfloat16)       # head 5 looks at that key only
-    for split in ((), (128, 6), (0, 1, 16)):
+    for split in ((), (128, 6), (0, 1, 16), (256, 3, 4)):
         got = ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
                                          d, 1.0, 0, 1, *split).cpu().float()
         assert torch.allclose(got[0, 5 * d:6 * d], vp[page, 0, :, off].float(), atol=2e-2)
@@ -411,12 +415,13 @@ def test_mfma_attention_one_far_key_stands_out(far):
 def test_attention_plan():
     plan = ops().attention_plan
     lds = 160 * 1024
-    assert plan(8, 4, 1, 2048, 8, 64, lds) == (16, 0, 1)        # decoding: the wavefronts of a workgroup share the keys
+    assert plan(8, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)       # decoding: partitions for workgroups, blocks for wavefronts
+    assert plan(64, 4, 1, 2048, 8, 64, lds) == (8, 0, 1)         # enough sequences: wavefronts only
+    assert plan(1, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)
     assert plan(8, 4, 1, 200, 8, 64, lds) == (4, 0, 1)
     assert plan(1, 4, 2048, 2048, 8, 64, lds) == (1, 0, 1)      # a long prompt portion: one wavefront per query tile
     assert plan(2, 4, 1, 50, 8, 64, lds) == (1, 0, 1)
-    assert plan(1, 8, 1, 100000, 4, 128, lds) == (1, 2048, 49)  # one very long sequence: keys split between workgroups too
-    assert plan(8, 1, 1, 4096, 8, 256, lds) == (8, 0, 1)        # wide heads: fewer wavefronts fit LDS
+    assert plan(1, 8, 1, 100000, 4, 128, lds) == (8, 4096, 25)
 
 
 # ----------------------------------------------------------------------------------- fused decode products
@@ -466,7 +471,7 @@ def test_decode_linear_gated(m, inter, k):
     assert rel_err(o.decode_linear(x.cuda(), w.cuda(), o.EPI_GATED), want) <= 1e-2
 
 
-@pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 32, 16), (32, 4, 64, 16), (3, 1, 96, 32), (8, 8, 128, 16)])
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 32, 16), (32, 4, 64, 16), (3, 1, 96, 32), (8, 8, 128, 16), (5, 1, 48, 16), (2, 2, 16, 8)])
 @pytest.mark.parametrize("m", [1, 7, 16])
 def test_decode_linear_rotary_and_cache_write(heads, kv_heads, d, bs, m):
     from paged_llm_amd.parts.registry import BuildEnv
