@@ -124,6 +124,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (reported as such)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="time only the 2048-token prefill (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -141,6 +142,11 @@ def main() -> int:
 
     with tempfile.TemporaryDirectory() as folder:
         engine = make_engine(cfg, folder, args.dtype, max(64, args.batch), args.context)
+        if args.prefill_only:
+            psec = time_prefill(engine, PREFILL_TOKENS, seed=100)
+            print(json.dumps({"prefill_ms": round(psec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / psec, 1),
+                              "frac": round(prefill_flops(cfg, PREFILL_TOKENS, 1) / psec / PEAK_FLOPS[short], 4)}))
+            return 0
         sec = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
         value = args.batch / sec
         decode_bytes = numbers["weight_bytes"] + args.batch * args.context * numbers["kv_bytes_per_token"]

@@ -401,12 +401,22 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
 
 PLLM_API int pllm_attention_mfma_head_dim() { return D; }
 
+static long pllm_max_lds() {
+  static long cached = 0;
+  if (!cached) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess) cached = v;
+    if (cached <= 0) cached = 64 * 1024;
+  }
+  return cached;
+}
+
 // LDS floats of the several-wavefront variant.
 static size_t merge_lds_bytes(int ncb, int waves) { return (size_t)(2 * waves * ncb * 16 + waves * ncb * DBLOCKS * 4 * 64) * sizeof(float); }
 
 // waves == 1: every work item is one wavefront that walks its key range.
-// waves in {4, 8, 16}: the wavefronts of a workgroup share the key range of one work item and merge
-//   through LDS; needs max_q_len * G <= 64 (decoding, tiny portions).
+// waves in {4, 8, 16}: the wavefronts of a workgroup share the key range of one work item (they take
+//   its blocks of 64 keys in turn, with the next block already requested) and merge through LDS.
 // partition_size == 0: a work item's key range is everything its queries may see; it writes the result.
 // partition_size > 0 (a multiple of 64): num_partitions work items per tile each take one aligned
 //   partition of the keys and write partials into `partials` (total_q * heads * num_partitions *
@@ -415,7 +425,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
                                        int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                        const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                                        int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                       int num_partitions, float* partials, int waves, hipStream_t stream) {
+                                       int num_partitions, float* partials, int waves, int column_blocks, hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
   const int G = num_heads / num_kv_heads;
@@ -423,10 +433,14 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   if (partition_size < 0 || (partition_size & 63) || (partition_size > 0 && (!partials || num_partitions < 1))) return -2;
   if (partition_size == 0) num_partitions = 1;
   const int max_cols = max_q_len * G;
-  const int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
+  // column_blocks (1, 2 or 4 blocks of 16 columns per work item; 0 = as many as the columns need, up to 4)
+  int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
+  if (column_blocks == 1 || column_blocks == 2 || column_blocks == 4) ncb = column_blocks < ncb ? column_blocks : ncb;
+  else if (column_blocks != 0) return -2;
   const int tiles = (max_cols + 16 * ncb - 1) / (16 * ncb);
   if (num_kv_heads * num_partitions > 65535 || num_seqs > 65535) return -2;
-  if (waves != 1 && (tiles != 1 || (waves != 4 && waves != 8 && waves != 16))) return -2;
+  if (waves != 1 && waves != 4 && waves != 8 && waves != 16) return -2;
+  if (waves > 1 && (long)merge_lds_bytes(ncb, waves) > pllm_max_lds()) return -2;
   dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64 * waves);
   const size_t lds = waves > 1 ? merge_lds_bytes(ncb, waves) : 0;
 #define PLLM_LAUNCH(NCB_, WAVES_)                                                                                                    \

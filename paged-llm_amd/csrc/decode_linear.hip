@@ -91,7 +91,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   // ---- request this wavefront's slabs of the first unit, then build the rows in LDS while they travel
   const int num_slabs = (K + kSlab - 1) / kSlab;
   const int my_slabs = wave < num_slabs ? (num_slabs - wave + WAVES - 1) / WAVES : 0;
-  constexpr int PRE = 3;                                        // slabs in flight per wavefront (registers)
+  constexpr int PRE = WAVES >= 16 ? 3 : 2;                      // slabs in flight per wavefront (registers)
   bf16x8 wbuf[PRE][4];
   const bf16* wrow = p.W;
   auto load_w = [&](int nth, bf16x8 (&dst)[4]) {                // nth slab of this wavefront, from wrow

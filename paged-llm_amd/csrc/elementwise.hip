@@ -16,7 +16,14 @@ __global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __rest
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range; never fault
   const T* src = table + (size_t)id * hidden;
   T* dst = out + (size_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  constexpr int V = 16 / sizeof(T);                              // elements per 16-byte piece
+  if (hidden % V == 0 && ((uintptr_t)table % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+    const uint4* s4 = reinterpret_cast<const uint4*>(src);
+    uint4* d4 = reinterpret_cast<uint4*>(dst);
+    for (int i = threadIdx.x; i < hidden / V; i += blockDim.x) d4[i] = s4[i];
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  }
 }
 
 PLLM_API int pllm_embed_gather(int dtype, const int* ids, const void* table, void* out, int num_tokens,
@@ -45,20 +52,51 @@ __global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const in
   const int r = blockIdx.x;
   const size_t src = row_index ? (size_t)row_index[r] : (size_t)r;
   const T* xr = x + src * hidden;
+  T* o = out + (size_t)r * hidden;
+  constexpr int V = 16 / sizeof(T);                              // elements per 16-byte piece
+  struct alignas(16) Piece { T v[V]; };
+  const bool wide = hidden % V == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                    (!delta || ((uintptr_t)delta % 16) == 0) && (!x_out || ((uintptr_t)x_out % 16) == 0);
   float acc = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    float v = to_f32(xr[i]);
-    if (delta) {
-      v = to_f32(from_f32<T>(v + to_f32(delta[src * hidden + i])));
-      if (x_out) x_out[src * hidden + i] = from_f32<T>(v);
+  if (wide) {
+    for (int c = threadIdx.x; c < hidden / V; c += blockDim.x) {
+      Piece px = reinterpret_cast<const Piece*>(xr)[c];
+      if (delta) {
+        const Piece pd = reinterpret_cast<const Piece*>(delta + src * hidden)[c];
+#pragma unroll
+        for (int j = 0; j < V; ++j) px.v[j] = from_f32<T>(to_f32(px.v[j]) + to_f32(pd.v[j]));
+        if (x_out) reinterpret_cast<Piece*>(x_out + src * hidden)[c] = px;
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const float v = to_f32(px.v[j]);
+        row[c * V + j] = v;
+        acc += v * v;
+      }
     }
-    row[i] = v;
-    acc += v * v;
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      float v = to_f32(xr[i]);
+      if (delta) {
+        v = to_f32(from_f32<T>(v + to_f32(delta[src * hidden + i])));
+        if (x_out) x_out[src * hidden + i] = from_f32<T>(v);
+      }
+      row[i] = v;
+      acc += v * v;
+    }
   }
   const float total = block_sum(acc, scratch);
   const float inv = rsqrtf(total / (float)hidden + eps);
-  T* o = out + (size_t)r * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_f32<T>((row[i] * inv) * w[i]);
+  if (wide) {
+    for (int c = threadIdx.x; c < hidden / V; c += blockDim.x) {
+      Piece po;
+#pragma unroll
+      for (int j = 0; j < V; ++j) po.v[j] = from_f32<T>((row[c * V + j] * inv) * w[c * V + j]);
+      reinterpret_cast<Piece*>(o)[c] = po;
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_f32<T>((row[i] * inv) * w[i]);
+  }
 }
 
 PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int* row_index, const float* w, float eps,
@@ -78,25 +116,39 @@ PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int
 
 // ---------------------------------------------------------------------------------------------
 // Gated activation: out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z / (1 + exp(-z)).
-template <typename T>
+template <typename T, int V>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
-  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // Each thread handles V consecutive outputs of one row (V = 1, or a 16-byte piece).
+  struct alignas(sizeof(T) * V) Piece { T v[V]; };
+  const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   if (idx >= total) return;
   const size_t t = idx / inter;
   const int i = (int)(idx - t * inter);
-  const float g = to_f32(gu[t * 2 * inter + i]);
-  const float u = to_f32(gu[t * 2 * inter + inter + i]);
-  out[idx] = from_f32<T>((g / (1.f + expf(-g))) * u);
+  const Piece pg = *reinterpret_cast<const Piece*>(gu + t * 2 * inter + i);
+  const Piece pu = *reinterpret_cast<const Piece*>(gu + t * 2 * inter + inter + i);
+  Piece po;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const float g = to_f32(pg.v[j]), u = to_f32(pu.v[j]);
+    po.v[j] = from_f32<T>((g / (1.f + expf(-g))) * u);
+  }
+  *reinterpret_cast<Piece*>(out + idx) = po;
 }
 
 PLLM_API int pllm_silu_mul(int dtype, const void* gate_up, void* out, int num_tokens, int inter, hipStream_t stream) {
   const size_t total = (size_t)num_tokens * inter;
   if (total == 0) return 0;
-  dim3 block(256), grid((unsigned)((total + 255) / 256));
-  if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total);
-  else
-    hipLaunchKernelGGL(silu_mul_kernel<bf16>, grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total);
+  const int elem = dtype == PLLM_F32 ? 4 : 2, wide = 16 / elem;
+  const bool vec = inter % wide == 0 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const size_t items = vec ? total / wide : total;
+  dim3 block(256), grid((unsigned)((items + 255) / 256));
+  if (dtype == PLLM_F32) {
+    if (vec) hipLaunchKernelGGL((silu_mul_kernel<float, 4>), grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total);
+    else hipLaunchKernelGGL((silu_mul_kernel<float, 1>), grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total);
+  } else {
+    if (vec) hipLaunchKernelGGL((silu_mul_kernel<bf16, 8>), grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total);
+    else hipLaunchKernelGGL((silu_mul_kernel<bf16, 1>), grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total);
+  }
   PLLM_RETURN_LAST_ERROR();
 }
 
@@ -124,21 +176,48 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
   const int off = slot >= 0 ? slot - page * block_size : 0;
 
   const int rot_heads = write_kv ? num_heads + num_kv_heads : num_heads;
-  for (int w = threadIdx.x; w < rot_heads * half; w += blockDim.x) {
-    const int head = w / half, i = w - head * half;
-    T* h = row + (size_t)head * head_dim;
-    const float lo = to_f32(h[i]), hi = to_f32(h[i + half]);
-    const float c = cs ? cs[i] : 1.f, s = sn ? sn[i] : 0.f;
-    const T out_lo = from_f32<T>(lo * c - hi * s);
-    const T out_hi = from_f32<T>(hi * c + lo * s);
-    if (head < num_heads) {
-      h[i] = out_lo;
-      h[i + half] = out_hi;
-    } else if (slot >= 0) {
-      const int kvh = head - num_heads;
-      T* dst = k_pages + (((size_t)page * num_kv_heads + kvh) * block_size + off) * head_dim;
-      dst[i] = out_lo;
-      dst[i + half] = out_hi;
+  struct alignas(16) Piece { T v[8]; };
+  const bool wide = (half % 8 == 0) && ((uintptr_t)qkv % 16) == 0 && (row_stride % 8 == 0) && ((uintptr_t)k_pages % 16) == 0;
+  if (wide) {
+    // 8 pairs per work item: 16-byte pieces of the lower and the upper half of a head
+    const int per_head = half / 8;
+    for (int w = threadIdx.x; w < rot_heads * per_head; w += blockDim.x) {
+      const int head = w / per_head, i = (w - head * per_head) * 8;
+      T* h = row + (size_t)head * head_dim;
+      const Piece lo = *reinterpret_cast<const Piece*>(h + i), hi = *reinterpret_cast<const Piece*>(h + i + half);
+      Piece out_lo, out_hi;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float c = cs ? cs[i + j] : 1.f, s = sn ? sn[i + j] : 0.f;
+        const float l = to_f32(lo.v[j]), u = to_f32(hi.v[j]);
+        out_lo.v[j] = from_f32<T>(l * c - u * s);
+        out_hi.v[j] = from_f32<T>(u * c + l * s);
+      }
+      T* dst = nullptr;
+      if (head < num_heads) dst = h;
+      else if (slot >= 0) dst = k_pages + (((size_t)page * num_kv_heads + (head - num_heads)) * block_size + off) * head_dim;
+      if (dst) {
+        *reinterpret_cast<Piece*>(dst + i) = out_lo;
+        *reinterpret_cast<Piece*>(dst + i + half) = out_hi;
+      }
+    }
+  } else {
+    for (int w = threadIdx.x; w < rot_heads * half; w += blockDim.x) {
+      const int head = w / half, i = w - head * half;
+      T* h = row + (size_t)head * head_dim;
+      const float lo = to_f32(h[i]), hi = to_f32(h[i + half]);
+      const float c = cs ? cs[i] : 1.f, s = sn ? sn[i] : 0.f;
+      const T out_lo = from_f32<T>(lo * c - hi * s);
+      const T out_hi = from_f32<T>(hi * c + lo * s);
+      if (head < num_heads) {
+        h[i] = out_lo;
+        h[i + half] = out_hi;
+      } else if (slot >= 0) {
+        const int kvh = head - num_heads;
+        T* dst = k_pages + (((size_t)page * num_kv_heads + kvh) * block_size + off) * head_dim;
+        dst[i] = out_lo;
+        dst[i + half] = out_hi;
+      }
     }
   }
   if (slot >= 0) {

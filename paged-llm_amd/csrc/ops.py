@@ -438,7 +438,7 @@ def gemm_large_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
+             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p]
 _attn_scratch: dict = {}
 
 
@@ -479,7 +479,8 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
                          cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
                          head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
-                         num_partitions: int = 1, waves: int = 1, out: torch.Tensor | None = None) -> torch.Tensor:
+                         num_partitions: int = 1, waves: int = 1, column_blocks: int = 0,
+                         out: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
     work item into aligned partitions that a second kernel merges; ``waves`` > 1 shares the keys
@@ -495,8 +496,10 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     _need(out.shape == (T, num_heads * head_dim) and out.stride(1) == 1 and out.dtype == q.dtype and out.stride(0) % 4 == 0,
           "bad attention output")
     _need(max_q_len >= 1 and partition_size % 64 == 0 and waves in (1, 4, 8, 16), "bad launch parameters")
-    _need(waves == 1 or max_q_len * (num_heads // num_kv_heads) <= 64,
-          "several wavefronts per work item need at most 64 (query, head) columns per kv head")
+    ncb = min(column_blocks or 4, 1 if max_q_len * (num_heads // num_kv_heads) <= 16 else (2 if max_q_len * (num_heads // num_kv_heads) <= 32 else 4))
+    _need(column_blocks in (0, 1, 2, 4), "column_blocks is 0 (automatic), 1, 2 or 4")
+    _need(waves == 1 or (2 * waves * ncb * 16 + waves * ncb * (head_dim // 16) * 4 * 64) * 4 <= _max_lds_bytes(q.device),
+          "the merge buffers of that many wavefronts do not fit LDS")
     ws = None
     if partition_size > 0:
         floats = T * num_heads * num_partitions * (head_dim + 2)
@@ -508,7 +511,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
     _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
              block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
-             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), _stream()),
+             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), _stream()),
            "paged_attention_mfma")
     return out
 
@@ -521,7 +524,9 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
     if mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
         waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, num_heads // num_kv_heads,
                                             head_dim, _max_lds_bytes(q.device))
+        # Prompt portions: 32 columns per wavefront leave registers for two wavefronts per SIMD
+        # (measured faster than 64 columns at one).
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
-                                    head_dim, scale, window, ctx.max_q_len, size, parts, waves)
+                                    head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window)
