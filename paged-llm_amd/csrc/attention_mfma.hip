@@ -351,6 +351,267 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Prompt portions: one workgroup of four wavefronts per (sequence, kv head, 128 columns).  All four
+// walk the same blocks of 64 keys, each for its own 32 columns, so the block is fetched once into
+// LDS (each wavefront fetches the 16 keys and values of one tile: one page lookup, uniform in the
+// wavefront) and the next block travels while the current one is used: global -> registers while
+// computing, registers -> the other LDS buffer, one barrier per block.
+//
+// LDS layouts: keys [64 rows][D + 8] (row = key), values [D rows][64 + 8] (row = channel) with the
+// keys of each half of 32 stored in operand order (lane group g, tile h, key i -> g*8 + h*4 + i), so
+// that both A operands are single 16-byte reads and rows that differ by one land 36 banks apart.
+constexpr int kKRow = D + 8;                 // elements per key row in LDS
+constexpr int kVRow = 64 + 8;                // elements per channel row in LDS
+constexpr int kKChunks = 16 * D / 8;         // 16-byte pieces of one tile of keys (16 rows of D)
+constexpr int kVChunks = 2 * D;              // 16-byte pieces of one tile of values (D channels x 2 halves of 8 keys)
+constexpr int kKPerLane = (kKChunks + 63) / 64;
+constexpr int kVPerLane = (kVChunks + 63) / 64;
+
+struct MaskedTag { static constexpr bool value = true; };
+struct PlainTag { static constexpr bool value = false; };
+
+template <int NCB>
+__global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
+    int block_size, float scale, int window, int paired) {
+  __shared__ __attribute__((aligned(16))) bf16 k_s[2][64 * kKRow];
+  __shared__ __attribute__((aligned(16))) bf16 v_s[2][D * kVRow];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const int seq = blockIdx.z, kvh = blockIdx.y;
+  const int G = num_heads / num_kv_heads;
+  const int q_begin = cu_seqlens_q[seq], num_q = cu_seqlens_q[seq + 1] - q_begin;
+  const int len_k = seq_lens_k[seq];
+  const int num_cols = num_q * G;
+  constexpr int kWgCols = 4 * 16 * NCB;
+  const int my_tiles = (num_cols + kWgCols - 1) / kWgCols;
+  // Later tiles see more keys.  Unpaired: they are started first, so that the short ones fill the
+  // tail.  Paired (few workgroups, all resident at once): a workgroup takes tile t from the far end
+  // and then its mirror image from the near end, so that every workgroup has the same amount to do.
+  const int far_tile = my_tiles - 1 - (int)blockIdx.x;
+  if (far_tile < 0) return;
+  const int passes = (paired && (int)blockIdx.x < far_tile) ? 2 : 1;
+  if (paired && (int)blockIdx.x > far_tile) return;
+  for (int pass = 0; pass < passes; ++pass) {
+  const int wg_col0 = (pass == 0 ? far_tile : (int)blockIdx.x) * kWgCols;
+  const int pos0 = len_k - num_q;
+  // key range of the whole workgroup
+  const int wg_last = min(wg_col0 + kWgCols, num_cols) - 1;
+  const int wg_qmin = pos0 + wg_col0 / G, wg_qmax = pos0 + wg_last / G;
+  const int k_hi = wg_qmax + 1;
+  const int k_lo = ((window > 0 && wg_qmin - window + 1 > 0) ? wg_qmin - window + 1 : 0) & ~63;
+  // this wavefront's columns
+  const int col0 = wg_col0 + wave * 16 * NCB;
+  const bool wave_on = col0 < num_cols;
+  const int last_col = min(col0 + 16 * NCB, num_cols) - 1;
+  const int qpos_min = pos0 + col0 / G, qpos_max = wave_on ? pos0 + last_col / G : -1;
+  const int vis_hi = qpos_max + 1;
+  const int vis_lo = (window > 0 && qpos_min - window + 1 > 0) ? qpos_min - window + 1 : 0;
+
+  int my_qpos[NCB], my_first[NCB];
+  bool my_valid[NCB];
+  size_t my_out[NCB];
+  bf16x8 qreg[NCB][KSTEPS];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int c = col0 + cb * 16 + r;
+    my_valid[cb] = c < num_cols;
+    const int tok = my_valid[cb] ? c / G : 0, hg = my_valid[cb] ? c - tok * G : 0;
+    my_qpos[cb] = my_valid[cb] ? pos0 + tok : -1;
+    my_first[cb] = (window > 0 && my_qpos[cb] - window + 1 > 0) ? my_qpos[cb] - window + 1 : 0;
+    const size_t row = (size_t)(q_begin + tok) * q_stride + (size_t)(kvh * G + hg) * D;
+    my_out[cb] = (size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int dd = s * 32 + g * 8;
+      qreg[cb][s] = (my_valid[cb] && dd < D) ? *reinterpret_cast<const bf16x8*>(q + row + dd) : zero8();
+    }
+  }
+  floatx4 acc[NCB][DBLOCKS];
+  float m_run[NCB], l_run[NCB];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    m_run[cb] = -INFINITY;
+    l_run[cb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) acc[cb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float sl2 = scale * kLog2e;
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  const size_t page_elems = (size_t)block_size * D;
+  const size_t page_stride = page_elems * num_kv_heads;
+
+  // ---- fetch of one tile (16 keys) per wavefront: wavefront w fetches tile w of the block
+  struct Fetched {
+    bf16x8 k[kKPerLane], v[kVPerLane];
+  };
+  auto fetch = [&](Fetched& f, int n0) {
+    const int nk = n0 + wave * 16;
+    const bool on = nk < k_hi;                                   // past the range: table entry unread, zeros stored
+    const bf16* kbase = k_pages;
+    const bf16* vbase = v_pages;
+    if (on) {
+      const int page = bt[nk / block_size];
+      const int off = nk & (block_size - 1);
+      const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
+      kbase = k_pages + base + (size_t)off * D;                  // 16 rows of D, contiguous
+      vbase = v_pages + base + off;                              // + channel * block_size + key
+    }
+#pragma unroll
+    for (int i = 0; i < kKPerLane; ++i) {
+      const int c = lane + i * 64;
+      f.k[i] = (on && c < kKChunks) ? *reinterpret_cast<const bf16x8*>(kbase + (size_t)c * 8) : zero8();
+    }
+#pragma unroll
+    for (int i = 0; i < kVPerLane; ++i) {
+      const int c = lane + i * 64;                                // c = channel * 2 + half
+      f.v[i] = (on && c < kVChunks) ? *reinterpret_cast<const bf16x8*>(vbase + (size_t)(c >> 1) * block_size + (c & 1) * 8) : zero8();
+    }
+  };
+  auto stash = [&](const Fetched& f, int buf) {
+#pragma unroll
+    for (int i = 0; i < kKPerLane; ++i) {
+      const int c = lane + i * 64;
+      if (c < kKChunks) {
+        const int row = c / (D / 8), part = c - row * (D / 8);
+        *reinterpret_cast<bf16x8*>(&k_s[buf][(wave * 16 + row) * kKRow + part * 8]) = f.k[i];
+      }
+    }
+    const int a = wave >> 1, h = wave & 1;                        // tile `wave` is half h of the 32-key group a
+#pragma unroll
+    for (int i = 0; i < kVPerLane; ++i) {
+      const int c = lane + i * 64;
+      if (c < kVChunks) {
+        const int ch = c >> 1, half = c & 1;
+        bf16* dst = &v_s[buf][ch * kVRow + a * 32 + h * 4];
+        // keys half*8 .. half*8+7 of the tile: lane groups g = half*2 and half*2 + 1, four keys each
+        bf16x4 lo4, hi4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { lo4[j] = f.v[i][j]; hi4[j] = f.v[i][4 + j]; }
+        *reinterpret_cast<bf16x4*>(dst + (half * 2) * 8) = lo4;
+        *reinterpret_cast<bf16x4*>(dst + (half * 2 + 1) * 8) = hi4;
+      }
+    }
+  };
+
+  // `masked` is a compile-time flag: blocks whose 64 keys every column of the wavefront may see take
+  // the version without any comparison.
+  auto compute = [&](int buf, int n0, auto masked_tag) {
+    constexpr bool kMasked = decltype(masked_tag)::value;
+    const bf16* kb = k_s[buf];
+    const bf16* vb = v_s[buf];
+    floatx4 s_t[4][NCB];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
+      if (kMasked && n0 + kt * 16 >= vis_hi) continue;            // uniform in the wavefront: nothing of this tile is visible
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        const int dd = s * 32 + g * 8;
+        const bf16x8 kop = (dd < D) ? *reinterpret_cast<const bf16x8*>(kb + (kt * 16 + r) * kKRow + dd) : zero8();
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qreg[cb][s], s_t[kt][cb], 0, 0, 0);
+      }
+    }
+    bf16x8 p_op[2][NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      // The maximum is taken over the raw dot products (the scale is positive); the running
+      // maximum m_run is kept in scaled log2 units.
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (kMasked) {
+            const int n = n0 + kt * 16 + g * 4 + i;
+            if (!(n <= my_qpos[cb] && n >= my_first[cb])) s_t[kt][cb][i] = -INFINITY;
+          }
+          mx = fmaxf(mx, s_t[kt][cb][i]);
+        }
+      mx = group_max(mx) * sl2;
+      const float m_new = fmaxf(m_run[cb], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run[cb] - m_safe);
+      m_run[cb] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = fast_exp2(fmaf(s_t[kt][cb][i], sl2, -m_safe));
+          psum += p;
+          p_op[kt >> 1][cb][(kt & 1) * 4 + i] = (__bf16)p;
+        }
+      l_run[cb] = l_run[cb] * alpha + psum;
+      if (!__all(alpha == 1.f)) {                                 // the maximum seldom moves after the first blocks
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; ++db) acc[cb][db] *= alpha;
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      if (kMasked && n0 + a * 32 >= vis_hi) continue;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) {
+        bf16x8 vreg = *reinterpret_cast<const bf16x8*>(vb + (db * 16 + r) * kVRow + a * 32 + g * 8);
+        if (kMasked) {
+          // values of keys that no column of this wavefront may see are zeroed (stale data, 0 * NaN)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int n = n0 + (2 * a + (j >> 2)) * 16 + g * 4 + (j & 3);
+            if (n >= vis_hi || n < vis_lo) vreg[j] = (__bf16)0.0f;
+          }
+        }
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) acc[cb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg, p_op[a][cb], acc[cb][db], 0, 0, 0);
+      }
+    }
+  };
+  const int full_from = window > 0 ? max(qpos_max - window + 1, 0) : 0;   // blocks from here on are inside every column's window
+  const bool all_cols = col0 + 16 * NCB <= num_cols;
+
+  // ---- the blocks.  Block i is computed from LDS while block i + 1 sits in registers (requested one
+  //      step earlier, written to the other LDS buffer after the computation) and block i + 2 is being
+  //      requested: a fetch has two steps to arrive.
+  auto step = [&](int n0, int buf, Fetched& arriving, Fetched& free_regs) {
+    if (n0 + 128 < k_hi) fetch(free_regs, n0 + 128);
+    if (wave_on && n0 < vis_hi && n0 + 64 > vis_lo) {
+      if (all_cols && n0 + 63 <= qpos_min && n0 >= full_from) compute(buf, n0, PlainTag{});
+      else compute(buf, n0, MaskedTag{});
+    }
+    if (n0 + 64 < k_hi) stash(arriving, buf ^ 1);
+    __syncthreads();
+  };
+  Fetched regs_a, regs_b;
+  fetch(regs_a, k_lo);
+  if (k_lo + 64 < k_hi) fetch(regs_b, k_lo + 64);
+  stash(regs_a, 0);
+  __syncthreads();
+  for (int n0 = k_lo; n0 < k_hi; n0 += 128) {
+    step(n0, 0, regs_b, regs_a);                                  // block n0 in buffer 0; n0 + 64 arrives in regs_b
+    if (n0 + 64 < k_hi) step(n0 + 64, 1, regs_a, regs_b);
+  }
+
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    if (!my_valid[cb]) continue;
+    const float inv = 1.f / group_sum(l_run[cb]);
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+      bf16x4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = (__bf16)(acc[cb][db][i] * inv);
+      *reinterpret_cast<bf16x4*>(out + my_out[cb] + db * 16 + g * 4) = o;
+    }
+  }
+  __syncthreads();                                                // the LDS buffers are reused by the next pass
+  }  // pass
+}
+
 // Merge of the partitions of one (token, head), one wavefront each:
 //   out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p   over the partitions that hold a visible key,
 // added in partition order.  The maxima are fetched by different lanes at once, then every lane
@@ -425,7 +686,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
                                        int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                        const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                                        int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                       int num_partitions, float* partials, int waves, int column_blocks, hipStream_t stream) {
+                                       int num_partitions, float* partials, int waves, int column_blocks, int pair_tiles, hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
   const int G = num_heads / num_kv_heads;
@@ -441,6 +702,21 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   if (num_kv_heads * num_partitions > 65535 || num_seqs > 65535) return -2;
   if (waves != 1 && waves != 4 && waves != 8 && waves != 16) return -2;
   if (waves > 1 && (long)merge_lds_bytes(ncb, waves) > pllm_max_lds()) return -2;
+  if (waves == 1 && partition_size == 0 && max_cols > 64 && column_blocks != 1 && column_blocks != 4) {
+    // prompt portions: workgroups of four wavefronts that share every block of keys through LDS
+    constexpr int kCols = 4 * 16 * 2;
+    const int ptiles = (max_cols + kCols - 1) / kCols;
+    // pair_tiles: the caller knows that the queries span most of the context (a prompt from its
+    // start), so late tiles have far more keys than early ones.  If all workgroups are resident at
+    // once anyway, and pairing still leaves one per compute unit, far and near tiles are paired.
+    const long wgs = (long)ptiles * num_kv_heads * num_seqs;
+    const int paired = (pair_tiles && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
+    dim3 pgrid(paired ? (ptiles + 1) / 2 : ptiles, num_kv_heads, num_seqs);
+    hipLaunchKernelGGL((paged_attention_prefill_kernel<2>), pgrid, dim3(256), 0, stream, (const bf16*)q, q_stride,
+                       (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q,
+                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, paired);
+    return (int)hipGetLastError();
+  }
   dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64 * waves);
   const size_t lds = waves > 1 ? merge_lds_bytes(ncb, waves) : 0;
 #define PLLM_LAUNCH(NCB_, WAVES_)                                                                                                    \
