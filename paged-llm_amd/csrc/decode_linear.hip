@@ -57,8 +57,23 @@ __device__ __forceinline__ bf16x8 zero8() {
 //   rotary/cache rows 0-7: columns j*8 .. j*8+7 of the lower half of a head, rows 8-15: their partners
 //                in the upper half (element i turns with element i + d/2)
 // so that both members of a pair are in one tile and the epilogue finds them in LDS.
-template <int EPI>
+//
+// HALF (at most 8 input rows): a unit is 8 weight rows.  Tile rows 0-7 hold them for the even slab of a
+// pair of K slabs, tile rows 8-15 hold the same weight rows for the odd slab; the B operand carries
+// the input rows for the even slab in columns 0-7 and for the odd slab in columns 8-15.  The two
+// diagonal 8 x 8 blocks of the result are the two halves of the sum; the other two are ignored.
+// Twice as many units of half the size: small matrices then put work on every compute unit.
+template <int EPI, bool HALF>
 __device__ __forceinline__ int unit_row(const DecodeLinearParams& p, int unit, int r) {
+  if (HALF) {
+    const int rr = r & 7;
+    if (EPI == EPI_ROPE_KV) {
+      const int half = p.head_dim >> 1, per_head = half >> 2;
+      const int head = unit / per_head, j = unit - head * per_head;
+      return head * p.head_dim + j * 4 + (rr & 3) + (rr < 4 ? 0 : half);
+    }
+    return min(unit * 8 + rr, p.N - 1);
+  }
   if (EPI == EPI_GATED) {
     const int n = min(unit * 8 + (r & 7), p.N - 1);
     return r < 8 ? n : n + p.N;                                 // up rows follow the gate rows
@@ -71,13 +86,54 @@ __device__ __forceinline__ int unit_row(const DecodeLinearParams& p, int unit, i
   return min(unit * 16 + r, p.N - 1);
 }
 
+// Rotary epilogue for one pair (element ri of the lower half, its partner in the upper half) of
+// head `head` of input row m: q is rotated and written out, k is rotated and written to its page,
+// v is written to its (transposed) page.
+__device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, int head, int ri, float lo, float hi) {
+  const int d = p.head_dim, half = d >> 1;
+  const int nh = p.num_heads, nkv = p.num_kv_heads;
+  if (head < nh + nkv) {
+    // q and k are rounded to bfloat16 by the projection before they are rotated
+    lo = __bfloat162float(__float2bfloat16(lo));
+    hi = __bfloat162float(__float2bfloat16(hi));
+    float cs = 1.f, sn = 0.f;
+    if (p.cos_t) {
+      const int pos = p.positions[m];
+      cs = p.cos_t[(size_t)pos * half + ri];
+      sn = p.sin_t[(size_t)pos * half + ri];
+    }
+    const bf16 out_lo = __float2bfloat16(lo * cs - hi * sn), out_hi = __float2bfloat16(hi * cs + lo * sn);
+    if (head < nh) {
+      bf16* q = (bf16*)p.out + (size_t)m * p.ldo + (size_t)head * d;
+      q[ri] = out_lo;
+      q[ri + half] = out_hi;
+    } else {
+      const int slot = p.slots[m];
+      if (slot >= 0) {
+        const int page = slot / p.block_size, off = slot - page * p.block_size;
+        bf16* k = p.k_pages + (((size_t)page * nkv + (head - nh)) * p.block_size + off) * d;
+        k[ri] = out_lo;
+        k[ri + half] = out_hi;
+      }
+    }
+  } else {
+    const int slot = p.slots[m];
+    if (slot >= 0) {
+      const int page = slot / p.block_size, off = slot - page * p.block_size;
+      bf16* v = p.v_pages + ((size_t)page * nkv + (head - nh - nkv)) * d * p.block_size + off;
+      v[(size_t)ri * p.block_size] = __float2bfloat16(lo);
+      v[(size_t)(ri + half) * p.block_size] = __float2bfloat16(hi);
+    }
+  }
+}
+
 #ifdef PLLM_TRACE
 #define PLLM_STAMP(i) do { if (p.trace && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1)) p.trace[(blockIdx.x ? 16 : 0) + (i)] = wall_clock64(); } while (0)
 #else
 #define PLLM_STAMP(i) do { } while (0)
 #endif
 
-template <int EPI, int WAVES>
+template <int EPI, int WAVES, bool HALF>
 __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p, int num_units) {
   PLLM_STAMP(0);
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -89,7 +145,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   const int r = lane & 15, g = lane >> 4;
 
   // ---- request this wavefront's slabs of the first unit, then build the rows in LDS while they travel
-  const int num_slabs = (K + kSlab - 1) / kSlab;
+  constexpr int kStep = HALF ? 2 * kSlab : kSlab;               // k range one wavefront consumes per step
+  const int khalf = HALF ? (r >> 3) * kSlab : 0;                // HALF: tile rows / columns 8-15 work on the odd slab
+  const int xrow = HALF ? (r & 7) : r;                          // input row this lane's B operand column belongs to
+  const int num_slabs = (K + kStep - 1) / kStep;
   const int my_slabs = wave < num_slabs ? (num_slabs - wave + WAVES - 1) / WAVES : 0;
   constexpr int PRE = WAVES >= 16 ? 3 : 2;                      // slabs in flight per wavefront (registers)
   bf16x8 wbuf[PRE][4];
@@ -98,12 +157,12 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
     const int slab = wave + nth * WAVES;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kk = slab * kSlab + j * 32 + g * 8;
+      const int kk = slab * kStep + khalf + j * 32 + g * 8;
       dst[j] = (kk < K) ? *reinterpret_cast<const bf16x8*>(wrow + kk) : zero8();
     }
   };
   auto request_unit = [&](int unit) {
-    wrow = p.W + (size_t)unit_row<EPI>(p, unit, r) * p.ldw;
+    wrow = p.W + (size_t)unit_row<EPI, HALF>(p, unit, r) * p.ldw;
 #pragma unroll
     for (int s = 0; s < PRE; ++s)
       if (s < my_slabs) load_w(s, wbuf[s]);
@@ -147,8 +206,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   PLLM_STAMP(2);
 
   auto x_operand = [&](int nth, int j) {
-    const int kk = (wave + nth * WAVES) * kSlab + j * 32 + g * 8;
-    return (r < M && kk < K) ? *reinterpret_cast<const bf16x8*>(xs + (size_t)r * row_len + kk) : zero8();
+    const int kk = (wave + nth * WAVES) * kStep + khalf + j * 32 + g * 8;
+    return (xrow < M && kk < K) ? *reinterpret_cast<const bf16x8*>(xs + (size_t)xrow * row_len + kk) : zero8();
   };
 
   // ---- units of this workgroup, one after the other; the next unit's weights are requested as
@@ -182,8 +241,25 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
         for (int w = 0; w < WAVES; ++w) s += part[w * 256 + i * 64 + ln];
         return s;
       };
-      const int m = r, row = g * 4 + i;                         // row of the tile
-      if (m < M) {
+      const int m = r, row = g * 4 + i;                         // column (input row) and row of the tile
+      if (HALF) {
+        // useful blocks: (rows 0-7, columns 0-7) + (rows 8-15, columns 8-15), 40 lanes further
+        if (m < M && m < 8 && row < 8) {
+          if (EPI == EPI_BF16 || EPI == EPI_F32) {
+            const int n = unit * 8 + row;
+            if (n < N) {
+              const float v = total(lane) + total(lane + 40);
+              if (EPI == EPI_F32) ((float*)p.out)[(size_t)m * p.ldo + n] = v;
+              else ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(v);
+            }
+          } else if (EPI == EPI_ROPE_KV && row < 4) {
+            const int d = p.head_dim, half = d >> 1, per_head = half >> 2;
+            const int head = unit / per_head, ri = (unit - head * per_head) * 4 + row;
+            const float lo = total(lane) + total(lane + 40), hi = total(lane + 16) + total(lane + 56);   // tile rows row + 4
+            rope_store(p, m, head, ri, lo, hi);
+          }
+        }
+      } else if (m < M) {
         if (EPI == EPI_BF16 || EPI == EPI_F32) {
           const int n = unit * 16 + row;
           if (n < N) {
@@ -200,41 +276,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
         } else if (row < 8) {  // EPI_ROPE_KV
           const int d = p.head_dim, half = d >> 1, per_head = half >> 3;
           const int head = unit / per_head, ri = (unit - head * per_head) * 8 + row;   // rotation index in [0, half)
-          float lo = total(lane), hi = total(lane + 32);
-          const int nh = p.num_heads, nkv = p.num_kv_heads;
-          if (head < nh + nkv) {
-            // q and k are rounded to bfloat16 by the projection before they are rotated
-            lo = __bfloat162float(__float2bfloat16(lo));
-            hi = __bfloat162float(__float2bfloat16(hi));
-            float cs = 1.f, sn = 0.f;
-            if (p.cos_t) {
-              const int pos = p.positions[m];
-              cs = p.cos_t[(size_t)pos * half + ri];
-              sn = p.sin_t[(size_t)pos * half + ri];
-            }
-            const bf16 out_lo = __float2bfloat16(lo * cs - hi * sn), out_hi = __float2bfloat16(hi * cs + lo * sn);
-            if (head < nh) {
-              bf16* q = (bf16*)p.out + (size_t)m * p.ldo + (size_t)head * d;
-              q[ri] = out_lo;
-              q[ri + half] = out_hi;
-            } else {
-              const int slot = p.slots[m];
-              if (slot >= 0) {
-                const int page = slot / p.block_size, off = slot - page * p.block_size;
-                bf16* k = p.k_pages + (((size_t)page * nkv + (head - nh)) * p.block_size + off) * d;
-                k[ri] = out_lo;
-                k[ri + half] = out_hi;
-              }
-            }
-          } else {
-            const int slot = p.slots[m];
-            if (slot >= 0) {
-              const int page = slot / p.block_size, off = slot - page * p.block_size;
-              bf16* v = p.v_pages + ((size_t)page * nkv + (head - nh - nkv)) * d * p.block_size + off;
-              v[(size_t)ri * p.block_size] = __float2bfloat16(lo);
-              v[(size_t)(ri + half) * p.block_size] = __float2bfloat16(hi);
-            }
-          }
+          rope_store(p, m, head, ri, total(lane), total(lane + 32));
         }
       }
     }
@@ -243,9 +285,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   }
 }
 
-template <int EPI, int WAVES>
+template <int EPI, int WAVES, bool HALF>
 static int launch(const DecodeLinearParams& p, int units, int blocks, size_t lds, hipStream_t stream) {
-  auto kernel = decode_linear_kernel<EPI, WAVES>;
+  auto kernel = decode_linear_kernel<EPI, WAVES, HALF>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -312,17 +354,27 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
       break;
     default: return -3;
   }
+  // Small matrices with at most 8 rows: units of 8 weight rows, so that every compute unit gets one.
+  const bool half = M <= 8 && epi != EPI_GATED && units < num_compute_units() && K >= 512;
+  if (half) units *= 2;
   // Up to two workgroups per compute unit stay resident; more units than that are dealt evenly
   // to that many workgroups, which walk them with the next unit's weights already on their way.
   const int resident = 2 * num_compute_units();
   const int per_block = (units + resident - 1) / resident;
   const int blocks = (units + per_block - 1) / per_block;
-#define GO(EPI_) return waves == 16 ? launch<EPI_, 16>(p, units, blocks, lds, stream) : launch<EPI_, 8>(p, units, blocks, lds, stream)
+#define GO(EPI_, HALF_) return waves == 16 ? launch<EPI_, 16, HALF_>(p, units, blocks, lds, stream) : launch<EPI_, 8, HALF_>(p, units, blocks, lds, stream)
+  if (half) {
+    switch (epi) {
+      case EPI_BF16: GO(EPI_BF16, true);
+      case EPI_F32: GO(EPI_F32, true);
+      case EPI_ROPE_KV: GO(EPI_ROPE_KV, true);
+    }
+  }
   switch (epi) {
-    case EPI_BF16: GO(EPI_BF16);
-    case EPI_F32: GO(EPI_F32);
-    case EPI_GATED: GO(EPI_GATED);
-    case EPI_ROPE_KV: GO(EPI_ROPE_KV);
+    case EPI_BF16: GO(EPI_BF16, false);
+    case EPI_F32: GO(EPI_F32, false);
+    case EPI_GATED: GO(EPI_GATED, false);
+    case EPI_ROPE_KV: GO(EPI_ROPE_KV, false);
   }
 #undef GO
   return -3;
