@@ -89,26 +89,20 @@ __device__ __forceinline__ int unit_row(const DecodeLinearParams& p, int unit, i
 // Rotary epilogue for one pair (element ri of the lower half, its partner in the upper half) of
 // head `head` of input row m: q is rotated and written out, k is rotated and written to its page,
 // v is written to its (transposed) page.
-__device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, int head, int ri, float lo, float hi) {
+__device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, int head, int ri, float lo, float hi, float cs,
+                                           float sn, int slot) {
   const int d = p.head_dim, half = d >> 1;
   const int nh = p.num_heads, nkv = p.num_kv_heads;
   if (head < nh + nkv) {
     // q and k are rounded to bfloat16 by the projection before they are rotated
     lo = __bfloat162float(__float2bfloat16(lo));
     hi = __bfloat162float(__float2bfloat16(hi));
-    float cs = 1.f, sn = 0.f;
-    if (p.cos_t) {
-      const int pos = p.positions[m];
-      cs = p.cos_t[(size_t)pos * half + ri];
-      sn = p.sin_t[(size_t)pos * half + ri];
-    }
     const bf16 out_lo = __float2bfloat16(lo * cs - hi * sn), out_hi = __float2bfloat16(hi * cs + lo * sn);
     if (head < nh) {
       bf16* q = (bf16*)p.out + (size_t)m * p.ldo + (size_t)head * d;
       q[ri] = out_lo;
       q[ri + half] = out_hi;
     } else {
-      const int slot = p.slots[m];
       if (slot >= 0) {
         const int page = slot / p.block_size, off = slot - page * p.block_size;
         bf16* k = p.k_pages + (((size_t)page * nkv + (head - nh)) * p.block_size + off) * d;
@@ -117,7 +111,6 @@ __device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, i
       }
     }
   } else {
-    const int slot = p.slots[m];
     if (slot >= 0) {
       const int page = slot / p.block_size, off = slot - page * p.block_size;
       bf16* v = p.v_pages + ((size_t)page * nkv + (head - nh - nkv)) * d * p.block_size + off;
@@ -170,6 +163,12 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   int unit = blockIdx.x;
   if (unit < num_units) request_unit(unit);
   PLLM_STAMP(1);
+  // Rotary epilogue: what depends only on the input row is fetched now, not after the product.
+  int rope_pos = 0, rope_slot = -1;
+  if (EPI == EPI_ROPE_KV && tid < 256 && (HALF ? (r & 7) : r) < M && (!HALF || r < 8)) {
+    rope_pos = p.cos_t ? p.positions[r] : 0;
+    rope_slot = p.slots[r];
+  }
 
   for (int m = wave; m < M; m += WAVES) {
     const size_t src = p.row_index ? (size_t)p.row_index[m] : (size_t)m;
@@ -214,6 +213,19 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   //      soon as the current unit's have been consumed, and travel during the reduction
   for (; unit < num_units; unit += gridDim.x) {
     floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+    float rope_cs = 1.f, rope_sn = 0.f;
+    if (EPI == EPI_ROPE_KV && tid < 256 && p.cos_t) {
+      // thread (i = tid >> 6, lane) will finish tile row g * 4 + i of input row r: fetch its angle now
+      const int half = p.head_dim >> 1, per_head = HALF ? (half >> 2) : (half >> 3), rows = HALF ? 4 : 8;
+      const int row = g * 4 + (tid >> 6);
+      if (row < rows && r < M && (!HALF || r < 8)) {
+        const int head = unit / per_head, ri = (unit - head * per_head) * rows + row;
+        if (head < p.num_heads + p.num_kv_heads) {
+          rope_cs = p.cos_t[(size_t)rope_pos * half + ri];
+          rope_sn = p.sin_t[(size_t)rope_pos * half + ri];
+        }
+      }
+    }
     for (int base = 0; base < my_slabs; base += PRE) {
 #pragma unroll
       for (int s = 0; s < PRE; ++s) {
@@ -256,7 +268,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
             const int d = p.head_dim, half = d >> 1, per_head = half >> 2;
             const int head = unit / per_head, ri = (unit - head * per_head) * 4 + row;
             const float lo = total(lane) + total(lane + 40), hi = total(lane + 16) + total(lane + 56);   // tile rows row + 4
-            rope_store(p, m, head, ri, lo, hi);
+            rope_store(p, m, head, ri, lo, hi, rope_cs, rope_sn, rope_slot);
           }
         }
       } else if (m < M) {
@@ -276,7 +288,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
         } else if (row < 8) {  // EPI_ROPE_KV
           const int d = p.head_dim, half = d >> 1, per_head = half >> 3;
           const int head = unit / per_head, ri = (unit - head * per_head) * 8 + row;   // rotation index in [0, half)
-          rope_store(p, m, head, ri, total(lane), total(lane + 32));
+          rope_store(p, m, head, ri, total(lane), total(lane + 32), rope_cs, rope_sn, rope_slot);
         }
       }
     }
