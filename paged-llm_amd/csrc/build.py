@@ -142,18 +142,16 @@ def load_library(source: str, defines: dict | None = None) -> ctypes.CDLL:
 
 
 # Sources every model needs, and the specialised ones per head size.
-COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip"]
+COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip", "decode_linear.hip",
+                  "gemm_skinny.hip"]
+# Head sizes whose attention library a full build makes (others are compiled at first use).
+USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
 
 
 def all_targets() -> list[tuple[str, dict]]:
     """Everything a full build compiles: the common sources plus the usual specialisations."""
     targets: list[tuple[str, dict]] = [(s, {}) for s in COMMON_SOURCES]
-    for extra in ("gemm_skinny.hip", "gemm_mfma.hip"):
-        if os.path.exists(os.path.join(CSRC, extra)):
-            targets.append((extra, {}))
-    if os.path.exists(os.path.join(CSRC, "attention_mfma.hip")):
-        for d in (16, 32, 64, 128):
-            targets.append(("attention_mfma.hip", {"HEAD_DIM": d}))
+    targets += [("attention_mfma.hip", {"HEAD_DIM": d}) for d in USUAL_HEAD_DIMS]
     return targets
 
 

@@ -358,9 +358,7 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
 
 # ------------------------------------------------------------------------------------------- choices
 SKINNY_MAX_ROWS = 64
-_SKINNY_SIG = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p,
-               c_void_p, c_void_p]
-_skinny_scratch: dict = {}
+_SKINNY_SIG = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
 
 
 def _skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -369,52 +367,20 @@ def _skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def _skinny_split(n_out_tiles: int, K: int) -> int:
-    """How many workgroups share the K range of one tile: enough to put work on every CU, while
-    every wavefront still gets at least one slab of 128."""
-    # Measured on MI355X: the cross-workgroup fix-up (device-scope fences) costs tens of
-    # microseconds, far more than the under-filled GPU it was meant to cure.  One split.
-    return 1
-
-
-def _skinny_buffers(device, floats: int, counters: int):
-    """Workspace for split-K partials and the arrival counters (zero once; kernels reset them)."""
-    key = str(device)
-    ws, cnt = _skinny_scratch.get(key, (None, None))
-    if ws is None or ws.numel() < floats:
-        ws = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=device)
-    if cnt is None or cnt.numel() < counters:
-        cnt = torch.zeros(max(counters, 4096), dtype=torch.int32, device=device)
-    _skinny_scratch[key] = (ws, cnt)
-    return ws, cnt
-
-
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None, gated: bool = False,
-                ksplit: int | None = None) -> torch.Tensor:
-    """a [M <= 64, K] times w [N, K]^T (gated: w is [gate; up], result silu(a Wg^T) * (a Wu^T))."""
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """a [M <= 64, K] times w [N, K]^T on the matrix cores, streaming w once; float or bfloat16 out."""
     _on_gpu(a, w)
     _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], f"gemm shapes {tuple(a.shape)} x {tuple(w.shape)}^T")
     _need(_skinny_ok(a, w), "gemm_skinny needs bfloat16 operands with K, row strides and addresses in multiples of 8 elements")
     M, K = a.shape
     _need(0 < M <= SKINNY_MAX_ROWS, f"gemm_skinny takes 1..{SKINNY_MAX_ROWS} rows, got {M}")
     N = w.shape[0]
-    if gated:
-        _need(N % 2 == 0, "gated product needs [gate; up] rows")
-        N //= 2
     out_dtype = out_dtype or torch.bfloat16
     _need(out_dtype in (torch.bfloat16, torch.float32), "output is bfloat16 or float32")
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    tiles_out = 1 if (gated or M <= 32) else 2
-    blocks = (N + tiles_out * 16 - 1) // (tiles_out * 16)
-    if ksplit is None:
-        ksplit = _skinny_split(blocks, K)
-    ws = cnt = None
-    if ksplit > 1:
-        floats = _fn("gemm_skinny.hip", "pllm_gemm_skinny_workspace_floats", signature=[c_int, c_int, c_int])(M, N, ksplit)
-        ws, cnt = _skinny_buffers(a.device, floats, blocks)
     _check(_fn("gemm_skinny.hip", "pllm_gemm_skinny", signature=_SKINNY_SIG)(
         _ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), M, N, K, 1 if out_dtype == torch.float32 else 0,
-        1 if gated else 0, ksplit, _ptr(ws), _ptr(cnt), _stream()), "gemm_skinny")
+        _stream()), "gemm_skinny")
     return out
 
 

@@ -39,7 +39,7 @@ class ModelRunner:
                        for pos, ss in model.state_specs().items()}
 
     # ------------------------------------------------------------------ batch -> device tensors
-    def _stage(self, entries: list, fixed_blocks: int | None = None):
+    def _stage(self, entries: list, fixed_blocks: int | None = None, fast: bool = True):
         """Checks the batch and lays all its integer arrays out in one host buffer.
 
         Returns (buffer, offsets, sizes, host) where piece i is buffer[offsets[i]: offsets[i] + sizes[i]]
@@ -49,7 +49,7 @@ class ModelRunner:
         """
         if not entries:
             raise StepError("a step needs at least one entry")
-        if fixed_blocks is not None and all(len(e.tokens) == 1 for e in entries):
+        if fast and fixed_blocks is not None and all(len(e.tokens) == 1 for e in entries):
             return self._stage_decode(entries, fixed_blocks)
         bs = self.block_size
         vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions

@@ -1,0 +1,92 @@
+"""The step function's host side: what it checks before any kernel runs, and the layout of the
+staged integer arrays (the device is not needed for either)."""
+
+import numpy as np
+import pytest
+import torch
+
+from paged_llm_amd.cache import NO_PAGE
+from paged_llm_amd.engine import StepEntry
+from paged_llm_amd.engine.loading import build_model, build_runtime
+from paged_llm_amd.engine.runner import StepError
+from paged_llm_amd.weights import fill_random
+from tests.tiny_configs import TINY_A
+
+
+@pytest.fixture(scope="module")
+def runtime():
+    model = build_model(TINY_A, "float32", "cpu")
+    fill_random(model, seed=0)
+    manager, storage, runner = build_runtime(model, 16, 12, 4, enable_prefix_caching=False)
+    return manager, runner
+
+
+def entry(manager, rid, tokens, start, want=()):
+    assert manager.allocate(rid, start, len(tokens))
+    g = next(iter(manager.groups))
+    return StepEntry(rid, list(tokens), start, {g: manager.block_table(rid, g)}, None, list(want))
+
+
+def test_layout_of_a_mixed_batch(runtime):
+    manager, runner = runtime
+    a = entry(manager, "a", [5, 6, 7, 8, 9], 0, want=[4])
+    b = entry(manager, "b", list(range(20)), 0)
+    manager.allocate("c", 0, 17)
+    c = entry(manager, "c", [3], 17, want=[0])
+    buf, offsets, sizes, host = runner._stage([a, b, c])
+    piece = lambda i: buf[offsets[i]: offsets[i] + sizes[i]]
+    assert piece(0).tolist() == [5, 6, 7, 8, 9] + list(range(20)) + [3]                    # token ids
+    assert piece(1).tolist() == list(range(5)) + list(range(20)) + [17]                    # positions
+    assert piece(2).tolist() == [0, 5, 25, 26] and piece(3).tolist() == [5, 20, 18]        # query offsets, context lengths
+    assert piece(6).tolist() == [4, 25]                                                    # rows whose logits are wanted
+    tables = piece(7).reshape(3, 2)
+    g = next(iter(manager.groups))
+    assert tables[1].tolist() == manager.block_table("b", g) and tables[0, 1] == 0        # short tables are padded with 0
+    slots = piece(8)
+    tc = manager.block_table("c", g)
+    assert slots[-1] == tc[1] * 16 + 1 and slots[0] == manager.block_table("a", g)[0] * 16
+    assert all(o % 4 == 0 for o in offsets)                                                # 16-byte aligned pieces
+    assert host["q_lens"] == [5, 20, 1] and host["k_lens"] == [5, 20, 18]
+    for r in "abc":
+        manager.free(r)
+
+
+def test_decode_staging_fast_path_equals_the_general_one(runtime):
+    manager, runner = runtime
+    entries = []
+    for i, start in enumerate([3, 16, 31, 0]):
+        rid = f"d{i}"
+        if start:
+            manager.allocate(rid, 0, start)
+        entries.append(entry(manager, rid, [10 + i], start, want=[0] if i != 1 else []))
+    fast = runner._stage(entries, fixed_blocks=4)
+    slow = runner._stage(entries, fixed_blocks=4, fast=False)
+    assert np.array_equal(fast[0], slow[0]) and fast[1] == slow[1] and fast[2] == slow[2]
+    assert fast[3]["k_lens"] == slow[3]["k_lens"] and fast[3]["table_shapes"] == slow[3]["table_shapes"]
+    for i in range(4):
+        manager.free(f"d{i}")
+
+
+@pytest.mark.parametrize("fast", [True, False])
+def test_bad_batches_are_refused_before_anything_runs(runtime, fast):
+    manager, runner = runtime
+    g = next(iter(manager.groups))
+    fixed = 4 if fast else None
+    ok = entry(manager, "ok", [1], 0)
+    with pytest.raises(StepError, match="token id"):
+        runner._stage([StepEntry("x", [256], 0, {g: [0]})], fixed)
+    with pytest.raises(StepError, match="position"):
+        runner._stage([StepEntry("x", [1], 256, {g: list(range(12)) + [0] * 5})], fixed)
+    with pytest.raises(StepError, match="twice"):
+        runner._stage([ok, ok], fixed)
+    with pytest.raises(StepError, match="page"):
+        runner._stage([StepEntry("x", [1], 20, {g: [0]})], fixed)                     # two pages needed, one given
+    with pytest.raises(StepError, match="page id"):
+        runner._stage([StepEntry("x", [1], 3, {g: [99]})], fixed)
+    with pytest.raises(StepError, match="page id"):
+        runner._stage([StepEntry("x", [1], 3, {g: [NO_PAGE]})], fixed)                # a released page inside the visible range
+    with pytest.raises(StepError, match="wanted row"):
+        runner._stage([StepEntry("x", [1], 0, {g: [0]}, None, [1])], fixed)
+    with pytest.raises(StepError):
+        runner._stage([], fixed)
+    manager.free("ok")
