@@ -24,9 +24,8 @@ def llama3_rescale(inv_freq: torch.Tensor, factor: float, low_freq_factor: float
     low_wl = original_max_position_embeddings / low_freq_factor
     high_wl = original_max_position_embeddings / high_freq_factor
     smooth = (original_max_position_embeddings / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
-    slowed = inv_freq / factor
-    blended = (1 - smooth) * slowed + smooth * inv_freq
-    out = torch.where(wavelen > low_wl, slowed, inv_freq)
+    blended = (1 - smooth) * inv_freq / factor + smooth * inv_freq
+    out = torch.where(wavelen > low_wl, inv_freq / factor, inv_freq)
     middle = (wavelen <= low_wl) & (wavelen >= high_wl)
     return torch.where(middle, blended, out)
 

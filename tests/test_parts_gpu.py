@@ -1,0 +1,279 @@
+"""Each part a layer is put together from, built alone through the part registries at sizes that no
+tiny configuration uses, with hand-made step contexts, against the plain function of the same part."""
+
+import math
+
+import pytest
+import torch
+
+from tests.plain import llama_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+HIDDEN, HEADS, KV_HEADS, HEAD_DIM, INTER, VOCAB = 96, 6, 3, 32, 200, 301
+EPS, THETA, BLOCK = 3e-6, 5000.0, 16
+DTYPES = [("float32", 3e-5), ("bfloat16", 3e-2)]
+
+
+def env_for(dtype: str, hidden: int = HIDDEN, max_positions: int = 256):
+    from paged_llm_amd.parts.registry import BuildEnv
+    return BuildEnv(hidden_size=hidden, dtype=getattr(torch, dtype), device=torch.device("cuda:0"),
+                    max_positions=max_positions, shared={})
+
+
+def build(family: str, kind: str, params: dict, env):
+    from paged_llm_amd.parts import PartSpec
+    from paged_llm_amd.parts.registry import build as build_part
+    return build_part(family, PartSpec(kind, params), env)
+
+
+def give_weights(part, seed: int, dtype: str, std: float = 0.08) -> dict:
+    """Random tensors for everything the part declares; returns them as float CPU tensors, rounded
+    to the type the part stores them in, for the plain side."""
+    gen = torch.Generator().manual_seed(seed)
+    plain_side = {}
+    for name, spec in part.weight_specs().items():
+        if spec.role == "vector":
+            t = 1.0 + 0.3 * torch.randn(spec.shape, generator=gen)
+        else:
+            t = std * torch.randn(spec.shape, generator=gen)
+            t = t.to(getattr(torch, dtype)).float()
+        part.assign(name, t)
+        plain_side[name] = t
+    part.finalize()
+    return plain_side
+
+
+def rel(got: torch.Tensor, want: torch.Tensor) -> float:
+    got, want = got.detach().float().cpu(), want.float()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-6))
+
+
+def rows(n: int, seed: int, dtype: str, hidden: int = HIDDEN) -> torch.Tensor:
+    gen = torch.Generator().manual_seed(seed)
+    return torch.randn(n, hidden, generator=gen).to(getattr(torch, dtype))
+
+
+def step_context(portions, tables, group: str, dtype: str):
+    """portions: one (start, n) per sequence; tables: one list of pages per sequence."""
+    from paged_llm_amd.engine.batch import GroupView, StepContext
+    dev = torch.device("cuda:0")
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    positions, slots, cu, k_lens = [], [], [0], []
+    for (start, n), table in zip(portions, tables):
+        for p in range(start, start + n):
+            positions.append(p)
+            slots.append(table[p // BLOCK] * BLOCK + p % BLOCK)
+        cu.append(cu[-1] + n)
+        k_lens.append(start + n)
+    width = max(len(t) for t in tables)
+    padded = [list(t) + [0] * (width - len(t)) for t in tables]
+    q_lens = [n for _, n in portions]
+    view = GroupView(i32(padded), i32(slots), BLOCK)
+    return StepContext(num_tokens=len(positions), num_seqs=len(portions), input_ids=i32([0] * len(positions)),
+                       positions=i32(positions), cu_seqlens_q=i32(cu), seq_lens_k=i32(k_lens),
+                       state_slots=i32([-1] * len(portions)), seq_starts=i32([s for s, _ in portions]),
+                       logits_index=i32([]), groups={group: view}, q_lens=q_lens, k_lens=k_lens,
+                       state_slot_list=[-1] * len(portions), max_q_len=max(q_lens), max_k_len=max(k_lens),
+                       dtype=getattr(torch, dtype), device=dev)
+
+
+def layer_cache(mixer, dtype: str, pages: int):
+    from paged_llm_amd.cache.kv_cache import LayerCache
+    spec = mixer.cache_spec()
+    dev = torch.device("cuda:0")
+    k = torch.zeros((pages, spec.num_kv_heads, BLOCK, spec.head_dim), dtype=getattr(torch, dtype), device=dev)
+    v = torch.zeros((pages, spec.num_kv_heads, spec.head_dim, BLOCK), dtype=getattr(torch, dtype), device=dev)
+    return LayerCache(k, v, spec.group_name(), BLOCK, pages)
+
+
+# ------------------------------------------------------------------------------------------- norm
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_norm_part(dtype, tol):
+    env = env_for(dtype)
+    norm = build("norm", "rmsnorm", {"eps": EPS}, env)
+    w = give_weights(norm, 1, dtype)["weight"]
+    x, delta = rows(9, 2, dtype), rows(9, 3, dtype)
+    want = plain.rms_norm(x.float(), w, EPS)
+    assert rel(norm.forward(x.cuda()), want) <= tol
+    # the sum is rounded once to the stream's type before the norm sees it
+    summed = (x.float() + delta.float()).to(x.dtype)
+    xd = x.cuda()
+    got = norm.add_norm(xd, delta.cuda())
+    assert rel(got, plain.rms_norm(summed.float(), w, EPS)) <= tol
+    assert torch.equal(xd.cpu(), summed)
+    # lazy form: rows of chosen rows; the residual afterwards
+    index = torch.tensor([7, 0, 3], dtype=torch.int32, device="cuda")
+    pend = norm.pending(x.cuda(), delta.cuda(), index, write_residual=False)
+    assert rel(pend.rows(), plain.rms_norm(summed.float()[[7, 0, 3]], w, EPS)) <= tol
+    pend = norm.pending(x.cuda(), delta.cuda())
+    assert torch.equal(pend.residual().cpu(), summed)
+
+
+def test_norm_eps_is_inside_the_root():
+    env = env_for("float32", hidden=16)
+    norm = build("norm", "rmsnorm", {"eps": 0.5}, env)
+    norm.assign("weight", torch.ones(16))
+    x = torch.full((1, 16), 1e-3)
+    want = 1e-3 / math.sqrt(1e-6 + 0.5)
+    assert abs(float(norm.forward(x.cuda())[0, 0]) - want) < 1e-9
+
+
+# --------------------------------------------------------------------------------------- position
+@pytest.mark.parametrize("scaling", [None, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                            "high_freq_factor": 4.0, "original_max_position_embeddings": 64}])
+def test_position_encoding_part(scaling):
+    env = env_for("float32", max_positions=300)
+    rot = build("position_encoding", "rotary", {"head_dim": 48, "theta": 777.0, "scaling": scaling}, env)
+    rot.prepare(300)
+    inv = plain.inverse_frequencies(48, 777.0, scaling)
+    # the part works in float like the reference, the plain function in double: the blend weight holds a
+    # difference of nearby numbers, so a few units in the last place are lost there, no more ...
+    assert float(((rot.inverse_frequencies() - inv) / inv).abs().max()) <= 1e-6
+    # ... and the tables are the cosines and sines of position * frequency, formed in float
+    angles = plain.rotary_angles(torch.arange(300), rot.inverse_frequencies())
+    assert rot.cos.shape == (300, 24)
+    assert float((rot.cos.cpu() - angles.cos()).abs().max()) < 1e-6
+    assert float((rot.sin.cpu() - angles.sin()).abs().max()) < 1e-6
+    from paged_llm_amd.parts import PartSpec
+    spec = PartSpec("rotary", {"head_dim": 48, "theta": 777.0, "scaling": scaling})
+    shared, again = env.position_encoding(spec), env.position_encoding(PartSpec(spec.kind, dict(spec.params)))
+    assert shared is again                     # layers with the same spec share one table
+
+
+# ------------------------------------------------------------------------------------------ mixer
+def attention_reference(w: dict, x: torch.Tensor, window=None, scale=None):
+    cfg = {"num_attention_heads": HEADS, "num_key_value_heads": KV_HEADS, "head_dim": HEAD_DIM}
+    inv = plain.inverse_frequencies(HEAD_DIM, THETA, None)
+    if scale is None:
+        return plain.attention_block(x, torch.arange(x.shape[0]), w, "", cfg, inv, window)
+    # another scale than d^-0.5: the same steps with that scale
+    T = x.shape[0]
+    q = (x @ w["q_proj.weight"].T).view(T, HEADS, HEAD_DIM)
+    k = (x @ w["k_proj.weight"].T).view(T, KV_HEADS, HEAD_DIM)
+    v = (x @ w["v_proj.weight"].T).view(T, KV_HEADS, HEAD_DIM)
+    ang = plain.rotary_angles(torch.arange(T), inv)
+    o = plain.causal_attention(plain.apply_rotary(q, ang), plain.apply_rotary(k, ang), v, scale, window)
+    return o.reshape(T, HEADS * HEAD_DIM) @ w["o_proj.weight"].T
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("options", [{}, {"window": 11}, {"scale": 0.3}])
+def test_attention_part_whole_in_portions_and_token_by_token(dtype, tol, options):
+    env = env_for(dtype)
+    params = {"num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM,
+              "position": {"kind": "rotary", "params": {"head_dim": HEAD_DIM, "theta": THETA, "scaling": None}}}
+    params.update(options)
+    mixer = build("mixer", "paged_attention", params, env)
+    w = give_weights(mixer, 5, dtype)
+    group = mixer.cache_spec().group_name()
+    L = 76
+    x = rows(L, 6, dtype)
+    want = attention_reference(w, x.float(), options.get("window"), options.get("scale"))
+    table = [9, 2, 7, 4, 11]                               # pages in no order
+    # whole
+    cache = layer_cache(mixer, dtype, 12)
+    got = mixer.forward(x.cuda(), step_context([(0, L)], [table], group, dtype), cache, None)
+    assert rel(got, want) <= tol, "whole"
+    # portions cut inside pages, then single tokens; a second sequence rides along in other pages
+    cache = layer_cache(mixer, dtype, 12)
+    other = rows(40, 7, dtype)
+    other_want = attention_reference(w, other.float(), options.get("window"), options.get("scale"))
+    other_table = [0, 5, 1]
+    out, out_other = [], []
+    cuts = [(0, 37), (37, 2), (39, 31)] + [(p, 1) for p in range(70, L)]
+    other_cuts = [(0, 3), (3, 30), (33, 1)] + [(34 + i, 1) for i in range(6)]
+    for i, (start, n) in enumerate(cuts):
+        portions, tables, xs = [(start, n)], [table], [x[start:start + n]]
+        if i < len(other_cuts):
+            s2, n2 = other_cuts[i]
+            portions.append((s2, n2)); tables.append(other_table); xs.append(other[s2:s2 + n2])
+        got = mixer.forward(torch.cat(xs).cuda(), step_context(portions, tables, group, dtype), cache, None)
+        out.append(got[:n])
+        if len(portions) == 2:
+            out_other.append(got[n:])
+    assert rel(torch.cat(out), want) <= tol, "portions"
+    assert rel(torch.cat(out_other), other_want) <= tol, "second sequence"
+
+
+def test_attention_part_refuses_sizes_its_kernels_do_not_take():
+    env = env_for("bfloat16")
+    with pytest.raises(ValueError, match="steps of 16"):
+        build("mixer", "paged_attention", {"num_heads": 4, "num_kv_heads": 2, "head_dim": 24}, env)
+    with pytest.raises(ValueError, match="multiple"):
+        build("mixer", "paged_attention", {"num_heads": 5, "num_kv_heads": 2, "head_dim": 32}, env)
+
+
+# ----------------------------------------------------------------------------------- feed-forward
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("num_rows", [1, 5, 16, 40, 130])
+def test_feed_forward_part(dtype, tol, num_rows):
+    env = env_for(dtype)
+    ff = build("feed_forward", "gated_mlp", {"intermediate_size": INTER}, env)
+    w = give_weights(ff, 8, dtype)
+    x = rows(num_rows, 9, dtype)
+    want = plain.swiglu(x.float(), w["gate_proj.weight"], w["up_proj.weight"], w["down_proj.weight"])
+    assert rel(ff.forward(x.cuda(), None), want) <= tol
+    # fed by a norm that has not run yet
+    norm = build("norm", "rmsnorm", {"eps": EPS}, env)
+    nw = give_weights(norm, 10, dtype)["weight"]
+    h = plain.rms_norm(x.float(), nw, EPS).to(x.dtype).float()
+    want = plain.swiglu(h, w["gate_proj.weight"], w["up_proj.weight"], w["down_proj.weight"])
+    assert rel(ff.forward(norm.pending(x.cuda()), None), want) <= tol
+
+
+def test_feed_forward_part_refuses_other_activations():
+    with pytest.raises(NotImplementedError):
+        build("feed_forward", "gated_mlp", {"intermediate_size": 64, "activation": "gelu"}, env_for("bfloat16"))
+
+
+# ------------------------------------------------------------------------------------------ block
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("num_rows", [4, 45])
+def test_block_part(dtype, tol, num_rows):
+    env = env_for(dtype)
+    block = build("block", "prenorm", {"mixer_norm": "input_layernorm", "mixer": "self_attn",
+                                       "feed_forward_norm": "post_attention_layernorm", "feed_forward": "mlp"}, env)
+    mixer = build("mixer", "paged_attention", {
+        "num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM,
+        "position": {"kind": "rotary", "params": {"head_dim": HEAD_DIM, "theta": THETA, "scaling": None}}}, env)
+    block.attach(build("norm", "rmsnorm", {"eps": EPS}, env), mixer, build("norm", "rmsnorm", {"eps": 2 * EPS}, env),
+                 build("feed_forward", "gated_mlp", {"intermediate_size": INTER}, env))
+    names = set(block.weight_specs())
+    assert {"input_layernorm.weight", "self_attn.q_proj.weight", "mlp.down_proj.weight",
+            "post_attention_layernorm.weight"} <= names and len(names) == 9
+    w = give_weights(block, 11, dtype)
+    x, delta = rows(num_rows, 12, dtype), rows(num_rows, 13, dtype)
+    # plain: the stream is x + delta; two pre-norm branches (pagedllm/model/llama.py:174-185)
+    s = x.float() + delta.float()
+    attn_w = {k[len("self_attn."):]: v for k, v in w.items() if k.startswith("self_attn.")}
+    s = s + attention_reference(attn_w, plain.rms_norm(s, w["input_layernorm.weight"], EPS))
+    branch = plain.swiglu(plain.rms_norm(s, w["post_attention_layernorm.weight"], 2 * EPS), w["mlp.gate_proj.weight"],
+                          w["mlp.up_proj.weight"], w["mlp.down_proj.weight"])
+    cache = layer_cache(mixer, dtype, 4)
+    ctx = step_context([(0, num_rows)], [[3, 1, 2]], mixer.cache_spec().group_name(), dtype)
+    got_x, got_delta = block.forward(x.cuda(), delta.cuda(), ctx, cache, None)
+    assert rel(got_x, s) <= tol
+    assert rel(got_delta, branch) <= tol
+
+
+# ----------------------------------------------------------------------------- embedding and head
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_embedding_and_head_parts(dtype, tol):
+    env = env_for(dtype)
+    emb = build("embedding", "token_embedding", {"vocab_size": VOCAB}, env)
+    table = give_weights(emb, 14, dtype)["weight"]
+    ids = torch.tensor([0, VOCAB - 1, 17, 17, 5], dtype=torch.int32)
+    assert torch.equal(emb.forward(ids.cuda()).float().cpu(), table[ids.long()])
+    x = rows(5, 15, dtype)
+    tied = build("head", "lm_head", {"vocab_size": VOCAB, "tied": True}, env)
+    assert tied.weight_specs() == {}
+    tied.tie(emb.table)
+    logits = tied.forward(x.cuda())
+    assert logits.dtype == torch.float32 and rel(logits, x.float() @ table.T) <= tol
+    own = build("head", "lm_head", {"vocab_size": VOCAB}, env)
+    hw = give_weights(own, 16, dtype)["weight"]
+    assert rel(own.forward(x.cuda()), x.float() @ hw.T) <= tol
+    for many in (33, 100):                                   # other row counts take other kernels
+        xm = rows(many, 17, dtype)
+        assert rel(own.forward(xm.cuda()), xm.float() @ hw.T) <= tol
