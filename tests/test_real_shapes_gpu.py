@@ -1,0 +1,62 @@
+"""Layers of real size (TinyLlama-1.1B, Llama-3.2-1B and Llama-3.1-8B shapes: widths, head counts,
+intermediate sizes, vocabularies, rotary constants and tying as in those models) with random weights
+(all 22 layers of the first, a few of the others, so that the plain implementation stays quick): a prompt in one step,
+tokens decoded one by one, and a second request fed in portions beside them; in true 32-bit and in
+bfloat16 against the plain implementation."""
+
+import pytest
+
+from tests import helpers
+from tests.helpers import TraceBuilder
+
+pytestmark = pytest.mark.gpu
+
+LLAMA3 = lambda factor: {"rope_type": "llama3", "factor": factor, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                         "original_max_position_embeddings": 8192}
+BASE = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "rms_norm_eps": 1e-5, "torch_dtype": "bfloat16",
+        "max_position_embeddings": 4096}
+# name -> (configuration, layers of the model it is taken from)
+SHAPES = {
+    "tinyllama_1b": (dict(BASE, num_hidden_layers=22, hidden_size=2048, num_attention_heads=32, num_key_value_heads=4,
+                          head_dim=64, intermediate_size=5632, vocab_size=32000, rope_theta=10000.0,
+                          tie_word_embeddings=False), 22),
+    "llama32_1b": (dict(BASE, num_hidden_layers=4, hidden_size=2048, num_attention_heads=32, num_key_value_heads=8,
+                        head_dim=64, intermediate_size=8192, vocab_size=128256, rope_theta=500000.0,
+                        rope_scaling=LLAMA3(32.0), tie_word_embeddings=True), 16),
+    "llama31_8b": (dict(BASE, num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                        head_dim=128, intermediate_size=14336, vocab_size=128256, rope_theta=500000.0,
+                        rope_scaling=LLAMA3(8.0), tie_word_embeddings=False), 32),
+}
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+
+
+@pytest.fixture(scope="module", params=list(SHAPES))
+def case(request, tmp_path_factory):
+    cfg, _ = SHAPES[request.param]
+    folder = helpers.make_folder(tmp_path_factory.mktemp(request.param), cfg, seed=21, stored="bfloat16")
+    vocab = cfg["vocab_size"]
+    reqs = {"p": helpers.random_tokens(308, vocab, seed=1), "q": helpers.random_tokens(90, vocab, seed=2)}
+    want = {rid: helpers.plain_logits(folder, toks) for rid, toks in reqs.items()}
+    return folder, reqs, want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_decoding_and_portions_at_real_sizes(case, dtype):
+    from paged_llm_amd.engine.replay import ReplaySession
+    folder, reqs, want = case
+    p, q = reqs["p"], reqs["q"]
+    session = ReplaySession(folder, dtype, 320 + 128, None)
+    trace = TraceBuilder()
+    trace.step([("p", p[:300], [0, 63, 64, 255, 299])])
+    portions = iter([q[:50], q[50:52], q[52:90]])
+    for i in range(300, 308):
+        entries = [("p", p[i:i + 1], "all")]
+        part = next(portions, None)
+        if part is not None:
+            entries.append(("q", part, "last"))
+        trace.step(entries)
+    got = helpers.replay_in_process(session, trace)
+    assert len(got) == 5 + 8 + 3
+    for (rid, pos), row in got.items():
+        err = helpers.worst(row, want[rid][pos])
+        assert err <= TOL[dtype], f"request {rid} position {pos}: relative error {err:.3g} > {TOL[dtype]}"
