@@ -27,6 +27,18 @@ TINYLLAMA = {
     "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 4096,
     "torch_dtype": "bfloat16",
 }
+_LLAMA3 = lambda factor: {"rope_type": "llama3", "factor": factor, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                          "original_max_position_embeddings": 8192}
+# Other layer sizes to measure at (--model); the default record stays on TinyLlama-1.1B.
+MODELS = {
+    "tinyllama-1.1b": ("TinyLlama-1.1B shapes", TINYLLAMA),
+    "llama-3.2-1b": ("Llama-3.2-1B shapes", dict(
+        TINYLLAMA, num_hidden_layers=16, num_key_value_heads=8, intermediate_size=8192, vocab_size=128256,
+        rope_theta=500000.0, rope_scaling=_LLAMA3(32.0), tie_word_embeddings=True, max_position_embeddings=131072)),
+    "llama-3.1-8b": ("Llama-3.1-8B shapes", dict(
+        TINYLLAMA, num_hidden_layers=32, hidden_size=4096, num_key_value_heads=8, head_dim=128, intermediate_size=14336,
+        vocab_size=128256, rope_theta=500000.0, rope_scaling=_LLAMA3(8.0), max_position_embeddings=131072)),
+}
 # Published peaks of the MI355X: HBM3E bandwidth and dense MFMA rates.
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -121,6 +133,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--model", default="tinyllama-1.1b", choices=sorted(MODELS), help="layer sizes to run at")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (reported as such)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
@@ -131,7 +144,8 @@ def main() -> int:
         return 2
 
     import torch
-    cfg = dict(TINYLLAMA)
+    model_name, cfg = MODELS[args.model]
+    cfg = dict(cfg)
     model_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -152,10 +166,10 @@ def main() -> int:
         decode_bytes = numbers["weight_bytes"] + args.batch * args.context * numbers["kv_bytes_per_token"]
         achieved = decode_bytes / sec / 1e9
         record = {
-            "metric": "decode tokens/s (TinyLlama-1.1B shapes, random weights)", "value": round(value, 1), "unit": "tokens/s",
+            "metric": f"decode tokens/s ({model_name}, random weights)", "value": round(value, 1), "unit": "tokens/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
-            "config": {"model": "TinyLlama-1.1B shapes", "layers": cfg["num_hidden_layers"], "layers_of_model": model_layers,
+            "config": {"model": model_name, "layers": cfg["num_hidden_layers"], "layers_of_model": model_layers,
                        "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                        "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
                        "global_batch": args.batch, "seq_len": args.context, "block_size": 16, "weights": "random seed 0",

@@ -7,13 +7,14 @@
 //   epilogue              plain (bfloat16 or float out) | silu(gate) * up | rotary encoding of q and
 //                         k and the write of k, v into their cache pages
 //
-// One workgroup owns units of 16 weight rows over all of K.  Its wavefronts deal the K slabs of
-// 128 round-robin; per slab a lane issues four 16-byte loads of one weight row, laid out so that the
-// four lanes that share a row read 64 contiguous bytes in each load instruction; the loaded pieces
-// are the A operands of v_mfma_f32_16x16x32_bf16 (the rows use the same k assignment).  The first slab's weights are requested
-// before the prologue runs, so the prologue hides behind HBM latency.  The rows (after the norm)
-// sit in LDS and are the B operand of every wavefront.  Partial sums of the wavefronts are added
-// through LDS in wave order: every output is summed in one fixed order.
+// One workgroup of 8 wavefronts owns units of 16 weight rows over all of K.  Its wavefronts deal the K
+// slabs of 128 round-robin; per slab a lane issues four 16-byte loads of one weight row, laid out so that
+// the four lanes that share a row read 64 contiguous bytes in each load instruction; the loaded pieces are
+// the A operands of v_mfma_f32_16x16x32_bf16 (the rows use the same k assignment).  A wavefront first
+// requests its share of the input rows (cache hits), then the first slabs of weights (HBM), and works on
+// the rows while the weights travel.  The rows (after the norm) sit in LDS and are the B operand of every
+// wavefront.  Partial sums of the wavefronts are added through LDS in wave order: every output is summed
+// in one fixed order.
 #include "common.h"
 
 using namespace pllm;
@@ -129,12 +130,17 @@ __device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, i
 template <int EPI, int WAVES, bool HALF>
 __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p, int num_units) {
   PLLM_STAMP(0);
+  // Fetch the arguments the first loads depend on in one go (left alone, the compiler fetches each where
+  // it is first used, and every fetch is a wait of its own).
+  asm volatile("" ::"s"(p.x), "s"(p.delta), "s"(p.norm_w), "s"(p.row_index), "s"(p.W), "s"(p.x_out), "s"(p.ldx), "s"(p.ldd),
+               "s"(p.ldw), "s"(p.ldxo), "s"(p.M), "s"(p.K), "s"(p.N), "s"(num_units));
+  if (EPI == EPI_ROPE_KV) asm volatile("" ::"s"(p.positions), "s"(p.slots), "s"(p.cos_t), "s"(p.head_dim), "s"(p.num_heads), "s"(p.num_kv_heads));
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int M = p.M, N = p.N, K = p.K;
   const int row_len = K + kPad;
   bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                       // [M][K + kPad]
   float* part = reinterpret_cast<float*>(lds_raw + (((size_t)M * row_len * 2 + 15) & ~(size_t)15));   // [WAVES][256]
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
 
   // ---- request this wavefront's slabs of the first unit, then build the rows in LDS while they travel
@@ -143,62 +149,135 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   const int xrow = HALF ? (r & 7) : r;                          // input row this lane's B operand column belongs to
   const int num_slabs = (K + kStep - 1) / kStep;
   const int my_slabs = wave < num_slabs ? (num_slabs - wave + WAVES - 1) / WAVES : 0;
-  constexpr int PRE = WAVES >= 16 ? 3 : 2;                      // slabs in flight per wavefront (registers)
+  constexpr int PRE = 2;                                        // slabs in flight per wavefront (registers)
   bf16x8 wbuf[PRE][4];
   const bf16* wrow = p.W;
   auto load_w = [&](int nth, bf16x8 (&dst)[4]) {                // nth slab of this wavefront, from wrow
     const int slab = wave + nth * WAVES;
+    // No condition on the loads (the compiler would turn one into a branch around them, and could then no
+    // longer tell how many loads are under way).  Past the end of K a lane rereads the row's last piece,
+    // which meets zeros in the rows' operand; a slab this wavefront does not have is one address for all lanes.
+    const bool mine = nth < my_slabs;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int kk = slab * kStep + khalf + j * 32 + g * 8;
-      dst[j] = (kk < K) ? *reinterpret_cast<const bf16x8*>(wrow + kk) : zero8();
+      dst[j] = *reinterpret_cast<const bf16x8*>(mine ? wrow + min(kk, K - 8) : p.W);
     }
   };
-  auto request_unit = [&](int unit) {
+  auto request_unit = [&](int unit) {                           // PRE slabs, needed or not
     wrow = p.W + (size_t)unit_row<EPI, HALF>(p, unit, r) * p.ldw;
 #pragma unroll
-    for (int s = 0; s < PRE; ++s)
-      if (s < my_slabs) load_w(s, wbuf[s]);
+    for (int s = 0; s < PRE; ++s) load_w(s, wbuf[s]);
   };
-  int unit = blockIdx.x;
-  if (unit < num_units) request_unit(unit);
-  PLLM_STAMP(1);
+  int unit = blockIdx.x;                                        // below num_units: the grid has no more workgroups than units
+
+  // ---- the rows into LDS.  A wavefront owns a group of 64 pieces of 8 columns and walks rows with it, up
+  // to kBatch rows at a time.  It requests the pieces of its first batch, then its weights, and only then
+  // touches the first piece: loads return in the order they were issued, so the rows (cache hits) must not
+  // queue behind the weights (HBM), and the weight loads carry no condition, so that the compiler can
+  // count exactly how many loads may still be under way when a piece is used.  Sums of squares: per lane
+  // over its 8 elements, over the wavefront, then over the column groups of a row in ascending order: one
+  // fixed order, whatever else is in the batch.
+  constexpr int kBatch = 4;
+  const int ipr = ((K >> 3) + 63) >> 6;                         // column groups per row
+  const int cg = min(ipr, WAVES), rpp = WAVES / cg;             // groups and rows under way at a time
+  const int wc = wave % cg, wr = wave / cg;                     // this wavefront's first group and row
+  const bool active = wr < rpp;
+  float* sq = part;                                             // [M][ipr] (the buffer is free until the product ends)
+  int src_lane = lane < M ? lane : 0;                           // lane m holds the source row of input row m
+  if (p.row_index) src_lane = p.row_index[src_lane];
+  const bool has_delta = p.delta != nullptr, has_norm = p.norm_w != nullptr;
+  bf16x8 xv[kBatch], dv[kBatch];
+  float4 nw0, nw1;
+  auto column = [&](int c) { return min((c * 64 + lane) * 8, K - 8); };   // loads stay inside the row ...
+  auto inside = [&](int c) { return (c * 64 + lane) * 8 < K; };           // ... and this says whether they count
+  auto issue = [&](int c, int m0) {                             // rows m0, m0 + rpp, ... of column group c
+    const int k0 = column(c);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, min(m0 + u * rpp, M - 1));
+      xv[u] = *reinterpret_cast<const bf16x8*>(p.x + src * p.ldx + k0);
+    }
+    if (has_delta) {
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, min(m0 + u * rpp, M - 1));
+        dv[u] = *reinterpret_cast<const bf16x8*>(p.delta + src * p.ldd + k0);
+      }
+    }
+  };
+  auto issue_norm = [&](int c) {
+    if (has_norm) {
+      nw0 = *reinterpret_cast<const float4*>(p.norm_w + column(c));
+      nw1 = *reinterpret_cast<const float4*>(p.norm_w + column(c) + 4);
+    }
+  };
+  auto sum_rows = [&](int c, int m0) {                          // pass 1 on the issued batch
+    const int k0 = column(c);
+    const bool in = inside(c);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int m = m0 + u * rpp;
+      if (!active || m >= M) continue;                          // the same for the whole wavefront
+      bf16x8 v = xv[u];
+      if (has_delta) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (__bf16)((float)v[i] + (float)dv[u][i]);     // float sum, rounded once
+        if (p.x_out && blockIdx.x == 0 && in) {
+          const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, m);
+          *reinterpret_cast<bf16x8*>(p.x_out + src * p.ldxo + k0) = v;
+        }
+      }
+      if (in) *reinterpret_cast<bf16x8*>(xs + (size_t)m * row_len + k0) = v;            // as stored in bfloat16
+      if (has_norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
+        ss = wave_sum(in ? ss : 0.f);
+        if (lane == 0) sq[m * ipr + c] = ss;
+      }
+    }
+  };
+  auto scale_rows = [&](int c, int m0) {                        // pass 2 with the norm weights of column group c loaded
+    const int k0 = column(c);
+    if (!active || !inside(c)) return;
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int m = m0 + u * rpp;
+      if (m >= M) continue;
+      float total = 0.f;
+      for (int j = 0; j < ipr; ++j) total += sq[m * ipr + j];
+      const float inv = rsqrtf(total / (float)K + p.eps);
+      bf16* at = xs + (size_t)m * row_len + k0;                 // each lane rereads only what it wrote
+      bf16x8 v = *reinterpret_cast<const bf16x8*>(at);
+      const float w[8] = {nw0.x, nw0.y, nw0.z, nw0.w, nw1.x, nw1.y, nw1.z, nw1.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = (__bf16)(((float)v[i] * inv) * w[i]);
+      *reinterpret_cast<bf16x8*>(at) = v;
+    }
+  };
+
+  issue(wc, wr);
+  issue_norm(wc);
   // Rotary epilogue: what depends only on the input row is fetched now, not after the product.
   int rope_pos = 0, rope_slot = -1;
   if (EPI == EPI_ROPE_KV && tid < 256 && (HALF ? (r & 7) : r) < M && (!HALF || r < 8)) {
     rope_pos = p.cos_t ? p.positions[r] : 0;
     rope_slot = p.slots[r];
   }
-
-  for (int m = wave; m < M; m += WAVES) {
-    const size_t src = p.row_index ? (size_t)p.row_index[m] : (size_t)m;
-    const bf16* xr = p.x + src * p.ldx;
-    bf16* dst = xs + (size_t)m * row_len;
-    float ss = 0.f;
-    // pass 1: the (summed) row goes to LDS exactly as it is stored in bfloat16
-    for (int k0 = lane * 8; k0 < K; k0 += 512) {
-      bf16x8 v = *reinterpret_cast<const bf16x8*>(xr + k0);
-      if (p.delta) {
-        const bf16x8 d = *reinterpret_cast<const bf16x8*>(p.delta + src * p.ldd + k0);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (__bf16)((float)v[i] + (float)d[i]);       // float sum, rounded once
-        if (p.x_out && blockIdx.x == 0) *reinterpret_cast<bf16x8*>(p.x_out + src * p.ldxo + k0) = v;
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
-      *reinterpret_cast<bf16x8*>(dst + k0) = v;
+  request_unit(unit);                                           // the first unit's weights: on their way during all that follows
+  PLLM_STAMP(1);
+  sum_rows(wc, wr);
+  for (int c = wc; c < ipr; c += cg)
+    for (int m0 = (c == wc) ? wr + kBatch * rpp : wr; m0 < M; m0 += kBatch * rpp) {
+      issue(c, m0);
+      sum_rows(c, m0);
     }
-    if (p.norm_w) {
-      // pass 2: scale in place (each lane rereads only what it wrote)
-      const float inv = rsqrtf(wave_sum(ss) / (float)K + p.eps);
-      for (int k0 = lane * 8; k0 < K; k0 += 512) {
-        bf16x8 v = *reinterpret_cast<const bf16x8*>(dst + k0);
-        const float4 w0 = *reinterpret_cast<const float4*>(p.norm_w + k0), w1 = *reinterpret_cast<const float4*>(p.norm_w + k0 + 4);
-        const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (__bf16)(((float)v[i] * inv) * w[i]);
-        *reinterpret_cast<bf16x8*>(dst + k0) = v;
-      }
+  if (has_norm) {
+    __syncthreads();
+    for (int c = wc; c < ipr; c += cg) {
+      if (c != wc) issue_norm(c);
+      for (int m0 = wr; m0 < M; m0 += kBatch * rpp) scale_rows(c, m0);
     }
   }
   __syncthreads();
@@ -316,6 +395,16 @@ PLLM_API long pllm_max_lds_bytes() {
   return v;
 }
 
+// LDS of one compute unit (what resident workgroups share); on this GPU the same as one workgroup's limit.
+static long pllm_lds_bytes_per_cu() {
+  static long bytes = 0;
+  if (!bytes) {
+    const long v = pllm_max_lds_bytes();
+    bytes = v > 0 ? v : 64 * 1024;
+  }
+  return bytes;
+}
+
 // Bytes of LDS a call needs; the caller checks them against the device's limit.
 PLLM_API long pllm_decode_linear_lds_bytes(int M, int K, int waves) {
   const long rows = (((long)M * (K + kPad) * 2) + 15) & ~15L;
@@ -342,7 +431,7 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
                                 void* x_out, int ldxo, const int* row_index, const void* W, int ldw, void* out, int ldo, int M,
                                 int N, int K, const int* positions, const float* cos_t, const float* sin_t, const int* slots,
                                 void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim, int block_size,
-                                hipStream_t stream) {
+                                int tune, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 16 || K <= 0 || (K & 7) || (ldx & 7) || (ldw & 7) || (delta && (ldd & 7)) || (x_out && (ldxo & 7))) return -2;
   DecodeLinearParams p;
@@ -354,8 +443,6 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
 #ifdef PLLM_TRACE
   p.trace = pllm_trace_buffer;
 #endif
-  const int waves = (K >= 4096) ? 16 : 8;
-  const size_t lds = (size_t)pllm_decode_linear_lds_bytes(M, K, waves);
   int units;
   switch (epi) {
     case EPI_BF16: case EPI_F32: units = (N + 15) / 16; break;
@@ -366,15 +453,29 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
       break;
     default: return -3;
   }
-  // Small matrices with at most 8 rows: units of 8 weight rows, so that every compute unit gets one.
-  const bool half = M <= 8 && epi != EPI_GATED && units < num_compute_units() && K >= 512;
+  // Shape of the work.  A unit of 8 weight rows (at most 8 input rows, not the gated product) when that
+  // leaves the busiest compute unit with at most 3/4 of what units of 16 would give it to stream.  One or two workgroups per
+  // compute unit: two overlap one's prologue and reduction with the other's streaming, and are taken when
+  // their rows fit into LDS side by side and the busiest compute unit gets no more units that way; more
+  // units than workgroups are dealt evenly, and a workgroup walks its units with the next one's weights
+  // already on their way.  `tune` overrides the choice for measurements: bit 2/3 = units of 16/8 weight
+  // rows, bit 4/5 = one/two workgroups per compute unit.
+  const int cus = num_compute_units();
+  constexpr int waves = 8;
+  const size_t lds = (size_t)pllm_decode_linear_lds_bytes(M, K, waves);
+  auto ceil_div = [](int a, int b) { return (a + b - 1) / b; };
+  bool half = M <= 8 && epi != EPI_GATED && K >= 512 && 2 * ceil_div(2 * units, cus) <= 3 * ceil_div(units, cus);   // at most 3/4
+  if (tune & 4) half = false;
+  if (tune & 8) half = M <= 8 && epi != EPI_GATED;
   if (half) units *= 2;
-  // Up to two workgroups per compute unit stay resident; more units than that are dealt evenly
-  // to that many workgroups, which walk them with the next unit's weights already on their way.
-  const int resident = 2 * num_compute_units();
-  const int per_block = (units + resident - 1) / resident;
-  const int blocks = (units + per_block - 1) / per_block;
-#define GO(EPI_, HALF_) return waves == 16 ? launch<EPI_, 16, HALF_>(p, units, blocks, lds, stream) : launch<EPI_, 8, HALF_>(p, units, blocks, lds, stream)
+  const int per_block2 = ceil_div(units, 2 * cus), blocks2 = ceil_div(units, per_block2);
+  const int busiest2 = per_block2 * (blocks2 > cus ? 2 : 1), busiest1 = ceil_div(units, cus);
+  bool two = 2 * lds <= (size_t)pllm_lds_bytes_per_cu() && busiest2 <= busiest1;
+  if (tune & 16) two = false;
+  if (tune & 32) two = true;
+  const int per_block = two ? per_block2 : busiest1;
+  const int blocks = ceil_div(units, per_block);
+#define GO(EPI_, HALF_) return launch<EPI_, waves, HALF_>(p, units, blocks, lds, stream)
   if (half) {
     switch (epi) {
       case EPI_BF16: GO(EPI_BF16, true);

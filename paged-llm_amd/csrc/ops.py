@@ -274,7 +274,7 @@ EPI_BF16, EPI_F32, EPI_GATED, EPI_ROPE_KV = 0, 1, 2, 3
 DECODE_MAX_ROWS = 16
 _DECODE_SIG = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
                c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-               c_void_p]
+               c_int, c_void_p]
 _lds_limit: dict = {}
 
 
@@ -295,20 +295,21 @@ def decode_linear_takes(rows: int, K: int, x: torch.Tensor, w: torch.Tensor) -> 
     if not (x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return False
-    waves = 16 if K >= 4096 else 8
+    waves = 8
     need = ((rows * (K + 8) * 2 + 15) // 16) * 16 + waves * 256 * 4
     return need <= _max_lds_bytes(x.device)
 
 
 def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: torch.Tensor | None = None,
                   norm_weight: torch.Tensor | None = None, eps: float = 0.0, x_out: torch.Tensor | None = None,
-                  row_index: torch.Tensor | None = None, rope: dict | None = None) -> torch.Tensor:
+                  row_index: torch.Tensor | None = None, rope: dict | None = None, tune: int = 0) -> torch.Tensor:
     """rows = x[row_index] (+ delta) -> optional RMS norm -> rows W^T -> epilogue, in one kernel.
 
     epi EPI_BF16 / EPI_F32: [M, N] out.  EPI_GATED: w = [gate; up], out = silu(gate) * up [M, N/2].
     EPI_ROPE_KV: w = [q; k; v] rows; q is rotated and returned [M, heads * d]; k (rotated) and v go
     into the cache pages; ``rope`` = dict(positions, cos, sin, slots, k_pages, v_pages, num_heads,
     num_kv_heads, head_dim, block_size).  ``x_out`` receives x + delta (the new residual).
+    ``tune`` (measurements only) overrides the kernel's choice of work shape.
     """
     _on_gpu(x, w, delta, norm_weight, x_out, row_index)
     M = row_index.numel() if row_index is not None else x.shape[0]
@@ -352,7 +353,7 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
              _ptr(x_out), x_out.stride(0) if x_out is not None else 0, _ptr(row_index), _ptr(w), w.stride(0), _ptr(out),
              out.stride(0), M, N, K, _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")),
              _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)),
-             int(r.get("head_dim", 0)), int(r.get("block_size", 0)), _stream()), "decode_linear")
+             int(r.get("head_dim", 0)), int(r.get("block_size", 0)), int(tune), _stream()), "decode_linear")
     return out
 
 
