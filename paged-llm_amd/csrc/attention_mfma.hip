@@ -246,7 +246,11 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   // With several wavefronts per work item the blocks are dealt round-robin; their partial
   // results are merged through LDS below.
   constexpr int kStride = WAVES * 64;
-  if (WAVES > 1) {
+  // Registers of one block: with small heads two blocks fit and the next one travels while the current
+  // one is used; with large heads one block is all there is room for (the caller then sizes partitions
+  // so that a wavefront has a single block).
+  constexpr bool kTwoBlocks = 4 * KSTEPS * 4 + 4 * DBLOCKS * 2 <= 64;
+  if constexpr (WAVES > 1 && kTwoBlocks) {
     KVBlock blk_a, blk_b;
     int n0 = k_lo + wave * 64;
     if (n0 < k_hi) {
@@ -267,7 +271,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     }
   } else {
     KVBlock blk;
-    for (int n0 = k_lo; n0 < k_hi; n0 += 64) {
+    for (int n0 = k_lo + (WAVES > 1 ? wave * 64 : 0); n0 < k_hi; n0 += kStride) {
       load_block(blk, n0);
       compute_block(blk, n0);
     }
@@ -676,7 +680,7 @@ static long pllm_max_lds() {
 static size_t merge_lds_bytes(int ncb, int waves) { return (size_t)(2 * waves * ncb * 16 + waves * ncb * DBLOCKS * 4 * 64) * sizeof(float); }
 
 // waves == 1: every work item is one wavefront that walks its key range.
-// waves in {4, 8, 16}: the wavefronts of a workgroup share the key range of one work item (they take
+// waves in {4, 8}: the wavefronts of a workgroup share the key range of one work item (they take
 //   its blocks of 64 keys in turn, with the next block already requested) and merge through LDS.
 // partition_size == 0: a work item's key range is everything its queries may see; it writes the result.
 // partition_size > 0 (a multiple of 64): num_partitions work items per tile each take one aligned
@@ -700,7 +704,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   else if (column_blocks != 0) return -2;
   const int tiles = (max_cols + 16 * ncb - 1) / (16 * ncb);
   if (num_kv_heads * num_partitions > 65535 || num_seqs > 65535) return -2;
-  if (waves != 1 && waves != 4 && waves != 8 && waves != 16) return -2;
+  if (waves != 1 && waves != 4 && waves != 8) return -2;
   if (waves > 1 && (long)merge_lds_bytes(ncb, waves) > pllm_max_lds()) return -2;
   if (waves == 1 && partition_size == 0 && max_cols > 64 && column_blocks != 1 && column_blocks != 4) {
     // prompt portions: workgroups of four wavefronts that share every block of keys through LDS
@@ -733,7 +737,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
 #define PLLM_BY_WAVES(NCB_)                                                                          \
   do {                                                                                               \
     if (waves == 1) PLLM_LAUNCH(NCB_, 1); else if (waves == 4) PLLM_LAUNCH(NCB_, 4);                 \
-    else if (waves == 8) PLLM_LAUNCH(NCB_, 8); else PLLM_LAUNCH(NCB_, 16);                           \
+    else PLLM_LAUNCH(NCB_, 8);                                                                       \
   } while (0)
   if (ncb == 1) PLLM_BY_WAVES(1); else if (ncb == 2) PLLM_BY_WAVES(2); else PLLM_BY_WAVES(4);
 #undef PLLM_BY_WAVES
@@ -751,7 +755,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
 // Largest number of wavefronts per work item whose merge buffers fit `lds_limit` bytes (0: none).
 PLLM_API int pllm_attention_mfma_max_waves(int max_cols, long lds_limit) {
   const int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
-  for (int w = 16; w >= 4; w /= 2)
+  for (int w = 8; w >= 4; w /= 2)
     if ((long)merge_lds_bytes(ncb, w) <= lds_limit) return w;
   return 0;
 }

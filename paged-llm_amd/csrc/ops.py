@@ -432,14 +432,27 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
     if max_waves < 4:
         return 1, 0, 1
     items = num_seqs * num_kv_heads
-    want_parts = max(1, 384 // items)
-    size = 256                                        # at least four blocks of 64 keys per workgroup
-    while (max_k_len + size - 1) // size > want_parts:
-        size *= 2
+    if 4 * ((head_dim + 31) // 32) * 4 + 4 * (head_dim // 16) * 2 <= 64:
+        # Small heads: a wavefront holds two blocks of 64 keys, one travelling while the other is used, so
+        # it may walk many blocks; partitions only as far as they are needed to fill the GPU.
+        want_parts = max(1, 384 // items)
+        size = 256                                    # at least four blocks of 64 keys per workgroup
+        while (max_k_len + size - 1) // size > want_parts:
+            size *= 2
+        waves = max_waves
+        while waves > 4 and (waves // 2) * 64 >= min(size, max_k_len):
+            waves //= 2
+    else:
+        # Large heads: registers hold one block, so a partition is one block per wavefront: 8 wavefronts
+        # if that still gives every compute unit a workgroup, else 4.  Very long contexts keep the number
+        # of partitions bounded and let the wavefronts walk several blocks.
+        waves = max_waves
+        if waves > 4 and (max_k_len <= 256 or items * ((max_k_len + 511) // 512) < 256):
+            waves = 4
+        size = waves * 64
+        while (max_k_len + size - 1) // size > 128:
+            size *= 2
     parts = (max_k_len + size - 1) // size
-    waves = max_waves
-    while waves > 4 and (waves // 2) * 64 >= min(size, max_k_len):
-        waves //= 2
     return (waves, size, parts) if parts > 1 else (waves, 0, 1)
 
 
@@ -462,7 +475,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
         out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
     _need(out.shape == (T, num_heads * head_dim) and out.stride(1) == 1 and out.dtype == q.dtype and out.stride(0) % 4 == 0,
           "bad attention output")
-    _need(max_q_len >= 1 and partition_size % 64 == 0 and waves in (1, 4, 8, 16), "bad launch parameters")
+    _need(max_q_len >= 1 and partition_size % 64 == 0 and waves in (1, 4, 8), "bad launch parameters")
     ncb = min(column_blocks or 4, 1 if max_q_len * (num_heads // num_kv_heads) <= 16 else (2 if max_q_len * (num_heads // num_kv_heads) <= 32 else 4))
     _need(column_blocks in (0, 1, 2, 4), "column_blocks is 0 (automatic), 1, 2 or 4")
     _need(waves == 1 or (2 * waves * ncb * 16 + waves * ncb * (head_dim // 16) * 4 * 64) * 4 <= _max_lds_bytes(q.device),

@@ -336,7 +336,7 @@ def test_paged_attention_mfma(heads, kv_heads, d, bs, lens, num_q):
     if max(num_q) * (heads // kv_heads) <= 64:
         cols = max(num_q) * (heads // kv_heads)
         ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
-        for waves in (4, 8, 16):
+        for waves in (4, 8):
             if (2 * waves * ncb * 16 + waves * ncb * (d // 16) * 4 * 64) * 4 <= 160 * 1024:
                 assert rel_err(ops().paged_attention_mfma(*args, 0, 1, waves), want) <= 1.6e-2, f"{waves} wavefronts"
                 parts = (max(lens) + 255) // 256
@@ -384,7 +384,7 @@ def test_mfma_attention_one_far_key_stands_out(far):
     q, kp, vp, tables, cu, sl = paged_case([700], [1], heads, kv_heads, d, bs, torch.bfloat16, seed=4)
     page, off = int(tables[0, far // bs]), far % bs
     kp[page, 0, off, :] = (q[0, 5 * d:6 * d].float() * 40).to(torch.bfloat16)       # head 5 looks at that key only
-    for split in ((), (128, 6), (0, 1, 16), (256, 3, 4)):
+    for split in ((), (128, 6), (0, 1, 8), (256, 3, 4)):
         got = ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
                                          d, 1.0, 0, 1, *split).cpu().float()
         assert torch.allclose(got[0, 5 * d:6 * d], vp[page, 0, :, off].float(), atol=2e-2)
@@ -393,13 +393,15 @@ def test_mfma_attention_one_far_key_stands_out(far):
 def test_attention_plan():
     plan = ops().attention_plan
     lds = 160 * 1024
-    assert plan(8, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)       # decoding: partitions for workgroups, blocks for wavefronts
+    assert plan(8, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)       # decoding: partitions for workgroups, one block per wavefront
     assert plan(64, 4, 1, 2048, 8, 64, lds) == (8, 0, 1)         # enough sequences: wavefronts only
     assert plan(1, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)
     assert plan(8, 4, 1, 200, 8, 64, lds) == (4, 0, 1)
     assert plan(1, 4, 2048, 2048, 8, 64, lds) == (1, 0, 1)      # a long prompt portion: one wavefront per query tile
     assert plan(2, 4, 1, 50, 8, 64, lds) == (1, 0, 1)
-    assert plan(1, 8, 1, 100000, 4, 128, lds) == (8, 4096, 25)
+    assert plan(8, 8, 1, 2048, 4, 128, lds) == (8, 512, 4)      # large heads: one block per wavefront
+    assert plan(1, 8, 1, 2048, 4, 128, lds) == (4, 256, 8)
+    assert plan(1, 8, 1, 100000, 4, 128, lds) == (8, 1024, 98)  # bounded number of partitions
 
 
 # ----------------------------------------------------------------------------------- fused decode products
