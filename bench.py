@@ -126,6 +126,66 @@ def time_prefill(engine, tokens: int, seed: int, repeats: int = 3) -> float:
     return best
 
 
+# The reference's own end-to-end workload (benchmarks/bench.py:27-45,109-132 there): 64 prompts of seeded random
+# ids, greedy, exactly `out` tokens each (EOS ignored), at most `batch` requests at a time; output
+# tokens / wall time of generate() including the prompts.  `published` = the reference's numbers on one
+# RTX 4090 in fp16 (benchmarks/results/latest.md there), for orientation only: other hardware.
+E2E_CASES = [
+    dict(name="256in_128out_b1", batch=1, published=135.0), dict(name="256in_128out_b8", batch=8, published=1015.0),
+    dict(name="256in_128out_b32", batch=32, published=3467.0), dict(name="256in_128out_b64", batch=64, published=5827.0),
+    dict(name="ragged_b32", batch=32, var_len=True, published=2691.0), dict(name="ragged_b64", batch=64, var_len=True, published=4210.0),
+    dict(name="shared_prefix_b32", batch=32, shared_prefix=0.75, published=3744.0),
+]
+
+
+def e2e_prompts(num_prompts: int, input_len: int, output_len: int, shared_prefix: float, var_len: bool, vocab: int, seed: int = 0):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    shared_len = int(input_len * shared_prefix)
+    shared = torch.randint(100, vocab, (shared_len,), generator=g).tolist()
+    prompts, out_lens = [], []
+    for _ in range(num_prompts):
+        in_len, out_len = input_len, output_len
+        if var_len:
+            in_len = int(torch.randint(max(shared_len + 1, input_len // 4), input_len + 1, (1,), generator=g))
+            out_len = int(torch.randint(max(1, output_len // 4), output_len + 1, (1,), generator=g))
+        prompts.append(shared + torch.randint(100, vocab, (in_len - shared_len,), generator=g).tolist())
+        out_lens.append(out_len)
+    return prompts, out_lens
+
+
+def run_e2e(cfg: dict, dtype: str) -> dict:
+    import torch
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    results = {}
+    with tempfile.TemporaryDirectory() as folder:
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        for case in E2E_CASES:
+            # a fresh engine per case: nothing of an earlier case's prompts is left in the prefix cache
+            engine = LLMEngine(folder, EngineConfig(block_size=16, num_gpu_blocks=64 * 26 + 64, max_num_seqs=case["batch"],
+                                                    max_num_batched_tokens=4096, max_model_len=256 + 128, dtype=dtype, seed=0,
+                                                    enable_prefix_caching=True), random_weights=0)
+            for seed in (1, 0):                          # other prompts first: that pass captures the graphs this case needs
+                prompts, out_lens = e2e_prompts(64, 256, 128, case.get("shared_prefix", 0.0), case.get("var_len", False), 32000, seed)
+                sps = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True) for n in out_lens]
+                hits0, steps0 = engine.cache_manager.num_cache_hits, engine.stats.num_steps
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                outs = engine.generate(prompts, sps)
+                torch.cuda.synchronize()
+                elapsed = time.perf_counter() - t0
+            assert all(len(o.token_ids) == n for o, n in zip(outs, out_lens))
+            results[case["name"]] = {"output_tok_per_s": round(sum(out_lens) / elapsed, 1), "elapsed_s": round(elapsed, 3),
+                                     "steps": engine.stats.num_steps - steps0,
+                                     "prefix_cache_hits": engine.cache_manager.num_cache_hits - hits0,
+                                     "published_rtx4090_fp16": case["published"]}
+            del engine
+            torch.cuda.empty_cache()
+    return results
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -138,6 +198,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time only the 2048-token prefill (for profiling)")
+    ap.add_argument("--e2e", action="store_true", help="the reference's end-to-end workload (64 requests, 256 in / 128 out) instead")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -153,6 +214,11 @@ def main() -> int:
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     nbytes = 2 if short == "bf16" else 4
     numbers = model_numbers(cfg, nbytes)
+
+    if args.e2e:
+        print(json.dumps({"metric": f"end-to-end output tokens/s ({model_name}, random weights, 64 requests)", "dtype": short,
+                          "unit": "tokens/s", "cases": run_e2e(cfg, args.dtype)}))
+        return 0
 
     with tempfile.TemporaryDirectory() as folder:
         engine = make_engine(cfg, folder, args.dtype, max(64, args.batch), args.context)
