@@ -20,6 +20,7 @@ from __future__ import annotations
 import hashlib
 import struct
 from collections import OrderedDict
+import itertools
 from dataclasses import dataclass, field
 
 NO_PAGE = -1
@@ -143,6 +144,7 @@ class _Holding:
     """What one request holds."""
     tables: dict[str, list[int]]
     state_slot: int | None = None
+    version: int = 0          # a new number whenever any table changes (never reused by another holding)
 
 
 class CacheManager:
@@ -163,6 +165,7 @@ class CacheManager:
         self.slots = StateSlotPool(num_state_slots)
         self.uses_state = num_state_slots > 0
         self._held: dict[object, _Holding] = {}
+        self._versions = itertools.count(1)
         self._pending: dict[str, list[PageCopy]] = {g.name: [] for g in groups}
         self.num_cache_queries = 0
         self.num_cache_hits = 0
@@ -194,6 +197,12 @@ class CacheManager:
 
     def block_table(self, request, group: str) -> list[int]:
         return self._held[request].tables[group]
+
+    def table_version(self, request) -> int:
+        """A number that changes whenever any block table of ``request`` does (a page appended, copied
+        for a write, or given back by a window), and that no other state of any request shares: who
+        has read the tables at this number need not read them again."""
+        return self._held[request].version
 
     def state_slot(self, request) -> int | None:
         h = self._held.get(request)
@@ -262,6 +271,19 @@ class CacheManager:
         first_key = num_computed - g.window + 1
         return max(0, first_key) // self.block_size
 
+    def _nothing_to_do(self, hold: _Holding, num_computed: int, num_new: int, total_pages: int) -> bool:
+        """The usual decode step: the pages are there, the one written to is the request's alone, and
+        no window has moved past a page."""
+        bs = self.block_size
+        idx = num_computed // bs
+        for name, g in self.groups.items():
+            table = hold.tables[name]
+            if g.kind != "full" or len(table) < total_pages:
+                return False
+            if num_new > 0 and num_computed % bs != 0 and self.pools[name].refs[table[idx]] > 1:
+                return False
+        return True
+
     def allocate(self, request, num_computed: int, num_new: int,
                  cached: dict[str, list[int]] | None = None) -> bool:
         """Make ``request`` hold pages for positions [0, num_computed + num_new) in every group
@@ -273,8 +295,10 @@ class CacheManager:
         bs = self.block_size
         hold = self._held.get(request)
         new_request = hold is None
-        cached = cached or {}
         total_pages = self.pages_for(num_computed + num_new)
+        if hold is not None and not cached and self._nothing_to_do(hold, num_computed, num_new, total_pages):
+            return True
+        cached = cached or {}
         plan = {}
         for name, g in self.groups.items():
             pool = self.pools[name]
@@ -307,12 +331,15 @@ class CacheManager:
             if self.uses_state:
                 hold.state_slot = self.slots.acquire()
             self._held[request] = hold
+        changed = new_request
         for name, (hits, need, cow_index, first_needed) in plan.items():
             pool, table = self.pools[name], hold.tables[name]
+            changed = changed or bool(hits) or need > 0 or cow_index is not None
             for i in range(min(first_needed, len(table))):
                 if table[i] != NO_PAGE:
                     pool.drop(table[i])
                     table[i] = NO_PAGE
+                    changed = True
             for p in hits:
                 pool.share(p)
             table.extend(hits)
@@ -325,6 +352,8 @@ class CacheManager:
                 self._pending[name].append(PageCopy(shared, fresh))
                 pool.drop(shared)
                 table[cow_index] = fresh
+        if changed:
+            hold.version = next(self._versions)
         return True
 
     def fork(self, parent, child) -> None:
@@ -345,6 +374,7 @@ class CacheManager:
                         if p != NO_PAGE:
                             self.pools[name].drop(p)
                 raise RuntimeError("no free state slot for a fork")
+        hold.version = next(self._versions)
         self._held[child] = hold
 
     def free(self, request) -> None:

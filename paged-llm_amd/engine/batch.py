@@ -22,6 +22,10 @@ class StepEntry:
     block_tables: dict             # group name -> list of page ids (NO_PAGE where a window has passed)
     state_slot: int | None = None
     want: list = field(default_factory=list)   # indices into `tokens` whose logits are returned
+    # Optional: a value that is different whenever the block tables differ from what an earlier entry of
+    # this request held (the cache manager's table_version).  The step function may then skip reading
+    # tables it has already staged; None means "always read".
+    table_version: object = None
 
 
 @dataclass

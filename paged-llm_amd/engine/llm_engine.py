@@ -161,7 +161,8 @@ class LLMEngine:
             entries.append(StepEntry(
                 req.request_id, req.token_ids[start:start + n], start,
                 {g: self.cache_manager.block_table(req.request_id, g) for g in self.groups},
-                self.cache_manager.state_slot(req.request_id), [n - 1] if item.needs_sampling else []))
+                self.cache_manager.state_slot(req.request_id), [n - 1] if item.needs_sampling else [],
+                self.cache_manager.table_version(req.request_id)))
             if item.needs_sampling:
                 sampled_items.append(req)
         logits = self.runner.step(entries, self.cache_manager.take_pending_copies())

@@ -246,15 +246,85 @@ class ModelRunner:
         self._graphs[key] = entry
         return entry
 
+    def _restage_decode(self, entry: dict, entries: list) -> None:
+        """Write a decode step's arrays into the pinned buffer of its graph, in the layout of
+        ``_stage_decode`` and with the same checks, but reading only the block tables that changed
+        since the buffer was last written: the buffer keeps the rows of the step before, and an entry
+        whose ``table_version`` is the one staged in its row leaves that row alone."""
+        bs, S = self.block_size, len(entries)
+        vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions
+        view, offsets, sizes = entry["view"], entry["offsets"], entry["sizes"]
+        ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=S)
+        starts = np.fromiter((e.start for e in entries), dtype=np.int64, count=S)
+        rids = [e.request_id for e in entries]
+        if len(set(rids)) != S:
+            raise StepError("a request appears twice in one step")
+        if ids.min() < 0 or ids.max() >= vocab:
+            raise StepError(f"token id outside [0, {vocab})")
+        if starts.min() < 0 or starts.max() + 1 > max_pos:
+            raise StepError(f"a position exceeds the model's {max_pos} positions")
+        logits_idx = []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                if w != 0:
+                    raise StepError(f"request {e.request_id!r}: wanted row {w} outside its 1 token")
+                logits_idx.append(i)
+        slots_state = np.fromiter((-1 if e.state_slot is None else e.state_slot for e in entries), dtype=np.int32, count=S)
+        if self.states and (slots_state < 0).any():
+            raise StepError("this model keeps per-request state: every entry needs a state slot")
+        k_lens = starts + 1
+        need = (k_lens + bs - 1) // bs
+        staged = entry["staged_rows"]                 # per row: (request id, table version) as last written
+        stale = [s for s, e in enumerate(entries) if e.table_version is None or staged[s] != (rids[s], e.table_version)]
+
+        def put(i, values):
+            view[offsets[i]: offsets[i] + sizes[i]] = values
+
+        put(0, ids); put(1, starts); put(3, k_lens); put(4, slots_state); put(5, starts); put(6, logits_idx)
+        for gi, (name, cs) in enumerate(self.group_specs.items()):
+            num_pages = self.kv.num_pages[name]
+            fixed = entry["table_shapes"][name][1]
+            tables = view[offsets[7 + 2 * gi]: offsets[7 + 2 * gi] + S * fixed].reshape(S, fixed)
+            held = entry["table_lens"][name]
+            for s in stale:
+                e = entries[s]
+                table = e.block_tables.get(name)
+                if table is None:
+                    raise StepError(f"request {e.request_id!r} has no block table for cache group {name!r}")
+                n = min(len(table), fixed)
+                row = np.asarray(table[:n], dtype=np.int64)
+                first_key = max(0, e.start - cs.window + 1) if cs.window > 0 else 0
+                live = row[first_key // bs:]
+                if live.size and (live.min() < 0 or live.max() >= num_pages):
+                    raise StepError(f"request {e.request_id!r}: page id outside [0, {num_pages}) in group {name!r}")
+                tables[s, :n] = np.where(row == NO_PAGE, 0, row)
+                tables[s, n:] = 0
+                held[s] = n
+            short = need > held
+            if short.any():
+                s = int(np.argmax(short))
+                raise StepError(f"request {rids[s]!r}: too few pages in group {name!r} for {int(k_lens[s])} positions")
+            last_page = tables[np.arange(S), need - 1].astype(np.int64)
+            put(8 + 2 * gi, last_page * bs + starts % bs)
+        for s in stale:
+            staged[s] = (rids[s], entries[s].table_version)
+
     def _graph_step(self, key, entries: list) -> torch.Tensor:
         S, n_want, bound = key
-        buf, offsets, sizes, host = self._stage(entries, fixed_blocks=(bound + self.block_size - 1) // self.block_size)
         entry = self._graphs.get(key)
         if entry is None:
+            buf, offsets, sizes, host = self._stage(entries, fixed_blocks=(bound + self.block_size - 1) // self.block_size)
             entry = self._capture(key, buf, offsets, sizes, host)
-        assert entry["offsets"] == offsets and entry["sizes"] == sizes
-        entry["pinned"].numpy()[:] = buf
+            entry["view"] = entry["pinned"].numpy()
+            entry["table_shapes"] = host["table_shapes"]
+            entry["staged_rows"] = [None] * S
+            entry["table_lens"] = {name: np.zeros(S, dtype=np.int64) for name in self.group_specs}
+            entry["copied"] = torch.cuda.Event()
+        else:
+            entry["copied"].synchronize()                  # the last step's copy has left the pinned buffer
+        self._restage_decode(entry, entries)
         entry["static"].copy_(entry["pinned"], non_blocking=True)
+        entry["copied"].record()
         entry["graph"].replay()
         return entry["logits"].clone()
 

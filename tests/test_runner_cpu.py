@@ -90,3 +90,66 @@ def test_bad_batches_are_refused_before_anything_runs(runtime, fast):
     with pytest.raises(StepError):
         runner._stage([], fixed)
     manager.free("ok")
+
+
+def test_decode_steps_restaged_in_place_equal_fresh_staging(runtime):
+    """Graph replays rewrite their pinned buffer in place and skip block tables whose version they
+    have already staged: over steps with requests that grow, end, and are replaced in their row, the
+    buffer must equal a fresh staging of every step."""
+    manager, runner = runtime
+    g = next(iter(manager.groups))
+    rng = np.random.default_rng(3)
+    live = {}                                            # row -> [request id, next position]
+    serial = skipped = 0
+    entry = None
+    for step in range(60):
+        for row in range(3):
+            if row not in live or live[row][1] >= 40 or rng.random() < 0.08:
+                if row in live:
+                    manager.free(live[row][0])
+                serial += 1
+                rid, start = f"q{serial}", int(rng.integers(0, 20))
+                if start:
+                    assert manager.allocate(rid, 0, start)
+                live[row] = [rid, start]
+        entries = []
+        for row in range(3):
+            rid, start = live[row]
+            assert manager.allocate(rid, start, 1)
+            entries.append(StepEntry(rid, [int(rng.integers(0, 256))], start, {g: manager.block_table(rid, g)}, None,
+                                     [0] if row != 1 else [], manager.table_version(rid)))
+            live[row][1] = start + 1
+        fresh, offsets, sizes, host = runner._stage_decode(entries, 4)
+        if entry is None:
+            entry = dict(view=fresh.copy(), offsets=offsets, sizes=sizes, table_shapes=host["table_shapes"],
+                         staged_rows=[None] * 3, table_lens={g: np.zeros(3, dtype=np.int64)})
+            entry["view"][offsets[7]: offsets[7] + sizes[7]] = -7          # nothing of the first staging may be relied on
+        before = list(entry["staged_rows"])
+        runner._restage_decode(entry, entries)
+        assert np.array_equal(entry["view"], fresh), f"step {step}"
+        skipped += sum(before[r] == entry["staged_rows"][r] for r in range(3))
+    assert skipped > 90                                  # most rows were left alone
+    # a table that did not grow although the position needs another page is refused
+    rid, start = live[0]
+    bad = StepEntry(rid, [1], 63, {g: manager.block_table(rid, g)}, None, [0], manager.table_version(rid))
+    others = [StepEntry(live[r][0], [1], live[r][1], {g: manager.block_table(live[r][0], g)}, None,
+                        [0] if r != 1 else [], manager.table_version(live[r][0])) for r in (1, 2)]
+    with pytest.raises(StepError, match="too few pages"):
+        runner._restage_decode(entry, [bad] + others)
+    for row in range(3):
+        manager.free(live[row][0])
+
+
+def test_table_version_changes_exactly_when_a_table_does(runtime):
+    manager, _ = runtime
+    assert manager.allocate("v", 0, 5)
+    v0 = manager.table_version("v")
+    assert manager.allocate("v", 5, 1) and manager.table_version("v") == v0          # same page
+    assert manager.allocate("v", 6, 10) and manager.table_version("v") == v0         # still the first page
+    assert manager.allocate("v", 16, 1) and manager.table_version("v") != v0         # a second page
+    v1 = manager.table_version("v")
+    manager.fork("v", "w")
+    assert manager.table_version("w") not in (v0, v1)
+    assert manager.allocate("w", 17, 1)                                               # writes into a shared page: copy
+    assert manager.table_version("w") != manager.table_version("v") and manager.take_pending_copies()
+    manager.free("v"); manager.free("w")
