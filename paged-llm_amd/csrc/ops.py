@@ -431,27 +431,16 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
         max_waves //= 2
     if max_waves < 4:
         return 1, 0, 1
+    # Partitions only as far as they are needed to fill the GPU: fewer, longer work items are faster than
+    # many short ones plus a larger merge (measured for head sizes 64 and 128).
     items = num_seqs * num_kv_heads
-    if 4 * ((head_dim + 31) // 32) * 4 + 4 * (head_dim // 16) * 2 <= 64:
-        # Small heads: a wavefront holds two blocks of 64 keys, one travelling while the other is used, so
-        # it may walk many blocks; partitions only as far as they are needed to fill the GPU.
-        want_parts = max(1, 384 // items)
-        size = 256                                    # at least four blocks of 64 keys per workgroup
-        while (max_k_len + size - 1) // size > want_parts:
-            size *= 2
-        waves = max_waves
-        while waves > 4 and (waves // 2) * 64 >= min(size, max_k_len):
-            waves //= 2
-    else:
-        # Large heads: registers hold one block, so a partition is one block per wavefront: 8 wavefronts
-        # if that still gives every compute unit a workgroup, else 4.  Very long contexts keep the number
-        # of partitions bounded and let the wavefronts walk several blocks.
-        waves = max_waves
-        if waves > 4 and (max_k_len <= 256 or items * ((max_k_len + 511) // 512) < 256):
-            waves = 4
-        size = waves * 64
-        while (max_k_len + size - 1) // size > 128:
-            size *= 2
+    want_parts = max(1, 384 // items)
+    size = 256                                        # at least four blocks of 64 keys per workgroup
+    while (max_k_len + size - 1) // size > want_parts:
+        size *= 2
+    waves = max_waves
+    while waves > 4 and (waves // 2) * 64 >= min(size, max_k_len):
+        waves //= 2
     parts = (max_k_len + size - 1) // size
     return (waves, size, parts) if parts > 1 else (waves, 0, 1)
 

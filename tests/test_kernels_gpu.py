@@ -393,15 +393,14 @@ def test_mfma_attention_one_far_key_stands_out(far):
 def test_attention_plan():
     plan = ops().attention_plan
     lds = 160 * 1024
-    assert plan(8, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)       # decoding: partitions for workgroups, one block per wavefront
+    assert plan(8, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)       # decoding: partitions for workgroups, blocks for wavefronts
     assert plan(64, 4, 1, 2048, 8, 64, lds) == (8, 0, 1)         # enough sequences: wavefronts only
     assert plan(1, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)
     assert plan(8, 4, 1, 200, 8, 64, lds) == (4, 0, 1)
     assert plan(1, 4, 2048, 2048, 8, 64, lds) == (1, 0, 1)      # a long prompt portion: one wavefront per query tile
     assert plan(2, 4, 1, 50, 8, 64, lds) == (1, 0, 1)
-    assert plan(8, 8, 1, 2048, 4, 128, lds) == (8, 512, 4)      # large heads: one block per wavefront
-    assert plan(1, 8, 1, 2048, 4, 128, lds) == (4, 256, 8)
-    assert plan(1, 8, 1, 100000, 4, 128, lds) == (8, 1024, 98)  # bounded number of partitions
+    assert plan(8, 8, 1, 2048, 4, 128, lds) == (8, 512, 4)
+    assert plan(1, 8, 1, 100000, 4, 128, lds) == (8, 4096, 25)
 
 
 # ----------------------------------------------------------------------------------- fused decode products
