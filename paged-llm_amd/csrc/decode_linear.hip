@@ -127,7 +127,7 @@ __device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, i
 #define PLLM_STAMP(i) do { } while (0)
 #endif
 
-template <int EPI, int WAVES, bool HALF>
+template <int EPI, int WAVES, bool HALF, bool DIRECT>
 __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p, int num_units) {
   PLLM_STAMP(0);
   // Fetch the arguments the first loads depend on in one go (left alone, the compiler fetches each where
@@ -138,8 +138,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int M = p.M, N = p.N, K = p.K;
   const int row_len = K + kPad;
-  bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                       // [M][K + kPad]
-  float* part = reinterpret_cast<float*>(lds_raw + (((size_t)M * row_len * 2 + 15) & ~(size_t)15));   // [WAVES][256]
+  bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                       // [M][K + kPad] (not DIRECT)
+  float* part = reinterpret_cast<float*>(lds_raw + (DIRECT ? 0 : (((size_t)M * row_len * 2 + 15) & ~(size_t)15)));   // [WAVES][256]
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
 
@@ -164,13 +164,49 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
       dst[j] = *reinterpret_cast<const bf16x8*>(mine ? wrow + min(kk, K - 8) : p.W);
     }
   };
+  // DIRECT (rows that need no sum and no norm): the rows' operand comes straight from memory with the
+  // weights of the same slab and never passes through LDS.  Tile columns past M read row M - 1; what they
+  // produce is never stored.
+  bf16x8 xbuf[DIRECT ? PRE : 1][4];
+  const bf16* xsrc = p.x;
+  if (DIRECT) {
+    const int row = min(xrow, M - 1);
+    xsrc = p.x + (size_t)(p.row_index ? p.row_index[row] : row) * p.ldx;
+  }
+  auto load_x = [&](int nth, bf16x8 (&dst)[4]) {
+    const int slab = wave + nth * WAVES;
+    const bool mine = nth < my_slabs;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kk = slab * kStep + khalf + j * 32 + g * 8;
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(mine ? xsrc + min(kk, K - 8) : p.x);
+      dst[j] = kk < K ? v : zero8();                            // zeros past the end of K (the weights reread their last piece there)
+    }
+  };
   auto request_unit = [&](int unit) {                           // PRE slabs, needed or not
     wrow = p.W + (size_t)unit_row<EPI, HALF>(p, unit, r) * p.ldw;
+    if (DIRECT) {
+#pragma unroll
+      for (int s = 0; s < PRE; ++s) load_x(s, xbuf[s]);
+    }
 #pragma unroll
     for (int s = 0; s < PRE; ++s) load_w(s, wbuf[s]);
   };
   int unit = blockIdx.x;                                        // below num_units: the grid has no more workgroups than units
 
+  // Rotary epilogue: what depends only on the input row is fetched early, not after the product.
+  int rope_pos = 0, rope_slot = -1;
+  auto rope_inputs = [&]() {
+    if (EPI == EPI_ROPE_KV && tid < 256 && (HALF ? (r & 7) : r) < M && (!HALF || r < 8)) {
+      rope_pos = p.cos_t ? p.positions[r] : 0;
+      rope_slot = p.slots[r];
+    }
+  };
+  if constexpr (DIRECT) {
+    rope_inputs();
+    request_unit(unit);
+    PLLM_STAMP(1);
+  } else {
   // ---- the rows into LDS.  A wavefront owns a group of 64 pieces of 8 columns and walks rows with it, up
   // to kBatch rows at a time.  It requests the pieces of its first batch, then its weights, and only then
   // touches the first piece: loads return in the order they were issued, so the rows (cache hits) must not
@@ -259,12 +295,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
 
   issue(wc, wr);
   issue_norm(wc);
-  // Rotary epilogue: what depends only on the input row is fetched now, not after the product.
-  int rope_pos = 0, rope_slot = -1;
-  if (EPI == EPI_ROPE_KV && tid < 256 && (HALF ? (r & 7) : r) < M && (!HALF || r < 8)) {
-    rope_pos = p.cos_t ? p.positions[r] : 0;
-    rope_slot = p.slots[r];
-  }
+  rope_inputs();
   request_unit(unit);                                           // the first unit's weights: on their way during all that follows
   PLLM_STAMP(1);
   sum_rows(wc, wr);
@@ -281,9 +312,11 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
     }
   }
   __syncthreads();
+  }
   PLLM_STAMP(2);
 
-  auto x_operand = [&](int nth, int j) {
+  auto x_operand = [&](int nth, int j, int s) {
+    if (DIRECT) return xbuf[s][j];
     const int kk = (wave + nth * WAVES) * kStep + khalf + j * 32 + g * 8;
     return (xrow < M && kk < K) ? *reinterpret_cast<const bf16x8*>(xs + (size_t)xrow * row_len + kk) : zero8();
   };
@@ -312,8 +345,11 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
         if (nth >= my_slabs) break;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[s][j], x_operand(nth, j), acc, 0, 0, 0);
-        if (nth + PRE < my_slabs) load_w(nth + PRE, wbuf[s]);   // keep PRE slabs in flight
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[s][j], x_operand(nth, j, s), acc, 0, 0, 0);
+        if (nth + PRE < my_slabs) {                             // keep PRE slabs in flight
+          if (DIRECT) load_x(nth + PRE, xbuf[s]);
+          load_w(nth + PRE, wbuf[s]);
+        }
       }
     }
     PLLM_STAMP(3);
@@ -376,9 +412,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   }
 }
 
-template <int EPI, int WAVES, bool HALF>
+template <int EPI, int WAVES, bool HALF, bool DIRECT>
 static int launch(const DecodeLinearParams& p, int units, int blocks, size_t lds, hipStream_t stream) {
-  auto kernel = decode_linear_kernel<EPI, WAVES, HALF>;
+  auto kernel = decode_linear_kernel<EPI, WAVES, HALF, DIRECT>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -459,10 +495,13 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   // their rows fit into LDS side by side and the busiest compute unit gets no more units that way; more
   // units than workgroups are dealt evenly, and a workgroup walks its units with the next one's weights
   // already on their way.  `tune` overrides the choice for measurements: bit 2/3 = units of 16/8 weight
-  // rows, bit 4/5 = one/two workgroups per compute unit.
+  // rows, bit 4/5 = one/two workgroups per compute unit, bit 6 = rows through LDS even without a sum or norm.
   const int cus = num_compute_units();
   constexpr int waves = 8;
-  const size_t lds = (size_t)pllm_decode_linear_lds_bytes(M, K, waves);
+  // Rows that need no sum and no norm are read straight from memory (no LDS for them, any K).
+  bool direct = !delta && !norm_w;
+  if (tune & 64) direct = false;
+  const size_t lds = direct ? (size_t)waves * 256 * sizeof(float) : (size_t)pllm_decode_linear_lds_bytes(M, K, waves);
   auto ceil_div = [](int a, int b) { return (a + b - 1) / b; };
   bool half = M <= 8 && epi != EPI_GATED && K >= 512 && 2 * ceil_div(2 * units, cus) <= 3 * ceil_div(units, cus);   // at most 3/4
   if (tune & 4) half = false;
@@ -475,7 +514,7 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   if (tune & 32) two = true;
   const int per_block = two ? per_block2 : busiest1;
   const int blocks = ceil_div(units, per_block);
-#define GO(EPI_, HALF_) return launch<EPI_, waves, HALF_>(p, units, blocks, lds, stream)
+#define GO(EPI_, HALF_) return direct ? launch<EPI_, waves, HALF_, true>(p, units, blocks, lds, stream) : launch<EPI_, waves, HALF_, false>(p, units, blocks, lds, stream)
   if (half) {
     switch (epi) {
       case EPI_BF16: GO(EPI_BF16, true);

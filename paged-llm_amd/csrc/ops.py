@@ -288,13 +288,19 @@ def _max_lds_bytes(device) -> int:
     return _lds_limit[key]
 
 
-def decode_linear_takes(rows: int, K: int, x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether the fused decode product takes these operands (else the caller runs the parts apart)."""
+def decode_linear_takes(rows: int, K: int, x: torch.Tensor, w: torch.Tensor, staged: bool = True) -> bool:
+    """Whether the fused decode product takes these operands (else the caller runs the parts apart).
+    ``staged``: a residual sum or a norm runs in front, so the rows must fit into LDS; plain rows are read
+    straight from memory and may be of any length."""
     if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < rows <= DECODE_MAX_ROWS and K % 8 == 0):
         return False
     if not (x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return False
+    if not staged:
+        # With more than 8 rows every unit rereads as many bytes of rows as it streams of weights; for long
+        # rows the library's product is then faster (measured at K = 5632 and 14336).
+        return rows <= 8 or K <= 4096
     waves = 8
     need = ((rows * (K + 8) * 2 + 15) // 16) * 16 + waves * 256 * 4
     return need <= _max_lds_bytes(x.device)
@@ -315,7 +321,9 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
     M = row_index.numel() if row_index is not None else x.shape[0]
     K = x.shape[1]
     _need(x.dim() == 2 and w.dim() == 2 and w.shape[1] == K, f"decode_linear shapes {tuple(x.shape)} x {tuple(w.shape)}^T")
-    _need(decode_linear_takes(M, K, x, w), "decode_linear takes bfloat16, 1..16 rows, K a multiple of 8, rows that fit LDS")
+    staged = delta is not None or norm_weight is not None or bool(tune & 64)
+    _need(decode_linear_takes(M, K, x, w, staged),
+          "decode_linear takes bfloat16, 1..16 rows, K a multiple of 8, and with a sum or norm in front rows that fit LDS")
     if delta is not None:
         _need(delta.shape == x.shape and delta.dtype == x.dtype and delta.stride(1) == 1 and delta.stride(0) % 8 == 0
               and delta.data_ptr() % 16 == 0, "delta must match x")

@@ -28,7 +28,7 @@ def _fused(x, weight: torch.Tensor, epi: int, rope: dict | None = None):
             x.fused_done(args)
             return out
         x = x.rows()
-    if x.dtype == torch.bfloat16 and ops.decode_linear_takes(x.shape[0], x.shape[1], x, weight):
+    if x.dtype == torch.bfloat16 and ops.decode_linear_takes(x.shape[0], x.shape[1], x, weight, staged=False):
         return ops.decode_linear(x, weight, epi, rope=rope)
     return None
 
