@@ -186,6 +186,68 @@ def run_e2e(cfg: dict, dtype: str) -> dict:
     return results
 
 
+# The reference's attention micro-benchmark (benchmarks/bench_kernel.py:31-33 there): its cases at its shape
+# (32 heads / 8 kv heads / head size 128, pages of 16) and at TinyLlama's; `published` = microseconds of the
+# reference's Triton kernel on one RTX 4090 in fp16 (benchmarks/results/kernel.md there), other hardware.
+ATTENTION_PUBLISHED = {("decode", 1, 512): 39, ("decode", 1, 2048): 135, ("decode", 1, 8192): 445, ("decode", 8, 512): 50,
+                       ("decode", 8, 2048): 162, ("decode", 8, 8192): 529, ("decode", 32, 512): 125, ("decode", 32, 2048): 425,
+                       ("decode", 32, 8192): 1479, ("decode", 64, 512): 208, ("decode", 64, 2048): 669, ("decode", 64, 8192): 2540,
+                       ("prefill", 1, 512): 66, ("prefill", 1, 2048): 526, ("chunked_prefill_512_new", 4, 2048): 808}
+
+
+def run_attention_cases() -> dict:
+    """Microseconds per call of the attention op (kernel + merge where keys are partitioned), timed as replays of
+    a HIP graph that holds calls on several copies of the cache, so that caches do not flatter."""
+    import types
+    import torch
+    from paged_llm_amd.csrc import ops
+    cases = [("decode", b, ctx, 1) for b in (1, 8, 32, 64) for ctx in (512, 2048, 8192)]
+    cases += [("prefill", 1, n, n) for n in (512, 2048)] + [("chunked_prefill_512_new", 4, 2048, 512)]
+    out = {}
+    for label, (nh, nkv, d) in (("h32_kv8_d128", (32, 8, 128)), ("h32_kv4_d64", (32, 4, 64))):
+        rows = {}
+        for name, S, ctx, T in cases:
+            bs = 16
+            pages_per = (ctx + bs - 1) // bs
+            P = S * pages_per
+            kv_bytes = S * ctx * nkv * d * 2 * 2
+            copies = max(2, min(6, int(1.0e9 // kv_bytes)))
+            g = torch.Generator(device="cuda").manual_seed(0)
+            kps = [torch.randn(P, nkv, bs, d, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(copies)]
+            vps = [torch.randn(P, nkv, d, bs, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(copies)]
+            tables = torch.randperm(P, device="cuda", generator=g).to(torch.int32).view(S, pages_per)
+            q = torch.randn(S * T, nh * d, device="cuda", dtype=torch.bfloat16, generator=g)
+            cu = torch.arange(0, S * T + 1, T, device="cuda", dtype=torch.int32)
+            sl = torch.full((S,), ctx, device="cuda", dtype=torch.int32)
+            ctx_info = types.SimpleNamespace(num_seqs=S, max_q_len=T, max_k_len=ctx)
+            fn = lambda i: ops.paged_attention(q, kps[i % copies], vps[i % copies], tables, cu, sl, nh, nkv, d, d ** -0.5, 0, ctx_info)
+            fn(0)
+            torch.cuda.synchronize()
+            stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(2 * copies):
+                    fn(i)
+            graph.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                graph.replay()
+            torch.cuda.synchronize()
+            us = (time.perf_counter() - t0) / (10 * copies) * 1e6
+            row = {"us": round(us, 1)}
+            if T == 1:
+                row["kv_gb_per_s"] = round(kv_bytes / us / 1e3, 1)
+            else:
+                pairs = S * sum(ctx - T + i + 1 for i in range(T))
+                row["tflops"] = round(4 * nh * d * pairs / us / 1e6, 1)
+            if label == "h32_kv8_d128":
+                row["published_rtx4090_fp16_us"] = ATTENTION_PUBLISHED[(name, S, ctx)]
+            rows[f"{name}_b{S}_ctx{ctx}"] = row
+            del kps, vps
+        out[label] = rows
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -198,6 +260,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time only the 2048-token prefill (for profiling)")
+    ap.add_argument("--attention", action="store_true", help="the reference's attention micro-benchmark cases instead")
     ap.add_argument("--e2e", action="store_true", help="the reference's end-to-end workload (64 requests, 256 in / 128 out) instead")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -215,6 +278,9 @@ def main() -> int:
     nbytes = 2 if short == "bf16" else 4
     numbers = model_numbers(cfg, nbytes)
 
+    if args.attention:
+        print(json.dumps({"metric": "attention op, microseconds per call (bf16, pages of 16 positions)", "cases": run_attention_cases()}))
+        return 0
     if args.e2e:
         print(json.dumps({"metric": f"end-to-end output tokens/s ({model_name}, random weights, 64 requests)", "dtype": short,
                           "unit": "tokens/s", "cases": run_e2e(cfg, args.dtype)}))
