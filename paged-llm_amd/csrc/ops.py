@@ -31,12 +31,19 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
 
 
-def _stream() -> c_void_p:
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
-def _ptr(t: torch.Tensor | None) -> c_void_p:
-    return c_void_p(0) if t is None else c_void_p(t.data_ptr())
+def _stream():
+    """The current HIP stream of the current device, as what ctypes passes for a pointer."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
 
 
 def _check(code: int, what: str) -> None:
@@ -74,7 +81,7 @@ _FUNCS: dict = {}
 
 
 def _fn(source: str, name: str, defines: dict | None = None, signature: list | None = None):
-    key = (source, name, tuple(sorted((defines or {}).items())))
+    key = (source, name, tuple(sorted(defines.items()))) if defines else (source, name)
     f = _FUNCS.get(key)
     if f is None:
         lib = build.load_library(source, defines)
