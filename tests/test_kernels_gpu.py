@@ -390,6 +390,36 @@ def test_mfma_attention_one_far_key_stands_out(far):
         assert torch.allclose(got[0, 5 * d:6 * d], vp[page, 0, :, off].float(), atol=2e-2)
 
 
+@pytest.mark.parametrize("heads,kv_heads,d", [(32, 4, 64), (8, 2, 128), (6, 1, 96)])
+@pytest.mark.parametrize("batch", [1, 9])
+def test_long_contexts_through_the_planned_launch(heads, kv_heads, d, batch):
+    """Decoding at contexts of thousands of keys, launched as the engine launches it (partitions, wavefronts
+    and merge as planned for the batch).  In every sequence one head looks at one key only, somewhere among
+    the thousands (the first, both sides of a block and of a partition edge, the last): its output must be
+    that key's value.  All heads of the first and the last sequence are compared with dense attention."""
+    import types
+    bs = 16
+    lens = [6000 + 517 * i for i in range(batch)]
+    q, kp, vp, tables, cu, sl = paged_case(lens, [1] * batch, heads, kv_heads, d, bs, torch.bfloat16, seed=9)
+    far = [0, 63, 64, 255, 256, 4095, 4096, 5999, 2048][:batch]
+    for s, n in enumerate(far):
+        page, off = int(tables[s, n // bs]), n % bs
+        head = s % heads
+        kp[page, head // (heads // kv_heads), off, :] = (q[s, head * d:(head + 1) * d].float() * 40).to(torch.bfloat16)
+    ctx = types.SimpleNamespace(num_seqs=batch, max_q_len=1, max_k_len=max(lens))
+    got = ops().paged_attention(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d,
+                                1.0, 0, ctx).cpu().float()
+    for s, n in enumerate(far):
+        page, off = int(tables[s, n // bs]), n % bs
+        head = s % heads
+        assert torch.allclose(got[s, head * d:(head + 1) * d], vp[page, head // (heads // kv_heads), :, off].float(), atol=2e-2), \
+            f"sequence {s}: key {n} of {lens[s]}"
+    pick = sorted({0, batch - 1})                              # dense attention of the first and the last sequence
+    want = dense_attention(q[pick], kp, vp, tables[pick], torch.arange(len(pick) + 1, dtype=torch.int32), sl[pick], heads,
+                           kv_heads, d, 1.0)
+    assert rel_err(got[pick], want) <= 1.6e-2
+
+
 def test_attention_plan():
     plan = ops().attention_plan
     lds = 160 * 1024
