@@ -154,21 +154,26 @@ def e2e_prompts(num_prompts: int, input_len: int, output_len: int, shared_prefix
     return prompts, out_lens
 
 
-def run_e2e(cfg: dict, dtype: str) -> dict:
+def run_e2e(cfg: dict, dtype: str, cases: list, num_prompts: int = 64, input_len: int = 256, output_len: int = 128,
+            block_size: int = 16, max_num_batched_tokens: int = 4096, prefix_caching: bool = True) -> dict:
     import torch
     from paged_llm_amd import EngineConfig, SamplingParams
     from paged_llm_amd.engine.llm_engine import LLMEngine
     results = {}
+    vocab = min(cfg["vocab_size"], 32000)
+    pages_per_request = (input_len + output_len + block_size - 1) // block_size + 1
     with tempfile.TemporaryDirectory() as folder:
         with open(os.path.join(folder, "config.json"), "w") as f:
             json.dump(cfg, f)
-        for case in E2E_CASES:
+        for case in cases:
             # a fresh engine per case: nothing of an earlier case's prompts is left in the prefix cache
-            engine = LLMEngine(folder, EngineConfig(block_size=16, num_gpu_blocks=64 * 26 + 64, max_num_seqs=case["batch"],
-                                                    max_num_batched_tokens=4096, max_model_len=256 + 128, dtype=dtype, seed=0,
-                                                    enable_prefix_caching=True), random_weights=0)
+            engine = LLMEngine(folder, EngineConfig(
+                block_size=block_size, num_gpu_blocks=max(num_prompts, case["batch"]) * pages_per_request + 64,
+                max_num_seqs=case["batch"], max_num_batched_tokens=max_num_batched_tokens, max_model_len=input_len + output_len,
+                dtype=dtype, seed=0, enable_prefix_caching=prefix_caching), random_weights=0)
             for seed in (1, 0):                          # other prompts first: that pass captures the graphs this case needs
-                prompts, out_lens = e2e_prompts(64, 256, 128, case.get("shared_prefix", 0.0), case.get("var_len", False), 32000, seed)
+                prompts, out_lens = e2e_prompts(num_prompts, input_len, output_len, case.get("shared_prefix", 0.0),
+                                                case.get("var_len", False), vocab, seed)
                 sps = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True) for n in out_lens]
                 hits0, steps0 = engine.cache_manager.num_cache_hits, engine.stats.num_steps
                 torch.cuda.synchronize()
@@ -178,9 +183,10 @@ def run_e2e(cfg: dict, dtype: str) -> dict:
                 elapsed = time.perf_counter() - t0
             assert all(len(o.token_ids) == n for o, n in zip(outs, out_lens))
             results[case["name"]] = {"output_tok_per_s": round(sum(out_lens) / elapsed, 1), "elapsed_s": round(elapsed, 3),
+                                     "total_tok_per_s": round((sum(len(p) for p in prompts) + sum(out_lens)) / elapsed, 1),
                                      "steps": engine.stats.num_steps - steps0,
                                      "prefix_cache_hits": engine.cache_manager.num_cache_hits - hits0,
-                                     "published_rtx4090_fp16": case["published"]}
+                                     "published_rtx4090_fp16": case.get("published")}
             del engine
             torch.cuda.empty_cache()
     return results
@@ -261,7 +267,17 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time only the 2048-token prefill (for profiling)")
     ap.add_argument("--attention", action="store_true", help="the reference's attention micro-benchmark cases instead")
-    ap.add_argument("--e2e", action="store_true", help="the reference's end-to-end workload (64 requests, 256 in / 128 out) instead")
+    ap.add_argument("--e2e", action="store_true", help="the reference's end-to-end workload (64 requests, 256 in / 128 out) instead: "
+                    "its published cases, or one case given by the options below (names as in the reference's benchmarks/bench.py)")
+    ap.add_argument("--num-prompts", type=int, default=64)
+    ap.add_argument("--input-len", type=int, default=256)
+    ap.add_argument("--output-len", type=int, default=128)
+    ap.add_argument("--batch-size", type=int, default=None, help="requests at a time (max_num_seqs); gives one --e2e case")
+    ap.add_argument("--shared-prefix", type=float, default=0.0)
+    ap.add_argument("--var-len", action="store_true", help="ragged workload: random input/output lengths per request")
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--max-num-batched-tokens", type=int, default=4096)
+    ap.add_argument("--no-prefix-caching", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -282,8 +298,14 @@ def main() -> int:
         print(json.dumps({"metric": "attention op, microseconds per call (bf16, pages of 16 positions)", "cases": run_attention_cases()}))
         return 0
     if args.e2e:
-        print(json.dumps({"metric": f"end-to-end output tokens/s ({model_name}, random weights, 64 requests)", "dtype": short,
-                          "unit": "tokens/s", "cases": run_e2e(cfg, args.dtype)}))
+        cases = E2E_CASES
+        if args.batch_size is not None:
+            cases = [dict(name=f"{args.input_len}in_{args.output_len}out_b{args.batch_size}", batch=args.batch_size,
+                          shared_prefix=args.shared_prefix, var_len=args.var_len)]
+        print(json.dumps({"metric": f"end-to-end output tokens/s ({model_name}, random weights, {args.num_prompts} requests)", "dtype": short,
+                          "unit": "tokens/s", "cases": run_e2e(
+                              cfg, args.dtype, cases, args.num_prompts, args.input_len, args.output_len, args.block_size,
+                              args.max_num_batched_tokens, not args.no_prefix_caching)}))
         return 0
 
     with tempfile.TemporaryDirectory() as folder:
