@@ -211,10 +211,22 @@ class ModelRunner:
         return self._context(staged, offsets, sizes, host)
 
     # ------------------------------------------------------------------ decode steps as HIP graphs
+    @staticmethod
+    def _bucket(n: int) -> int:
+        """Batch sizes graphs are captured for: 1, 2, 3, 4, 6, 8, 12, 16, 24, 32, ... (at most half as
+        many rows again as the batch has)."""
+        if n <= 4:
+            return n
+        p = 1 << (n - 1).bit_length()                       # the power of two at or above n
+        return p if n > 3 * p // 4 else 3 * p // 4
+
     def _graph_key(self, entries: list):
         """Decode-only steps (one token per request) of a model whose parts launch kernels only can
         be replayed from a captured graph.  The key holds everything launch shapes depend on: the
-        number of requests, of wanted rows, and a bound on the context length."""
+        number of rows, of wanted rows, and a bound on the context length.  Rows and wanted rows are
+        rounded up to a few sizes, so that a batch that shrinks by one request at a time does not
+        capture a graph per size; the extra rows are empty requests that read one key, write nothing
+        and whose logits nobody sees (only for models without per-request state)."""
         if not self.use_graphs or len(entries) > self.max_graph_batch:
             return None
         if any(len(e.tokens) != 1 for e in entries):
@@ -222,15 +234,45 @@ class ModelRunner:
         longest = max(e.start + 1 for e in entries)
         bound = ((longest + 511) // 512) * 512 if longest <= 8192 else 1 << (longest - 1).bit_length()
         bound = min(bound, max(self.model.max_positions, longest))
-        return (len(entries), sum(len(e.want) for e in entries), bound)
+        rows, wanted = len(entries), sum(len(e.want) for e in entries)
+        if not self.states:
+            rows = self._bucket(rows)
+            wanted = min(self._bucket(wanted), rows) if wanted else 0
+            wanted = max(wanted, sum(len(e.want) for e in entries))
+        return (rows, wanted, bound)
 
-    def _capture(self, key, buf, offsets, sizes, host):
+    def _decode_layout(self, S: int, n_want: int, fixed: int):
+        """(offsets, sizes, table shapes) of a decode step's buffer: the layout ``_stage_decode`` produces."""
+        sizes = [S, S, S + 1, S, S, S, n_want]
+        table_shapes = {}
+        for name in self.group_specs:
+            sizes += [S * fixed, S]
+            table_shapes[name] = (S, fixed)
+        offsets, cursor = [], 0
+        for n in sizes:                                       # each piece starts on a 16-byte boundary
+            offsets.append(cursor)
+            cursor += n + (-n) % 4
+        return offsets, sizes, table_shapes, cursor
+
+    def _new_graph_entry(self, key, pinned: torch.Tensor | None = None) -> dict:
+        """Layout and buffers of a decode step of ``key``'s size, filled with an all-empty batch."""
         S, n_want, bound = key
-        pinned = torch.empty(buf.size, dtype=torch.int32, pin_memory=True)
-        pinned.numpy()[:] = buf
-        static = torch.empty(buf.size, dtype=torch.int32, device=self.device)
-        static.copy_(pinned)
-        ctx = self._context(static, offsets, sizes, host, max_k_len=bound, capturing=True)
+        offsets, sizes, table_shapes, total = self._decode_layout(S, n_want, (bound + self.block_size - 1) // self.block_size)
+        on_gpu = self.device.type == "cuda"
+        if pinned is None:
+            pinned = torch.zeros(max(total, 1), dtype=torch.int32, pin_memory=on_gpu)
+        view = pinned.numpy()
+        view[offsets[2]: offsets[2] + S + 1] = np.arange(S + 1)
+        return dict(key=key, pinned=pinned, view=view, offsets=offsets, sizes=sizes, table_shapes=table_shapes,
+                    static=torch.zeros(max(total, 1), dtype=torch.int32, device=self.device), staged_rows=[None] * S,
+                    table_lens={name: np.zeros(S, dtype=np.int64) for name in self.group_specs},
+                    copied=torch.cuda.Event() if on_gpu else None)
+
+    def _capture(self, entry: dict) -> None:
+        S, n_want, bound = entry["key"]
+        entry["static"].copy_(entry["pinned"])
+        host = dict(T=S, S=S, q_lens=[1] * S, k_lens=[bound] * S, slots_state=[-1] * S, table_shapes=entry["table_shapes"])
+        ctx = self._context(entry["static"], entry["offsets"], entry["sizes"], host, max_k_len=bound, capturing=True)
         stream = torch.cuda.Stream(device=self.device)
         stream.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(stream):
@@ -240,24 +282,27 @@ class ModelRunner:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
             logits = self.model.forward(ctx, self.kv, self.states)
-        entry = dict(graph=graph, pinned=pinned, static=static, logits=logits, ctx=ctx, offsets=offsets, sizes=sizes)
-        if len(self._graphs) >= 48:
+        entry.update(graph=graph, logits=logits, ctx=ctx)
+        if len(self._graphs) >= 64:
             self._graphs.pop(next(iter(self._graphs)))
-        self._graphs[key] = entry
-        return entry
+        self._graphs[entry["key"]] = entry
 
     def _restage_decode(self, entry: dict, entries: list) -> None:
         """Write a decode step's arrays into the pinned buffer of its graph, in the layout of
         ``_stage_decode`` and with the same checks, but reading only the block tables that changed
         since the buffer was last written: the buffer keeps the rows of the step before, and an entry
-        whose ``table_version`` is the one staged in its row leaves that row alone."""
-        bs, S = self.block_size, len(entries)
+        whose ``table_version`` is the one staged in its row leaves that row alone.  Rows past the
+        entries are empty requests: token 0 at position 0, block table [0], no slot to write to."""
+        bs, S = self.block_size, len(entry["staged_rows"])
+        R = len(entries)
         vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions
         view, offsets, sizes = entry["view"], entry["offsets"], entry["sizes"]
-        ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=S)
-        starts = np.fromiter((e.start for e in entries), dtype=np.int64, count=S)
+        ids = np.zeros(S, dtype=np.int64)
+        starts = np.zeros(S, dtype=np.int64)
+        ids[:R] = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
+        starts[:R] = np.fromiter((e.start for e in entries), dtype=np.int64, count=R)
         rids = [e.request_id for e in entries]
-        if len(set(rids)) != S:
+        if len(set(rids)) != R:
             raise StepError("a request appears twice in one step")
         if ids.min() < 0 or ids.max() >= vocab:
             raise StepError(f"token id outside [0, {vocab})")
@@ -269,13 +314,17 @@ class ModelRunner:
                 if w != 0:
                     raise StepError(f"request {e.request_id!r}: wanted row {w} outside its 1 token")
                 logits_idx.append(i)
-        slots_state = np.fromiter((-1 if e.state_slot is None else e.state_slot for e in entries), dtype=np.int32, count=S)
+        n_want = len(logits_idx)
+        logits_idx += [0] * (sizes[6] - n_want)               # rows nobody asked for repeat row 0
+        slots_state = np.full(S, -1, dtype=np.int32)
+        slots_state[:R] = np.fromiter((-1 if e.state_slot is None else e.state_slot for e in entries), dtype=np.int32, count=R)
         if self.states and (slots_state < 0).any():
             raise StepError("this model keeps per-request state: every entry needs a state slot")
         k_lens = starts + 1
         need = (k_lens + bs - 1) // bs
-        staged = entry["staged_rows"]                 # per row: (request id, table version) as last written
+        staged = entry["staged_rows"]                 # per row: (request id, table version) as last written, or "empty"
         stale = [s for s, e in enumerate(entries) if e.table_version is None or staged[s] != (rids[s], e.table_version)]
+        emptied = [s for s in range(R, S) if staged[s] != "empty"]
 
         def put(i, values):
             view[offsets[i]: offsets[i] + sizes[i]] = values
@@ -300,33 +349,36 @@ class ModelRunner:
                 tables[s, :n] = np.where(row == NO_PAGE, 0, row)
                 tables[s, n:] = 0
                 held[s] = n
+            for s in emptied:
+                tables[s, :] = 0
+                held[s] = 1
             short = need > held
             if short.any():
                 s = int(np.argmax(short))
                 raise StepError(f"request {rids[s]!r}: too few pages in group {name!r} for {int(k_lens[s])} positions")
-            last_page = tables[np.arange(S), need - 1].astype(np.int64)
-            put(8 + 2 * gi, last_page * bs + starts % bs)
+            slots = tables[np.arange(S), need - 1].astype(np.int64) * bs + starts % bs
+            slots[R:] = -1                                        # empty rows write nothing
+            put(8 + 2 * gi, slots)
         for s in stale:
             staged[s] = (rids[s], entries[s].table_version)
+        for s in emptied:
+            staged[s] = "empty"
+        return n_want
 
     def _graph_step(self, key, entries: list) -> torch.Tensor:
-        S, n_want, bound = key
         entry = self._graphs.get(key)
-        if entry is None:
-            buf, offsets, sizes, host = self._stage(entries, fixed_blocks=(bound + self.block_size - 1) // self.block_size)
-            entry = self._capture(key, buf, offsets, sizes, host)
-            entry["view"] = entry["pinned"].numpy()
-            entry["table_shapes"] = host["table_shapes"]
-            entry["staged_rows"] = [None] * S
-            entry["table_lens"] = {name: np.zeros(S, dtype=np.int64) for name in self.group_specs}
-            entry["copied"] = torch.cuda.Event()
+        fresh = entry is None
+        if fresh:
+            entry = self._new_graph_entry(key)
         else:
             entry["copied"].synchronize()                  # the last step's copy has left the pinned buffer
-        self._restage_decode(entry, entries)
+        n_want = self._restage_decode(entry, entries)
+        if fresh:
+            self._capture(entry)
         entry["static"].copy_(entry["pinned"], non_blocking=True)
         entry["copied"].record()
         entry["graph"].replay()
-        return entry["logits"].clone()
+        return entry["logits"][:n_want].clone()
 
     # ------------------------------------------------------------------ run
     @torch.no_grad()

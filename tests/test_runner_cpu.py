@@ -153,3 +153,41 @@ def test_table_version_changes_exactly_when_a_table_does(runtime):
     assert manager.allocate("w", 17, 1)                                               # writes into a shared page: copy
     assert manager.table_version("w") != manager.table_version("v") and manager.take_pending_copies()
     manager.free("v"); manager.free("w")
+
+
+def test_graph_sizes_are_few_and_extra_rows_are_empty_requests(runtime):
+    manager, runner = runtime
+    g = next(iter(manager.groups))
+    sizes = sorted({runner._bucket(n) for n in range(1, 300)})
+    assert sizes[:10] == [1, 2, 3, 4, 6, 8, 12, 16, 24, 32] and all(runner._bucket(n) >= n for n in range(1, 300))
+    assert all(2 * runner._bucket(n) <= 3 * n for n in range(4, 300))               # at most half as many rows again
+    entries = []
+    for i, start in enumerate([3, 16, 31, 0, 20]):
+        rid = f"p{i}"
+        if start:
+            manager.allocate(rid, 0, start)
+        assert manager.allocate(rid, start, 1)
+        entries.append(StepEntry(rid, [10 + i], start, {g: manager.block_table(rid, g)}, None, [0] if i != 1 else [],
+                                 manager.table_version(rid)))
+    entry = runner._new_graph_entry((6, 6, 64))                                      # five requests run as six rows
+    assert runner._restage_decode(entry, entries) == 4
+    fresh, offsets, sizes, _ = runner._stage_decode(entries, 4)
+    piece = lambda buf, offs, szs, i: buf[offs[i]: offs[i] + szs[i]]
+    got = lambda i: piece(entry["view"], entry["offsets"], entry["sizes"], i)
+    for i in (0, 1, 3, 4, 5, 8):                                                     # ids, positions, lengths, state, starts, slots
+        assert got(i)[:5].tolist() == piece(fresh, offsets, sizes, i).tolist()
+    assert got(0)[5] == 0 and got(1)[5] == 0 and got(3)[5] == 1 and got(8)[5] == -1  # the empty row: one key, no slot
+    assert got(2).tolist() == list(range(7))
+    assert got(6).tolist() == [0, 2, 3, 4, 0, 0]                                     # rows nobody asked for repeat row 0
+    tables = got(7).reshape(6, 4)
+    assert np.array_equal(tables[:5], piece(fresh, offsets, sizes, 7).reshape(5, 4)) and not tables[5].any()
+    # the batch shrinks: row 4 becomes empty too
+    for e in entries[:4]:
+        e.start += 1
+        assert manager.allocate(e.request_id, e.start, 1)
+        e.block_tables = {g: manager.block_table(e.request_id, g)}
+        e.table_version = manager.table_version(e.request_id)
+    runner._restage_decode(entry, entries[:4])
+    assert got(8)[4] == -1 and got(3)[4] == 1 and not got(7).reshape(6, 4)[4].any()
+    for i in range(5):
+        manager.free(f"p{i}")
