@@ -1,5 +1,5 @@
-"""Minimal usage (options as in the reference's examples/generate.py:10-15; --backend is gone
-because there is one attention implementation):
+"""Minimal usage (options as in the reference's examples/generate.py:10-15; --backend takes "auto" or
+"hip", the one attention implementation there is):
 
     python examples/generate.py --model DIR --max-tokens 64 --temperature 0.0
     python examples/generate.py --model DIR --random-weights 0 --prompt-ids 1,2,3 --prompt-ids 4,5
@@ -22,6 +22,7 @@ def main(argv=None) -> int:
     logging.basicConfig(level=logging.INFO, format="%(message)s")
     ap = argparse.ArgumentParser()
     ap.add_argument("--model", required=True, help="folder with config.json and *.safetensors")
+    ap.add_argument("--backend", default="auto", choices=["auto", "hip"])
     ap.add_argument("--max-tokens", type=int, default=64)
     ap.add_argument("--temperature", type=float, default=0.0)
     ap.add_argument("--top-k", type=int, default=-1)
@@ -43,7 +44,7 @@ def main(argv=None) -> int:
         overrides["random_weights"] = args.random_weights
     engine = LLMEngine(args.model, EngineConfig(
         block_size=args.block_size, num_gpu_blocks=args.num_gpu_blocks, max_num_batched_tokens=args.max_num_batched_tokens,
-        max_model_len=args.max_model_len, dtype=args.dtype, seed=args.seed), **overrides)
+        max_model_len=args.max_model_len, dtype=args.dtype, seed=args.seed, attention_backend=args.backend), **overrides)
     if args.prompt_ids:
         prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     elif engine.tokenizer is not None:
@@ -62,7 +63,7 @@ def main(argv=None) -> int:
         print(f"--- [{out.finish_reason}] cached_prefix_tokens={out.num_cached_tokens}\n{shown}\n")
     s = engine.stats
     print(f"steps={s.num_steps} prefill_tokens={s.num_prefill_tokens} decode_tokens={s.num_decode_tokens} "
-          f"preemptions={s.num_preemptions} dtype={engine.dtype}")
+          f"preemptions={s.num_preemptions} attention={engine.attention_backend} dtype={engine.dtype}")
     return 0
 
 

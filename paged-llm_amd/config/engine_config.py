@@ -17,6 +17,9 @@ class EngineConfig:
     max_model_len: int = 4096
     enable_prefix_caching: bool = True
     enable_chunked_prefill: bool = True
+    # "auto" | "hip": this engine's own kernels (there is one implementation; the reference's "triton",
+    # "flash" and "torch" are refused).
+    attention_backend: str = "auto"
     dtype: str = "auto"            # "auto" | "bfloat16" | "float32"
     device: str = "cuda"
     seed: int = 0
@@ -28,5 +31,8 @@ class EngineConfig:
             raise ValueError("block_size must be a power of two (kernels split positions with shift and mask)")
         if self.max_num_batched_tokens < self.block_size:
             raise ValueError("max_num_batched_tokens must be >= block_size")
+        if self.attention_backend not in ("auto", "hip"):
+            raise ValueError(f"attention_backend={self.attention_backend!r}: this engine has one attention implementation, "
+                             "its HIP kernels (\"auto\" or \"hip\")")
         if self.max_num_seqs <= 0:
             raise ValueError("max_num_seqs must be positive")

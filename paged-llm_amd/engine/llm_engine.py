@@ -76,6 +76,8 @@ class LLMEngine:
             self.model = build_model(hf_cfg, cfg.dtype, self.device, cfg.max_model_len)
             fill_random(self.model, int(random_seed))
         self.dtype = self.model.dtype
+        # What runs the attention (the reference reports its backend's name here, pagedllm/engine.py:117-118).
+        self.attention_backend = "hip"
         log.info("loaded %s in %.1fs (dtype=%s)", model, time.perf_counter() - t0, self.dtype)
 
         num_pages = cfg.num_gpu_blocks or self._profile_num_pages()

@@ -98,3 +98,11 @@ def test_sampling_params():
     sp = SamplingParams()
     assert (sp.temperature, sp.top_p, sp.top_k, sp.max_tokens, sp.ignore_eos, sp.stop_token_ids) == (1.0, 1.0, -1, 128, False, ())
     assert SamplingParams(temperature=0.0).greedy and not sp.greedy
+
+
+def test_attention_backend_names():
+    from paged_llm_amd import EngineConfig
+    assert EngineConfig().attention_backend == "auto" and EngineConfig(attention_backend="hip").attention_backend == "hip"
+    for other in ("triton", "flash", "torch"):
+        with pytest.raises(ValueError, match="one attention implementation"):
+            EngineConfig(attention_backend=other)
