@@ -39,7 +39,7 @@ class ModelRunner:
                        for pos, ss in model.state_specs().items()}
 
     # ------------------------------------------------------------------ batch -> device tensors
-    def _stage(self, entries: list, fixed_blocks: int | None = None, fast: bool = True):
+    def _stage(self, entries: list, fixed_blocks: int | None = None):
         """Checks the batch and lays all its integer arrays out in one host buffer.
 
         Returns (buffer, offsets, sizes, host) where piece i is buffer[offsets[i]: offsets[i] + sizes[i]]
@@ -49,8 +49,6 @@ class ModelRunner:
         """
         if not entries:
             raise StepError("a step needs at least one entry")
-        if fast and fixed_blocks is not None and all(len(e.tokens) == 1 for e in entries):
-            return self._stage_decode(entries, fixed_blocks)
         bs = self.block_size
         vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions
         seen = set()
@@ -135,62 +133,6 @@ class ModelRunner:
         host = dict(T=T, S=S, q_lens=q_lens, k_lens=k_lens, slots_state=slots_state.tolist(), table_shapes=table_shapes)
         return np.concatenate(padded), offsets, [p.size for p in pieces], host
 
-    def _stage_decode(self, entries: list, fixed_blocks: int):
-        """``_stage`` for steps of one token per request (the layout and the checks are the same;
-        the arrays are built without a Python loop over positions)."""
-        bs, S = self.block_size, len(entries)
-        vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions
-        ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=S)
-        starts = np.fromiter((e.start for e in entries), dtype=np.int64, count=S)
-        if len({e.request_id for e in entries}) != S:
-            raise StepError("a request appears twice in one step")
-        if ids.min() < 0 or ids.max() >= vocab:
-            raise StepError(f"token id outside [0, {vocab})")
-        if starts.min() < 0 or starts.max() + 1 > max_pos:
-            raise StepError(f"a position exceeds the model's {max_pos} positions")
-        logits_idx = []
-        for i, e in enumerate(entries):
-            for w in e.want:
-                if w != 0:
-                    raise StepError(f"request {e.request_id!r}: wanted row {w} outside its 1 token")
-                logits_idx.append(i)
-        k_lens = starts + 1
-        need = (k_lens + bs - 1) // bs
-        pieces = [ids.astype(np.int32), starts.astype(np.int32), np.arange(S + 1, dtype=np.int32), k_lens.astype(np.int32)]
-        slots_state = np.asarray([-1 if e.state_slot is None else e.state_slot for e in entries], dtype=np.int32)
-        if self.states and (slots_state < 0).any():
-            raise StepError("this model keeps per-request state: every entry needs a state slot")
-        pieces += [slots_state, starts.astype(np.int32), np.asarray(logits_idx, dtype=np.int32)]
-        table_shapes = {}
-        for name, cs in self.group_specs.items():
-            num_pages = self.kv.num_pages[name]
-            tables = np.zeros((S, fixed_blocks), dtype=np.int32)
-            last_page = np.empty(S, dtype=np.int64)
-            for s, e in enumerate(entries):
-                table = e.block_tables.get(name)
-                n = int(need[s])
-                if table is None or len(table) < n:
-                    raise StepError(f"request {e.request_id!r}: too few pages in group {name!r} for {int(k_lens[s])} positions")
-                row = np.asarray(table[:n], dtype=np.int64)
-                first_key = max(0, e.start - cs.window + 1) if cs.window > 0 else 0
-                live = row[first_key // bs:]
-                if live.min() < 0 or live.max() >= num_pages:
-                    raise StepError(f"request {e.request_id!r}: page id outside [0, {num_pages}) in group {name!r}")
-                tables[s, :n] = np.where(row == NO_PAGE, 0, row)
-                last_page[s] = row[n - 1]
-            table_shapes[name] = tables.shape
-            pieces += [tables.reshape(-1), (last_page * bs + starts % bs).astype(np.int32)]
-        padded, offsets, cursor = [], [], 0
-        for p in pieces:
-            offsets.append(cursor)
-            pad = (-p.size) % 4
-            padded.append(p)
-            if pad:
-                padded.append(np.zeros(pad, dtype=np.int32))
-            cursor += p.size + pad
-        host = dict(T=S, S=S, q_lens=[1] * S, k_lens=k_lens.tolist(), slots_state=slots_state.tolist(), table_shapes=table_shapes)
-        return np.concatenate(padded), offsets, [p.size for p in pieces], host
-
     def _context(self, staged: torch.Tensor, offsets: list, sizes: list, host: dict, max_k_len: int | None = None,
                  capturing: bool = False) -> StepContext:
         def piece(i):
@@ -242,7 +184,8 @@ class ModelRunner:
         return (rows, wanted, bound)
 
     def _decode_layout(self, S: int, n_want: int, fixed: int):
-        """(offsets, sizes, table shapes) of a decode step's buffer: the layout ``_stage_decode`` produces."""
+        """(offsets, sizes, table shapes) of a decode step's buffer: the layout ``_stage`` produces
+        for one token per request with block tables of ``fixed`` entries."""
         sizes = [S, S, S + 1, S, S, S, n_want]
         table_shapes = {}
         for name in self.group_specs:
@@ -289,7 +232,7 @@ class ModelRunner:
 
     def _restage_decode(self, entry: dict, entries: list) -> None:
         """Write a decode step's arrays into the pinned buffer of its graph, in the layout of
-        ``_stage_decode`` and with the same checks, but reading only the block tables that changed
+        ``_stage`` and with the same checks, but reading only the block tables that changed
         since the buffer was last written: the buffer keeps the rows of the step before, and an entry
         whose ``table_version`` is the one staged in its row leaves that row alone.  Rows past the
         entries are empty requests: token 0 at position 0, block table [0], no slot to write to."""

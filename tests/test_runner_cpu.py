@@ -51,27 +51,10 @@ def test_layout_of_a_mixed_batch(runtime):
         manager.free(r)
 
 
-def test_decode_staging_fast_path_equals_the_general_one(runtime):
-    manager, runner = runtime
-    entries = []
-    for i, start in enumerate([3, 16, 31, 0]):
-        rid = f"d{i}"
-        if start:
-            manager.allocate(rid, 0, start)
-        entries.append(entry(manager, rid, [10 + i], start, want=[0] if i != 1 else []))
-    fast = runner._stage(entries, fixed_blocks=4)
-    slow = runner._stage(entries, fixed_blocks=4, fast=False)
-    assert np.array_equal(fast[0], slow[0]) and fast[1] == slow[1] and fast[2] == slow[2]
-    assert fast[3]["k_lens"] == slow[3]["k_lens"] and fast[3]["table_shapes"] == slow[3]["table_shapes"]
-    for i in range(4):
-        manager.free(f"d{i}")
-
-
-@pytest.mark.parametrize("fast", [True, False])
-def test_bad_batches_are_refused_before_anything_runs(runtime, fast):
+@pytest.mark.parametrize("fixed", [4, None])
+def test_bad_batches_are_refused_before_anything_runs(runtime, fixed):
     manager, runner = runtime
     g = next(iter(manager.groups))
-    fixed = 4 if fast else None
     ok = entry(manager, "ok", [1], 0)
     with pytest.raises(StepError, match="token id"):
         runner._stage([StepEntry("x", [256], 0, {g: [0]})], fixed)
@@ -119,7 +102,7 @@ def test_decode_steps_restaged_in_place_equal_fresh_staging(runtime):
             entries.append(StepEntry(rid, [int(rng.integers(0, 256))], start, {g: manager.block_table(rid, g)}, None,
                                      [0] if row != 1 else [], manager.table_version(rid)))
             live[row][1] = start + 1
-        fresh, offsets, sizes, host = runner._stage_decode(entries, 4)
+        fresh, offsets, sizes, host = runner._stage(entries, 4)
         if entry is None:
             entry = dict(view=fresh.copy(), offsets=offsets, sizes=sizes, table_shapes=host["table_shapes"],
                          staged_rows=[None] * 3, table_lens={g: np.zeros(3, dtype=np.int64)})
@@ -171,7 +154,7 @@ def test_graph_sizes_are_few_and_extra_rows_are_empty_requests(runtime):
                                  manager.table_version(rid)))
     entry = runner._new_graph_entry((6, 6, 64))                                      # five requests run as six rows
     assert runner._restage_decode(entry, entries) == 4
-    fresh, offsets, sizes, _ = runner._stage_decode(entries, 4)
+    fresh, offsets, sizes, _ = runner._stage(entries, 4)
     piece = lambda buf, offs, szs, i: buf[offs[i]: offs[i] + szs[i]]
     got = lambda i: piece(entry["view"], entry["offsets"], entry["sizes"], i)
     for i in (0, 1, 3, 4, 5, 8):                                                     # ids, positions, lengths, state, starts, slots
@@ -191,3 +174,29 @@ def test_graph_sizes_are_few_and_extra_rows_are_empty_requests(runtime):
     assert got(8)[4] == -1 and got(3)[4] == 1 and not got(7).reshape(6, 4)[4].any()
     for i in range(5):
         manager.free(f"p{i}")
+
+
+def test_replayed_decode_steps_refuse_bad_batches_too(runtime):
+    manager, runner = runtime
+    g = next(iter(manager.groups))
+    ok = entry(manager, "ok2", [1], 0)
+
+    def run(*entries):
+        runner._restage_decode(runner._new_graph_entry((len(entries), 0, 64)), list(entries))
+
+    run(ok)
+    with pytest.raises(StepError, match="token id"):
+        run(StepEntry("x", [256], 0, {g: [0]}))
+    with pytest.raises(StepError, match="position"):
+        run(StepEntry("x", [1], 256, {g: list(range(12)) + [0] * 5}))
+    with pytest.raises(StepError, match="twice"):
+        run(ok, ok)
+    with pytest.raises(StepError, match="too few pages"):
+        run(StepEntry("x", [1], 20, {g: [0]}))
+    with pytest.raises(StepError, match="page id"):
+        run(StepEntry("x", [1], 3, {g: [99]}))
+    with pytest.raises(StepError, match="page id"):
+        run(StepEntry("x", [1], 3, {g: [NO_PAGE]}))
+    with pytest.raises(StepError, match="wanted row"):
+        runner._restage_decode(runner._new_graph_entry((1, 1, 64)), [StepEntry("x", [1], 0, {g: [0]}, None, [1])])
+    manager.free("ok2")
