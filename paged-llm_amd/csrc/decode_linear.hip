@@ -127,7 +127,7 @@ __device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, i
 #define PLLM_STAMP(i) do { } while (0)
 #endif
 
-template <int EPI, int WAVES, bool HALF, bool DIRECT>
+template <int EPI, int WAVES, bool HALF, bool DIRECT, int PRE>
 __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p, int num_units) {
   PLLM_STAMP(0);
   // Fetch the arguments the first loads depend on in one go (left alone, the compiler fetches each where
@@ -149,10 +149,13 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   const int xrow = HALF ? (r & 7) : r;                          // input row this lane's B operand column belongs to
   const int num_slabs = (K + kStep - 1) / kStep;
   const int my_slabs = wave < num_slabs ? (num_slabs - wave + WAVES - 1) / WAVES : 0;
-  constexpr int PRE = 2;                                        // slabs in flight per wavefront (registers)
+  // PRE slabs are in flight per wavefront (registers).  A unit is walked in rounds of PRE slabs (the last
+  // round of a unit may hold slabs the wavefront does not have: they cost one cached address), and a
+  // slot that has been consumed is refilled at once with the slab PRE positions further on, which may
+  // belong to the next unit: the weights stream without a gap at unit boundaries.
+  const int padded_slabs = max(PRE, (my_slabs + PRE - 1) / PRE * PRE);
   bf16x8 wbuf[PRE][4];
-  const bf16* wrow = p.W;
-  auto load_w = [&](int nth, bf16x8 (&dst)[4]) {                // nth slab of this wavefront, from wrow
+  auto load_w = [&](const bf16* wrow, int nth, bf16x8 (&dst)[4]) {      // nth slab of this wavefront of a unit's rows
     const int slab = wave + nth * WAVES;
     // No condition on the loads (the compiler would turn one into a branch around them, and could then no
     // longer tell how many loads are under way).  Past the end of K a lane rereads the row's last piece,
@@ -183,16 +186,17 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
       dst[j] = kk < K ? v : zero8();                            // zeros past the end of K (the weights reread their last piece there)
     }
   };
-  auto request_unit = [&](int unit) {                           // PRE slabs, needed or not
-    wrow = p.W + (size_t)unit_row<EPI, HALF>(p, unit, r) * p.ldw;
+  auto rows_of_unit = [&](int unit) { return p.W + (size_t)unit_row<EPI, HALF>(p, unit, r) * p.ldw; };
+  int unit = blockIdx.x;                                        // below num_units: the grid has no more workgroups than units
+  const bf16* wrow = rows_of_unit(unit);
+  auto request_first = [&]() {                                  // the first PRE slabs of the first unit, needed or not
     if (DIRECT) {
 #pragma unroll
       for (int s = 0; s < PRE; ++s) load_x(s, xbuf[s]);
     }
 #pragma unroll
-    for (int s = 0; s < PRE; ++s) load_w(s, wbuf[s]);
+    for (int s = 0; s < PRE; ++s) load_w(wrow, s, wbuf[s]);
   };
-  int unit = blockIdx.x;                                        // below num_units: the grid has no more workgroups than units
 
   // Rotary epilogue: what depends only on the input row is fetched early, not after the product.
   int rope_pos = 0, rope_slot = -1;
@@ -204,7 +208,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   };
   if constexpr (DIRECT) {
     rope_inputs();
-    request_unit(unit);
+    request_first();
     PLLM_STAMP(1);
   } else {
   // ---- the rows into LDS.  A wavefront owns a group of 64 pieces of 8 columns and walks rows with it, up
@@ -296,7 +300,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   issue(wc, wr);
   issue_norm(wc);
   rope_inputs();
-  request_unit(unit);                                           // the first unit's weights: on their way during all that follows
+  request_first();                                              // the first unit's weights: on their way during all that follows
   PLLM_STAMP(1);
   sum_rows(wc, wr);
   for (int c = wc; c < ipr; c += cg)
@@ -321,8 +325,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
     return (xrow < M && kk < K) ? *reinterpret_cast<const bf16x8*>(xs + (size_t)xrow * row_len + kk) : zero8();
   };
 
-  // ---- units of this workgroup, one after the other; the next unit's weights are requested as
-  //      soon as the current unit's have been consumed, and travel during the reduction
+  // ---- units of this workgroup, one after the other
   for (; unit < num_units; unit += gridDim.x) {
     floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
     float rope_cs = 1.f, rope_sn = 0.f;
@@ -338,23 +341,29 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
         }
       }
     }
-    for (int base = 0; base < my_slabs; base += PRE) {
+    const int next = unit + gridDim.x;
+    const bf16* wrow_next = next < num_units ? rows_of_unit(next) : p.W;
+    for (int base = 0; base < padded_slabs; base += PRE) {
 #pragma unroll
       for (int s = 0; s < PRE; ++s) {
         const int nth = base + s;
-        if (nth >= my_slabs) break;
+        if (nth < my_slabs) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[s][j], x_operand(nth, j, s), acc, 0, 0, 0);
-        if (nth + PRE < my_slabs) {                             // keep PRE slabs in flight
-          if (DIRECT) load_x(nth + PRE, xbuf[s]);
-          load_w(nth + PRE, wbuf[s]);
+          for (int j = 0; j < 4; ++j)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[s][j], x_operand(nth, j, s), acc, 0, 0, 0);
+        }
+        const int ahead = nth + PRE;                            // refill the slot: this unit's slab, or the next unit's
+        if (ahead < padded_slabs) {
+          if (DIRECT) load_x(ahead, xbuf[s]);
+          load_w(wrow, ahead, wbuf[s]);
+        } else if (next < num_units) {
+          if (DIRECT) load_x(ahead - padded_slabs, xbuf[s]);
+          load_w(wrow_next, ahead - padded_slabs, wbuf[s]);
         }
       }
     }
+    wrow = wrow_next;
     PLLM_STAMP(3);
-    const int next = unit + gridDim.x;
-    if (next < num_units) request_unit(next);
 
     // acc[i] = element (tile row g*4 + i, input row r); add the wavefronts in wave order
 #pragma unroll
@@ -412,9 +421,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   }
 }
 
-template <int EPI, int WAVES, bool HALF, bool DIRECT>
+template <int EPI, int WAVES, bool HALF, bool DIRECT, int PRE>
 static int launch(const DecodeLinearParams& p, int units, int blocks, size_t lds, hipStream_t stream) {
-  auto kernel = decode_linear_kernel<EPI, WAVES, HALF, DIRECT>;
+  auto kernel = decode_linear_kernel<EPI, WAVES, HALF, DIRECT, PRE>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -514,7 +523,11 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   if (tune & 32) two = true;
   const int per_block = two ? per_block2 : busiest1;
   const int blocks = ceil_div(units, per_block);
-#define GO(EPI_, HALF_) return direct ? launch<EPI_, waves, HALF_, true>(p, units, blocks, lds, stream) : launch<EPI_, waves, HALF_, false>(p, units, blocks, lds, stream)
+#define GO(EPI_, HALF_)                                                                                                   \
+  do {                                                                                                                    \
+    if (direct) return launch<EPI_, waves, HALF_, true, 2>(p, units, blocks, lds, stream);                                \
+    return launch<EPI_, waves, HALF_, false, 2>(p, units, blocks, lds, stream);                                           \
+  } while (0)
   if (half) {
     switch (epi) {
       case EPI_BF16: GO(EPI_BF16, true);
