@@ -81,13 +81,18 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
     return [torch.randint(100, vocab, (length,), generator=g).tolist() for _ in range(n)]
 
 
-def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int) -> float:
-    """Seconds per decode step at `batch` requests whose contexts end at `context` tokens."""
+def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int):
+    """(seconds per decode step, mean context length over the timed steps) at `batch` requests whose
+    contexts end at (or just under) `context` tokens."""
     import torch
     from paged_llm_amd import SamplingParams
-    prompt_len = context - (steps + warmup)
+    # Requests whose prompt is done go on decoding while the others' prompts are still computed, so some
+    # are a few tokens ahead: leave room for that, so that no context passes `context` while timed.
+    budget = engine.scheduler.config.max_num_batched_tokens
+    ahead = batch * context // budget + 1
+    prompt_len = context - (steps + warmup) - ahead
     assert prompt_len >= 1, "context too short for this many steps"
-    sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 40, ignore_eos=True)
+    sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + ahead + 40, ignore_eos=True)
     for p in random_prompts(batch, prompt_len, engine.model.spec.vocab_size, seed):
         engine.add_request(p, sp)
     while any(not r.is_prefill_done for r in engine.scheduler.running) or engine.scheduler.waiting:
@@ -96,15 +101,18 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed:
     for _ in range(warmup):
         engine.step()
     torch.cuda.synchronize()
+    before = sum(r.num_tokens for r in engine.scheduler.running)
     t0 = time.perf_counter()
     for _ in range(steps):
         out = engine.step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     assert len(out) == batch
+    after = sum(r.num_tokens for r in engine.scheduler.running)
+    assert max(r.num_tokens for r in engine.scheduler.running) <= context + 1, "a context passed the one asked for"
     for r in list(engine.scheduler.running):
         engine.abort_request(r.request_id)
-    return elapsed / steps
+    return elapsed / steps, (before + after) / 2.0 / batch
 
 
 def time_prefill(engine, tokens: int, seed: int, repeats: int = 3) -> float:
@@ -315,9 +323,9 @@ def main() -> int:
             print(json.dumps({"prefill_ms": round(psec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / psec, 1),
                               "frac": round(prefill_flops(cfg, PREFILL_TOKENS, 1) / psec / PEAK_FLOPS[short], 4)}))
             return 0
-        sec = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
+        sec, mean_context = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
         value = args.batch / sec
-        decode_bytes = numbers["weight_bytes"] + args.batch * args.context * numbers["kv_bytes_per_token"]
+        decode_bytes = numbers["weight_bytes"] + args.batch * mean_context * numbers["kv_bytes_per_token"]
         achieved = decode_bytes / sec / 1e9
         record = {
             "metric": f"decode tokens/s ({model_name}, random weights)", "value": round(value, 1), "unit": "tokens/s",
@@ -326,7 +334,7 @@ def main() -> int:
             "config": {"model": model_name, "layers": cfg["num_hidden_layers"], "layers_of_model": model_layers,
                        "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                        "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-                       "global_batch": args.batch, "seq_len": args.context, "block_size": 16, "weights": "random seed 0",
+                       "global_batch": args.batch, "seq_len": args.context, "mean_context_timed": round(mean_context, 1), "block_size": 16, "weights": "random seed 0",
                        "parallelism": "single GPU"},
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(achieved / PEAK_HBM_GBS, 4)},
@@ -334,7 +342,7 @@ def main() -> int:
         if not args.no_points:
             points = {}
             for b in (1, 64):
-                s = time_decode(engine, b, args.context, max(16, args.steps // 2), max(4, args.warmup // 2), seed=10 + b)
+                s, _ = time_decode(engine, b, args.context, max(16, args.steps // 2), max(4, args.warmup // 2), seed=10 + b)
                 points[f"decode_b{b}"] = round(b / s, 1)
             record["points"] = points
             psec = time_prefill(engine, PREFILL_TOKENS, seed=100)
