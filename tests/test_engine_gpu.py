@@ -221,3 +221,35 @@ def test_decode_steps_replayed_from_graphs_equal_eager_steps(folder_a):
     assert eager.keys() == graphed.keys()
     for key in eager:
         assert helpers.worst(graphed[key], eager[key]) <= 1e-6, key
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_settings_give_the_plain_greedy_tokens(folder_a, folder_b, seed):
+    """Random engine settings (page size, pool size down to where requests are preempted, token budget,
+    requests at a time, prefix reuse, prompt portions, graph replay) and random requests, some with a
+    shared beginning: whatever the settings, the tokens are the plain implementation's and every page
+    comes back."""
+    from paged_llm_amd import SamplingParams
+    rng = np.random.default_rng(1000 + seed)
+    folder, vocab = (folder_a, 256) if seed % 2 == 0 else (folder_b, 512)
+    block = int(rng.choice([8, 16, 32]))
+    shared = helpers.random_tokens(int(rng.integers(0, 40)), vocab, seed=seed)
+    prompts, wants = [], []
+    for i in range(int(rng.integers(3, 9))):
+        own = helpers.random_tokens(int(rng.integers(1, 50)), vocab, seed=seed * 100 + i)
+        prompts.append((shared + own) if rng.random() < 0.5 else own)
+        wants.append(int(rng.integers(1, 14)))
+    longest = max(len(p) + w for p, w in zip(prompts, wants))
+    pages_one = (longest + block - 1) // block + 1
+    chunked = bool(rng.random() < 0.7)
+    budget = int(rng.integers(block, 65)) if chunked else max(64, max(len(p) for p in prompts) + 16)
+    engine = engine_for(folder, block_size=block, num_gpu_blocks=int(pages_one * rng.uniform(1.0, 4.0)) + 1,
+                        max_num_batched_tokens=max(budget, block), max_num_seqs=int(rng.integers(1, 7)),
+                        enable_prefix_caching=bool(rng.random() < 0.6), enable_chunked_prefill=chunked,
+                        enable_hip_graphs=bool(rng.random() < 0.7), max_model_len=longest + 1)
+    total = engine.cache_manager.num_pages()
+    outs = engine.generate(prompts, [SamplingParams(temperature=0.0, max_tokens=w, ignore_eos=True) for w in wants])
+    for p, w, o in zip(prompts, wants, outs):
+        assert o.token_ids == plain_greedy(folder, p, w), f"prompt of {len(p)} tokens, {w} wanted, {o.num_preemptions} preemptions"
+    assert engine.cache_manager.num_free_pages() == total
+    engine.cache_manager.check_invariants()
