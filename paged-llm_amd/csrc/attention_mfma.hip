@@ -751,11 +751,3 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   }
   return err;
 }
-
-// Largest number of wavefronts per work item whose merge buffers fit `lds_limit` bytes (0: none).
-PLLM_API int pllm_attention_mfma_max_waves(int max_cols, long lds_limit) {
-  const int ncb = max_cols <= 16 ? 1 : (max_cols <= 32 ? 2 : 4);
-  for (int w = 8; w >= 4; w /= 2)
-    if ((long)merge_lds_bytes(ncb, w) <= lds_limit) return w;
-  return 0;
-}

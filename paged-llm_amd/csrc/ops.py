@@ -308,9 +308,9 @@ def decode_linear_takes(rows: int, K: int, x: torch.Tensor, w: torch.Tensor, sta
         # With more than 8 rows every unit rereads as many bytes of rows as it streams of weights; for long
         # rows the library's product is then faster (measured at K = 5632 and 14336).
         return rows <= 8 or K <= 4096
-    waves = 8
-    need = ((rows * (K + 8) * 2 + 15) // 16) * 16 + waves * 256 * 4
-    return need <= _max_lds_bytes(x.device)
+    f = _fn("decode_linear.hip", "pllm_decode_linear_lds_bytes", signature=[c_int, c_int, c_int])
+    f.restype = c_long
+    return int(f(rows, K, 8)) <= _max_lds_bytes(x.device)
 
 
 def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: torch.Tensor | None = None,
@@ -422,11 +422,18 @@ def gemm_large_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p]
 _attn_scratch: dict = {}
+_attn_checked: set = set()
 
 
 def mfma_attention_takes(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int, block_size: int) -> bool:
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size >= 16
             and block_size & (block_size - 1) == 0 and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 64)
+
+
+def _merge_lds_bytes(column_blocks: int, waves: int, head_dim: int) -> int:
+    """LDS of the attention kernel's several-wavefront variant (as merge_lds_bytes in attention_mfma.hip):
+    maximum and weight per column and wavefront, and every wavefront's partial output."""
+    return (2 * waves * column_blocks * 16 + waves * column_blocks * (head_dim // 16) * 4 * 64) * 4
 
 
 def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: int, group: int, head_dim: int,
@@ -442,7 +449,7 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
         return 1, 0, 1
     ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
     max_waves = 8
-    while max_waves >= 4 and (2 * max_waves * ncb * 16 + max_waves * ncb * (head_dim // 16) * 4 * 64) * 4 > lds_limit:
+    while max_waves >= 4 and _merge_lds_bytes(ncb, max_waves, head_dim) > lds_limit:
         max_waves //= 2
     if max_waves < 4:
         return 1, 0, 1
@@ -482,7 +489,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     _need(max_q_len >= 1 and partition_size % 64 == 0 and waves in (1, 4, 8), "bad launch parameters")
     ncb = min(column_blocks or 4, 1 if max_q_len * (num_heads // num_kv_heads) <= 16 else (2 if max_q_len * (num_heads // num_kv_heads) <= 32 else 4))
     _need(column_blocks in (0, 1, 2, 4), "column_blocks is 0 (automatic), 1, 2 or 4")
-    _need(waves == 1 or (2 * waves * ncb * 16 + waves * ncb * (head_dim // 16) * 4 * 64) * 4 <= _max_lds_bytes(q.device),
+    _need(waves == 1 or _merge_lds_bytes(ncb, waves, head_dim) <= _max_lds_bytes(q.device),
           "the merge buffers of that many wavefronts do not fit LDS")
     ws = None
     if partition_size > 0:
@@ -492,6 +499,10 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
         if ws is None or ws.numel() < floats:
             ws = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=q.device)
             _attn_scratch[key] = ws
+    if head_dim not in _attn_checked:                 # the library on disk is the one compiled for this head size
+        built = _fn("attention_mfma.hip", "pllm_attention_mfma_head_dim", {"HEAD_DIM": head_dim}, [])()
+        _need(built == head_dim, f"attention library for head size {head_dim} reports head size {built}")
+        _attn_checked.add(head_dim)
     f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
     _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
              block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,

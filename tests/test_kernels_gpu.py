@@ -337,7 +337,7 @@ def test_paged_attention_mfma(heads, kv_heads, d, bs, lens, num_q):
         cols = max(num_q) * (heads // kv_heads)
         ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
         for waves in (4, 8):
-            if (2 * waves * ncb * 16 + waves * ncb * (d // 16) * 4 * 64) * 4 <= 160 * 1024:
+            if ops()._merge_lds_bytes(ncb, waves, d) <= 160 * 1024:
                 assert rel_err(ops().paged_attention_mfma(*args, 0, 1, waves), want) <= 1.6e-2, f"{waves} wavefronts"
                 parts = (max(lens) + 255) // 256
                 assert rel_err(ops().paged_attention_mfma(*args, 256, parts, waves), want) <= 1.6e-2, f"{waves} wavefronts, partitions"
