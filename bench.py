@@ -115,6 +115,31 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed:
     return elapsed / steps, (before + after) / 2.0 / batch
 
 
+def measured_peaks() -> dict:
+    """What this GPU gives to the simplest programs, beside the published peaks: GB/s of a kernel that only
+    reads 1 GiB with every load issued early, and TFLOP/s of the library's large bfloat16 product (8192^3)."""
+    import torch
+    from paged_llm_amd.csrc import ops
+    def best(fn, repeats=5):
+        fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(repeats):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); fn(); b.record()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b) * 1e-3)
+        return min(times)
+    x = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
+    read = x.numel() * 2 / best(lambda: ops.stream_read(x)) / 1e9
+    del x
+    n = 8192
+    a = torch.randn(n, n, dtype=torch.bfloat16, device="cuda")
+    b = torch.randn(n, n, dtype=torch.bfloat16, device="cuda")
+    mfma = 2.0 * n ** 3 / best(lambda: torch.mm(a, b.t())) / 1e12
+    return {"hbm_read_gbs": round(read, 1), "bf16_product_tflops": round(mfma, 1)}
+
+
 def time_prefill(engine, tokens: int, seed: int, repeats: int = 3) -> float:
     """Seconds of one step that computes a whole prompt of `tokens` tokens (best of a few)."""
     import torch
@@ -349,6 +374,13 @@ def main() -> int:
             flops = prefill_flops(cfg, PREFILL_TOKENS, 1)
             record["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3),
                                  "frac": round(flops / psec / PEAK_FLOPS[short], 4)}
+            if short == "bf16":
+                # the same two fractions against what the GPU gives to a plain large read and a plain large product
+                del engine
+                torch.cuda.empty_cache()
+                peaks = measured_peaks()
+                record["measured_peaks"] = dict(peaks, decode_frac=round(achieved / peaks["hbm_read_gbs"], 4),
+                                                prefill_frac=round(flops / psec / (peaks["bf16_product_tflops"] * 1e12), 4))
     print(json.dumps(record))
     return 0
 

@@ -268,3 +268,27 @@ PLLM_API int pllm_copy_pages(int dtype, void* pages, const int* src, const int* 
     hipLaunchKernelGGL(copy_pages_kernel<bf16>, grid, block, 0, stream, (bf16*)pages, src, dst, (size_t)page_elems);
   PLLM_RETURN_LAST_ERROR();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Measurement only: read `bytes` (a multiple of 16) with 16-byte loads, eight under way per thread, and
+// write nothing (the store's condition never holds).  Its time is what streaming a buffer costs here.
+__global__ __launch_bounds__(256) void stream_read_kernel(const float4* __restrict__ src, size_t pieces, float* __restrict__ out) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  float s = 0.f;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 7 * stride < pieces; i += 8 * stride) {
+    float4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[i + u * stride];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u].x + v[u].y + v[u].z + v[u].w;
+  }
+  for (; i < pieces; i += stride) s += src[i].x;
+  if (s == 12345.678f) out[0] = s;
+}
+
+PLLM_API int pllm_stream_read(const void* src, long bytes, float* out, int blocks, hipStream_t stream) {
+  if (bytes <= 0 || (bytes & 15) || blocks <= 0) return -2;
+  hipLaunchKernelGGL(stream_read_kernel, dim3(blocks), dim3(256), 0, stream, (const float4*)src, (size_t)bytes / 16, out);
+  PLLM_RETURN_LAST_ERROR();
+}

@@ -276,6 +276,21 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     return out
 
 
+def stream_read(buffer: torch.Tensor, blocks: int = 2048) -> None:
+    """Measurement only: read all of ``buffer`` once (what streaming that many bytes costs on this GPU)."""
+    _on_gpu(buffer)
+    nbytes = buffer.numel() * buffer.element_size()
+    _need(buffer.is_contiguous() and nbytes % 16 == 0 and buffer.data_ptr() % 16 == 0, "stream_read takes whole 16-byte pieces")
+    sink = _stream_sink.get(str(buffer.device))
+    if sink is None:
+        sink = _stream_sink[str(buffer.device)] = torch.zeros(1, dtype=torch.float32, device=buffer.device)
+    f = _fn("elementwise.hip", "pllm_stream_read", signature=[c_void_p, c_long, c_void_p, c_int, c_void_p])
+    _check(f(_ptr(buffer), nbytes, _ptr(sink), int(blocks), _stream()), "stream_read")
+
+
+_stream_sink: dict = {}
+
+
 # ------------------------------------------------------------------------------------------- fused decode products
 EPI_BF16, EPI_F32, EPI_GATED, EPI_ROPE_KV = 0, 1, 2, 3
 DECODE_MAX_ROWS = 16
