@@ -32,15 +32,34 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// Reductions over a wavefront without LDS traffic or lane-index arithmetic: two swaps inside groups of
+// four lanes, a mirror inside groups of 8 and of 16 (data-parallel-primitive moves; after each step all
+// lanes of the group hold the group's result), then the four rows of 16 are read out and combined in row
+// order.  Every lane gets the result; the order of operations is fixed.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppSwap1 = 0xB1;        // quad_perm [1, 0, 3, 2]
+constexpr int kDppSwap2 = 0x4E;        // quad_perm [2, 3, 0, 1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <- lane 7 - i of its group of 8
+constexpr int kDppMirror = 0x140;      // lane i <- lane 15 - i of its row of 16
+__device__ __forceinline__ float row_lane(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  return v;
+  v += dpp_move<kDppSwap1>(v);
+  v += dpp_move<kDppSwap2>(v);
+  v += dpp_move<kDppHalfMirror>(v);
+  v += dpp_move<kDppMirror>(v);
+  return ((row_lane(v, 0) + row_lane(v, 16)) + row_lane(v, 32)) + row_lane(v, 48);
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-  return v;
+  v = fmaxf(v, dpp_move<kDppSwap1>(v));
+  v = fmaxf(v, dpp_move<kDppSwap2>(v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_move<kDppMirror>(v));
+  return fmaxf(fmaxf(row_lane(v, 0), row_lane(v, 16)), fmaxf(row_lane(v, 32), row_lane(v, 48)));
 }
 
 // Sum over a workgroup whose size is a multiple of 64 (at most 1024). `scratch` holds 16 floats
