@@ -2,7 +2,8 @@
 // because at these sizes a kernel launch costs as much as the weights take to stream:
 //
 //   prologue (optional)   rows = x (+ delta), the residual sum in float rounded once; the new
-//                         residual is written out by workgroup 0; RMS norm of the rows in float
+//                         residual is written out by workgroup 0; RMS norm in float: the elements
+//                         take the norm's weights here, the row's 1 / rms goes onto the finished sums
 //   product               rows[M, K] * W[N, K]^T on the matrix cores, float accumulation
 //   epilogue              plain (bfloat16 or float out) | silu(gate) * up | rotary encoding of q and
 //                         k and the write of k, v into their cache pages
@@ -24,6 +25,7 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 
 constexpr int kSlab = 128;
 constexpr int kPad = 8;            // bf16 elements of padding per LDS row (spreads rows over banks)
+constexpr int kSquares = 512;      // floats of LDS for the rows' sums of squares: 16 rows x up to 32 column groups of 512
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_GATED = 2, EPI_ROPE_KV = 3 };
 
@@ -140,6 +142,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   const int row_len = K + kPad;
   bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                       // [M][K + kPad] (not DIRECT)
   float* part = reinterpret_cast<float*>(lds_raw + (DIRECT ? 0 : (((size_t)M * row_len * 2 + 15) & ~(size_t)15)));   // [WAVES][256]
+  float* sq = part + WAVES * 256;                               // [M][column groups] sums of squares, kSquares floats
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
 
@@ -223,7 +226,6 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   const int cg = min(ipr, WAVES), rpp = WAVES / cg;             // groups and rows under way at a time
   const int wc = wave % cg, wr = wave / cg;                     // this wavefront's first group and row
   const bool active = wr < rpp;
-  float* sq = part;                                             // [M][ipr] (the buffer is free until the product ends)
   int src_lane = lane < M ? lane : 0;                           // lane m holds the source row of input row m
   if (p.row_index) src_lane = p.row_index[src_lane];
   const bool has_delta = p.delta != nullptr, has_norm = p.norm_w != nullptr;
@@ -268,56 +270,44 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
           *reinterpret_cast<bf16x8*>(p.x_out + src * p.ldxo + k0) = v;
         }
       }
-      if (in) *reinterpret_cast<bf16x8*>(xs + (size_t)m * row_len + k0) = v;            // as stored in bfloat16
       if (has_norm) {
+        // The row's scale 1 / rms is applied to the finished sums (it is the same for the whole row);
+        // here the elements take the norm's weights, and their squares are summed.
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
+        const float w[8] = {nw0.x, nw0.y, nw0.z, nw0.w, nw1.x, nw1.y, nw1.z, nw1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (__bf16)((float)v[i] * w[i]);
         ss = wave_sum(in ? ss : 0.f);
         if (lane == 0) sq[m * ipr + c] = ss;
       }
+      if (in) *reinterpret_cast<bf16x8*>(xs + (size_t)m * row_len + k0) = v;
     }
   };
-  auto scale_rows = [&](int c, int m0) {                        // pass 2 with the norm weights of column group c loaded
-    const int k0 = column(c);
-    if (!active || !inside(c)) return;
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const int m = m0 + u * rpp;
-      if (m >= M) continue;
-      float total = 0.f;
-      for (int j = 0; j < ipr; ++j) total += sq[m * ipr + j];
-      const float inv = rsqrtf(total / (float)K + p.eps);
-      bf16* at = xs + (size_t)m * row_len + k0;                 // each lane rereads only what it wrote
-      bf16x8 v = *reinterpret_cast<const bf16x8*>(at);
-      const float w[8] = {nw0.x, nw0.y, nw0.z, nw0.w, nw1.x, nw1.y, nw1.z, nw1.w};
-#pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = (__bf16)(((float)v[i] * inv) * w[i]);
-      *reinterpret_cast<bf16x8*>(at) = v;
-    }
-  };
-
   issue(wc, wr);
   issue_norm(wc);
   rope_inputs();
   request_first();                                              // the first unit's weights: on their way during all that follows
   PLLM_STAMP(1);
   sum_rows(wc, wr);
-  for (int c = wc; c < ipr; c += cg)
+  for (int c = wc; c < ipr; c += cg) {
+    if (c != wc) issue_norm(c);
     for (int m0 = (c == wc) ? wr + kBatch * rpp : wr; m0 < M; m0 += kBatch * rpp) {
       issue(c, m0);
       sum_rows(c, m0);
-    }
-  if (has_norm) {
-    __syncthreads();
-    for (int c = wc; c < ipr; c += cg) {
-      if (c != wc) issue_norm(c);
-      for (int m0 = wr; m0 < M; m0 += kBatch * rpp) scale_rows(c, m0);
     }
   }
   __syncthreads();
   }
   PLLM_STAMP(2);
+  // 1 / rms of the input row this thread's results belong to (tile column r), from the sums of squares
+  float row_scale = 1.f;
+  if (!DIRECT && p.norm_w && r < M) {
+    float total = 0.f;
+    for (int j = 0; j < ((K >> 3) + 63) >> 6; ++j) total += sq[r * (((K >> 3) + 63) >> 6) + j];
+    row_scale = rsqrtf(total * (1.f / (float)K) + p.eps);
+  }
 
   auto x_operand = [&](int nth, int j, int s) {
     if (DIRECT) return xbuf[s][j];
@@ -384,14 +374,14 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
           if (EPI == EPI_BF16 || EPI == EPI_F32) {
             const int n = unit * 8 + row;
             if (n < N) {
-              const float v = total(lane) + total(lane + 40);
+              const float v = (total(lane) + total(lane + 40)) * row_scale;
               if (EPI == EPI_F32) ((float*)p.out)[(size_t)m * p.ldo + n] = v;
               else ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(v);
             }
           } else if (EPI == EPI_ROPE_KV && row < 4) {
             const int d = p.head_dim, half = d >> 1, per_head = half >> 2;
             const int head = unit / per_head, ri = (unit - head * per_head) * 4 + row;
-            const float lo = total(lane) + total(lane + 40), hi = total(lane + 16) + total(lane + 56);   // tile rows row + 4
+            const float lo = (total(lane) + total(lane + 40)) * row_scale, hi = (total(lane + 16) + total(lane + 56)) * row_scale;   // tile rows row + 4
             rope_store(p, m, head, ri, lo, hi, rope_cs, rope_sn, rope_slot);
           }
         }
@@ -399,20 +389,20 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
         if (EPI == EPI_BF16 || EPI == EPI_F32) {
           const int n = unit * 16 + row;
           if (n < N) {
-            const float v = total(lane);
+            const float v = total(lane) * row_scale;
             if (EPI == EPI_F32) ((float*)p.out)[(size_t)m * p.ldo + n] = v;
             else ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(v);
           }
         } else if (EPI == EPI_GATED) {
           const int n = unit * 8 + row;
           if (row < 8 && n < N) {
-            const float gate = total(lane), up = total(lane + 32);    // same outputs, 8 tile rows further
+            const float gate = total(lane) * row_scale, up = total(lane + 32) * row_scale;    // same outputs, 8 tile rows further
             ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16((gate / (1.f + expf(-gate))) * up);
           }
         } else if (row < 8) {  // EPI_ROPE_KV
           const int d = p.head_dim, half = d >> 1, per_head = half >> 3;
           const int head = unit / per_head, ri = (unit - head * per_head) * 8 + row;   // rotation index in [0, half)
-          rope_store(p, m, head, ri, total(lane), total(lane + 32), rope_cs, rope_sn, rope_slot);
+          rope_store(p, m, head, ri, total(lane) * row_scale, total(lane + 32) * row_scale, rope_cs, rope_sn, rope_slot);
         }
       }
     }
@@ -453,7 +443,7 @@ static long pllm_lds_bytes_per_cu() {
 // Bytes of LDS a call needs; the caller checks them against the device's limit.
 PLLM_API long pllm_decode_linear_lds_bytes(int M, int K, int waves) {
   const long rows = (((long)M * (K + kPad) * 2) + 15) & ~15L;
-  return rows + (long)waves * 256 * 4;
+  return rows + (long)waves * 256 * 4 + kSquares * 4;
 }
 
 #ifdef PLLM_TRACE
@@ -510,6 +500,7 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   // Rows that need no sum and no norm are read straight from memory (no LDS for them, any K).
   bool direct = !delta && !norm_w;
   if (tune & 64) direct = false;
+  if (!direct && (long)M * (((K >> 3) + 63) >> 6) > kSquares) return -2;
   const size_t lds = direct ? (size_t)waves * 256 * sizeof(float) : (size_t)pllm_decode_linear_lds_bytes(M, K, waves);
   auto ceil_div = [](int a, int b) { return (a + b - 1) / b; };
   bool half = M <= 8 && epi != EPI_GATED && K >= 512 && 2 * ceil_div(2 * units, cus) <= 3 * ceil_div(units, cus);   // at most 3/4

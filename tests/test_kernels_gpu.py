@@ -464,10 +464,13 @@ def test_decode_linear_with_residual_sum_norm_and_row_choice(m, k):
     h2 = plain.rms_norm(x.float()[idx.long()], nw, 1e-4).to(torch.bfloat16)
     got = o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32, norm_weight=nw.cuda(), eps=1e-4, row_index=idx.cuda())
     assert rel_err(got, h2.double() @ w.double().T) <= 1e-2
-    # the fused norm against the norm kernel followed by the plain product
+    # the fused norm against the norm kernel followed by the plain product: the same numbers up to where
+    # the rounding to bfloat16 happens (the norm kernel rounds x * w / rms, the fused kernel rounds x * w and
+    # scales the finished sums by 1 / rms), so each is held to the exact result
     sep = o.decode_linear(o.rmsnorm(x.cuda(), nw.cuda(), 1e-4), w.cuda(), o.EPI_F32)
     fused = o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32, norm_weight=nw.cuda(), eps=1e-4)
-    assert rel_err(fused, sep) <= 2e-3
+    exact = plain.rms_norm(x.double(), nw.double(), 1e-4) @ w.double().T
+    assert rel_err(fused, exact) <= 4e-3 and rel_err(sep, exact) <= 4e-3
 
 
 @pytest.mark.parametrize("m", [1, 8, 16])
