@@ -618,8 +618,11 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
 
 // Merge of the partitions of one (token, head), one wavefront each:
 //   out = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p   over the partitions that hold a visible key,
-// added in partition order.  The maxima are fetched by different lanes at once, then every lane
-// walks the partitions for its channels with independent loads.
+// added in partition order.  The kernel is a chain of waits for memory, so the chain is kept short: with
+// one query per sequence (decoding) the token is the sequence, and the partials of every partition are
+// requested before the lengths that say which of them count have arrived (what does not count is dropped
+// by a select, never multiplied: it may be anything).
+template <bool ONE_QUERY>
 __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ partials, bf16* __restrict__ out, int out_stride,
                                                              const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k,
                                                              int num_seqs, int total_q, int num_heads, int window, int partition_size,
@@ -628,33 +631,44 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (item >= total_q * num_heads) return;
   const int tok = item / num_heads, head = item - tok * num_heads;
-  int lo = 0, hi = num_seqs - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (cu_seqlens_q[mid] <= tok) lo = mid; else hi = mid - 1;
+  const float* base = partials + (size_t)item * num_partitions * kPartialFloats;
+  // maxima of up to 64 partitions at a time, one per lane, requested at once
+  float m_mine = -INFINITY;
+  if (lane < num_partitions) m_mine = base[(size_t)lane * kPartialFloats];
+  int seq = tok, q_begin = tok, num_q = 1;
+  if (!ONE_QUERY) {
+    int lo = 0, hi = num_seqs - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (cu_seqlens_q[mid] <= tok) lo = mid; else hi = mid - 1;
+    }
+    seq = lo;
+    q_begin = cu_seqlens_q[lo];
+    num_q = cu_seqlens_q[lo + 1] - q_begin;
   }
-  const int q_begin = cu_seqlens_q[lo], num_q = cu_seqlens_q[lo + 1] - q_begin;
-  const int qpos = seq_lens_k[lo] - num_q + (tok - q_begin);
+  const int qpos = seq_lens_k[seq] - num_q + (tok - q_begin);
   const int first_key = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
   const int p_lo = first_key / partition_size, p_hi = min(qpos / partition_size, num_partitions - 1);
-  const float* base = partials + (size_t)item * num_partitions * kPartialFloats;
-  float M = -INFINITY;
-  for (int p = p_lo + lane; p <= p_hi; p += 64) M = fmaxf(M, base[(size_t)p * kPartialFloats]);
+  float M = (lane >= p_lo && lane <= p_hi) ? m_mine : -INFINITY;
+  for (int p = 64 + lane; p <= p_hi; p += 64)
+    if (p >= p_lo) M = fmaxf(M, base[(size_t)p * kPartialFloats]);
   M = wave_max(M);
   float l = 0.f;
   float o[(D + 63) / 64];
 #pragma unroll
   for (int j = 0; j < (D + 63) / 64; ++j) o[j] = 0.f;
 #pragma unroll 4
-  for (int p = p_lo; p <= p_hi; ++p) {
+  for (int p = 0; p < num_partitions; ++p) {                     // all of them: the loads wait for nothing
     const float* pp = base + (size_t)p * kPartialFloats;
-    const float w = fast_exp2(pp[0] - M);
-    l += w * pp[1];
+    const bool counts = p >= p_lo && p <= p_hi;
+    const float m_p = pp[0], l_p = pp[1];
+    float a[(D + 63) / 64];
 #pragma unroll
-    for (int j = 0; j < (D + 63) / 64; ++j) {
-      const int i = lane + j * 64;
-      if (i < D) o[j] += w * pp[2 + i];
-    }
+    for (int j = 0; j < (D + 63) / 64; ++j) a[j] = pp[2 + min(lane + j * 64, D - 1)];
+    const float w = counts ? fast_exp2(m_p - M) : 0.f;
+    l += counts ? w * l_p : 0.f;
+#pragma unroll
+    for (int j = 0; j < (D + 63) / 64; ++j) o[j] += counts ? w * a[j] : 0.f;
   }
   const float inv = 1.f / l;
 #pragma unroll
@@ -745,8 +759,13 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   int err = (int)hipGetLastError();
   if (err) return err;
   if (partition_size > 0) {
-    hipLaunchKernelGGL(attention_merge_kernel, dim3((total_q * num_heads + 3) / 4), dim3(256), 0, stream, partials, (bf16*)out,
-                       out_stride, cu_seqlens_q, seq_lens_k, num_seqs, total_q, num_heads, window, partition_size, num_partitions);
+    // one query per sequence: total_q == num_seqs and no sequence is empty (max_q_len bounds them all)
+    if (max_q_len == 1 && total_q == num_seqs)
+      hipLaunchKernelGGL(attention_merge_kernel<true>, dim3((total_q * num_heads + 3) / 4), dim3(256), 0, stream, partials, (bf16*)out,
+                         out_stride, cu_seqlens_q, seq_lens_k, num_seqs, total_q, num_heads, window, partition_size, num_partitions);
+    else
+      hipLaunchKernelGGL(attention_merge_kernel<false>, dim3((total_q * num_heads + 3) / 4), dim3(256), 0, stream, partials, (bf16*)out,
+                         out_stride, cu_seqlens_q, seq_lens_k, num_seqs, total_q, num_heads, window, partition_size, num_partitions);
     err = (int)hipGetLastError();
   }
   return err;
