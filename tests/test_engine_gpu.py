@@ -253,3 +253,17 @@ def test_random_settings_give_the_plain_greedy_tokens(folder_a, folder_b, seed):
         assert o.token_ids == plain_greedy(folder, p, w), f"prompt of {len(p)} tokens, {w} wanted, {o.num_preemptions} preemptions"
     assert engine.cache_manager.num_free_pages() == total
     engine.cache_manager.check_invariants()
+
+
+def test_page_pool_sized_from_free_memory(folder_a):
+    """Without num_gpu_blocks the pool is what fits the memory budget after one probing step of
+    max_num_batched_tokens tokens (more than the model has positions for must not index out of range),
+    capped by what max_num_seqs requests of max_model_len could ever hold."""
+    from paged_llm_amd import SamplingParams
+    engine = engine_for(folder_a, num_gpu_blocks=None, max_num_batched_tokens=512, max_num_seqs=4, max_model_len=128,
+                        gpu_memory_utilization=0.5)
+    assert engine.cache_manager.num_pages() == 4 * 8                    # the cap: plenty of memory for a tiny model
+    out = engine.generate([helpers.random_tokens(9, 256, seed=1)], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))[0]
+    assert out.token_ids == plain_greedy(folder_a, out.prompt_token_ids, 5)
+    with pytest.raises(RuntimeError, match="not enough GPU memory"):
+        engine_for(folder_a, num_gpu_blocks=None, gpu_memory_utilization=1e-6)
