@@ -42,9 +42,6 @@ struct DecodeLinearParams {
   const int* positions; const float* cos_t; const float* sin_t; const int* slots;
   bf16* k_pages; bf16* v_pages;
   int num_heads, num_kv_heads, head_dim, block_size;
-#ifdef PLLM_TRACE
-  long long* trace;
-#endif
 };
 
 __device__ __forceinline__ bf16x8 zero8() {
@@ -123,15 +120,8 @@ __device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, i
   }
 }
 
-#ifdef PLLM_TRACE
-#define PLLM_STAMP(i) do { if (p.trace && threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1)) p.trace[(blockIdx.x ? 16 : 0) + (i)] = wall_clock64(); } while (0)
-#else
-#define PLLM_STAMP(i) do { } while (0)
-#endif
-
 template <int EPI, int WAVES, bool HALF, bool DIRECT, int PRE>
 __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p, int num_units) {
-  PLLM_STAMP(0);
   // Fetch the arguments the first loads depend on in one go (left alone, the compiler fetches each where
   // it is first used, and every fetch is a wait of its own).
   asm volatile("" ::"s"(p.x), "s"(p.delta), "s"(p.norm_w), "s"(p.row_index), "s"(p.W), "s"(p.x_out), "s"(p.ldx), "s"(p.ldd),
@@ -212,7 +202,6 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   if constexpr (DIRECT) {
     rope_inputs();
     request_first();
-    PLLM_STAMP(1);
   } else {
   // ---- the rows into LDS.  A wavefront owns a group of 64 pieces of 8 columns and walks rows with it, up
   // to kBatch rows at a time.  It requests the pieces of its first batch, then its weights, and only then
@@ -289,7 +278,6 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   issue_norm(wc);
   rope_inputs();
   request_first();                                              // the first unit's weights: on their way during all that follows
-  PLLM_STAMP(1);
   sum_rows(wc, wr);
   for (int c = wc; c < ipr; c += cg) {
     if (c != wc) issue_norm(c);
@@ -300,7 +288,6 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   }
   __syncthreads();
   }
-  PLLM_STAMP(2);
   // 1 / rms of the input row this thread's results belong to (tile column r), from the sums of squares
   float row_scale = 1.f;
   if (!DIRECT && p.norm_w && r < M) {
@@ -353,7 +340,6 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
       }
     }
     wrow = wrow_next;
-    PLLM_STAMP(3);
 
     // acc[i] = element (tile row g*4 + i, input row r); add the wavefronts in wave order
 #pragma unroll
@@ -407,7 +393,6 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
       }
     }
     __syncthreads();                                            // the partial sums are read: the buffer may be reused
-    PLLM_STAMP(4);
   }
 }
 
@@ -446,10 +431,6 @@ PLLM_API long pllm_decode_linear_lds_bytes(int M, int K, int waves) {
   return rows + (long)waves * 256 * 4 + kSquares * 4;
 }
 
-#ifdef PLLM_TRACE
-static long long* pllm_trace_buffer = nullptr;
-PLLM_API void pllm_set_trace(long long* buf) { pllm_trace_buffer = buf; }
-#endif
 
 static int num_compute_units() {
   static int cus = 0;
@@ -475,9 +456,6 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   p.M = M; p.N = N; p.K = K; p.positions = positions; p.cos_t = cos_t; p.sin_t = sin_t; p.slots = slots;
   p.k_pages = (bf16*)k_pages; p.v_pages = (bf16*)v_pages; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads;
   p.head_dim = head_dim; p.block_size = block_size;
-#ifdef PLLM_TRACE
-  p.trace = pllm_trace_buffer;
-#endif
   int units;
   switch (epi) {
     case EPI_BF16: case EPI_F32: units = (N + 15) / 16; break;
