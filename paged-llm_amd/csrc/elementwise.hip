@@ -99,18 +99,82 @@ __global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const in
   }
 }
 
+// The same for rows of at most 64 * P pieces of 16 bytes: one wavefront per row keeps the row in registers
+// (P pieces per lane), so there is no LDS and no barrier, and a workgroup of four wavefronts does four rows.
+// The sum of squares is taken per lane over its pieces in order, then over the wavefront.
+template <typename T, int P>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* __restrict__ delta, const int* __restrict__ row_index,
+                                                           const float* __restrict__ w, float eps, T* __restrict__ out, T* x_out,
+                                                           int hidden, int rows) {
+  constexpr int V = 16 / sizeof(T);
+  struct alignas(16) Piece { T v[V]; };
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const size_t src = row_index ? (size_t)row_index[r] : (size_t)r;
+  const int pieces = hidden / V;
+  const Piece* xr = reinterpret_cast<const Piece*>(x + src * hidden);
+  Piece px[P], pd[P];
+#pragma unroll
+  for (int i = 0; i < P; ++i) {
+    const int c = min(lane + i * 64, pieces - 1);                // inside the row; what lies past it is not used
+    px[i] = xr[c];
+    if (delta) pd[i] = reinterpret_cast<const Piece*>(delta + src * hidden)[c];
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < P; ++i) {
+    const int c = lane + i * 64;
+    if (c >= pieces) continue;
+    if (delta) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) px[i].v[j] = from_f32<T>(to_f32(px[i].v[j]) + to_f32(pd[i].v[j]));
+      if (x_out) reinterpret_cast<Piece*>(x_out + src * hidden)[c] = px[i];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc += to_f32(px[i].v[j]) * to_f32(px[i].v[j]);
+  }
+  const float inv = rsqrtf(wave_sum(acc) / (float)hidden + eps);
+  Piece* o = reinterpret_cast<Piece*>(out + (size_t)r * hidden);
+#pragma unroll
+  for (int i = 0; i < P; ++i) {
+    const int c = lane + i * 64;
+    if (c >= pieces) continue;
+    Piece po;
+#pragma unroll
+    for (int j = 0; j < V; ++j) po.v[j] = from_f32<T>((to_f32(px[i].v[j]) * inv) * w[c * V + j]);
+    o[c] = po;
+  }
+}
+
+template <typename T>
+static void launch_rmsnorm(const T* x, const T* delta, const int* row_index, const float* w, float eps, T* out, T* x_out, int rows,
+                           int hidden, hipStream_t stream) {
+  constexpr int V = 16 / sizeof(T);
+  const bool wide = hidden % V == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
+                    (!delta || ((uintptr_t)delta % 16) == 0) && (!x_out || ((uintptr_t)x_out % 16) == 0);
+  const int per_lane = wide ? (hidden / V + 63) / 64 : 0;
+  dim3 grid4((rows + 3) / 4), block(256);
+#define PLLM_ROWS(P_) hipLaunchKernelGGL((rmsnorm_rows_kernel<T, P_>), grid4, block, 0, stream, x, delta, row_index, w, eps, out, x_out, hidden, rows)
+  if (wide && per_lane <= 2) PLLM_ROWS(2);
+  else if (wide && per_lane <= 4) PLLM_ROWS(4);
+  else if (wide && per_lane <= 8) PLLM_ROWS(8);
+  else if (wide && per_lane <= 16) PLLM_ROWS(16);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(rows), block, ((size_t)hidden + 16) * sizeof(float), stream, x, delta, row_index, w,
+                       eps, out, x_out, hidden);
+#undef PLLM_ROWS
+}
+
 PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int* row_index, const float* w, float eps,
                           void* out, void* x_out, int rows, int hidden, hipStream_t stream) {
   if (rows <= 0) return 0;
   const size_t lds = ((size_t)hidden + 16) * sizeof(float);
-  if (lds > 64 * 1024) return -2;  // row does not fit the staging buffer
-  dim3 grid(rows), block(256);
+  if (lds > 64 * 1024) return -2;  // row does not fit the staging buffer of the one-row-per-workgroup kernel
   if (dtype == PLLM_F32)
-    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, lds, stream, (const float*)x, (const float*)delta, row_index, w, eps,
-                       (float*)out, (float*)x_out, hidden);
+    launch_rmsnorm<float>((const float*)x, (const float*)delta, row_index, w, eps, (float*)out, (float*)x_out, rows, hidden, stream);
   else
-    hipLaunchKernelGGL(rmsnorm_kernel<bf16>, grid, block, lds, stream, (const bf16*)x, (const bf16*)delta, row_index, w, eps,
-                       (bf16*)out, (bf16*)x_out, hidden);
+    launch_rmsnorm<bf16>((const bf16*)x, (const bf16*)delta, row_index, w, eps, (bf16*)out, (bf16*)x_out, rows, hidden, stream);
   PLLM_RETURN_LAST_ERROR();
 }
 
