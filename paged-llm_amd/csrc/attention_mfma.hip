@@ -391,13 +391,22 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
   const int num_cols = num_q * G;
   constexpr int kWgCols = 4 * 16 * NCB;
   const int my_tiles = (num_cols + kWgCols - 1) / kWgCols;
-  // Later tiles see more keys.  Unpaired: they are started first, so that the short ones fill the
-  // tail.  Paired (few workgroups, all resident at once): a workgroup takes tile t from the far end
+  // Later tiles see more keys.  paired == 0: they are started first, so that the short ones fill the
+  // tail.  paired == 1 (few workgroups, all resident at once): a workgroup takes tile t from the far end
   // and then its mirror image from the near end, so that every workgroup has the same amount to do.
-  const int far_tile = my_tiles - 1 - (int)blockIdx.x;
-  if (far_tile < 0) return;
-  const int passes = (paired && (int)blockIdx.x < far_tile) ? 2 : 1;
-  if (paired && (int)blockIdx.x > far_tile) return;
+  // paired == 2 (two workgroups resident per compute unit): the first half of the (sequence, kv head) groups
+  // walks its tiles from the far end and the second half from the near end, so that the two workgroups that share a compute
+  // unit (launched half a grid apart) have a far and a near tile between them and overlap each other's
+  // matrix and vector work.
+  int far_tile = my_tiles - 1 - (int)blockIdx.x;
+  if (far_tile < 0) return;                                     // this sequence has fewer tiles than the longest
+  if (paired == 2) {
+    // whole (sequence, kv head) groups change direction, so that every tile of a group is taken once
+    const int group = (int)(blockIdx.z * gridDim.y + blockIdx.y), groups = (int)(gridDim.y * gridDim.z);
+    if (2 * group >= groups) far_tile = (int)blockIdx.x;
+  }
+  const int passes = (paired == 1 && (int)blockIdx.x < far_tile) ? 2 : 1;
+  if (paired == 1 && (int)blockIdx.x > far_tile) return;
   for (int pass = 0; pass < passes; ++pass) {
   const int wg_col0 = (pass == 0 ? far_tile : (int)blockIdx.x) * kWgCols;
   const int pos0 = len_k - num_q;
@@ -728,8 +737,11 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // start), so late tiles have far more keys than early ones.  If all workgroups are resident at
     // once anyway, and pairing still leaves one per compute unit, far and near tiles are paired.
     const long wgs = (long)ptiles * num_kv_heads * num_seqs;
-    const int paired = (pair_tiles && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
-    dim3 pgrid(paired ? (ptiles + 1) / 2 : ptiles, num_kv_heads, num_seqs);
+    int paired = (pair_tiles && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
+    // small heads leave registers for two workgroups per compute unit: with exactly that many workgroups
+    // the mirrored order is the faster one (measured at head size 64; at 128 one workgroup fills a unit)
+    if (D <= 64 && ptiles > 1 && wgs > 256 && wgs <= 512) paired = 2;
+    dim3 pgrid(paired == 1 ? (ptiles + 1) / 2 : ptiles, num_kv_heads, num_seqs);
     hipLaunchKernelGGL((paged_attention_prefill_kernel<2>), pgrid, dim3(256), 0, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q,
                        seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, paired);
