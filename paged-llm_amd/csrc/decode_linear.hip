@@ -396,6 +396,174 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
   }
 }
 
+// 17 to 64 input rows (decoding with many requests): the same units, slabs and fixed order of sums, with
+// MT tiles of 16 input rows side by side.  A weight slab is loaded once per wavefront and multiplied with
+// each tile's rows, which come straight from memory (cache hits) beside it; there is no sum or norm in
+// front of this form (the caller runs the norm on its own) and no LDS for the rows.
+template <int EPI, int MT>
+__global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLinearParams p, int num_units) {
+  constexpr int WAVES = 8, PRE = 2;
+  asm volatile("" ::"s"(p.x), "s"(p.row_index), "s"(p.W), "s"(p.ldx), "s"(p.ldw), "s"(p.M), "s"(p.K), "s"(p.N), "s"(num_units));
+  if (EPI == EPI_ROPE_KV) asm volatile("" ::"s"(p.positions), "s"(p.slots), "s"(p.cos_t), "s"(p.head_dim), "s"(p.num_heads), "s"(p.num_kv_heads));
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  float* part = reinterpret_cast<float*>(lds_raw);              // [WAVES][MT][256]
+  const int M = p.M, N = p.N, K = p.K;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int num_slabs = (K + kSlab - 1) / kSlab;
+  const int my_slabs = wave < num_slabs ? (num_slabs - wave + WAVES - 1) / WAVES : 0;
+  const int padded_slabs = max(PRE, (my_slabs + PRE - 1) / PRE * PRE);
+  bf16x8 wbuf[PRE][4], xbuf[PRE][MT][4];
+  const bf16* xsrc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {                                // tile columns past M read row M - 1; never stored
+    const int row = min(t * 16 + r, M - 1);
+    xsrc[t] = p.x + (size_t)(p.row_index ? p.row_index[row] : row) * p.ldx;
+  }
+  auto load_w = [&](const bf16* wrow, int nth, bf16x8 (&dst)[4]) {      // unconditional, as in the kernel above
+    const int slab = wave + nth * WAVES;
+    const bool mine = nth < my_slabs;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kk = slab * kSlab + j * 32 + g * 8;
+      dst[j] = *reinterpret_cast<const bf16x8*>(mine ? wrow + min(kk, K - 8) : p.W);
+    }
+  };
+  auto load_x = [&](int nth, bf16x8 (&dst)[MT][4]) {
+    const int slab = wave + nth * WAVES;
+    const bool mine = nth < my_slabs;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int kk = slab * kSlab + j * 32 + g * 8;
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(mine ? xsrc[t] + min(kk, K - 8) : p.x);
+        dst[t][j] = kk < K ? v : zero8();
+      }
+    }
+  };
+  auto rows_of_unit = [&](int unit) { return p.W + (size_t)unit_row<EPI, false>(p, unit, r) * p.ldw; };
+  int unit = blockIdx.x;
+  const bf16* wrow = rows_of_unit(unit);
+  int rope_pos[MT], rope_slot[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    rope_pos[t] = 0;
+    rope_slot[t] = -1;
+    if (EPI == EPI_ROPE_KV && tid < 256 && t * 16 + r < M) {
+      rope_pos[t] = p.cos_t ? p.positions[t * 16 + r] : 0;
+      rope_slot[t] = p.slots[t * 16 + r];
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < PRE; ++s) {
+    load_x(s, xbuf[s]);
+    load_w(wrow, s, wbuf[s]);
+  }
+
+  for (; unit < num_units; unit += gridDim.x) {
+    floatx4 acc[MT];
+    float rope_cs[MT], rope_sn[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+      rope_cs[t] = 1.f;
+      rope_sn[t] = 0.f;
+    }
+    if (EPI == EPI_ROPE_KV && tid < 256 && p.cos_t) {
+      const int half = p.head_dim >> 1, per_head = half >> 3;
+      const int row = g * 4 + (tid >> 6);
+      const int head = unit / per_head, ri = (unit - head * per_head) * 8 + row;
+      if (row < 8 && head < p.num_heads + p.num_kv_heads) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          if (t * 16 + r < M) {
+            rope_cs[t] = p.cos_t[(size_t)rope_pos[t] * half + ri];
+            rope_sn[t] = p.sin_t[(size_t)rope_pos[t] * half + ri];
+          }
+        }
+      }
+    }
+    const int next = unit + gridDim.x;
+    const bf16* wrow_next = next < num_units ? rows_of_unit(next) : p.W;
+    for (int base = 0; base < padded_slabs; base += PRE) {
+#pragma unroll
+      for (int s = 0; s < PRE; ++s) {
+        const int nth = base + s;
+        if (nth < my_slabs) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wbuf[s][j], xbuf[s][t][j], acc[t], 0, 0, 0);
+          }
+        }
+        const int ahead = nth + PRE;
+        if (ahead < padded_slabs) {
+          load_x(ahead, xbuf[s]);
+          load_w(wrow, ahead, wbuf[s]);
+        } else if (next < num_units) {
+          load_x(ahead - padded_slabs, xbuf[s]);
+          load_w(wrow_next, ahead - padded_slabs, wbuf[s]);
+        }
+      }
+    }
+    wrow = wrow_next;
+
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[(wave * MT + t) * 256 + i * 64 + lane] = acc[t][i];
+    }
+    __syncthreads();
+    if (tid < 256) {
+      const int i = tid >> 6, row = g * 4 + i;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        auto total = [&](int ln) {
+          float s = 0.f;
+#pragma unroll
+          for (int w = 0; w < WAVES; ++w) s += part[(w * MT + t) * 256 + i * 64 + ln];
+          return s;
+        };
+        const int m = t * 16 + r;
+        if (m >= M) continue;
+        if (EPI == EPI_BF16 || EPI == EPI_F32) {
+          const int n = unit * 16 + row;
+          if (n < N) {
+            const float v = total(lane);
+            if (EPI == EPI_F32) ((float*)p.out)[(size_t)m * p.ldo + n] = v;
+            else ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(v);
+          }
+        } else if (EPI == EPI_GATED) {
+          const int n = unit * 8 + row;
+          if (row < 8 && n < N) {
+            const float gate = total(lane), up = total(lane + 32);
+            ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16((gate / (1.f + expf(-gate))) * up);
+          }
+        } else if (row < 8) {  // EPI_ROPE_KV
+          const int half = p.head_dim >> 1, per_head = half >> 3;
+          const int head = unit / per_head, ri = (unit - head * per_head) * 8 + row;
+          rope_store(p, m, head, ri, total(lane), total(lane + 32), rope_cs[t], rope_sn[t], rope_slot[t]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <int EPI>
+static int launch_wide(const DecodeLinearParams& p, int units, int blocks, hipStream_t stream) {
+  const int tiles = (p.M + 15) / 16;
+  const size_t lds = (size_t)8 * tiles * 256 * sizeof(float);
+  switch (tiles) {
+    case 2: hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, 2>), dim3(blocks), dim3(512), lds, stream, p, units); break;
+    case 3: hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, 3>), dim3(blocks), dim3(512), lds, stream, p, units); break;
+    case 4: hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, 4>), dim3(blocks), dim3(512), lds, stream, p, units); break;
+    default: return -2;
+  }
+  return (int)hipGetLastError();
+}
+
 template <int EPI, int WAVES, bool HALF, bool DIRECT, int PRE>
 static int launch(const DecodeLinearParams& p, int units, int blocks, size_t lds, hipStream_t stream) {
   auto kernel = decode_linear_kernel<EPI, WAVES, HALF, DIRECT, PRE>;
@@ -449,7 +617,7 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
                                 void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim, int block_size,
                                 int tune, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 16 || K <= 0 || (K & 7) || (ldx & 7) || (ldw & 7) || (delta && (ldd & 7)) || (x_out && (ldxo & 7))) return -2;
+  if (M > 64 || (M > 16 && (delta || norm_w)) || K <= 0 || (K & 7) || (ldx & 7) || (ldw & 7) || (delta && (ldd & 7)) || (x_out && (ldxo & 7))) return -2;
   DecodeLinearParams p;
   p.x = (const bf16*)x; p.ldx = ldx; p.delta = (const bf16*)delta; p.ldd = ldd; p.norm_w = norm_w; p.eps = eps;
   p.x_out = (bf16*)x_out; p.ldxo = ldxo; p.row_index = row_index; p.W = (const bf16*)W; p.ldw = ldw; p.out = out; p.ldo = ldo;
@@ -475,6 +643,16 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   // rows, bit 4/5 = one/two workgroups per compute unit, bit 6 = rows through LDS even without a sum or norm.
   const int cus = num_compute_units();
   constexpr int waves = 8;
+  if (M > 16) {                                                 // tiles of 16 rows side by side, one workgroup per compute unit
+    const int per_block = (units + cus - 1) / cus, blocks = (units + per_block - 1) / per_block;
+    switch (epi) {
+      case EPI_BF16: return launch_wide<EPI_BF16>(p, units, blocks, stream);
+      case EPI_F32: return launch_wide<EPI_F32>(p, units, blocks, stream);
+      case EPI_GATED: return launch_wide<EPI_GATED>(p, units, blocks, stream);
+      case EPI_ROPE_KV: return launch_wide<EPI_ROPE_KV>(p, units, blocks, stream);
+    }
+    return -3;
+  }
   // Rows that need no sum and no norm are read straight from memory (no LDS for them, any K).
   bool direct = !delta && !norm_w;
   if (tune & 64) direct = false;

@@ -293,7 +293,8 @@ _stream_sink: dict = {}
 
 # ------------------------------------------------------------------------------------------- fused decode products
 EPI_BF16, EPI_F32, EPI_GATED, EPI_ROPE_KV = 0, 1, 2, 3
-DECODE_MAX_ROWS = 16
+DECODE_MAX_ROWS = 16          # rows of the fused form with a sum or norm in front
+DECODE_WIDE_MAX_ROWS = 64     # rows of the form for plain rows
 _DECODE_SIG = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
                c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                c_int, c_void_p]
@@ -313,19 +314,31 @@ def _max_lds_bytes(device) -> int:
 def decode_linear_takes(rows: int, K: int, x: torch.Tensor, w: torch.Tensor, staged: bool = True) -> bool:
     """Whether the fused decode product takes these operands (else the caller runs the parts apart).
     ``staged``: a residual sum or a norm runs in front, so the rows must fit into LDS; plain rows are read
-    straight from memory and may be of any length."""
-    if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < rows <= DECODE_MAX_ROWS and K % 8 == 0):
+    straight from memory, may be of any length, and there may be up to 64 of them."""
+    if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < rows <= (DECODE_MAX_ROWS if staged else DECODE_WIDE_MAX_ROWS) and K % 8 == 0):
         return False
     if not (x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return False
     if not staged:
-        # With more than 8 rows every unit rereads as many bytes of rows as it streams of weights; for long
-        # rows the library's product is then faster (measured at K = 5632 and 14336).
-        return rows <= 8 or K <= 4096
+        return True
     f = _fn("decode_linear.hip", "pllm_decode_linear_lds_bytes", signature=[c_int, c_int, c_int])
     f.restype = c_long
     return int(f(rows, K, 8)) <= _max_lds_bytes(x.device)
+
+
+def decode_linear_pays(rows: int, N: int, K: int, epi: int, staged: bool) -> bool:
+    """Whether the fused decode product is the faster choice for plain rows (measured against the library's
+    product; by sizes only).  Every unit of 16 weight rows rereads all rows from the cache: beyond 8 rows
+    that is as much as it streams of weights, and the library wins for long rows (K = 5632, 14336); beyond
+    16 rows it wins for all but small matrices (q/k/v and output projections of 2048-wide models), where
+    the fused kernel still fills the chip better; beyond 32 rows only the saved rotary kernel pays."""
+    if staged or rows <= 8:
+        return True
+    if rows <= 16:
+        return K <= 4096
+    small = N * K <= (1 << 23)
+    return small and (rows <= 32 or epi == EPI_ROPE_KV)
 
 
 def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: torch.Tensor | None = None,
@@ -345,7 +358,7 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
     _need(x.dim() == 2 and w.dim() == 2 and w.shape[1] == K, f"decode_linear shapes {tuple(x.shape)} x {tuple(w.shape)}^T")
     staged = delta is not None or norm_weight is not None or bool(tune & 64)
     _need(decode_linear_takes(M, K, x, w, staged),
-          "decode_linear takes bfloat16, 1..16 rows, K a multiple of 8, and with a sum or norm in front rows that fit LDS")
+          "decode_linear takes bfloat16, K a multiple of 8, 1..64 plain rows, or with a sum or norm in front 1..16 rows that fit LDS")
     if delta is not None:
         _need(delta.shape == x.shape and delta.dtype == x.dtype and delta.stride(1) == 1 and delta.stride(0) % 8 == 0
               and delta.data_ptr() % 16 == 0, "delta must match x")

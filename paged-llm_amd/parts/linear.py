@@ -3,6 +3,7 @@
 * float32: the plain kernel with float operands (the true 32-bit path), always.
 * bfloat16, at most 16 rows (decoding): the fused decode kernel, which also takes in a pending
   residual sum + norm in front and an activation or the rotary/cache write behind.
+* bfloat16, 17 to 64 rows and a small matrix: the same kernel's form for plain rows (the norm runs first).
 * bfloat16, more rows (prompt portions): the vendor's matrix-product library; float results
   (logits of many rows) come from the MFMA kernel for few rows, 64 rows at a time.
 * shapes none of these accept: the plain kernel.
@@ -28,7 +29,8 @@ def _fused(x, weight: torch.Tensor, epi: int, rope: dict | None = None):
             x.fused_done(args)
             return out
         x = x.rows()
-    if x.dtype == torch.bfloat16 and ops.decode_linear_takes(x.shape[0], x.shape[1], x, weight, staged=False):
+    if (x.dtype == torch.bfloat16 and ops.decode_linear_takes(x.shape[0], x.shape[1], x, weight, staged=False)
+            and ops.decode_linear_pays(x.shape[0], weight.shape[0], x.shape[1], epi, staged=False)):
         return ops.decode_linear(x, weight, epi, rope=rope)
     return None
 
