@@ -401,49 +401,17 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
 
 
 # ------------------------------------------------------------------------------------------- choices
-SKINNY_MAX_ROWS = 64
-_SKINNY_SIG = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
-
-
-def _skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
-    K = a.shape[1]
-    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and K % 8 == 0 and a.stride(1) == 1 and w.stride(1) == 1
-            and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
-
-
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """a [M <= 64, K] times w [N, K]^T on the matrix cores, streaming w once; float or bfloat16 out."""
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """a [M, K] times w [N, K]^T for more rows than the fused decode kernel takes (prompt portions, large
+    decode batches): the vendor's matrix-product library, as the reference's engine uses a library for
+    its products (nn.Linear, pagedllm/model/llama.py:141-144).  Float accumulation; the result is bfloat16
+    or, for logits, float32 straight from the accumulators."""
     _on_gpu(a, w)
-    _need(a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], f"gemm shapes {tuple(a.shape)} x {tuple(w.shape)}^T")
-    _need(_skinny_ok(a, w), "gemm_skinny needs bfloat16 operands with K, row strides and addresses in multiples of 8 elements")
-    M, K = a.shape
-    _need(0 < M <= SKINNY_MAX_ROWS, f"gemm_skinny takes 1..{SKINNY_MAX_ROWS} rows, got {M}")
-    N = w.shape[0]
-    out_dtype = out_dtype or torch.bfloat16
-    _need(out_dtype in (torch.bfloat16, torch.float32), "output is bfloat16 or float32")
-    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    _check(_fn("gemm_skinny.hip", "pllm_gemm_skinny", signature=_SKINNY_SIG)(
-        _ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), M, N, K, 1 if out_dtype == torch.float32 else 0,
-        _stream()), "gemm_skinny")
-    return out
-
-
-def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
-    """The fast bfloat16 products; None when neither takes the shape (the caller falls back to
-    the plain kernel).  The choice looks at the number of rows only."""
-    if not _skinny_ok(a, w):
-        return None
-    M = a.shape[0]
-    out_dtype = out_dtype or torch.bfloat16
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1],
+          f"gemm_bf16 takes bfloat16 [M, K] x [N, K]^T, got {tuple(a.shape)} {a.dtype} x {tuple(w.shape)} {w.dtype}")
     if out_dtype == torch.float32:
-        # Float results for many rows (logits of a whole prompt): the same kernel, 64 rows at a time.
-        return torch.cat([gemm_skinny(a[i:i + SKINNY_MAX_ROWS], w, out_dtype) for i in range(0, M, SKINNY_MAX_ROWS)], dim=0)
-    return gemm_large_bf16(a, w)
-
-
-def gemm_large_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """Many rows (prompt portions): the vendor's matrix-product library, as the reference's engine
-    uses a library for its products (nn.Linear, pagedllm/model/llama.py:141-144)."""
+        return torch.mm(a, w.t(), out_dtype=torch.float32)
+    _need(out_dtype in (None, torch.bfloat16), "output is bfloat16 or float32")
     return torch.mm(a, w.t())
 
 

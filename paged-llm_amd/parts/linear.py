@@ -4,9 +4,8 @@
 * bfloat16, at most 16 rows (decoding): the fused decode kernel, which also takes in a pending
   residual sum + norm in front and an activation or the rotary/cache write behind.
 * bfloat16, 17 to 64 rows and a small matrix: the same kernel's form for plain rows (the norm runs first).
-* bfloat16, more rows (prompt portions): the vendor's matrix-product library; float results
-  (logits of many rows) come from the MFMA kernel for few rows, 64 rows at a time.
-* shapes none of these accept: the plain kernel.
+* bfloat16, more rows (prompt portions): the vendor's matrix-product library, with bfloat16 or (logits)
+  float results.
 
 The choice depends on the number of rows and the sizes only, never on the rows' content.  ``x`` may
 be a tensor or a ``PendingNorm``.
@@ -42,10 +41,8 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> tor
         if out is not None:
             return out
     x = rows_of(x)
-    if x.dtype == torch.bfloat16:
-        fast = ops.gemm_bf16(x, weight, out_dtype)
-        if fast is not None:
-            return fast
+    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+        return ops.gemm_bf16(x, weight, out_dtype)
     return ops.gemm_generic(x, weight, out_dtype)
 
 

@@ -287,24 +287,21 @@ def test_sampling_frequencies_follow_the_filtered_distribution(temperature, top_
     assert chi2 < dof + 5 * math.sqrt(2 * max(dof, 1)) + 5, f"chi-square {chi2:.1f} for {dof} degrees of freedom"
 
 
-# ----------------------------------------------------------------------------------- bfloat16 products for few rows
-@pytest.mark.parametrize("m", [1, 5, 8, 16, 17, 33, 48, 64])
-@pytest.mark.parametrize("n,k", [(16, 64), (100, 96), (517, 176), (2048, 2048), (2048, 5632), (96, 1000)])
-def test_gemm_skinny(m, n, k):
+# ----------------------------------------------------------------------------------- bfloat16 products for many rows
+@pytest.mark.parametrize("m", [17, 64, 200])
+@pytest.mark.parametrize("n,k", [(100, 96), (517, 176), (2048, 5632), (96, 1000), (33, 37)])
+def test_library_product_float_and_bfloat16_out(m, n, k):
     a, w = rnd(m, k, seed=20, dtype=torch.bfloat16), rnd(n, k, seed=21, dtype=torch.bfloat16)
     want = a.double() @ w.double().T
-    assert rel_err(ops().gemm_skinny(a.cuda(), w.cuda(), torch.float32), want) <= 2e-5
-    out16 = ops().gemm_skinny(a.cuda(), w.cuda())
+    assert rel_err(ops().gemm_bf16(a.cuda(), w.cuda(), torch.float32), want) <= 2e-5
+    out16 = ops().gemm_bf16(a.cuda(), w.cuda())
     assert out16.dtype == torch.bfloat16 and rel_err(out16, want) <= 1e-2
 
 
-def test_gemm_skinny_strided_rows():
-    big = rnd(9, 300, seed=24, dtype=torch.bfloat16).cuda()
-    a = big[:, 40:40 + 176]                                       # row stride 300: not a multiple of 8
-    assert ops().gemm_bf16(a, rnd(64, 176, seed=25, dtype=torch.bfloat16).cuda()) is None
-    big = rnd(9, 304, seed=24, dtype=torch.bfloat16).cuda()
-    a, w = big[:, 40:40 + 176], rnd(64, 176, seed=25, dtype=torch.bfloat16).cuda()
-    assert rel_err(ops().gemm_skinny(a, w, torch.float32), a.double().cpu() @ w.double().cpu().T) <= 2e-5
+def test_library_product_strided_rows():
+    big = rnd(40, 300, seed=24, dtype=torch.bfloat16).cuda()
+    a, w = big[:, 41:41 + 176], rnd(64, 176, seed=25, dtype=torch.bfloat16).cuda()          # row stride and offset of no special form
+    assert rel_err(ops().gemm_bf16(a, w, torch.float32), a.double().cpu() @ w.double().cpu().T) <= 2e-5
 
 
 def test_large_bf16_product_and_float_rows():
