@@ -356,11 +356,15 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prompt portions: one workgroup of four wavefronts per (sequence, kv head, 128 columns).  All four
-// walk the same blocks of 64 keys, each for its own 32 columns, so the block is fetched once into
-// LDS (each wavefront fetches the 16 keys and values of one tile: one page lookup, uniform in the
-// wavefront) and the next block travels while the current one is used: global -> registers while
-// computing, registers -> the other LDS buffer, one barrier per block.
+// Prompt portions: one workgroup per (sequence, kv head, 128 columns), of KG groups of four wavefronts.
+// A step covers 64 * KG keys: the four wavefronts of group kg work on keys kg * 64 .. kg * 64 + 63 of the
+// step, each for its own 32 columns, so a step is fetched once into LDS (each wavefront fetches the 16
+// keys and values of one tile: one page lookup, uniform in the wavefront) and the next step travels while
+// the current one is used: global -> registers while computing, registers -> the other LDS buffer, one
+// barrier per step.  With KG = 2 the two groups hold two halves of every column's softmax, merged through
+// LDS at the end (group 0 first): a compute unit then holds two wavefronts per SIMD with equal work, which
+// overlap each other's matrix, vector and LDS phases (one wavefront alone leaves the SIMD idle for
+// most of its chain of dependent steps).
 //
 // LDS layouts: keys [64 rows][D + 8] (row = key), values [D rows][64 + 8] (row = channel) with the
 // keys of each half of 32 stored in operand order (lane group g, tile h, key i -> g*8 + h*4 + i), so
@@ -375,15 +379,21 @@ constexpr int kVPerLane = (kVChunks + 63) / 64;
 struct MaskedTag { static constexpr bool value = true; };
 struct PlainTag { static constexpr bool value = false; };
 
-template <int NCB>
-__global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
+template <int NCB, int KG>
+__global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
     int block_size, float scale, int window, int paired) {
-  __shared__ __attribute__((aligned(16))) bf16 k_s[2][64 * kKRow];
-  __shared__ __attribute__((aligned(16))) bf16 v_s[2][D * kVRow];
+  extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
+  constexpr int kKTile = 64 * kKRow, kVTile = D * kVRow;         // elements of one group's keys / values of a step
+  // keys [2 buffers][KG][64 rows][kKRow], then values [2 buffers][KG][D rows][kVRow].  Addresses are formed
+  // from the LDS symbol where they are used: a pointer kept in a register may be spilled, and comes back as
+  // a generic pointer whose accesses are no longer LDS instructions.
+#define PLLM_K_TILE(buf, group) (reinterpret_cast<bf16*>(prefill_lds) + ((buf) * KG + (group)) * kKTile)
+#define PLLM_V_TILE(buf, group) (reinterpret_cast<bf16*>(prefill_lds) + 2 * KG * kKTile + ((buf) * KG + (group)) * kVTile)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const int cw = wave & 3, kg = wave >> 2;                      // column share and key group of this wavefront
   const int seq = blockIdx.z, kvh = blockIdx.y;
   const int G = num_heads / num_kv_heads;
   const int q_begin = cu_seqlens_q[seq], num_q = cu_seqlens_q[seq + 1] - q_begin;
@@ -394,17 +404,8 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
   // Later tiles see more keys.  paired == 0: they are started first, so that the short ones fill the
   // tail.  paired == 1 (few workgroups, all resident at once): a workgroup takes tile t from the far end
   // and then its mirror image from the near end, so that every workgroup has the same amount to do.
-  // paired == 2 (two workgroups resident per compute unit): the first half of the (sequence, kv head) groups
-  // walks its tiles from the far end and the second half from the near end, so that the two workgroups that share a compute
-  // unit (launched half a grid apart) have a far and a near tile between them and overlap each other's
-  // matrix and vector work.
-  int far_tile = my_tiles - 1 - (int)blockIdx.x;
+  const int far_tile = my_tiles - 1 - (int)blockIdx.x;
   if (far_tile < 0) return;                                     // this sequence has fewer tiles than the longest
-  if (paired == 2) {
-    // whole (sequence, kv head) groups change direction, so that every tile of a group is taken once
-    const int group = (int)(blockIdx.z * gridDim.y + blockIdx.y), groups = (int)(gridDim.y * gridDim.z);
-    if (2 * group >= groups) far_tile = (int)blockIdx.x;
-  }
   const int passes = (paired == 1 && (int)blockIdx.x < far_tile) ? 2 : 1;
   if (paired == 1 && (int)blockIdx.x > far_tile) return;
   for (int pass = 0; pass < passes; ++pass) {
@@ -416,7 +417,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
   const int k_hi = wg_qmax + 1;
   const int k_lo = ((window > 0 && wg_qmin - window + 1 > 0) ? wg_qmin - window + 1 : 0) & ~63;
   // this wavefront's columns
-  const int col0 = wg_col0 + wave * 16 * NCB;
+  const int col0 = wg_col0 + cw * 16 * NCB;
   const bool wave_on = col0 < num_cols;
   const int last_col = min(col0 + 16 * NCB, num_cols) - 1;
   const int qpos_min = pos0 + col0 / G, qpos_max = wave_on ? pos0 + last_col / G : -1;
@@ -489,16 +490,16 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
       const int c = lane + i * 64;
       if (c < kKChunks) {
         const int row = c / (D / 8), part = c - row * (D / 8);
-        *reinterpret_cast<bf16x8*>(&k_s[buf][(wave * 16 + row) * kKRow + part * 8]) = f.k[i];
+        *reinterpret_cast<bf16x8*>(PLLM_K_TILE(buf, kg) + (cw * 16 + row) * kKRow + part * 8) = f.k[i];
       }
     }
-    const int a = wave >> 1, h = wave & 1;                        // tile `wave` is half h of the 32-key group a
+    const int a = cw >> 1, h = cw & 1;                            // tile `cw` of the group is half h of its 32 keys a
 #pragma unroll
     for (int i = 0; i < kVPerLane; ++i) {
       const int c = lane + i * 64;
       if (c < kVChunks) {
         const int ch = c >> 1, half = c & 1;
-        bf16* dst = &v_s[buf][ch * kVRow + a * 32 + h * 4];
+        bf16* dst = PLLM_V_TILE(buf, kg) + ch * kVRow + a * 32 + h * 4;
         // keys half*8 .. half*8+7 of the tile: lane groups g = half*2 and half*2 + 1, four keys each
         bf16x4 lo4, hi4;
 #pragma unroll
@@ -513,8 +514,8 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
   // the version without any comparison.
   auto compute = [&](int buf, int n0, auto masked_tag) {
     constexpr bool kMasked = decltype(masked_tag)::value;
-    const bf16* kb = k_s[buf];
-    const bf16* vb = v_s[buf];
+    const bf16* kb = PLLM_K_TILE(buf, kg);
+    const bf16* vb = PLLM_V_TILE(buf, kg);
     floatx4 s_t[4][NCB];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
@@ -587,32 +588,68 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
   const int full_from = window > 0 ? max(qpos_max - window + 1, 0) : 0;   // blocks from here on are inside every column's window
   const bool all_cols = col0 + 16 * NCB <= num_cols;
 
-  // ---- the blocks.  Block i is computed from LDS while block i + 1 sits in registers (requested one
-  //      step earlier, written to the other LDS buffer after the computation) and block i + 2 is being
+  // ---- the steps.  Step i is computed from LDS while step i + 1 sits in registers (requested one
+  //      step earlier, written to the other LDS buffer after the computation) and step i + 2 is being
   //      requested: a fetch has two steps to arrive.
+  constexpr int kStepKeys = 64 * KG;
   auto step = [&](int n0, int buf, Fetched& arriving, Fetched& free_regs) {
-    if (n0 + 128 < k_hi) fetch(free_regs, n0 + 128);
-    if (wave_on && n0 < vis_hi && n0 + 64 > vis_lo) {
-      if (all_cols && n0 + 63 <= qpos_min && n0 >= full_from) compute(buf, n0, PlainTag{});
-      else compute(buf, n0, MaskedTag{});
+    if (n0 + 2 * kStepKeys < k_hi) fetch(free_regs, n0 + 2 * kStepKeys);
+    const int mine = n0 + kg * 64;                                // this group's 64 keys of the step
+    if (wave_on && mine < vis_hi && mine + 64 > vis_lo) {
+      if (all_cols && mine + 63 <= qpos_min && mine >= full_from) compute(buf, mine, PlainTag{});
+      else compute(buf, mine, MaskedTag{});
     }
-    if (n0 + 64 < k_hi) stash(arriving, buf ^ 1);
+    if (n0 + kStepKeys < k_hi) stash(arriving, buf ^ 1);
     __syncthreads();
   };
   Fetched regs_a, regs_b;
   fetch(regs_a, k_lo);
-  if (k_lo + 64 < k_hi) fetch(regs_b, k_lo + 64);
+  if (k_lo + kStepKeys < k_hi) fetch(regs_b, k_lo + kStepKeys);
   stash(regs_a, 0);
   __syncthreads();
-  for (int n0 = k_lo; n0 < k_hi; n0 += 128) {
-    step(n0, 0, regs_b, regs_a);                                  // block n0 in buffer 0; n0 + 64 arrives in regs_b
-    if (n0 + 64 < k_hi) step(n0 + 64, 1, regs_a, regs_b);
+  for (int n0 = k_lo; n0 < k_hi; n0 += 2 * kStepKeys) {
+    step(n0, 0, regs_b, regs_a);                                  // step n0 in buffer 0; the next one arrives in regs_b
+    if (n0 + kStepKeys < k_hi) step(n0 + kStepKeys, 1, regs_a, regs_b);
+  }
+
+  if (KG == 2) {
+    // Group 1 hands its half of every column to group 0 through LDS (the last step ended with a barrier,
+    // so the key and value buffers are free): per wavefront [NCB][DBLOCKS * 4 + 2][64 lanes] floats.
+    float* hand = reinterpret_cast<float*>(prefill_lds) + (size_t)cw * NCB * (DBLOCKS * 4 + 2) * 64;
+    if (kg == 1) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) {
+        float* h = hand + cb * (DBLOCKS * 4 + 2) * 64 + lane;
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) h[(db * 4 + i) * 64] = acc[cb][db][i];
+        h[DBLOCKS * 4 * 64] = m_run[cb];
+        h[(DBLOCKS * 4 + 1) * 64] = l_run[cb];
+      }
+    }
+    __syncthreads();
+    if (kg == 0) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) {
+        const float* h = hand + cb * (DBLOCKS * 4 + 2) * 64 + lane;
+        const float m_other = h[DBLOCKS * 4 * 64], l_other = h[(DBLOCKS * 4 + 1) * 64];
+        const float m_new = fmaxf(m_run[cb], m_other);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float a_mine = fast_exp2(m_run[cb] - m_safe), a_other = fast_exp2(m_other - m_safe);   // 2^-inf = 0: an empty half adds nothing
+        l_run[cb] = l_run[cb] * a_mine + l_other * a_other;
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[cb][db][i] = acc[cb][db][i] * a_mine + h[(db * 4 + i) * 64] * a_other;
+      }
+    }
   }
 
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb) {
-    if (!my_valid[cb]) continue;
-    const float inv = 1.f / group_sum(l_run[cb]);
+    const float inv = 1.f / group_sum(l_run[cb]);                 // every lane takes part in the exchange
+    if (!my_valid[cb] || kg != 0) continue;
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) {
       bf16x4 o;
@@ -623,6 +660,8 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(
   }
   __syncthreads();                                                // the LDS buffers are reused by the next pass
   }  // pass
+#undef PLLM_K_TILE
+#undef PLLM_V_TILE
 }
 
 // Merge of the partitions of one (token, head), one wavefront each:
@@ -700,6 +739,13 @@ static long pllm_max_lds() {
 }
 
 // LDS floats of the several-wavefront variant.
+// LDS of the prompt kernel with kg key groups: two buffers of keys and values per group, reused at the
+// end for the hand-over of group 1's halves (four wavefronts x 2 column blocks).
+constexpr size_t prefill_lds_bytes(int kg) {
+  const size_t buffers = (size_t)2 * kg * (64 * kKRow + D * kVRow) * sizeof(bf16);
+  const size_t hand = (size_t)4 * 2 * (DBLOCKS * 4 + 2) * 64 * sizeof(float);
+  return buffers > hand ? buffers : hand;
+}
 static size_t merge_lds_bytes(int ncb, int waves) { return (size_t)(2 * waves * ncb * 16 + waves * ncb * DBLOCKS * 4 * 64) * sizeof(float); }
 
 // waves == 1: every work item is one wavefront that walks its key range.
@@ -737,12 +783,18 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // start), so late tiles have far more keys than early ones.  If all workgroups are resident at
     // once anyway, and pairing still leaves one per compute unit, far and near tiles are paired.
     const long wgs = (long)ptiles * num_kv_heads * num_seqs;
-    int paired = (pair_tiles && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
-    // small heads leave registers for two workgroups per compute unit: with exactly that many workgroups
-    // the mirrored order is the faster one (measured at head size 64; at 128 one workgroup fills a unit)
-    if (D <= 64 && ptiles > 1 && wgs > 256 && wgs <= 512) paired = 2;
+    const int paired = (pair_tiles && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
     dim3 pgrid(paired == 1 ? (ptiles + 1) / 2 : ptiles, num_kv_heads, num_seqs);
-    hipLaunchKernelGGL((paged_attention_prefill_kernel<2>), pgrid, dim3(256), 0, stream, (const bf16*)q, q_stride,
+    // two key groups (eight wavefronts) for the head sizes that then still fit into registers and LDS; else one
+    constexpr bool two = D <= 96 && prefill_lds_bytes(2) <= 160 * 1024;            // larger heads need more registers than eight wavefronts leave
+    constexpr size_t lds = prefill_lds_bytes(two ? 2 : 1);
+    if ((long)lds > pllm_max_lds()) return -2;
+    auto kern = paged_attention_prefill_kernel<2, two ? 2 : 1>;
+    if (lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kern, pgrid, dim3(two ? 512 : 256), lds, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q,
                        seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, paired);
     return (int)hipGetLastError();
