@@ -728,6 +728,17 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
 
 PLLM_API int pllm_attention_mfma_head_dim() { return D; }
 
+static int num_compute_units() {
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
 static long pllm_max_lds() {
   static long cached = 0;
   if (!cached) {
@@ -783,13 +794,21 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // start), so late tiles have far more keys than early ones.  If all workgroups are resident at
     // once anyway, and pairing still leaves one per compute unit, far and near tiles are paired.
     const long wgs = (long)ptiles * num_kv_heads * num_seqs;
-    const int paired = (pair_tiles && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
+    const int paired = ((pair_tiles & 1) && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
     dim3 pgrid(paired == 1 ? (ptiles + 1) / 2 : ptiles, num_kv_heads, num_seqs);
-    // two key groups (eight wavefronts) for the head sizes that then still fit into registers and LDS; else one
-    constexpr bool two = D <= 96 && prefill_lds_bytes(2) <= 160 * 1024;            // larger heads need more registers than eight wavefronts leave
-    constexpr size_t lds = prefill_lds_bytes(two ? 2 : 1);
+    // Two key groups (eight wavefronts, one workgroup per compute unit) when there are too few workgroups to
+    // give every compute unit two of the four-wavefront kind at a time, and for the head sizes that then still
+    // fit into registers and LDS; else one key group.  pair_tiles bits 1 and 2 force one or two (measurements).
+    constexpr bool two_fits = D <= 96 && prefill_lds_bytes(2) <= 160 * 1024;
+    bool two = two_fits && (long)pgrid.x * pgrid.y * pgrid.z < 2L * num_compute_units();
+    if (pair_tiles & 2) two = false;
+    if ((pair_tiles & 4) && two_fits) two = true;
+    const size_t lds = prefill_lds_bytes(two ? 2 : 1);
     if ((long)lds > pllm_max_lds()) return -2;
-    auto kern = paged_attention_prefill_kernel<2, two ? 2 : 1>;
+    auto kern = paged_attention_prefill_kernel<2, 1>;
+    if constexpr (two_fits) {
+      if (two) kern = paged_attention_prefill_kernel<2, 2>;
+    }
     if (lds > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) return (int)e;
