@@ -170,3 +170,31 @@ def test_long_decoding(folders, dtype):
     for i in range(6, len(toks)):
         trace.step([("long", toks[i:i + 1], "all")])
     check(helpers.replay_in_process(session, trace), folder, {"long": toks}, dtype)
+
+
+# Widths that are no multiple of 8 (or odd): the fused and vectorised kernels do not take them, and the
+# choice of another kernel must not change the result.
+ODD_BASE = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "rope_theta": 10000.0, "tie_word_embeddings": False,
+            "rms_norm_eps": 1e-5, "max_position_embeddings": 256}
+ODD_WIDTHS = {
+    "hidden100": dict(ODD_BASE, num_hidden_layers=2, hidden_size=100, num_attention_heads=2, num_key_value_heads=1, head_dim=16,
+                      intermediate_size=90, vocab_size=77),
+    "hidden33": dict(ODD_BASE, num_hidden_layers=1, hidden_size=33, num_attention_heads=1, num_key_value_heads=1, head_dim=16,
+                     intermediate_size=35, vocab_size=67),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(ODD_WIDTHS))
+def test_widths_that_are_no_multiple_of_eight(tmp_path, name, dtype):
+    cfg = ODD_WIDTHS[name]
+    folder = helpers.make_folder(tmp_path, cfg, seed=5, stored="bfloat16")
+    toks = helpers.random_tokens(70, cfg["vocab_size"], seed=1)
+    trace = TraceBuilder()
+    trace.step([("a", toks[:37], "all")])
+    trace.step([("a", toks[37:39], "all")])
+    for i in range(39, 70):
+        trace.step([("a", toks[i:i + 1], "all")])
+    got = helpers.replay_in_process(session_for(folder, dtype, 128), trace)
+    assert len(got) == 70
+    check(got, folder, {"a": toks}, dtype)
