@@ -186,12 +186,14 @@ def test_trace_run_program(folder_a, tmp_path, dtype):
         assert helpers.worst(row, helpers.plain_logits(folder_a, toks[rid])[pos]) <= tol
 
 
-def test_decode_steps_replayed_from_graphs_equal_eager_steps(folder_a):
+@pytest.mark.parametrize("live_requests", [3, 20, 40])
+def test_decode_steps_replayed_from_graphs_equal_eager_steps(folder_a, live_requests):
     """Decode steps captured into HIP graphs are replayed many times, with eager prefill steps of
-    other requests in between; every replay must give what the eager step function gives."""
+    other requests in between; every replay must give what the eager step function gives.  With 20 and 40
+    requests the graph holds the library's products (more than 16 rows) beside the engine's kernels."""
     from paged_llm_amd.engine.replay import ReplaySession
     import paged_llm_amd.engine.loading as loading
-    toks = {f"g{i}": helpers.random_tokens(60 + 7 * i, 256, seed=500 + i) for i in range(3)}
+    toks = {f"g{i}": helpers.random_tokens(60 + i % 5, 256, seed=500 + i) for i in range(live_requests)}
 
     def run(use_graphs):
         real = loading.build_runtime
@@ -201,7 +203,7 @@ def test_decode_steps_replayed_from_graphs_equal_eager_steps(folder_a):
         import paged_llm_amd.engine.replay as replay
         replay.build_runtime = patched
         try:
-            session = ReplaySession(folder_a, "bfloat16", 64 * 2 * 3, None)
+            session = ReplaySession(folder_a, "bfloat16", 64 * 2 * (live_requests + 1), None)
         finally:
             replay.build_runtime = real
         assert session.runner.use_graphs == use_graphs

@@ -75,3 +75,36 @@ def test_prompt_decoding_and_portions_at_real_sizes(case, dtype):
     got = helpers.replay_in_process(session, trace)
     assert len(got) == 5 + 8 + 3
     check_rows(got, want, dtype)
+
+
+def test_graph_replays_with_library_products_equal_eager_steps(tmp_path):
+    """24 requests decode together: beyond 16 rows the step's graph holds the library's products (gate/up,
+    down, head with float output) at their real sizes.  Every replay is held against the eager step."""
+    from paged_llm_amd.engine.replay import ReplaySession
+    import paged_llm_amd.engine.replay as replay
+    cfg, _ = SHAPES["llama32_1b"]
+    folder = helpers.make_folder(tmp_path, cfg, seed=22, stored="bfloat16")
+    toks = {f"g{i}": helpers.random_tokens(12 + i % 3, cfg["vocab_size"], seed=700 + i) for i in range(24)}
+
+    def run(use_graphs):
+        real = replay.build_runtime
+        replay.build_runtime = lambda *a, **kw: real(*a, **dict(kw, use_graphs=use_graphs))
+        try:
+            session = ReplaySession(folder, "bfloat16", 64 * 25, None)
+        finally:
+            replay.build_runtime = real
+        trace = TraceBuilder()
+        trace.step([(r, t[:6], "last") for r, t in toks.items()])
+        for i in range(6, 12):
+            live = [(r, t[i:i + 1], "all") for r, t in toks.items()]
+            trace.step(live if i % 2 else live[:19])
+            if i == 8:
+                trace.step([("late", toks["g0"][:9], "last")], end=["late"])      # an eager step between replays
+        return helpers.replay_in_process(session, trace), session
+
+    eager, _ = run(False)
+    graphed, session = run(True)
+    assert session.runner._graphs
+    assert eager.keys() == graphed.keys()
+    for key in eager:
+        assert helpers.worst(graphed[key], eager[key]) <= 1e-6, key
