@@ -402,8 +402,8 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
   constexpr int kWgCols = 4 * 16 * NCB;
   const int my_tiles = (num_cols + kWgCols - 1) / kWgCols;
   // Later tiles see more keys.  paired == 0: they are started first, so that the short ones fill the
-  // tail.  paired == 1 (few workgroups, all resident at once): a workgroup takes tile t from the far end
-  // and then its mirror image from the near end, so that every workgroup has the same amount to do.
+  // tail.  paired == 1: a workgroup takes tile t from the far end and then its mirror image from the
+  // near end, so that every workgroup of a sequence has the same amount to do.
   const int far_tile = my_tiles - 1 - (int)blockIdx.x;
   if (far_tile < 0) return;                                     // this sequence has fewer tiles than the longest
   const int passes = (paired == 1 && (int)blockIdx.x < far_tile) ? 2 : 1;
@@ -770,7 +770,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
                                        int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                        const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                                        int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                       int num_partitions, float* partials, int waves, int column_blocks, int pair_tiles, hipStream_t stream) {
+                                       int num_partitions, float* partials, int waves, int column_blocks, int tune, hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
   const int G = num_heads / num_kv_heads;
@@ -790,19 +790,19 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // prompt portions: workgroups of four wavefronts that share every block of keys through LDS
     constexpr int kCols = 4 * 16 * 2;
     const int ptiles = (max_cols + kCols - 1) / kCols;
-    // pair_tiles: the caller knows that the queries span most of the context (a prompt from its
-    // start), so late tiles have far more keys than early ones.  If all workgroups are resident at
-    // once anyway, and pairing still leaves one per compute unit, far and near tiles are paired.
-    const long wgs = (long)ptiles * num_kv_heads * num_seqs;
-    const int paired = ((pair_tiles & 1) && ptiles > 1 && wgs <= 1024 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= 256) ? 1 : 0;
+    // Far and near tiles of a sequence are paired in one workgroup whenever that still leaves a workgroup
+    // per compute unit: all workgroups of a sequence then have the same amount to do and no long one is
+    // left for the end (measured faster for one prompt and for many, at head sizes 64 and 128).
+    // `tune` (measurements): bit 0 = no pairing, bit 1 = one key group, bit 2 = two key groups.
+    const int paired = (!(tune & 1) && ptiles > 1 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= num_compute_units()) ? 1 : 0;
     dim3 pgrid(paired == 1 ? (ptiles + 1) / 2 : ptiles, num_kv_heads, num_seqs);
     // Two key groups (eight wavefronts, one workgroup per compute unit) when there are too few workgroups to
     // give every compute unit two of the four-wavefront kind at a time, and for the head sizes that then still
-    // fit into registers and LDS; else one key group.  pair_tiles bits 1 and 2 force one or two (measurements).
+    // fit into registers and LDS; else one key group.
     constexpr bool two_fits = D <= 96 && prefill_lds_bytes(2) <= 160 * 1024;
     bool two = two_fits && (long)pgrid.x * pgrid.y * pgrid.z < 2L * num_compute_units();
-    if (pair_tiles & 2) two = false;
-    if ((pair_tiles & 4) && two_fits) two = true;
+    if (tune & 2) two = false;
+    if ((tune & 4) && two_fits) two = true;
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
     if ((long)lds > pllm_max_lds()) return -2;
     auto kern = paged_attention_prefill_kernel<2, 1>;

@@ -466,7 +466,7 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
                          cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
                          head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
-                         num_partitions: int = 1, waves: int = 1, column_blocks: int = 0, pair_tiles: int = 0,
+                         num_partitions: int = 1, waves: int = 1, column_blocks: int = 0, tune: int = 0,
                          out: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
@@ -502,7 +502,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
     _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
              block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
-             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), int(pair_tiles), _stream()),
+             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), int(tune), _stream()),
            "paged_attention_mfma")
     return out
 
@@ -518,7 +518,6 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
         # Prompt portions: 32 columns per wavefront leave registers for two wavefronts per SIMD
         # (measured faster than 64 columns at one).
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
-                                    head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0,
-                                    pair_tiles=2 * ctx.max_q_len > ctx.max_k_len)
+                                    head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window)
