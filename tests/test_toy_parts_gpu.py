@@ -1,8 +1,9 @@
 """The framework's generality, shown with toy parts that are defined here and registered without a
 change to the framework's files: a mixer with per-request state of fixed size, a layer that runs
-twice, a layer that reads another layer's cache, and a windowed attention layer with pages of its
-own.  The toy model is replayed whole, in portions and mixed, and compared with a plain
-implementation written here."""
+twice, a layer that reads another layer's cache, a windowed attention layer with pages of its
+own, a feed-forward with a router and experts, and another position encoding (rotation angles on a
+linear grid of frequencies).  The toy model is replayed whole, in portions and mixed, and compared
+with a plain implementation written here."""
 
 import numpy as np
 import pytest
@@ -16,16 +17,18 @@ pytestmark = pytest.mark.gpu
 
 TOY = {"architectures": ["ToyHybridForCausalLM"], "vocab_size": 120, "hidden_size": 48, "intermediate_size": 72,
        "heads": 3, "kv_heads": 1, "head_dim": 16, "decay": 0.8, "window": 7, "eps": 1e-5, "theta": 100.0,
-       "max_position_embeddings": 256}
+       "experts": 3, "expert_size": 24, "linear_base": 0.37, "max_position_embeddings": 256}
 # step -> (layer, cache_from): layer 1 (the stateful mixer) runs twice, step 2 reads the cache of step 0
 SCHEDULE = [(0, None), (1, None), (2, 0), (3, None), (1, None)]
 
 
 def register_toy():
     from paged_llm_amd.config.registry import ARCHITECTURES, Architecture, register_architecture
-    from paged_llm_amd.parts import (LayerSpec, Mixer, ModelSpec, PartSpec, ScheduleStep, StateSpec, WeightSpec,
-                                     register_mixer)
-    from paged_llm_amd.parts.linear import linear
+    from paged_llm_amd.parts import (FeedForward, LayerSpec, Mixer, ModelSpec, PartSpec, PositionEncoding, ScheduleStep,
+                                     StateSpec, WeightSpec, register_feed_forward, register_mixer,
+                                     register_position_encoding)
+    from paged_llm_amd.parts.linear import gated_linear, linear
+    from paged_llm_amd.parts.norm import rows_of
     if "ToyHybridForCausalLM" in ARCHITECTURES:
         return
 
@@ -62,16 +65,72 @@ def register_toy():
 
     register_mixer("toy_decay", DecayMixer)
 
+    class SoftExperts(FeedForward):
+        """A router (logits and softmax in float, its matrix kept in float) and gated experts; the output is
+        the experts' outputs weighted by the router's probabilities.  Every expert sees every row here, so that
+        rounding cannot flip a choice in the comparison; a top-k choice would gather its rows in the same place."""
+
+        def __init__(self, params, env):
+            self.hidden, self.experts, self.inter = env.hidden_size, int(params["experts"]), int(params["expert_size"])
+            self.dtype, self.device, self._w = env.dtype, env.device, {}
+
+        def weight_specs(self):
+            specs = {"router.weight": WeightSpec((self.experts, self.hidden), role="vector")}
+            for e in range(self.experts):
+                specs[f"experts.{e}.gate_proj.weight"] = WeightSpec((self.inter, self.hidden))
+                specs[f"experts.{e}.up_proj.weight"] = WeightSpec((self.inter, self.hidden))
+                specs[f"experts.{e}.down_proj.weight"] = WeightSpec((self.hidden, self.inter))
+            return specs
+
+        def assign(self, name, tensor):
+            keep = torch.float32 if name == "router.weight" else self.dtype
+            self._w[name] = tensor.to(device=self.device, dtype=keep).contiguous()
+
+        def finalize(self):
+            self.router = self._w["router.weight"]
+            self.gate_up = [torch.cat([self._w[f"experts.{e}.gate_proj.weight"], self._w[f"experts.{e}.up_proj.weight"]]).contiguous()
+                            for e in range(self.experts)]
+            self.down = [self._w[f"experts.{e}.down_proj.weight"] for e in range(self.experts)]
+
+        def forward(self, h, ctx):
+            rows = rows_of(h)
+            probs = torch.softmax(rows.float() @ self.router.T, dim=-1)
+            out = torch.zeros(rows.shape, dtype=torch.float32, device=rows.device)
+            for e in range(self.experts):
+                out += probs[:, e:e + 1] * linear(gated_linear(rows, self.gate_up[e]), self.down[e]).float()
+            return out.to(rows.dtype)
+
+    register_feed_forward("toy_soft_experts", SoftExperts)
+
+    class LinearRotary(PositionEncoding):
+        """Rotation angles position * base * (i + 1) / (d / 2): the attention part only asks for the two tables."""
+
+        def __init__(self, params, env):
+            self.head_dim, self.base, self.device = int(params["head_dim"]), float(params["base"]), env.device
+            self.cos = self.sin = None
+
+        def prepare(self, max_positions):
+            half = self.head_dim // 2
+            angles = torch.outer(torch.arange(max_positions, dtype=torch.float32),
+                                 self.base * (torch.arange(half, dtype=torch.float32) + 1) / half)
+            self.cos, self.sin = angles.cos().to(self.device).contiguous(), angles.sin().to(self.device).contiguous()
+
+    register_position_encoding("toy_linear_rotary", LinearRotary)
+
     def build_spec(c):
         norm = PartSpec("rmsnorm", {"eps": c["eps"]})
         rotary = {"kind": "rotary", "params": {"head_dim": c["head_dim"], "theta": c["theta"], "scaling": None}}
-        def attention(**extra):
+        linear_grid = {"kind": "toy_linear_rotary", "params": {"head_dim": c["head_dim"], "base": c["linear_base"]}}
+        def attention(position=rotary, **extra):
             return PartSpec("paged_attention", {"num_heads": c["heads"], "num_kv_heads": c["kv_heads"], "head_dim": c["head_dim"],
-                                                "position": rotary, **extra})
+                                                "position": position, **extra})
         ffn = PartSpec("gated_mlp", {"intermediate_size": c["intermediate_size"]})
+        routed = PartSpec("toy_soft_experts", {"experts": c["experts"], "expert_size": c["expert_size"]})
         block = PartSpec("prenorm", {"mixer_norm": "norm1", "mixer": "mixer", "feed_forward_norm": "norm2", "feed_forward": "ffn"})
-        mixers = [attention(), PartSpec("toy_decay", {"decay": c["decay"]}), attention(kv_proj=False), attention(window=c["window"])]
-        layers = [LayerSpec(f"layers.{i}", block, m, ffn, norm, norm) for i, m in enumerate(mixers)]
+        # layers 0 and 2 share a cache, so they share the position encoding too (the linear grid); layer 3 has the experts
+        mixers = [attention(linear_grid), PartSpec("toy_decay", {"decay": c["decay"]}), attention(linear_grid, kv_proj=False),
+                  attention(window=c["window"])]
+        layers = [LayerSpec(f"layers.{i}", block, m, routed if i == 3 else ffn, norm, norm) for i, m in enumerate(mixers)]
         return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"],
                          embedding=PartSpec("token_embedding", {"vocab_size": c["vocab_size"]}), layers=layers, final_norm=norm,
                          head=PartSpec("lm_head", {"vocab_size": c["vocab_size"], "tied": False}),
@@ -84,7 +143,8 @@ def register_toy():
 def plain_toy(folder, tokens):
     c, w = TOY, {k: v.float() for k, v in plain.load_weights(folder).items()}
     T, nh, nkv, d = len(tokens), c["heads"], c["kv_heads"], c["head_dim"]
-    ang = plain.rotary_angles(torch.arange(T), plain.inverse_frequencies(d, c["theta"], None))
+    ang_usual = plain.rotary_angles(torch.arange(T), plain.inverse_frequencies(d, c["theta"], None))
+    ang_linear = plain.rotary_angles(torch.arange(T), c["linear_base"] * (torch.arange(d // 2, dtype=torch.float32) + 1) / (d // 2))
     x = w["embed.weight"][torch.tensor(tokens)]
     kept = {}
     for step, (layer, cache_from) in enumerate(SCHEDULE):
@@ -97,6 +157,7 @@ def plain_toy(folder, tokens):
                 rows.append(s)
             a = torch.stack(rows)
         else:
+            ang = ang_linear if layer in (0, 2) else ang_usual
             q = plain.apply_rotary((h @ w[p + "mixer.q_proj.weight"].T).view(T, nh, d), ang)
             if cache_from is None:
                 k = plain.apply_rotary((h @ w[p + "mixer.k_proj.weight"].T).view(T, nkv, d), ang)
@@ -108,7 +169,12 @@ def plain_toy(folder, tokens):
             a = o.reshape(T, nh * d) @ w[p + "mixer.o_proj.weight"].T
         x = x + a
         h = plain.rms_norm(x, w[p + "norm2.weight"], c["eps"])
-        x = x + plain.swiglu(h, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+        if layer == 3:
+            probs = torch.softmax(h @ w[p + "ffn.router.weight"].T, dim=-1)
+            x = x + sum(probs[:, e:e + 1] * plain.swiglu(h, *(w[p + f"ffn.experts.{e}.{n}_proj.weight"] for n in ("gate", "up", "down")))
+                        for e in range(c["experts"]))
+        else:
+            x = x + plain.swiglu(h, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
     return (plain.rms_norm(x, w["norm.weight"], c["eps"]) @ w["head.weight"].T).numpy()
 
 
