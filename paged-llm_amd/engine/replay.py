@@ -24,7 +24,9 @@ MAX_LIVE_REQUESTS = 16
 
 class ReplaySession:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, out_dir: str | None, device="cuda"):
-        self.model = load_model(model_dir, dtype, device)
+        # A request may hold up to max_tokens positions: the position tables reach that far even where the
+        # configuration names fewer (as max(max_position_embeddings, max_model_len) in pagedllm/model/loader.py:42-44).
+        self.model = load_model(model_dir, dtype, device, max_model_len=max_tokens)
         bs = REPLAY_BLOCK_SIZE
         num_pages = max(1, (max_tokens + bs - 1) // bs)
         self.manager, self.storage, self.runner = build_runtime(

@@ -198,3 +198,18 @@ def test_widths_that_are_no_multiple_of_eight(tmp_path, name, dtype):
     got = helpers.replay_in_process(session_for(folder, dtype, 128), trace)
     assert len(got) == 70
     check(got, folder, {"a": toks}, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_request_longer_than_the_configured_positions(folders, dtype):
+    """max_position_embeddings of configuration B is 128; the pool is made for more, and the position tables
+    follow the pool (the reference takes the larger of the two lengths, pagedllm/model/loader.py:42-44)."""
+    folder = folders["B", "bfloat16"]
+    toks = helpers.random_tokens(150, TINY_B["vocab_size"], seed=77)
+    trace = TraceBuilder()
+    trace.step([("long", toks[:120], [0, 119])])
+    for i in range(120, 150):
+        trace.step([("long", toks[i:i + 1], "all")])
+    got = helpers.replay_in_process(session_for(folder, dtype, 192), trace)
+    assert len(got) == 32
+    check(got, folder, {"long": toks}, dtype)
