@@ -1,4 +1,4 @@
-// Linear layers of a decode step (at most 16 rows) in bfloat16, each fused with what surrounds it,
+// Linear layers of a decode step (at most 16 rows; plain rows up to 64, see the second kernel) in bfloat16, each fused with what surrounds it,
 // because at these sizes a kernel launch costs as much as the weights take to stream:
 //
 //   prologue (optional)   rows = x (+ delta), the residual sum in float rounded once; the new

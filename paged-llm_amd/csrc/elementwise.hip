@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
 }
 
 template <typename T>
-static void launch_rmsnorm(const T* x, const T* delta, const int* row_index, const float* w, float eps, T* out, T* x_out, int rows,
+static int launch_rmsnorm(const T* x, const T* delta, const int* row_index, const float* w, float eps, T* out, T* x_out, int rows,
                            int hidden, hipStream_t stream) {
   constexpr int V = 16 / sizeof(T);
   const bool wide = hidden % V == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
@@ -160,22 +160,25 @@ static void launch_rmsnorm(const T* x, const T* delta, const int* row_index, con
   else if (wide && per_lane <= 4) PLLM_ROWS(4);
   else if (wide && per_lane <= 8) PLLM_ROWS(8);
   else if (wide && per_lane <= 16) PLLM_ROWS(16);
-  else
-    hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(rows), block, ((size_t)hidden + 16) * sizeof(float), stream, x, delta, row_index, w,
-                       eps, out, x_out, hidden);
+  else {
+    const size_t lds = ((size_t)hidden + 16) * sizeof(float);   // the row as floats, and the reduction's scratch
+    if (lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rmsnorm_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(rows), block, lds, stream, x, delta, row_index, w, eps, out, x_out, hidden);
+  }
 #undef PLLM_ROWS
+  return (int)hipGetLastError();
 }
 
 PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int* row_index, const float* w, float eps,
                           void* out, void* x_out, int rows, int hidden, hipStream_t stream) {
   if (rows <= 0) return 0;
-  const size_t lds = ((size_t)hidden + 16) * sizeof(float);
-  if (lds > 64 * 1024) return -2;  // row does not fit the staging buffer of the one-row-per-workgroup kernel
+  if (((size_t)hidden + 16) * sizeof(float) > 160 * 1024) return -2;  // a row must fit the LDS of the one-row-per-workgroup kernel
   if (dtype == PLLM_F32)
-    launch_rmsnorm<float>((const float*)x, (const float*)delta, row_index, w, eps, (float*)out, (float*)x_out, rows, hidden, stream);
-  else
-    launch_rmsnorm<bf16>((const bf16*)x, (const bf16*)delta, row_index, w, eps, (bf16*)out, (bf16*)x_out, rows, hidden, stream);
-  PLLM_RETURN_LAST_ERROR();
+    return launch_rmsnorm<float>((const float*)x, (const float*)delta, row_index, w, eps, (float*)out, (float*)x_out, rows, hidden, stream);
+  return launch_rmsnorm<bf16>((const bf16*)x, (const bf16*)delta, row_index, w, eps, (bf16*)out, (bf16*)x_out, rows, hidden, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -120,7 +120,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, delta: torch.Tens
     H = x.shape[1]
     _need(weight.dtype == torch.float32 and weight.shape == (H,) and weight.is_contiguous(),
           f"norm weight must be float32 [{H}], got {weight.dtype} {tuple(weight.shape)}")
-    _need(H + 16 <= 16384, f"rmsnorm kernel stages one row in LDS: hidden size {H} is above its limit of 16368")
+    _need((H + 16) * 4 <= min(_max_lds_bytes(x.device), 160 * 1024),
+          f"rmsnorm kernel stages one row in LDS as floats: hidden size {H} is above its limit")
     if delta is not None:
         _need(delta.shape == x.shape and delta.dtype == x.dtype and delta.is_contiguous(), "delta must match x")
     if row_index is not None:

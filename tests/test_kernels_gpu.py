@@ -39,7 +39,7 @@ def test_embed_gather(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden", [48, 200, 2048, 5000])
+@pytest.mark.parametrize("hidden", [48, 200, 2048, 5000, 8200, 16384, 20001])
 def test_rmsnorm(dtype, hidden):
     x = rnd(9, hidden, seed=1, dtype=dtype, scale=3.0)
     w = 1 + 0.3 * rnd(hidden, seed=2)
