@@ -1,4 +1,4 @@
-"""Layers of real size (TinyLlama-1.1B, Llama-3.2-1B and Llama-3.1-8B shapes: widths, head counts,
+"""Layers of real size (TinyLlama-1.1B, Llama-3.2-1B, Llama-3.1-8B and 70B shapes: widths, head counts,
 intermediate sizes, vocabularies, rotary constants and tying as in those models) with random weights
 (all 22 layers of the first, a few of the others, so that the plain implementation stays quick): a prompt in one step,
 tokens decoded one by one, and a second request fed in portions beside them; in true 32-bit and in
@@ -26,6 +26,10 @@ SHAPES = {
     "llama31_8b": (dict(BASE, num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
                         head_dim=128, intermediate_size=14336, vocab_size=128256, rope_theta=500000.0,
                         rope_scaling=LLAMA3(8.0), tie_word_embeddings=False), 32),
+    # one layer at the widths of the 70B model (rows too long for the fused kernels' LDS staging), smaller vocabulary
+    "llama31_70b": (dict(BASE, num_hidden_layers=1, hidden_size=8192, num_attention_heads=64, num_key_value_heads=8,
+                         head_dim=128, intermediate_size=28672, vocab_size=32000, rope_theta=500000.0,
+                         rope_scaling=LLAMA3(8.0), tie_word_embeddings=False), 80),
 }
 # float32: every row within 2e-5 of the plain implementation.
 # bfloat16: rounding noise grows with depth.  Measured over all 122 positions of this trace (error of a row =
