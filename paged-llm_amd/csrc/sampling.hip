@@ -163,7 +163,30 @@ __global__ __launch_bounds__(kThreads) void argmax_kernel(const float* __restric
   __shared__ ArgMax ascratch[16];
   const float* z = logits + (size_t)blockIdx.x * vocab;
   ArgMax best; best.v = -INFINITY; best.i = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += kThreads) { ArgMax c; c.v = z[i]; c.i = i; best = better(best, c); }
+  if ((vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(z) & 15) == 0) {
+    // pieces of four, four pieces requested before the first is looked at: the row is read by one compute
+    // unit, so what counts is how many loads are under way
+    const float4* z4 = reinterpret_cast<const float4*>(z);
+    const int pieces = vocab >> 2;
+    for (int i = threadIdx.x; i < pieces; i += 4 * kThreads) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = i + u * kThreads;
+        v[u] = j < pieces ? z4[j] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = i + u * kThreads;
+        if (j >= pieces) continue;
+        const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { ArgMax c; c.v = e[k]; c.i = 4 * j + k; best = better(best, c); }
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < vocab; i += kThreads) { ArgMax c; c.v = z[i]; c.i = i; best = better(best, c); }
+  }
   best = block_argmax(best, ascratch);
   if (threadIdx.x == 0) out[blockIdx.x] = best.i;
 }

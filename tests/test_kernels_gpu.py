@@ -238,12 +238,19 @@ def test_attention_one_far_key_stands_out():
 
 
 # ----------------------------------------------------------------------------------- sampling
-def test_argmax_takes_the_first_maximum():
-    z = rnd(5, 1000, seed=14)
+@pytest.mark.parametrize("vocab", [1000, 1001, 32000, 128256, 5003])
+def test_argmax_takes_the_first_maximum(vocab):
+    z = rnd(5, vocab, seed=14)
     z[1, 17] = z[1, 900] = 50.0
     z[2, :] = 0.0
+    z[3, vocab - 1] = 60.0                                             # the last element of a row
+    z[4, vocab - 2] = z[4, vocab - 1] = 70.0
     got = ops().argmax(z.cuda()).cpu()
-    assert got.tolist() == z.argmax(-1).tolist()[:1] + [17, 0] + z.argmax(-1).tolist()[3:]
+    assert got.tolist() == [int(z[0].argmax()), 17, 0, vocab - 1, vocab - 2]
+    # rows of a larger matrix: a row stride that leaves rows unaligned when the vocabulary is odd
+    wide = torch.zeros(5, vocab + 3)
+    wide[:, 1:vocab + 1] = z
+    assert ops().argmax(wide.cuda()[:, 1:vocab + 1].contiguous()).cpu().tolist() == got.tolist()
 
 
 def sample_rows(z, temperature, top_k, top_p, draws, seed=0):
