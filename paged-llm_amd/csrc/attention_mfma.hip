@@ -510,8 +510,9 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     }
   };
 
-  // `masked` is a compile-time flag: blocks whose 64 keys every column of the wavefront may see take
-  // the version without any comparison.
+  // `masked` is a compile-time flag: blocks whose 64 keys every valid column of the wavefront may see take
+  // the version without any comparison.  Columns past the end of the sequence (the last tile's surplus)
+  // carry zero queries and are never stored; they go along with either version.
   auto compute = [&](int buf, int n0, auto masked_tag) {
     constexpr bool kMasked = decltype(masked_tag)::value;
     const bf16* kb = PLLM_K_TILE(buf, kg);
@@ -586,7 +587,6 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     }
   };
   const int full_from = window > 0 ? max(qpos_max - window + 1, 0) : 0;   // blocks from here on are inside every column's window
-  const bool all_cols = col0 + 16 * NCB <= num_cols;
 
   // ---- the steps.  Step i is computed from LDS while step i + 1 sits in registers (requested one
   //      step earlier, written to the other LDS buffer after the computation) and step i + 2 is being
@@ -596,7 +596,7 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     if (n0 + 2 * kStepKeys < k_hi) fetch(free_regs, n0 + 2 * kStepKeys);
     const int mine = n0 + kg * 64;                                // this group's 64 keys of the step
     if (wave_on && mine < vis_hi && mine + 64 > vis_lo) {
-      if (all_cols && mine + 63 <= qpos_min && mine >= full_from) compute(buf, mine, PlainTag{});
+      if (mine + 63 <= qpos_min && mine >= full_from) compute(buf, mine, PlainTag{});
       else compute(buf, mine, MaskedTag{});
     }
     if (n0 + kStepKeys < k_hi) stash(arriving, buf ^ 1);
