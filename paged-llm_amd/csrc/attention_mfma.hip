@@ -384,7 +384,7 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
-    int block_size, float scale, int window, int paired) {
+    int block_size, float scale, int window) {
   extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
   constexpr int kKTile = 64 * kKRow, kVTile = D * kVRow;         // elements of one group's keys / values of a step
   // keys [2 buffers][KG][64 rows][kKRow], then values [2 buffers][KG][D rows][kVRow].  Addresses are formed
@@ -394,22 +394,21 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
 #define PLLM_V_TILE(buf, group) (reinterpret_cast<bf16*>(prefill_lds) + 2 * KG * kKTile + ((buf) * KG + (group)) * kVTile)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int cw = wave & 3, kg = wave >> 2;                      // column share and key group of this wavefront
-  const int seq = blockIdx.z, kvh = blockIdx.y;
+  // blockIdx.x = (sequence, kv head), blockIdx.y = tile slot: workgroups are handed out x first, so all
+  // long tiles of all sequences start before any short one
+  const int seq = blockIdx.x / num_kv_heads, kvh = blockIdx.x - seq * num_kv_heads;
+  const int slot = blockIdx.y;
   const int G = num_heads / num_kv_heads;
   const int q_begin = cu_seqlens_q[seq], num_q = cu_seqlens_q[seq + 1] - q_begin;
   const int len_k = seq_lens_k[seq];
   const int num_cols = num_q * G;
   constexpr int kWgCols = 4 * 16 * NCB;
   const int my_tiles = (num_cols + kWgCols - 1) / kWgCols;
-  // Later tiles see more keys.  paired == 0: they are started first, so that the short ones fill the
-  // tail.  paired == 1: a workgroup takes tile t from the far end and then its mirror image from the
-  // near end, so that every workgroup of a sequence has the same amount to do.
-  const int far_tile = my_tiles - 1 - (int)blockIdx.x;
-  if (far_tile < 0) return;                                     // this sequence has fewer tiles than the longest
-  const int passes = (paired == 1 && (int)blockIdx.x < far_tile) ? 2 : 1;
-  if (paired == 1 && (int)blockIdx.x > far_tile) return;
-  for (int pass = 0; pass < passes; ++pass) {
-  const int wg_col0 = (pass == 0 ? far_tile : (int)blockIdx.x) * kWgCols;
+  // Later tiles see more keys: slot 0 is every sequence's last tile, so the longest pieces of work start
+  // first and the short ones fill the tail.
+  const int tile = my_tiles - 1 - slot;
+  if (tile < 0) return;                                         // this sequence has fewer tiles than the longest
+  const int wg_col0 = tile * kWgCols;
   const int pos0 = len_k - num_q;
   // key range of the whole workgroup
   const int wg_last = min(wg_col0 + kWgCols, num_cols) - 1;
@@ -658,8 +657,6 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
       *reinterpret_cast<bf16x4*>(out + my_out[cb] + db * 16 + g * 4) = o;
     }
   }
-  __syncthreads();                                                // the LDS buffers are reused by the next pass
-  }  // pass
 #undef PLLM_K_TILE
 #undef PLLM_V_TILE
 }
@@ -790,17 +787,18 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // prompt portions: workgroups of four wavefronts that share every block of keys through LDS
     constexpr int kCols = 4 * 16 * 2;
     const int ptiles = (max_cols + kCols - 1) / kCols;
-    // Far and near tiles of a sequence are paired in one workgroup whenever that still leaves a workgroup
-    // per compute unit: all workgroups of a sequence then have the same amount to do and no long one is
-    // left for the end (measured faster for one prompt and for many, at head sizes 64 and 128).
-    // `tune` (measurements): bit 0 = no pairing, bit 1 = one key group, bit 2 = two key groups.
-    const int paired = (!(tune & 1) && ptiles > 1 && (long)((ptiles + 1) / 2) * num_kv_heads * num_seqs >= num_compute_units()) ? 1 : 0;
-    dim3 pgrid(paired == 1 ? (ptiles + 1) / 2 : ptiles, num_kv_heads, num_seqs);
+    // The grid is (sequence x kv head, tile slot): workgroups are handed out in that order, so the last
+    // tiles of all sequences (most keys) start first and the early tiles fill the tail; that keeps the compute
+    // units evenly loaded for any number and length of prompts (pairing far and near tiles in one workgroup
+    // was 5 % faster when the pairs filled the compute units exactly and up to 40 % slower just past that).
+    if (ptiles > 65535) return -2;
+    dim3 pgrid(num_kv_heads * num_seqs, ptiles, 1);
     // Two key groups (eight wavefronts, one workgroup per compute unit) when there are too few workgroups to
-    // give every compute unit two of the four-wavefront kind at a time, and for the head sizes that then still
-    // fit into registers and LDS; else one key group.
+    // keep two of the four-wavefront kind on every compute unit for most of the time (measured: faster up to
+    // about 2.5 workgroups per compute unit), and for the head sizes that then still fit into registers and
+    // LDS; else one key group.  `tune` (measurements): bit 1 = one key group, bit 2 = two key groups.
     constexpr bool two_fits = D <= 96 && prefill_lds_bytes(2) <= 160 * 1024;
-    bool two = two_fits && (long)pgrid.x * pgrid.y * pgrid.z < 2L * num_compute_units();
+    bool two = two_fits && 2L * pgrid.x * pgrid.y <= 5L * num_compute_units();
     if (tune & 2) two = false;
     if ((tune & 4) && two_fits) two = true;
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
@@ -815,7 +813,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     }
     hipLaunchKernelGGL(kern, pgrid, dim3(two ? 512 : 256), lds, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q,
-                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, paired);
+                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window);
     return (int)hipGetLastError();
   }
   dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64 * waves);
