@@ -508,14 +508,40 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     return out
 
 
+FEW_QUERY_COLUMNS = 64      # queries x heads per kv head that one tile of the decode kernel holds
+
+
 def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
                     scale, window, ctx) -> torch.Tensor:
-    """Attention of one step's queries over the paged cache: the MFMA kernel for bfloat16 where it
-    takes the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions."""
+    """Attention of one step's queries over the paged cache: the MFMA kernels for bfloat16 where they
+    take the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions.
+
+    A step that holds decoded tokens beside prompt portions is launched in two parts when the sequences with
+    few queries come first in the batch (the step function orders them so): those go to the kernel that cuts
+    their keys into partitions, the portions to the prompt kernel.  One launch for all would walk every decoded
+    token's whole context with a single wavefront (measured 49 us against 15 + 15 for a portion of 512 tokens
+    beside 7 decoded tokens at context 2048, 180 us at context 8192)."""
     bs = k_pages.shape[2]
     if mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
-        waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, num_heads // num_kv_heads,
-                                            head_dim, _max_lds_bytes(q.device))
+        group = num_heads // num_kv_heads
+        lds = _max_lds_bytes(q.device)
+        q_lens, k_lens = ctx.q_lens, ctx.k_lens
+        few = 0
+        while few < len(q_lens) and q_lens[few] * group <= FEW_QUERY_COLUMNS:
+            few += 1
+        if 0 < few < len(q_lens) and all(n * group > FEW_QUERY_COLUMNS for n in q_lens[few:]) and not ctx.capturing:
+            rows = sum(q_lens[:few])
+            out = torch.empty((q.shape[0], num_heads * head_dim), dtype=q.dtype, device=q.device)
+            max_q, max_k = max(q_lens[:few]), max(k_lens[:few])
+            waves, size, parts = attention_plan(few, num_kv_heads, max_q, max_k, group, head_dim, lds)
+            paged_attention_mfma(q[:rows], k_pages, v_pages, block_tables[:few], cu_seqlens_q[:few + 1], seq_lens_k[:few],
+                                 num_heads, num_kv_heads, head_dim, scale, window, max_q, size, parts, waves,
+                                 2 if waves == 1 else 0, out=out[:rows])
+            # the portions: rows, cu_seqlens_q and the output stay absolute, the per-sequence arrays start at `few`
+            paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
+                                 num_kv_heads, head_dim, scale, window, max(q_lens[few:]), 0, 1, 1, 2, out=out)
+            return out
+        waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, group, head_dim, lds)
         # Prompt portions: 32 columns per wavefront leave registers for two wavefronts per SIMD
         # (measured faster than 64 columns at one).
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,

@@ -46,6 +46,10 @@ class ModelRunner:
         in the order: ids, positions, cu_seqlens_q, seq_lens_k, state slots, starts, logits rows, then
         per cache group its block tables and slots.  ``fixed_blocks`` pads every block table to that
         many entries, so that the layout depends on the counts only (needed to replay a graph).
+
+        Inside the batch the entries stand in ascending order of their token counts (decoded tokens first, then
+        prompt portions, the order of equals kept): a part may then treat the sequences with few queries and
+        those with many as two contiguous runs.  The wanted rows keep the callers' order of entries.
         """
         if not entries:
             raise StepError("a step needs at least one entry")
@@ -53,7 +57,10 @@ class ModelRunner:
         vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions
         seen = set()
         q_lens, k_lens, starts = [], [], []
-        ids_parts, pos_parts, logits_idx = [], [], []
+        ids_parts, pos_parts = [], []
+        wanted_of: dict = {}                                          # request id -> batch rows of its wanted tokens
+        callers_order = [e.request_id for e in entries]
+        entries = sorted(entries, key=lambda e: len(e.tokens))        # stable
         offset = 0
         for e in entries:
             n = len(e.tokens)
@@ -71,7 +78,7 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= w < n:
                     raise StepError(f"request {e.request_id!r}: wanted row {w} outside its {n} tokens")
-                logits_idx.append(offset + w)
+            wanted_of[e.request_id] = [offset + w for w in e.want]
             ids_parts.append(toks)
             pos_parts.append(np.arange(e.start, e.start + n, dtype=np.int64))
             q_lens.append(n)
@@ -80,6 +87,7 @@ class ModelRunner:
             offset += n
         T, S = offset, len(entries)
         positions = np.concatenate(pos_parts)
+        logits_idx = [row for rid in callers_order for row in wanted_of[rid]]
 
         group_arrays = {}
         for name, cs in self.group_specs.items():

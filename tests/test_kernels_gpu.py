@@ -410,7 +410,7 @@ def test_long_contexts_through_the_planned_launch(heads, kv_heads, d, batch):
         page, off = int(tables[s, n // bs]), n % bs
         head = s % heads
         kp[page, head // (heads // kv_heads), off, :] = (q[s, head * d:(head + 1) * d].float() * 40).to(torch.bfloat16)
-    ctx = types.SimpleNamespace(num_seqs=batch, max_q_len=1, max_k_len=max(lens))
+    ctx = types.SimpleNamespace(num_seqs=batch, max_q_len=1, max_k_len=max(lens), q_lens=[1] * batch, k_lens=lens, capturing=False)
     got = ops().paged_attention(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d,
                                 1.0, 0, ctx).cpu().float()
     for s, n in enumerate(far):
@@ -422,6 +422,43 @@ def test_long_contexts_through_the_planned_launch(heads, kv_heads, d, batch):
     want = dense_attention(q[pick], kp, vp, tables[pick], torch.arange(len(pick) + 1, dtype=torch.int32), sl[pick], heads,
                            kv_heads, d, 1.0)
     assert rel_err(got[pick], want) <= 1.6e-2
+
+
+@pytest.mark.parametrize("heads,kv_heads,d", [(32, 4, 64), (8, 2, 128), (6, 1, 96), (4, 4, 32)])
+def test_decoded_tokens_beside_prompt_portions(heads, kv_heads, d):
+    """A step with decoded tokens (long contexts, cut into partitions) and small portions beside prompt portions:
+    launched in two parts, sequences with few queries first.  One decoded token looks at a single far key."""
+    import types
+    bs = 16
+    group = heads // kv_heads
+    few_q = [1, 1, 2, 1, 64 // group]                          # the last one fills the decode kernel's tile exactly
+    few_k = [3000, 17, 700, 4096, 900]
+    many_q = [64 // group + 1, 100, 300]
+    many_k = [2000, 100, 1300]
+    q_lens, k_lens = few_q + many_q, few_k + many_k
+    q, kp, vp, tables, cu, sl = paged_case(k_lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16, seed=12)
+    n = 1234                                                   # sequence 0, head 1 sees key 1234 only
+    page, off = int(tables[0, n // bs]), n % bs
+    kp[page, 1 // group, off, :] = (q[0, d:2 * d].float() * 40).to(torch.bfloat16)
+    ctx = types.SimpleNamespace(num_seqs=len(q_lens), max_q_len=max(q_lens), max_k_len=max(k_lens), q_lens=q_lens, k_lens=k_lens,
+                                capturing=False)
+    got = ops().paged_attention(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d,
+                                1.0, 0, ctx).cpu().float()
+    assert torch.allclose(got[0, d:2 * d], vp[page, 1 // group, :, off].float(), atol=2e-2)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, 1.0)
+    assert rel_err(got, want) <= 1.6e-2
+    # the same batch in one launch (sequences not in that order): the same numbers up to rounding
+    order = [5, 0, 6, 1, 2, 7, 3, 4]
+    rows = [list(range(int(cu[s]), int(cu[s + 1]))) for s in order]
+    q2 = q[[r for rs in rows for r in rs]]
+    cu2 = torch.tensor([0] + list(np.cumsum([len(rs) for rs in rows])), dtype=torch.int32)
+    ctx2 = types.SimpleNamespace(num_seqs=len(order), max_q_len=max(q_lens), max_k_len=max(k_lens), q_lens=[q_lens[s] for s in order],
+                                 k_lens=[k_lens[s] for s in order], capturing=False)
+    got2 = ops().paged_attention(q2.cuda(), kp.cuda(), vp.cuda(), tables[order].contiguous().cuda(), cu2.cuda(), sl[order].cuda(), heads,
+                                 kv_heads, d, 1.0, 0, ctx2).cpu().float()
+    back = torch.empty_like(got2)
+    back[[r for rs in rows for r in rs]] = got2
+    assert rel_err(back, want) <= 1.6e-2
 
 
 def test_attention_plan():

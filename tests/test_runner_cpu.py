@@ -35,18 +35,19 @@ def test_layout_of_a_mixed_batch(runtime):
     c = entry(manager, "c", [3], 17, want=[0])
     buf, offsets, sizes, host = runner._stage([a, b, c])
     piece = lambda i: buf[offsets[i]: offsets[i] + sizes[i]]
-    assert piece(0).tolist() == [5, 6, 7, 8, 9] + list(range(20)) + [3]                    # token ids
-    assert piece(1).tolist() == list(range(5)) + list(range(20)) + [17]                    # positions
-    assert piece(2).tolist() == [0, 5, 25, 26] and piece(3).tolist() == [5, 20, 18]        # query offsets, context lengths
-    assert piece(6).tolist() == [4, 25]                                                    # rows whose logits are wanted
+    # inside the batch the entries stand by ascending token count: c (1 token), a (5), b (20)
+    assert piece(0).tolist() == [3] + [5, 6, 7, 8, 9] + list(range(20))                    # token ids
+    assert piece(1).tolist() == [17] + list(range(5)) + list(range(20))                    # positions
+    assert piece(2).tolist() == [0, 1, 6, 26] and piece(3).tolist() == [18, 5, 20]         # query offsets, context lengths
+    assert piece(6).tolist() == [5, 0]                                                     # wanted rows, in the callers' order: a's, c's
     tables = piece(7).reshape(3, 2)
     g = next(iter(manager.groups))
-    assert tables[1].tolist() == manager.block_table("b", g) and tables[0, 1] == 0        # short tables are padded with 0
+    assert tables[2].tolist() == manager.block_table("b", g) and tables[1, 1] == 0        # short tables are padded with 0
     slots = piece(8)
     tc = manager.block_table("c", g)
-    assert slots[-1] == tc[1] * 16 + 1 and slots[0] == manager.block_table("a", g)[0] * 16
+    assert slots[0] == tc[1] * 16 + 1 and slots[1] == manager.block_table("a", g)[0] * 16
     assert all(o % 4 == 0 for o in offsets)                                                # 16-byte aligned pieces
-    assert host["q_lens"] == [5, 20, 1] and host["k_lens"] == [5, 20, 18]
+    assert host["q_lens"] == [1, 5, 20] and host["k_lens"] == [18, 5, 20]
     for r in "abc":
         manager.free(r)
 
