@@ -384,7 +384,7 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
-    int block_size, float scale, int window) {
+    int block_size, float scale, int window, const int* __restrict__ work) {
   extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
   constexpr int kKTile = 64 * kKRow, kVTile = D * kVRow;         // elements of one group's keys / values of a step
   // keys [2 buffers][KG][64 rows][kKRow], then values [2 buffers][KG][D rows][kVRow].  Addresses are formed
@@ -394,20 +394,28 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
 #define PLLM_V_TILE(buf, group) (reinterpret_cast<bf16*>(prefill_lds) + 2 * KG * kKTile + ((buf) * KG + (group)) * kVTile)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int cw = wave & 3, kg = wave >> 2;                      // column share and key group of this wavefront
-  // blockIdx.x = (sequence, kv head), blockIdx.y = tile slot: workgroups are handed out x first, so all
-  // long tiles of all sequences start before any short one
-  const int seq = blockIdx.x / num_kv_heads, kvh = blockIdx.x - seq * num_kv_heads;
-  const int slot = blockIdx.y;
+  // Workgroups are handed out x first.  With a work list (pairs of sequence and tile, those with the most keys
+  // first): blockIdx.x = kv head, blockIdx.y = entry of the list, so the longest pieces of work of all sequences
+  // start first and no workgroup is launched for nothing.  Without one: blockIdx.x = (sequence, kv head),
+  // blockIdx.y = tile slot counted from every sequence's last tile; sequences with fewer tiles than the
+  // longest leave their other slots empty.
+  int seq, kvh, listed_tile = -1;
+  if (work) {
+    kvh = blockIdx.x;
+    seq = work[2 * blockIdx.y];
+    listed_tile = work[2 * blockIdx.y + 1];
+  } else {
+    seq = blockIdx.x / num_kv_heads;
+    kvh = blockIdx.x - seq * num_kv_heads;
+  }
   const int G = num_heads / num_kv_heads;
   const int q_begin = cu_seqlens_q[seq], num_q = cu_seqlens_q[seq + 1] - q_begin;
   const int len_k = seq_lens_k[seq];
   const int num_cols = num_q * G;
   constexpr int kWgCols = 4 * 16 * NCB;
   const int my_tiles = (num_cols + kWgCols - 1) / kWgCols;
-  // Later tiles see more keys: slot 0 is every sequence's last tile, so the longest pieces of work start
-  // first and the short ones fill the tail.
-  const int tile = my_tiles - 1 - slot;
-  if (tile < 0) return;                                         // this sequence has fewer tiles than the longest
+  const int tile = work ? listed_tile : my_tiles - 1 - (int)blockIdx.y;
+  if (tile < 0 || tile >= my_tiles) return;                     // no such tile in this sequence
   const int wg_col0 = tile * kWgCols;
   const int pos0 = len_k - num_q;
   // key range of the whole workgroup
@@ -767,7 +775,8 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
                                        int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                        const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                                        int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                       int num_partitions, float* partials, int waves, int column_blocks, int tune, hipStream_t stream) {
+                                       int num_partitions, float* partials, int waves, int column_blocks, int tune, const int* work_list, int num_work,
+                                       hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
   const int G = num_heads / num_kv_heads;
@@ -791,14 +800,18 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // tiles of all sequences (most keys) start first and the early tiles fill the tail; that keeps the compute
     // units evenly loaded for any number and length of prompts (pairing far and near tiles in one workgroup
     // was 5 % faster when the pairs filled the compute units exactly and up to 40 % slower just past that).
-    if (ptiles > 65535) return -2;
+    if (ptiles > 65535 || num_work > 65535 || (work_list && num_work <= 0)) return -2;
     dim3 pgrid(num_kv_heads * num_seqs, ptiles, 1);
+    if (work_list) pgrid = dim3(num_kv_heads, num_work, 1);
     // Two key groups (eight wavefronts, one workgroup per compute unit) when there are too few workgroups to
     // keep two of the four-wavefront kind on every compute unit for most of the time (measured: faster up to
     // about 2.5 workgroups per compute unit), and for the head sizes that then still fit into registers and
     // LDS; else one key group.  `tune` (measurements): bit 1 = one key group, bit 2 = two key groups.
     constexpr bool two_fits = D <= 96 && prefill_lds_bytes(2) <= 160 * 1024;
-    bool two = two_fits && 2L * pgrid.x * pgrid.y <= 5L * num_compute_units();
+    // (workgroups that find work: a sequence has as many tiles as its own queries need, the grid as many slots
+    // as the longest)
+    const long busy = work_list ? (long)num_work * num_kv_heads : ((long)total_q * G / kCols + num_seqs) * num_kv_heads;
+    bool two = two_fits && 2L * busy <= 5L * num_compute_units();
     if (tune & 2) two = false;
     if ((tune & 4) && two_fits) two = true;
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
@@ -813,7 +826,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     }
     hipLaunchKernelGGL(kern, pgrid, dim3(two ? 512 : 256), lds, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q,
-                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window);
+                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, work_list);
     return (int)hipGetLastError();
   }
   dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64 * waves);

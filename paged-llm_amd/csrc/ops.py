@@ -11,6 +11,7 @@ from __future__ import annotations
 import ctypes
 from ctypes import c_float, c_int, c_long, c_longlong, c_ulonglong, c_void_p
 
+import numpy as np
 import torch
 
 from . import build
@@ -417,7 +418,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = 
 
 
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p]
+             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
 _attn_scratch: dict = {}
 _attn_checked: set = set()
 
@@ -468,11 +469,13 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                          cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
                          head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
                          num_partitions: int = 1, waves: int = 1, column_blocks: int = 0, tune: int = 0,
-                         out: torch.Tensor | None = None) -> torch.Tensor:
+                         out: torch.Tensor | None = None, work_list: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
     work item into aligned partitions that a second kernel merges; ``waves`` > 1 shares the keys
-    of a work item between the wavefronts of one workgroup (few queries per sequence only)."""
+    of a work item between the wavefronts of one workgroup (few queries per sequence only).  ``work_list``
+    (prompt portions): int32 [n, 2] pairs of (sequence, tile of 128 query columns), the order in which the
+    kernel's workgroups take them (``prompt_work_list``)."""
     S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
     _need(mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs),
           f"MFMA attention takes bfloat16, head sizes 16..256 in steps of 16, pages of >= 16 positions and groups of <= 64 "
@@ -488,6 +491,10 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     _need(column_blocks in (0, 1, 2, 4), "column_blocks is 0 (automatic), 1, 2 or 4")
     _need(waves == 1 or _merge_lds_bytes(ncb, waves, head_dim) <= _max_lds_bytes(q.device),
           "the merge buffers of that many wavefronts do not fit LDS")
+    if work_list is not None:
+        _on_gpu(work_list)
+        _need(work_list.dtype == torch.int32 and work_list.dim() == 2 and work_list.shape[1] == 2 and work_list.is_contiguous()
+              and 0 < work_list.shape[0] <= 65535, "work_list: int32 [n, 2], n in 1..65535")
     ws = None
     if partition_size > 0:
         floats = T * num_heads * num_partitions * (head_dim + 2)
@@ -503,12 +510,72 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
     _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
              block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
-             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), int(tune), _stream()),
+             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), int(tune), _ptr(work_list),
+             0 if work_list is None else work_list.shape[0], _stream()),
            "paged_attention_mfma")
     return out
 
 
+PROMPT_TILE_COLUMNS = 128   # query columns (queries x heads per kv head) of one workgroup of the prompt kernel
+_upload_buffers: dict = {}
+
+
+def _upload_ints(values: np.ndarray, device) -> torch.Tensor:
+    """int32 values to the device without stalling the host: through a pinned buffer (allocated once per
+    device) and a copy on the current stream.  A copy from pageable memory would hold the host until the
+    stream has caught up, and the kernels of the layers before could then no longer be issued ahead."""
+    key = str(device)
+    pinned, copied = _upload_buffers.get(key, (None, None))
+    if pinned is None or pinned.numel() < values.size:
+        pinned, copied = torch.empty(max(values.size, 1 << 14), dtype=torch.int32, pin_memory=True), torch.cuda.Event()
+        _upload_buffers[key] = (pinned, copied)
+    else:
+        copied.synchronize()                                   # the last upload has left the buffer
+    staged = pinned[:values.size].view(values.shape)
+    staged.copy_(torch.from_numpy(np.ascontiguousarray(values, dtype=np.int32)))
+    out = torch.empty(values.shape, dtype=torch.int32, device=device)
+    out.copy_(staged, non_blocking=True)
+    copied.record()
+    return out
+
+
+def prompt_work_list(ctx, first_seq: int, group: int) -> torch.Tensor | None:
+    """The prompt kernel's work for the sequences from ``first_seq`` on: int32 [n, 2] pairs (sequence counted
+    from ``first_seq``, tile), the tiles that see the most keys first.  Workgroups take them in that order, so
+    long pieces start first and none is launched for a tile that a shorter sequence does not have (with one
+    long and many short sequences most of a rectangular grid is empty, and handing out empty workgroups was
+    measured at 80 us for 3,800 of them).  Built from the host lengths once per step and kept in the context;
+    None when the sequences are all alike and the kernel's own grid does the same."""
+    cache = getattr(ctx, "launch_cache", None)
+    key = ("prompt_tiles", first_seq, group)
+    if cache is not None and key in cache:
+        return cache[key]
+    counts = {-(-n * group // PROMPT_TILE_COLUMNS) for n in ctx.q_lens[first_seq:]}
+    if len(counts) == 1 and len(set(ctx.k_lens[first_seq:])) == 1:
+        # every sequence has the same tiles with the same keys: the kernel's own grid (sequence x kv head, tiles
+        # from the last one down) has no empty workgroup and hands the work out in the same order
+        if cache is not None:
+            cache[key] = None
+        return None
+    seqs, tiles, keys = [], [], []
+    for s in range(first_seq, len(ctx.q_lens)):
+        n = -(-ctx.q_lens[s] * group // PROMPT_TILE_COLUMNS)
+        t = np.arange(n, dtype=np.int64)
+        seqs.append(np.full(n, s - first_seq, dtype=np.int64))
+        tiles.append(t)
+        keys.append(ctx.k_lens[s] - ctx.q_lens[s] + (t + 1) * PROMPT_TILE_COLUMNS // group)
+    seqs, tiles, keys = np.concatenate(seqs), np.concatenate(tiles), np.concatenate(keys)
+    work = None
+    if 0 < seqs.size <= 65535:
+        order = np.argsort(-keys, kind="stable")
+        work = _upload_ints(np.stack([seqs[order], tiles[order]], axis=1), ctx.device)
+    if cache is not None:
+        cache[key] = work
+    return work
+
+
 FEW_QUERY_COLUMNS = 64      # queries x heads per kv head that one tile of the decode kernel holds
+SPLIT_FROM_CONTEXT_TIMES_HEAD = 160_000   # context x head size of a few-query sequence from which two launches pay
 
 
 def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
@@ -516,11 +583,12 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
     """Attention of one step's queries over the paged cache: the MFMA kernels for bfloat16 where they
     take the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions.
 
-    A step that holds decoded tokens beside prompt portions is launched in two parts when the sequences with
-    few queries come first in the batch (the step function orders them so): those go to the kernel that cuts
-    their keys into partitions, the portions to the prompt kernel.  One launch for all would walk every decoded
-    token's whole context with a single wavefront (measured 49 us against 15 + 15 for a portion of 512 tokens
-    beside 7 decoded tokens at context 2048, 180 us at context 8192)."""
+    A step that holds decoded tokens beside prompt portions is one launch of the prompt kernel, in which a decoded
+    token is a tile of its own that one workgroup walks through its whole context; when such a context is long
+    (13 us per 1024 keys at head size 64, 34 us at 128) the step is launched in two parts instead, if the sequences
+    with few queries come first in the batch (the step function orders them so): those go to the kernel that cuts
+    their keys into partitions, the portions to the prompt kernel (a portion of 512 tokens beside 7 decoded tokens
+    at context 8192: 109 us in one launch, 36 us in two; at context 1024: 19 us and 24 us)."""
     bs = k_pages.shape[2]
     if mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
         group = num_heads // num_kv_heads
@@ -529,7 +597,8 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
         few = 0
         while few < len(q_lens) and q_lens[few] * group <= FEW_QUERY_COLUMNS:
             few += 1
-        if 0 < few < len(q_lens) and all(n * group > FEW_QUERY_COLUMNS for n in q_lens[few:]) and not ctx.capturing:
+        if (0 < few < len(q_lens) and max(k_lens[:few]) * head_dim >= SPLIT_FROM_CONTEXT_TIMES_HEAD and not ctx.capturing
+                and all(n * group > FEW_QUERY_COLUMNS for n in q_lens[few:])):
             rows = sum(q_lens[:few])
             out = torch.empty((q.shape[0], num_heads * head_dim), dtype=q.dtype, device=q.device)
             max_q, max_k = max(q_lens[:few]), max(k_lens[:few])
@@ -539,12 +608,15 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                                  2 if waves == 1 else 0, out=out[:rows])
             # the portions: rows, cu_seqlens_q and the output stay absolute, the per-sequence arrays start at `few`
             paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
-                                 num_kv_heads, head_dim, scale, window, max(q_lens[few:]), 0, 1, 1, 2, out=out)
+                                 num_kv_heads, head_dim, scale, window, max(q_lens[few:]), 0, 1, 1, 2, out=out,
+                                 work_list=prompt_work_list(ctx, few, group))
             return out
         waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, group, head_dim, lds)
         # Prompt portions: 32 columns per wavefront leave registers for two wavefronts per SIMD
         # (measured faster than 64 columns at one).
+        prompt = waves == 1 and ctx.max_q_len * group > FEW_QUERY_COLUMNS and not ctx.capturing
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
-                                    head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0)
+                                    head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0,
+                                    work_list=prompt_work_list(ctx, 0, group) if prompt else None)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window)

@@ -58,6 +58,9 @@ class StepContext:
     # True when the step is replayed from a captured HIP graph: launch shapes must then depend on
     # num_tokens/num_seqs only, and `max_k_len` is an upper bound, not the batch's own maximum.
     capturing: bool = False
+    # Device arrays that a part derives from the host lengths, kept for the other layers of the step
+    # (the list of prompt tiles the attention kernel works through, for one).
+    launch_cache: dict = field(default_factory=dict)
 
     @property
     def decode_only(self) -> bool:

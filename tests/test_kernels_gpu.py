@@ -410,7 +410,7 @@ def test_long_contexts_through_the_planned_launch(heads, kv_heads, d, batch):
         page, off = int(tables[s, n // bs]), n % bs
         head = s % heads
         kp[page, head // (heads // kv_heads), off, :] = (q[s, head * d:(head + 1) * d].float() * 40).to(torch.bfloat16)
-    ctx = types.SimpleNamespace(num_seqs=batch, max_q_len=1, max_k_len=max(lens), q_lens=[1] * batch, k_lens=lens, capturing=False)
+    ctx = types.SimpleNamespace(num_seqs=batch, max_q_len=1, max_k_len=max(lens), q_lens=[1] * batch, k_lens=lens, capturing=False, device=torch.device("cuda"))
     got = ops().paged_attention(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d,
                                 1.0, 0, ctx).cpu().float()
     for s, n in enumerate(far):
@@ -441,7 +441,7 @@ def test_decoded_tokens_beside_prompt_portions(heads, kv_heads, d):
     page, off = int(tables[0, n // bs]), n % bs
     kp[page, 1 // group, off, :] = (q[0, d:2 * d].float() * 40).to(torch.bfloat16)
     ctx = types.SimpleNamespace(num_seqs=len(q_lens), max_q_len=max(q_lens), max_k_len=max(k_lens), q_lens=q_lens, k_lens=k_lens,
-                                capturing=False)
+                                capturing=False, device=torch.device("cuda"))
     got = ops().paged_attention(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d,
                                 1.0, 0, ctx).cpu().float()
     assert torch.allclose(got[0, d:2 * d], vp[page, 1 // group, :, off].float(), atol=2e-2)
@@ -453,7 +453,7 @@ def test_decoded_tokens_beside_prompt_portions(heads, kv_heads, d):
     q2 = q[[r for rs in rows for r in rs]]
     cu2 = torch.tensor([0] + list(np.cumsum([len(rs) for rs in rows])), dtype=torch.int32)
     ctx2 = types.SimpleNamespace(num_seqs=len(order), max_q_len=max(q_lens), max_k_len=max(k_lens), q_lens=[q_lens[s] for s in order],
-                                 k_lens=[k_lens[s] for s in order], capturing=False)
+                                 k_lens=[k_lens[s] for s in order], capturing=False, device=torch.device("cuda"))
     got2 = ops().paged_attention(q2.cuda(), kp.cuda(), vp.cuda(), tables[order].contiguous().cuda(), cu2.cuda(), sl[order].cuda(), heads,
                                  kv_heads, d, 1.0, 0, ctx2).cpu().float()
     back = torch.empty_like(got2)
