@@ -258,7 +258,8 @@ def run_attention_cases() -> dict:
             q = torch.randn(S * T, nh * d, device="cuda", dtype=torch.bfloat16, generator=g)
             cu = torch.arange(0, S * T + 1, T, device="cuda", dtype=torch.int32)
             sl = torch.full((S,), ctx, device="cuda", dtype=torch.int32)
-            ctx_info = types.SimpleNamespace(num_seqs=S, max_q_len=T, max_k_len=ctx)
+            ctx_info = types.SimpleNamespace(num_seqs=S, max_q_len=T, max_k_len=ctx, q_lens=[T] * S, k_lens=[ctx] * S, capturing=False,
+                                             device=torch.device("cuda"), launch_cache={})
             fn = lambda i: ops.paged_attention(q, kps[i % copies], vps[i % copies], tables, cu, sl, nh, nkv, d, d ** -0.5, 0, ctx_info)
             fn(0)
             torch.cuda.synchronize()

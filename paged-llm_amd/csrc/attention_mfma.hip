@@ -595,28 +595,28 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
   };
   const int full_from = window > 0 ? max(qpos_max - window + 1, 0) : 0;   // blocks from here on are inside every column's window
 
-  // ---- the steps.  Step i is computed from LDS while step i + 1 sits in registers (requested one
-  //      step earlier, written to the other LDS buffer after the computation) and step i + 2 is being
-  //      requested: a fetch has two steps to arrive.
+  // ---- the steps.  Step i is computed from LDS while step i + 1 sits in registers (requested one step
+  //      earlier); after the computation it is written to the other LDS buffer and step i + 2 is requested
+  //      into the same registers: a fetch has a whole step to arrive.
   constexpr int kStepKeys = 64 * KG;
-  auto step = [&](int n0, int buf, Fetched& arriving, Fetched& free_regs) {
-    if (n0 + 2 * kStepKeys < k_hi) fetch(free_regs, n0 + 2 * kStepKeys);
+  Fetched regs;
+  auto step = [&](int n0, int buf) {
     const int mine = n0 + kg * 64;                                // this group's 64 keys of the step
     if (wave_on && mine < vis_hi && mine + 64 > vis_lo) {
       if (mine + 63 <= qpos_min && mine >= full_from) compute(buf, mine, PlainTag{});
       else compute(buf, mine, MaskedTag{});
     }
-    if (n0 + kStepKeys < k_hi) stash(arriving, buf ^ 1);
+    if (n0 + kStepKeys < k_hi) stash(regs, buf ^ 1);
+    if (n0 + 2 * kStepKeys < k_hi) fetch(regs, n0 + 2 * kStepKeys);
     __syncthreads();
   };
-  Fetched regs_a, regs_b;
-  fetch(regs_a, k_lo);
-  if (k_lo + kStepKeys < k_hi) fetch(regs_b, k_lo + kStepKeys);
-  stash(regs_a, 0);
+  fetch(regs, k_lo);
+  stash(regs, 0);
+  if (k_lo + kStepKeys < k_hi) fetch(regs, k_lo + kStepKeys);
   __syncthreads();
   for (int n0 = k_lo; n0 < k_hi; n0 += 2 * kStepKeys) {
-    step(n0, 0, regs_b, regs_a);                                  // step n0 in buffer 0; the next one arrives in regs_b
-    if (n0 + kStepKeys < k_hi) step(n0 + kStepKeys, 1, regs_a, regs_b);
+    step(n0, 0);
+    if (n0 + kStepKeys < k_hi) step(n0 + kStepKeys, 1);
   }
 
   if (KG == 2) {
@@ -803,15 +803,17 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     if (ptiles > 65535 || num_work > 65535 || (work_list && num_work <= 0)) return -2;
     dim3 pgrid(num_kv_heads * num_seqs, ptiles, 1);
     if (work_list) pgrid = dim3(num_kv_heads, num_work, 1);
-    // Two key groups (eight wavefronts, one workgroup per compute unit) when there are too few workgroups to
-    // keep two of the four-wavefront kind on every compute unit for most of the time (measured: faster up to
-    // about 2.5 workgroups per compute unit), and for the head sizes that then still fit into registers and
-    // LDS; else one key group.  `tune` (measurements): bit 1 = one key group, bit 2 = two key groups.
-    constexpr bool two_fits = D <= 96 && prefill_lds_bytes(2) <= 160 * 1024;
+    // Two key groups (eight wavefronts, one workgroup per compute unit) for the head sizes that then still fit
+    // into registers and LDS (up to 128): always where a wavefront of the four-wavefront kind needs more than half
+    // of a SIMD's registers (head sizes above 96: two groups are then the only way to two wavefronts per SIMD,
+    // measured 1.4 times faster at 128), else when there are too few workgroups to keep two of the four-wavefront
+    // kind on every compute unit for most of the time (measured: faster up to about 2.5 workgroups per compute
+    // unit).  `tune` (measurements): bit 1 = one key group, bit 2 = two key groups.
+    constexpr bool two_fits = D <= 128 && prefill_lds_bytes(2) <= 160 * 1024;
     // (workgroups that find work: a sequence has as many tiles as its own queries need, the grid as many slots
     // as the longest)
     const long busy = work_list ? (long)num_work * num_kv_heads : ((long)total_q * G / kCols + num_seqs) * num_kv_heads;
-    bool two = two_fits && 2L * busy <= 5L * num_compute_units();
+    bool two = two_fits && (D > 96 || 2L * busy <= 5L * num_compute_units());
     if (tune & 2) two = false;
     if ((tune & 4) && two_fits) two = true;
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
