@@ -120,6 +120,99 @@ __device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, i
   }
 }
 
+// The rows into LDS (kernels whose input needs a residual sum and / or a norm): rows = x[row_index] (+ delta),
+// the sum in float rounded once and written out by workgroup 0, the elements multiplied by the norm's
+// weights, and the rows' sums of squares into `sq` ([M][column groups]).  `after_first_requests` is called once
+// the first loads of the rows are issued: the caller requests its first weights there.
+template <int WAVES, class Early>
+__device__ __forceinline__ void stage_rows(const DecodeLinearParams& p, bf16* xs, float* sq, int row_len, int wave, int lane,
+                                           Early&& after_first_requests) {
+  const int M = p.M, K = p.K;
+  // ---- the rows into LDS.  A wavefront owns a group of 64 pieces of 8 columns and walks rows with it, up
+  // to kBatch rows at a time.  It requests the pieces of its first batch, then its weights, and only then
+  // touches the first piece: loads return in the order they were issued, so the rows (cache hits) must not
+  // queue behind the weights (HBM), and the weight loads carry no condition, so that the compiler can
+  // count exactly how many loads may still be under way when a piece is used.  Sums of squares: per lane
+  // over its 8 elements, over the wavefront, then over the column groups of a row in ascending order: one
+  // fixed order, whatever else is in the batch.
+  constexpr int kBatch = 4;
+  const int ipr = ((K >> 3) + 63) >> 6;                         // column groups per row
+  const int cg = min(ipr, WAVES), rpp = WAVES / cg;             // groups and rows under way at a time
+  const int wc = wave % cg, wr = wave / cg;                     // this wavefront's first group and row
+  const bool active = wr < rpp;
+  int src_lane = lane < M ? lane : 0;                           // lane m holds the source row of input row m
+  if (p.row_index) src_lane = p.row_index[src_lane];
+  const bool has_delta = p.delta != nullptr, has_norm = p.norm_w != nullptr;
+  bf16x8 xv[kBatch], dv[kBatch];
+  float4 nw0, nw1;
+  auto column = [&](int c) { return min((c * 64 + lane) * 8, K - 8); };   // loads stay inside the row ...
+  auto inside = [&](int c) { return (c * 64 + lane) * 8 < K; };           // ... and this says whether they count
+  auto issue = [&](int c, int m0) {                             // rows m0, m0 + rpp, ... of column group c
+    const int k0 = column(c);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, min(m0 + u * rpp, M - 1));
+      xv[u] = *reinterpret_cast<const bf16x8*>(p.x + src * p.ldx + k0);
+    }
+    if (has_delta) {
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, min(m0 + u * rpp, M - 1));
+        dv[u] = *reinterpret_cast<const bf16x8*>(p.delta + src * p.ldd + k0);
+      }
+    }
+  };
+  auto issue_norm = [&](int c) {
+    if (has_norm) {
+      nw0 = *reinterpret_cast<const float4*>(p.norm_w + column(c));
+      nw1 = *reinterpret_cast<const float4*>(p.norm_w + column(c) + 4);
+    }
+  };
+  auto sum_rows = [&](int c, int m0) {                          // pass 1 on the issued batch
+    const int k0 = column(c);
+    const bool in = inside(c);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int m = m0 + u * rpp;
+      if (!active || m >= M) continue;                          // the same for the whole wavefront
+      bf16x8 v = xv[u];
+      if (has_delta) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (__bf16)((float)v[i] + (float)dv[u][i]);     // float sum, rounded once
+        if (p.x_out && blockIdx.x == 0 && in) {
+          const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, m);
+          *reinterpret_cast<bf16x8*>(p.x_out + src * p.ldxo + k0) = v;
+        }
+      }
+      if (has_norm) {
+        // The row's scale 1 / rms is applied to the finished sums (it is the same for the whole row);
+        // here the elements take the norm's weights, and their squares are summed.
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
+        const float w[8] = {nw0.x, nw0.y, nw0.z, nw0.w, nw1.x, nw1.y, nw1.z, nw1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (__bf16)((float)v[i] * w[i]);
+        ss = wave_sum(in ? ss : 0.f);
+        if (lane == 0) sq[m * ipr + c] = ss;
+      }
+      if (in) *reinterpret_cast<bf16x8*>(xs + (size_t)m * row_len + k0) = v;
+    }
+  };
+  issue(wc, wr);
+  issue_norm(wc);
+  after_first_requests();                                       // the first unit's weights: on their way during all that follows
+  sum_rows(wc, wr);
+  for (int c = wc; c < ipr; c += cg) {
+    if (c != wc) issue_norm(c);
+    for (int m0 = (c == wc) ? wr + kBatch * rpp : wr; m0 < M; m0 += kBatch * rpp) {
+      issue(c, m0);
+      sum_rows(c, m0);
+    }
+  }
+  __syncthreads();
+}
+
 template <int EPI, int WAVES, bool HALF, bool DIRECT, int PRE>
 __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeLinearParams p, int num_units) {
   // Fetch the arguments the first loads depend on in one go (left alone, the compiler fetches each where
@@ -203,90 +296,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
     rope_inputs();
     request_first();
   } else {
-  // ---- the rows into LDS.  A wavefront owns a group of 64 pieces of 8 columns and walks rows with it, up
-  // to kBatch rows at a time.  It requests the pieces of its first batch, then its weights, and only then
-  // touches the first piece: loads return in the order they were issued, so the rows (cache hits) must not
-  // queue behind the weights (HBM), and the weight loads carry no condition, so that the compiler can
-  // count exactly how many loads may still be under way when a piece is used.  Sums of squares: per lane
-  // over its 8 elements, over the wavefront, then over the column groups of a row in ascending order: one
-  // fixed order, whatever else is in the batch.
-  constexpr int kBatch = 4;
-  const int ipr = ((K >> 3) + 63) >> 6;                         // column groups per row
-  const int cg = min(ipr, WAVES), rpp = WAVES / cg;             // groups and rows under way at a time
-  const int wc = wave % cg, wr = wave / cg;                     // this wavefront's first group and row
-  const bool active = wr < rpp;
-  int src_lane = lane < M ? lane : 0;                           // lane m holds the source row of input row m
-  if (p.row_index) src_lane = p.row_index[src_lane];
-  const bool has_delta = p.delta != nullptr, has_norm = p.norm_w != nullptr;
-  bf16x8 xv[kBatch], dv[kBatch];
-  float4 nw0, nw1;
-  auto column = [&](int c) { return min((c * 64 + lane) * 8, K - 8); };   // loads stay inside the row ...
-  auto inside = [&](int c) { return (c * 64 + lane) * 8 < K; };           // ... and this says whether they count
-  auto issue = [&](int c, int m0) {                             // rows m0, m0 + rpp, ... of column group c
-    const int k0 = column(c);
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, min(m0 + u * rpp, M - 1));
-      xv[u] = *reinterpret_cast<const bf16x8*>(p.x + src * p.ldx + k0);
-    }
-    if (has_delta) {
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, min(m0 + u * rpp, M - 1));
-        dv[u] = *reinterpret_cast<const bf16x8*>(p.delta + src * p.ldd + k0);
-      }
-    }
-  };
-  auto issue_norm = [&](int c) {
-    if (has_norm) {
-      nw0 = *reinterpret_cast<const float4*>(p.norm_w + column(c));
-      nw1 = *reinterpret_cast<const float4*>(p.norm_w + column(c) + 4);
-    }
-  };
-  auto sum_rows = [&](int c, int m0) {                          // pass 1 on the issued batch
-    const int k0 = column(c);
-    const bool in = inside(c);
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const int m = m0 + u * rpp;
-      if (!active || m >= M) continue;                          // the same for the whole wavefront
-      bf16x8 v = xv[u];
-      if (has_delta) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (__bf16)((float)v[i] + (float)dv[u][i]);     // float sum, rounded once
-        if (p.x_out && blockIdx.x == 0 && in) {
-          const size_t src = (size_t)__builtin_amdgcn_readlane(src_lane, m);
-          *reinterpret_cast<bf16x8*>(p.x_out + src * p.ldxo + k0) = v;
-        }
-      }
-      if (has_norm) {
-        // The row's scale 1 / rms is applied to the finished sums (it is the same for the whole row);
-        // here the elements take the norm's weights, and their squares are summed.
-        float ss = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
-        const float w[8] = {nw0.x, nw0.y, nw0.z, nw0.w, nw1.x, nw1.y, nw1.z, nw1.w};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (__bf16)((float)v[i] * w[i]);
-        ss = wave_sum(in ? ss : 0.f);
-        if (lane == 0) sq[m * ipr + c] = ss;
-      }
-      if (in) *reinterpret_cast<bf16x8*>(xs + (size_t)m * row_len + k0) = v;
-    }
-  };
-  issue(wc, wr);
-  issue_norm(wc);
-  rope_inputs();
-  request_first();                                              // the first unit's weights: on their way during all that follows
-  sum_rows(wc, wr);
-  for (int c = wc; c < ipr; c += cg) {
-    if (c != wc) issue_norm(c);
-    for (int m0 = (c == wc) ? wr + kBatch * rpp : wr; m0 < M; m0 += kBatch * rpp) {
-      issue(c, m0);
-      sum_rows(c, m0);
-    }
-  }
-  __syncthreads();
+  stage_rows<WAVES>(p, xs, sq, row_len, wave, lane, [&]() {
+    rope_inputs();
+    request_first();
+  });
   }
   // 1 / rms of the input row this thread's results belong to (tile column r), from the sums of squares
   float row_scale = 1.f;
