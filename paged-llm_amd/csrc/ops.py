@@ -420,6 +420,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = 
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
 _attn_scratch: dict = {}
+_attn_scratch_retired: list = []      # outgrown buffers stay allocated: captured graphs still hold their addresses
 _attn_checked: set = set()
 
 
@@ -501,6 +502,8 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
         key = str(q.device)
         ws = _attn_scratch.get(key)
         if ws is None or ws.numel() < floats:
+            if ws is not None:
+                _attn_scratch_retired.append(ws)
             ws = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=q.device)
             _attn_scratch[key] = ws
     if head_dim not in _attn_checked:                 # the library on disk is the one compiled for this head size

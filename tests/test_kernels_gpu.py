@@ -424,6 +424,28 @@ def test_long_contexts_through_the_planned_launch(heads, kv_heads, d, batch):
     assert rel_err(got[pick], want) <= 1.6e-2
 
 
+def test_an_outgrown_partition_buffer_stays_allocated():
+    """The buffer of the partitions' partial results grows with the batch; a captured graph still holds the
+    address of the one it was captured with, so an outgrown buffer must not go back to the allocator."""
+    o = ops()
+    heads, kv_heads, d, bs = 4, 1, 16, 16
+    def run(batch, parts):
+        lens = [parts * 64] * batch
+        q, kp, vp, tables, cu, sl = paged_case(lens, [1] * batch, heads, kv_heads, d, bs, torch.bfloat16, seed=3)
+        got = o.paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, 1.0, 0, 1,
+                                     64, parts).cpu().float()
+        pick = sorted({0, batch - 1})
+        want = dense_attention(q[pick], kp, vp, tables[pick], torch.arange(len(pick) + 1, dtype=torch.int32), sl[pick], heads,
+                               kv_heads, d, 1.0)
+        assert rel_err(got[pick], want) <= 1.6e-2
+    run(2, 2)
+    first = o._attn_scratch["cuda:0"]
+    need = first.numel() // (heads * (d + 2)) + 64            # rows x partitions that no longer fit
+    run(need // 16 + 1, 16)
+    assert o._attn_scratch["cuda:0"].numel() > first.numel()
+    assert any(t is first for t in o._attn_scratch_retired)
+
+
 @pytest.mark.parametrize("heads,kv_heads,d", [(32, 4, 64), (8, 2, 128), (6, 1, 96), (4, 4, 32)])
 def test_decoded_tokens_beside_prompt_portions(heads, kv_heads, d):
     """A step with decoded tokens (long contexts, cut into partitions) and small portions beside prompt portions:
