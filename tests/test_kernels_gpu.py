@@ -81,17 +81,27 @@ def test_silu_mul(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("slots", ["shuffled", "runs"])
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 16, 16), (3, 1, 48, 8), (8, 8, 128, 32)])
-def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs):
+def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs, slots):
+    """``runs``: the slots of prompt portions (consecutive positions): a portion from a page's start, one that
+    starts 3 slots into a page, and between them a token that writes nothing."""
     from paged_llm_amd.parts.registry import BuildEnv
     from paged_llm_amd.parts.rope import RotaryEncoding
-    T, pages = 23, 9
+    T, pages = (23, 9) if slots == "shuffled" else (61, 12)
     rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, dtype, torch.device("cuda"), 512, {}))
     rope.prepare(512)
     width = (heads + 2 * kv_heads) * d
     qkv = rnd(T, width, seed=7, dtype=dtype)
     positions = torch.tensor([(5 * t + 3) % 500 for t in range(T)], dtype=torch.int32)
     perm = torch.randperm(pages * bs, generator=torch.Generator().manual_seed(8))[:T].to(torch.int32)
+    if slots == "runs":
+        order = torch.randperm(pages, generator=torch.Generator().manual_seed(8)).tolist()
+        def portion(first_page, start, n):                       # n consecutive positions from `start` of a request
+            table = order[first_page:]
+            return [table[(start + i) // bs] * bs + (start + i) % bs for i in range(n)]
+        perm = torch.tensor(portion(0, 0, 32) + [-1] + portion(6, 3, 28), dtype=torch.int32)
+        assert perm.numel() == T
     k_pages = torch.zeros(pages, kv_heads, bs, d, dtype=dtype).cuda()
     v_pages = torch.zeros(pages, kv_heads, d, bs, dtype=dtype).cuda()
     g = qkv.cuda().clone()
@@ -105,13 +115,16 @@ def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs):
     assert rel_err(g[:, :heads * d].view(T, heads, d), q) <= TOL[dtype]
     kp, vp = k_pages.float().cpu(), v_pages.float().cpu()
     for t in range(T):
+        if int(perm[t]) < 0:
+            continue
         page, off = int(perm[t]) // bs, int(perm[t]) % bs
         assert rel_err(kp[page, :, off, :], k[t]) <= TOL[dtype]
-        assert torch.equal(vp[page, :, :, off], v[t].to(dtype).float())
+        assert torch.equal(vp[page, :, :, off], v[t].to(dtype).float()), f"token {t}"
     # untouched slots stay zero
     written = torch.zeros(pages * bs, dtype=torch.bool)
-    written[perm.long()] = True
+    written[perm[perm >= 0].long()] = True
     assert kp.permute(0, 2, 1, 3).reshape(pages * bs, -1)[~written].abs().max() == 0
+    assert vp.permute(0, 3, 1, 2).reshape(pages * bs, -1)[~written].abs().max() == 0
 
 
 def test_copy_pages():
