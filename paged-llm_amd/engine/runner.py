@@ -216,7 +216,7 @@ class ModelRunner:
         view[offsets[2]: offsets[2] + S + 1] = np.arange(S + 1)
         return dict(key=key, pinned=pinned, view=view, offsets=offsets, sizes=sizes, table_shapes=table_shapes,
                     static=torch.zeros(max(total, 1), dtype=torch.int32, device=self.device), staged_rows=[None] * S,
-                    table_lens={name: np.zeros(S, dtype=np.int64) for name in self.group_specs},
+                    table_lens={name: [0] * S for name in self.group_specs}, last_page={name: [None] * S for name in self.group_specs},
                     copied=torch.cuda.Event() if on_gpu else None)
 
     def _capture(self, entry: dict) -> None:
@@ -238,41 +238,39 @@ class ModelRunner:
             self._graphs.pop(next(iter(self._graphs)))
         self._graphs[entry["key"]] = entry
 
-    def _restage_decode(self, entry: dict, entries: list) -> None:
+    def _restage_decode(self, entry: dict, entries: list) -> int:
         """Write a decode step's arrays into the pinned buffer of its graph, in the layout of
         ``_stage`` and with the same checks, but reading only the block tables that changed
         since the buffer was last written: the buffer keeps the rows of the step before, and an entry
         whose ``table_version`` is the one staged in its row leaves that row alone.  Rows past the
-        entries are empty requests: token 0 at position 0, block table [0], no slot to write to."""
+        entries are empty requests: token 0 at position 0, block table [0], no slot to write to.
+        Runs once per decoded token of every request, before the GPU has anything to do: plain lists and
+        one array assignment per piece, no array arithmetic."""
         bs, S = self.block_size, len(entry["staged_rows"])
         R = len(entries)
+        pad = S - R
         vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions
         view, offsets, sizes = entry["view"], entry["offsets"], entry["sizes"]
-        ids = np.zeros(S, dtype=np.int64)
-        starts = np.zeros(S, dtype=np.int64)
-        ids[:R] = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
-        starts[:R] = np.fromiter((e.start for e in entries), dtype=np.int64, count=R)
-        rids = [e.request_id for e in entries]
-        if len(set(rids)) != R:
-            raise StepError("a request appears twice in one step")
-        if ids.min() < 0 or ids.max() >= vocab:
-            raise StepError(f"token id outside [0, {vocab})")
-        if starts.min() < 0 or starts.max() + 1 > max_pos:
-            raise StepError(f"a position exceeds the model's {max_pos} positions")
-        logits_idx = []
+        ids, starts, rids, slots_state, logits_idx = [], [], [], [], []
         for i, e in enumerate(entries):
+            ids.append(e.tokens[0])
+            starts.append(e.start)
+            rids.append(e.request_id)
+            slots_state.append(-1 if e.state_slot is None else e.state_slot)
             for w in e.want:
                 if w != 0:
                     raise StepError(f"request {e.request_id!r}: wanted row {w} outside its 1 token")
                 logits_idx.append(i)
+        if len(set(rids)) != R:
+            raise StepError("a request appears twice in one step")
+        if min(ids) < 0 or max(ids) >= vocab:
+            raise StepError(f"token id outside [0, {vocab})")
+        if min(starts) < 0 or max(starts) + 1 > max_pos:
+            raise StepError(f"a position exceeds the model's {max_pos} positions")
+        if self.states and min(slots_state) < 0:
+            raise StepError("this model keeps per-request state: every entry needs a state slot")
         n_want = len(logits_idx)
         logits_idx += [0] * (sizes[6] - n_want)               # rows nobody asked for repeat row 0
-        slots_state = np.full(S, -1, dtype=np.int32)
-        slots_state[:R] = np.fromiter((-1 if e.state_slot is None else e.state_slot for e in entries), dtype=np.int32, count=R)
-        if self.states and (slots_state < 0).any():
-            raise StepError("this model keeps per-request state: every entry needs a state slot")
-        k_lens = starts + 1
-        need = (k_lens + bs - 1) // bs
         staged = entry["staged_rows"]                 # per row: (request id, table version) as last written, or "empty"
         stale = [s for s, e in enumerate(entries) if e.table_version is None or staged[s] != (rids[s], e.table_version)]
         emptied = [s for s in range(R, S) if staged[s] != "empty"]
@@ -280,12 +278,15 @@ class ModelRunner:
         def put(i, values):
             view[offsets[i]: offsets[i] + sizes[i]] = values
 
-        put(0, ids); put(1, starts); put(3, k_lens); put(4, slots_state); put(5, starts); put(6, logits_idx)
+        starts_padded = starts + [0] * pad
+        put(0, ids + [0] * pad); put(1, starts_padded); put(3, [k + 1 for k in starts] + [1] * pad)
+        put(4, slots_state + [-1] * pad); put(5, starts_padded); put(6, logits_idx)
         for gi, (name, cs) in enumerate(self.group_specs.items()):
             num_pages = self.kv.num_pages[name]
             fixed = entry["table_shapes"][name][1]
             tables = view[offsets[7 + 2 * gi]: offsets[7 + 2 * gi] + S * fixed].reshape(S, fixed)
-            held = entry["table_lens"][name]
+            held = entry["table_lens"][name]          # entries of each row's table that are staged
+            last = entry["last_page"][name]           # per row: (entries needed, page of the newest position) as last looked up
             for s in stale:
                 e = entries[s]
                 table = e.block_tables.get(name)
@@ -300,16 +301,22 @@ class ModelRunner:
                 tables[s, :n] = np.where(row == NO_PAGE, 0, row)
                 tables[s, n:] = 0
                 held[s] = n
+                last[s] = None
             for s in emptied:
                 tables[s, :] = 0
                 held[s] = 1
-            short = need > held
-            if short.any():
-                s = int(np.argmax(short))
-                raise StepError(f"request {rids[s]!r}: too few pages in group {name!r} for {int(k_lens[s])} positions")
-            slots = tables[np.arange(S), need - 1].astype(np.int64) * bs + starts % bs
-            slots[R:] = -1                                        # empty rows write nothing
-            put(8 + 2 * gi, slots)
+                last[s] = None
+            slots = []
+            for s in range(R):
+                start = starts[s]
+                need = start // bs + 1                        # pages that start + 1 positions take
+                if need > held[s]:
+                    raise StepError(f"request {rids[s]!r}: too few pages in group {name!r} for {start + 1} positions")
+                known = last[s]
+                if known is None or known[0] != need:
+                    known = last[s] = (need, int(tables[s, need - 1]))
+                slots.append(known[1] * bs + start % bs)
+            put(8 + 2 * gi, slots + [-1] * pad)               # empty rows write nothing
         for s in stale:
             staged[s] = (rids[s], entries[s].table_version)
         for s in emptied:

@@ -106,7 +106,7 @@ def test_decode_steps_restaged_in_place_equal_fresh_staging(runtime):
         fresh, offsets, sizes, host = runner._stage(entries, 4)
         if entry is None:
             entry = dict(view=fresh.copy(), offsets=offsets, sizes=sizes, table_shapes=host["table_shapes"],
-                         staged_rows=[None] * 3, table_lens={g: np.zeros(3, dtype=np.int64)})
+                         staged_rows=[None] * 3, table_lens={g: [0] * 3}, last_page={g: [None] * 3})
             entry["view"][offsets[7]: offsets[7] + sizes[7]] = -7          # nothing of the first staging may be relied on
         before = list(entry["staged_rows"])
         runner._restage_decode(entry, entries)
