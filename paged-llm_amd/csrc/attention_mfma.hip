@@ -525,6 +525,27 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     const bf16* kb = PLLM_K_TILE(buf, kg);
     const bf16* vb = PLLM_V_TILE(buf, kg);
     floatx4 s_t[4][NCB];
+    if constexpr (!kMasked && KSTEPS <= 2) {
+      // All key operands of the block are requested from LDS before the first product: the reads then wait
+      // for each other's latency once, not one after the other between the matrix instructions.
+      bf16x8 kop[4][KSTEPS];
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          const int dd = s * 32 + g * 8;
+          kop[kt][s] = (dd < D) ? *reinterpret_cast<const bf16x8*>(kb + (kt * 16 + r) * kKRow + dd) : zero8();
+        }
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+          for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[kt][s], qreg[cb][s], s_t[kt][cb], 0, 0, 0);
+      }
+    } else {
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
 #pragma unroll
@@ -537,6 +558,16 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) s_t[kt][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qreg[cb][s], s_t[kt][cb], 0, 0, 0);
       }
+    }
+    }
+    // Unmasked blocks: the value operands are requested from LDS here, so that they arrive during the softmax.
+    constexpr bool kEarlyValues = !kMasked && DBLOCKS <= 4;
+    bf16x8 v_early[kEarlyValues ? 2 : 1][kEarlyValues ? DBLOCKS : 1];
+    if constexpr (kEarlyValues) {
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; ++db) v_early[a][db] = *reinterpret_cast<const bf16x8*>(vb + (db * 16 + r) * kVRow + a * 32 + g * 8);
     }
     bf16x8 p_op[2][NCB];
 #pragma unroll
@@ -579,7 +610,9 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
       if (kMasked && n0 + a * 32 >= vis_hi) continue;
 #pragma unroll
       for (int db = 0; db < DBLOCKS; ++db) {
-        bf16x8 vreg = *reinterpret_cast<const bf16x8*>(vb + (db * 16 + r) * kVRow + a * 32 + g * 8);
+        bf16x8 vreg;
+        if constexpr (kEarlyValues) vreg = v_early[a][db];
+        else vreg = *reinterpret_cast<const bf16x8*>(vb + (db * 16 + r) * kVRow + a * 32 + g * 8);
         if (kMasked) {
           // values of keys that no column of this wavefront may see are zeroed (stale data, 0 * NaN)
 #pragma unroll
