@@ -459,10 +459,16 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
     size = 256                                        # at least four blocks of 64 keys per workgroup
     while (max_k_len + size - 1) // size > want_parts:
         size *= 2
+    parts = (max_k_len + size - 1) // size
     waves = max_waves
     while waves > 4 and (waves // 2) * 64 >= min(size, max_k_len):
         waves //= 2
-    parts = (max_k_len + size - 1) // size
+    # Small heads (two blocks of keys under way per wavefront) and two or more work items per compute unit: two
+    # workgroups of four wavefronts on a compute unit stream faster than one of eight (64 sequences x 8 kv heads x
+    # 2048 keys at head size 64: a decode step of Llama-3.2-1B shapes 2.68 against 2.74 ms).  With one work item per
+    # compute unit, two partitions of four wavefronts each were slower in the step (2.81 against 2.75 ms at 4 kv heads).
+    if head_dim <= 64 and parts == 1 and items >= 512:
+        waves = 4
     return (waves, size, parts) if parts > 1 else (waves, 0, 1)
 
 

@@ -501,6 +501,8 @@ def test_attention_plan():
     lds = 160 * 1024
     assert plan(8, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)       # decoding: partitions for workgroups, blocks for wavefronts
     assert plan(64, 4, 1, 2048, 8, 64, lds) == (8, 0, 1)         # enough sequences: wavefronts only
+    assert plan(64, 8, 1, 2048, 4, 64, lds) == (4, 0, 1)         # two work items per compute unit: smaller workgroups
+    assert plan(64, 8, 1, 2048, 4, 128, lds) == (8, 0, 1)        # large heads keep eight (one block under way per wavefront)
     assert plan(1, 4, 1, 2048, 8, 64, lds) == (4, 256, 8)
     assert plan(8, 4, 1, 200, 8, 64, lds) == (4, 0, 1)
     assert plan(1, 4, 2048, 2048, 8, 64, lds) == (1, 0, 1)      # a long prompt portion: one wavefront per query tile
