@@ -167,7 +167,7 @@ class LLMEngine:
                 self.cache_manager.table_version(req.request_id)))
             if item.needs_sampling:
                 sampled_items.append(req)
-        logits = self.runner.step(entries, self.cache_manager.take_pending_copies())
+        logits = self.runner.step(entries, self.cache_manager.take_pending_copies(), borrow=True)    # sampled from at once
         if not sampled_items:
             return {}
         tokens = self.sampler.sample(logits, [r.sampling_params for r in sampled_items],

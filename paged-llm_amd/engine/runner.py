@@ -323,7 +323,7 @@ class ModelRunner:
             staged[s] = "empty"
         return n_want
 
-    def _graph_step(self, key, entries: list) -> torch.Tensor:
+    def _graph_step(self, key, entries: list, borrow: bool = False) -> torch.Tensor:
         entry = self._graphs.get(key)
         fresh = entry is None
         if fresh:
@@ -336,16 +336,19 @@ class ModelRunner:
         entry["static"].copy_(entry["pinned"], non_blocking=True)
         entry["copied"].record()
         entry["graph"].replay()
-        return entry["logits"][:n_want].clone()
+        logits = entry["logits"][:n_want]
+        return logits if borrow else logits.clone()
 
     # ------------------------------------------------------------------ run
     @torch.no_grad()
-    def step(self, entries: list, copies: dict | None = None) -> torch.Tensor:
-        """Float logits [wanted rows, vocab], in the order of the entries and of their ``want``."""
+    def step(self, entries: list, copies: dict | None = None, borrow: bool = False) -> torch.Tensor:
+        """Float logits [wanted rows, vocab], in the order of the entries and of their ``want``.
+        ``borrow``: the caller is done with the logits before its next step (a sampler that runs at once): a
+        replayed step then hands out its graph's own buffer, which the next replay overwrites, without a copy."""
         if copies:
             self.kv.apply_copies(copies)
         key = self._graph_key(entries)
         if key is not None:
-            return self._graph_step(key, entries)
+            return self._graph_step(key, entries, borrow)
         ctx = self.build_context(entries)
         return self.model.forward(ctx, self.kv, self.states)
