@@ -71,17 +71,6 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   const int seq = blockIdx.z;
   const int kvh = blockIdx.y / num_partitions, part = blockIdx.y - kvh * num_partitions;
   const int G = num_heads / num_kv_heads;
-  // With partitions and no window the first block of a wavefront starts at a key that the grid position alone
-  // gives: its pages are looked up together with the lengths, not after them (one wait for memory less in the
-  // chain lengths -> pages -> keys).  Entries past the sequence's own are inside its row and never used.
-  const bool early = partition_size > 0 && window == 0;
-  const int early_n0 = part * partition_size + (WAVES > 1 ? wave * 64 : 0);
-  int early_page[4] = {0, 0, 0, 0};
-  if (early) {
-    const int* row = block_tables + (size_t)seq * bt_stride;
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) early_page[kt] = row[min((early_n0 + kt * 16) / block_size, bt_stride - 1)];
-  }
   const int q_begin = cu_seqlens_q[seq], num_q = cu_seqlens_q[seq + 1] - q_begin;
   const int len_k = seq_lens_k[seq];
   const int num_cols = num_q * G;
@@ -150,7 +139,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
       const int nk = n0 + kt * 16;
       blk.on[kt] = nk < k_hi;                                   // uniform; tiles past the range: table entries stay unread
       if (!blk.on[kt]) continue;
-      const int page = (early && n0 == early_n0) ? early_page[kt] : bt[nk / block_size];
+      const int page = bt[nk / block_size];
       const int off = nk & (block_size - 1);
       const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
       const bf16* krow = k_pages + base + (size_t)(off + r) * D;
