@@ -766,6 +766,18 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
 
 PLLM_API int pllm_attention_mfma_head_dim() { return D; }
 
+// Registers per lane (vector and accumulation registers together) of the decode kernel's form with `waves`
+// wavefronts and one block of 16 columns, as the runtime reports them for the compiled kernel; -1 for another form.
+// Two workgroups of four wavefronts share a compute unit only up to 256: a test holds the kernel to that, since a
+// few registers more halve its throughput for large batches.
+PLLM_API int pllm_attention_decode_registers(int waves) {
+  hipFuncAttributes attr;
+  const void* fn = waves == 4 ? reinterpret_cast<const void*>(paged_attention_mfma_kernel<1, 4>)
+                 : waves == 8 ? reinterpret_cast<const void*>(paged_attention_mfma_kernel<1, 8>) : nullptr;
+  if (!fn || hipFuncGetAttributes(&attr, fn) != hipSuccess) return -1;
+  return attr.numRegs;
+}
+
 static int num_compute_units() {
   static int cus = 0;
   if (!cus) {

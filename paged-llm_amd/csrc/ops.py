@@ -429,6 +429,11 @@ def mfma_attention_takes(dtype: torch.dtype, num_heads: int, num_kv_heads: int, 
             and block_size & (block_size - 1) == 0 and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 64)
 
 
+def attention_decode_registers(head_dim: int, waves: int) -> int:
+    """Vector registers per lane of the compiled decode attention kernel (16 columns, ``waves`` wavefronts)."""
+    return int(_fn("attention_mfma.hip", "pllm_attention_decode_registers", {"HEAD_DIM": head_dim}, [c_int])(waves))
+
+
 def _merge_lds_bytes(column_blocks: int, waves: int, head_dim: int) -> int:
     """LDS of the attention kernel's several-wavefront variant (as merge_lds_bytes in attention_mfma.hip):
     maximum and weight per column and wavefront, and every wavefront's partial output."""

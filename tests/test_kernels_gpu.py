@@ -496,6 +496,14 @@ def test_decoded_tokens_beside_prompt_portions(heads, kv_heads, d):
     assert rel_err(back, want) <= 1.6e-2
 
 
+def test_decode_attention_kernel_leaves_room_for_two_workgroups():
+    """At head size 64 the decode kernel keeps two blocks of keys and values in registers; two of its workgroups of
+    four wavefronts share a compute unit only while it takes at most 256 registers per lane, vector and accumulation
+    registers together (the plan for large batches counts on that: a version that took a few more was measured half
+    as fast in the same launch)."""
+    assert 0 < ops().attention_decode_registers(64, 4) <= 256
+
+
 def test_attention_plan():
     plan = ops().attention_plan
     lds = 160 * 1024
