@@ -1,0 +1,45 @@
+"""Launch plans are plain functions of sizes; whatever they return must be something the kernels take."""
+
+import numpy as np
+
+from paged_llm_amd.csrc import ops
+
+
+def test_attention_plan_always_returns_a_launch_the_kernels_take():
+    rng = np.random.default_rng(7)
+    lds = 160 * 1024
+    for _ in range(3000):
+        seqs = int(rng.choice([1, 2, 3, 7, 8, 16, 33, 64, 100, 256, 1000]))
+        kv_heads = int(rng.choice([1, 2, 4, 8, 16]))
+        group = int(rng.choice([1, 2, 3, 4, 5, 8, 16]))
+        max_q = int(rng.choice([1, 1, 1, 2, 3, 8, 17, 64, 500]))
+        max_k = max(max_q, int(rng.choice([1, 15, 64, 65, 200, 256, 1000, 2048, 2049, 8192, 100000])))
+        d = int(rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 256]))
+        waves, size, parts = ops.attention_plan(seqs, kv_heads, max_q, max_k, group, d, lds)
+        what = f"plan({seqs}, {kv_heads}, {max_q}, {max_k}, {group}, {d}) = {(waves, size, parts)}"
+        assert waves in (1, 4, 8), what
+        assert size % 64 == 0 and size >= 0 and parts >= 1, what
+        if size == 0:
+            assert parts == 1, what
+        else:
+            assert parts > 1 and (parts - 1) * size < max_k <= parts * size, what     # the partitions cover the keys, none is empty
+            assert kv_heads * parts <= 65535, what                                  # a grid dimension
+        if max_q * group > 64:
+            assert (waves, size, parts) == (1, 0, 1), what                          # prompt portions: the other kernel
+        if waves > 1:
+            ncb = 1 if max_q * group <= 16 else (2 if max_q * group <= 32 else 4)
+            assert ops._merge_lds_bytes(ncb, waves, d) <= lds, what
+
+
+def test_attention_plan_depends_on_sizes_only():
+    a = ops.attention_plan(8, 4, 1, 2048, 8, 64, 160 * 1024)
+    assert a == ops.attention_plan(8, 4, 1, 2048, 8, 64, 160 * 1024) == (4, 256, 8)
+
+
+def test_graph_batch_sizes_cover_every_batch_with_at_most_half_as_many_rows_again():
+    from paged_llm_amd.engine.runner import ModelRunner
+    sizes = [ModelRunner._bucket(n) for n in range(1, 600)]
+    assert all(b >= n and 2 * b <= 3 * n + 1 for n, b in zip(range(1, 600), sizes))      # never fewer rows, at most half again
+    assert sizes == sorted(sizes)
+    assert len(set(sizes)) <= 24                                                       # few graphs for a batch that shrinks one by one
+    assert [ModelRunner._bucket(n) for n in (1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 64, 65)] == [1, 2, 3, 4, 6, 6, 8, 8, 12, 16, 64, 96]
