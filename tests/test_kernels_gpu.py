@@ -334,7 +334,7 @@ def test_large_bf16_product_and_float_rows():
 
 # ----------------------------------------------------------------------------------- attention on the matrix cores
 MFMA_SHAPES = [(4, 2, 32, 16), (8, 8, 64, 16), (32, 4, 64, 16), (3, 1, 48, 32), (5, 5, 16, 16), (6, 2, 128, 64), (2, 1, 256, 16),
-               (16, 1, 80, 16), (40, 1, 64, 16)]
+               (16, 1, 80, 16), (40, 1, 64, 16), (1, 1, 112, 16), (6, 2, 112, 16), (3, 3, 96, 16)]
 
 
 @pytest.mark.parametrize("heads,kv_heads,d,bs", MFMA_SHAPES)
