@@ -43,7 +43,8 @@ def _hipcc() -> str:
 
 def _digest(source: str, defines: dict) -> str:
     h = hashlib.sha256()
-    for path in (os.path.join(CSRC, "common.h"), os.path.join(CSRC, source)):
+    headers = sorted(os.path.join(CSRC, name) for name in os.listdir(CSRC) if name.endswith(".h"))
+    for path in (*headers, os.path.join(CSRC, source)):
         with open(path, "rb") as f:
             h.update(f.read())
     h.update(repr(sorted(defines.items())).encode())
@@ -144,7 +145,7 @@ def load_library(source: str, defines: dict | None = None) -> ctypes.CDLL:
 # Sources every model needs, and the specialised ones per head size.
 COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip", "decode_linear.hip"]
 # Head sizes whose attention library a full build makes (others are compiled at first use).
-USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
+USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 
 
 def all_targets() -> list[tuple[str, dict]]:
