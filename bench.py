@@ -88,38 +88,37 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed:
     from paged_llm_amd import SamplingParams
     # Requests whose prompt is done go on decoding while the others' prompts are still computed, so some
     # are a few tokens ahead: leave room for that, so that no context passes `context` while timed.
-    budget = engine.scheduler.config.max_num_batched_tokens
+    budget = engine.config.max_num_batched_tokens
     ahead = batch * context // budget + 1
     prompt_len = context - (steps + warmup) - ahead
     assert prompt_len >= 1, "context too short for this many steps"
     sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + ahead + 40, ignore_eos=True)
     for p in random_prompts(batch, prompt_len, engine.model.spec.vocab_size, seed):
         engine.add_request(p, sp)
-    while any(not r.is_prefill_done for r in engine.scheduler.running) or engine.scheduler.waiting:
+    while any(not r.decoding for r in engine.scheduler.active) or engine.scheduler.queue:
         engine.step()
-    assert len(engine.scheduler.running) == batch
+    assert len(engine.scheduler.active) == batch
     for _ in range(warmup):
         engine.step()
     torch.cuda.synchronize()
-    before = sum(r.num_tokens for r in engine.scheduler.running)
+    before = sum(len(r.tokens) for r in engine.scheduler.active)
     t0 = time.perf_counter()
     for _ in range(steps):
         out = engine.step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     assert len(out) == batch
-    after = sum(r.num_tokens for r in engine.scheduler.running)
-    assert max(r.num_tokens for r in engine.scheduler.running) <= context + 1, "a context passed the one asked for"
-    for r in list(engine.scheduler.running):
-        engine.abort_request(r.request_id)
+    after = sum(len(r.tokens) for r in engine.scheduler.active)
+    assert max(len(r.tokens) for r in engine.scheduler.active) <= context + 1, "a context passed the one asked for"
+    for r in list(engine.scheduler.active):
+        engine.abort_request(r.id)
     return elapsed / steps, (before + after) / 2.0 / batch
 
 
 def measured_peaks() -> dict:
-    """What this GPU gives to the simplest programs, beside the published peaks: GB/s of a kernel that only
-    reads 1 GiB with every load issued early, and TFLOP/s of the library's large bfloat16 product (8192^3)."""
+    """What this GPU gives to the simplest programs, beside the published peaks: GB/s of a device-to-device copy of
+    1 GiB (bytes read plus bytes written) and TFLOP/s of the library's large bfloat16 product (8192^3)."""
     import torch
-    from paged_llm_amd.csrc import ops
     def best(fn, repeats=5):
         fn()
         torch.cuda.synchronize()
@@ -131,13 +130,14 @@ def measured_peaks() -> dict:
             times.append(a.elapsed_time(b) * 1e-3)
         return min(times)
     x = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
-    read = x.numel() * 2 / best(lambda: ops.stream_read(x)) / 1e9
-    del x
+    y = torch.empty_like(x)
+    copy = 2 * x.numel() * 2 / best(lambda: y.copy_(x)) / 1e9
+    del x, y
     n = 8192
     a = torch.randn(n, n, dtype=torch.bfloat16, device="cuda")
     b = torch.randn(n, n, dtype=torch.bfloat16, device="cuda")
     mfma = 2.0 * n ** 3 / best(lambda: torch.mm(a, b.t())) / 1e12
-    return {"hbm_read_gbs": round(read, 1), "bf16_product_tflops": round(mfma, 1)}
+    return {"hbm_copy_gbs": round(copy, 1), "bf16_product_tflops": round(mfma, 1)}
 
 
 def time_prefill(engine, tokens: int, seed: int, repeats: int = 3) -> float:
@@ -380,7 +380,7 @@ def main() -> int:
                 del engine
                 torch.cuda.empty_cache()
                 peaks = measured_peaks()
-                record["measured_peaks"] = dict(peaks, decode_frac=round(achieved / peaks["hbm_read_gbs"], 4),
+                record["measured_peaks"] = dict(peaks, decode_frac=round(achieved / peaks["hbm_copy_gbs"], 4),
                                                 prefill_frac=round(flops / psec / (peaks["bf16_product_tflops"] * 1e12), 4))
     print(json.dumps(record))
     return 0

@@ -156,8 +156,11 @@ class CacheManager:
             raise ValueError("block_size must be a power of two")
         self.groups = {g.name: g for g in groups}
         self.block_size = block_size
-        # A windowed group forgets early pages, so a cached prefix cannot be re-entered.
-        self.prefix_caching = enable_prefix_caching and all(g.kind == "full" for g in groups) and bool(groups)
+        # A windowed group forgets early pages, so a cached prefix cannot be re-entered; and a state of fixed
+        # size exists only as of the last token run, so a request that skipped a cached prefix would start
+        # from a state that never saw it.  Prefix reuse is off in both cases.
+        self.prefix_caching = (enable_prefix_caching and bool(groups) and all(g.kind == "full" for g in groups)
+                               and num_state_slots == 0)
         self.pools: dict[str, PagePool] = {}
         for g in groups:
             n = num_pages[g.name] if isinstance(num_pages, dict) else num_pages
@@ -167,6 +170,7 @@ class CacheManager:
         self._held: dict[object, _Holding] = {}
         self._versions = itertools.count(1)
         self._pending: dict[str, list[PageCopy]] = {g.name: [] for g in groups}
+        self._pending_state: list[PageCopy] = []         # state slots to copy (after a fork), as (src, dst)
         self.num_cache_queries = 0
         self.num_cache_hits = 0
 
@@ -374,6 +378,7 @@ class CacheManager:
                         if p != NO_PAGE:
                             self.pools[name].drop(p)
                 raise RuntimeError("no free state slot for a fork")
+            self._pending_state.append(PageCopy(src.state_slot, hold.state_slot))
         hold.version = next(self._versions)
         self._held[child] = hold
 
@@ -394,6 +399,12 @@ class CacheManager:
     def take_pending_copies(self) -> dict[str, list[PageCopy]]:
         out = {g: ops for g, ops in self._pending.items() if ops}
         self._pending = {g: [] for g in self.groups}
+        return out
+
+    def take_pending_state_copies(self) -> list[PageCopy]:
+        """State slots whose content the step function must copy before the next forward pass
+        (a forked request starts from its parent's state)."""
+        out, self._pending_state = self._pending_state, []
         return out
 
     # ------------------------------------------------------------------ self-check (tests)

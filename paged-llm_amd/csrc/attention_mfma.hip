@@ -820,7 +820,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
                                        int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                        const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                                        int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                       int num_partitions, float* partials, int waves, int column_blocks, int tune, const int* work_list, int num_work,
+                                       int num_partitions, float* partials, int waves, int column_blocks, const int* work_list, int num_work,
                                        hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
@@ -853,14 +853,12 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // of a SIMD's registers (head sizes above 96: two groups are then the only way to two wavefronts per SIMD,
     // measured 1.4 times faster at 128), else when there are too few workgroups to keep two of the four-wavefront
     // kind on every compute unit for most of the time (measured: faster up to about 2.5 workgroups per compute
-    // unit).  `tune` (measurements): bit 1 = one key group, bit 2 = two key groups.
+    // unit).
     constexpr bool two_fits = D <= 128 && prefill_lds_bytes(2) <= 160 * 1024;
     // (workgroups that find work: a sequence has as many tiles as its own queries need, the grid as many slots
     // as the longest)
     const long busy = work_list ? (long)num_work * num_kv_heads : ((long)total_q * G / kCols + num_seqs) * num_kv_heads;
-    bool two = two_fits && (D > 96 || 2L * busy <= 5L * num_compute_units());
-    if (tune & 2) two = false;
-    if ((tune & 4) && two_fits) two = true;
+    const bool two = two_fits && (D > 96 || 2L * busy <= 5L * num_compute_units());
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
     if ((long)lds > pllm_max_lds()) return -2;
     auto kern = paged_attention_prefill_kernel<2, 1>;
@@ -983,7 +981,7 @@ PLLM_API int pllm_paged_attention_decode_noalloc(const void* q, int q_stride, co
   if (err) return err;
   const int rc = pllm_paged_attention_mfma(q, q_stride, k_pages, v_pages, out, out_stride, block_tables, bt_stride, cu_seqlens_q,
                                            seq_lens_k, num_seqs, total_q, max_q_len, num_heads, num_kv_heads, block_size, scale, window,
-                                           partition_size, num_partitions, partials, waves, 0, 0, nullptr, 0, stream);
+                                           partition_size, num_partitions, partials, waves, 0, nullptr, 0, stream);
   if (rc == -2) {
     snprintf(noalloc_error, sizeof noalloc_error, "the attention kernels refuse this shape (pages of %d positions, %d wavefronts, %d/%d heads)",
              block_size, waves, num_heads, num_kv_heads);

@@ -628,7 +628,7 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
                                 void* x_out, int ldxo, const int* row_index, const void* W, int ldw, void* out, int ldo, int M,
                                 int N, int K, const int* positions, const float* cos_t, const float* sin_t, const int* slots,
                                 void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim, int block_size,
-                                int tune, hipStream_t stream) {
+                                hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (M > 16 && (delta || norm_w)) || K <= 0 || (K & 7) || (ldx & 7) || (ldw & 7) || (delta && (ldd & 7)) || (x_out && (ldxo & 7))) return -2;
   DecodeLinearParams p;
@@ -652,8 +652,7 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   // compute unit: two overlap one's prologue and reduction with the other's streaming, and are taken when
   // their rows fit into LDS side by side and the busiest compute unit gets no more units that way; more
   // units than workgroups are dealt evenly, and a workgroup walks its units with the next one's weights
-  // already on their way.  `tune` overrides the choice for measurements: bit 2/3 = units of 16/8 weight
-  // rows, bit 4/5 = one/two workgroups per compute unit, bit 6 = rows through LDS even without a sum or norm.
+  // already on their way.
   const int cus = num_compute_units();
   constexpr int waves = 8;
   if (M > 16) {                                                 // tiles of 16 rows side by side, one workgroup per compute unit
@@ -667,20 +666,15 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
     return -3;
   }
   // Rows that need no sum and no norm are read straight from memory (no LDS for them, any K).
-  bool direct = !delta && !norm_w;
-  if (tune & 64) direct = false;
+  const bool direct = !delta && !norm_w;
   if (!direct && (long)M * (((K >> 3) + 63) >> 6) > kSquares) return -2;
   const size_t lds = direct ? (size_t)waves * 256 * sizeof(float) : (size_t)pllm_decode_linear_lds_bytes(M, K, waves);
   auto ceil_div = [](int a, int b) { return (a + b - 1) / b; };
-  bool half = M <= 8 && epi != EPI_GATED && K >= 512 && 2 * ceil_div(2 * units, cus) <= 3 * ceil_div(units, cus);   // at most 3/4
-  if (tune & 4) half = false;
-  if (tune & 8) half = M <= 8 && epi != EPI_GATED;
+  const bool half = M <= 8 && epi != EPI_GATED && K >= 512 && 2 * ceil_div(2 * units, cus) <= 3 * ceil_div(units, cus);   // at most 3/4
   if (half) units *= 2;
   const int per_block2 = ceil_div(units, 2 * cus), blocks2 = ceil_div(units, per_block2);
   const int busiest2 = per_block2 * (blocks2 > cus ? 2 : 1), busiest1 = ceil_div(units, cus);
-  bool two = 2 * lds <= (size_t)pllm_lds_bytes_per_cu() && busiest2 <= busiest1;
-  if (tune & 16) two = false;
-  if (tune & 32) two = true;
+  const bool two = 2 * lds <= (size_t)pllm_lds_bytes_per_cu() && busiest2 <= busiest1;
   const int per_block = two ? per_block2 : busiest1;
   const int blocks = ceil_div(units, per_block);
 #define GO(EPI_, HALF_)                                                                                                   \

@@ -220,9 +220,9 @@ PLLM_API int pllm_silu_mul(int dtype, const void* gate_up, void* out, int num_to
 }
 
 // ---------------------------------------------------------------------------------------------
-// Rotary encoding of q and k (half-split pairing: element i turns with element i + d/2 by the
-// angle pos * inv_freq[i]; cos/sin come from float tables [positions, d/2]) fused with the cache
-// write.  q is rotated in place inside the fused projection buffer
+// Rotary encoding of q and k fused with the cache write.  The first rotary_dim elements of a head are
+// rotated: pair i is (i, i + rotary_dim/2) (half-split) or (2i, 2i + 1) (interleaved) and turns by the
+// angle whose cos/sin stand in column i of the float tables [positions, rotary_dim/2].  q is rotated in place inside the fused projection buffer
 //   qkv[t] = [ q heads | k heads | v heads ],  row stride `row_stride` elements.
 // Rotated k goes to k_pages [page, kv_head, offset, d]; v goes, transposed, to
 // v_pages [page, kv_head, d, offset].  slot = page * block_size + offset; slot < 0 skips the write.
@@ -231,9 +231,10 @@ template <typename T>
 __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
                                     const float* __restrict__ cos_table, const float* __restrict__ sin_table,
                                     const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                    int num_heads, int num_kv_heads, int head_dim, int block_size, int write_kv) {
+                                    int num_heads, int num_kv_heads, int head_dim, int block_size, int write_kv,
+                                    int rotary_dim, int interleaved) {
   const int t = blockIdx.x;
-  const int half = head_dim >> 1;
+  const int half = rotary_dim >> 1;                      // pairs per head, and the tables' row length
   const int pos = positions[t];
   const float* cs = cos_table ? cos_table + (size_t)pos * half : nullptr;  // no tables: no rotation
   const float* sn = sin_table ? sin_table + (size_t)pos * half : nullptr;
@@ -244,7 +245,8 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
 
   const int rot_heads = write_kv ? num_heads + num_kv_heads : num_heads;
   struct alignas(16) Piece { T v[8]; };
-  const bool wide = (half % 8 == 0) && ((uintptr_t)qkv % 16) == 0 && (row_stride % 8 == 0) && ((uintptr_t)k_pages % 16) == 0;
+  const bool wide = rotary_dim == head_dim && !interleaved && (half % 8 == 0) && ((uintptr_t)qkv % 16) == 0 &&
+                    (row_stride % 8 == 0) && ((uintptr_t)k_pages % 16) == 0;
   if (wide) {
     // 8 pairs per work item: 16-byte pieces of the lower and the upper half of a head
     const int per_head = half / 8;
@@ -269,21 +271,31 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
       }
     }
   } else {
+    // Any rotary width and either pairing: pair i of a head is (i, i + half) or, interleaved, (2i, 2i + 1);
+    // elements from rotary_dim on are not rotated (of k they are copied to the page as they are).
     for (int w = threadIdx.x; w < rot_heads * half; w += blockDim.x) {
       const int head = w / half, i = w - head * half;
+      const int a = interleaved ? 2 * i : i, b = interleaved ? 2 * i + 1 : i + half;
       T* h = row + (size_t)head * head_dim;
-      const float lo = to_f32(h[i]), hi = to_f32(h[i + half]);
+      const float lo = to_f32(h[a]), hi = to_f32(h[b]);
       const float c = cs ? cs[i] : 1.f, s = sn ? sn[i] : 0.f;
       const T out_lo = from_f32<T>(lo * c - hi * s);
       const T out_hi = from_f32<T>(hi * c + lo * s);
       if (head < num_heads) {
-        h[i] = out_lo;
-        h[i + half] = out_hi;
+        h[a] = out_lo;
+        h[b] = out_hi;
       } else if (slot >= 0) {
         const int kvh = head - num_heads;
         T* dst = k_pages + (((size_t)page * num_kv_heads + kvh) * block_size + off) * head_dim;
-        dst[i] = out_lo;
-        dst[i + half] = out_hi;
+        dst[a] = out_lo;
+        dst[b] = out_hi;
+      }
+    }
+    const int tail = head_dim - rotary_dim;
+    if (tail > 0 && slot >= 0) {
+      for (int w = threadIdx.x; w < num_kv_heads * tail; w += blockDim.x) {
+        const int kvh = w / tail, i = rotary_dim + (w - kvh * tail);
+        k_pages[(((size_t)page * num_kv_heads + kvh) * block_size + off) * head_dim + i] = row[(size_t)(num_heads + kvh) * head_dim + i];
       }
     }
   }
@@ -296,20 +308,23 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
   }
 }
 
+// rotary_dim: how many leading elements of a head are rotated (even, at most head_dim; the tables hold
+// rotary_dim / 2 columns); interleaved: pairs are (2i, 2i + 1) instead of (i, i + rotary_dim / 2).
 PLLM_API int pllm_rope_scatter(int dtype, void* qkv, int row_stride, const int* positions, const float* cos_table,
                                const float* sin_table, const int* slot_mapping, void* k_pages, void* v_pages,
                                int num_tokens, int num_heads, int num_kv_heads, int head_dim, int block_size,
-                               int write_kv, hipStream_t stream) {
+                               int write_kv, int rotary_dim, int interleaved, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
+  if (rotary_dim < 0 || rotary_dim > head_dim || (rotary_dim & 1)) return -2;
   dim3 grid(num_tokens), block(256);
   if (dtype == PLLM_F32)
     hipLaunchKernelGGL(rope_scatter_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, positions, cos_table,
                        sin_table, slot_mapping, (float*)k_pages, (float*)v_pages, num_heads, num_kv_heads, head_dim,
-                       block_size, write_kv);
+                       block_size, write_kv, rotary_dim, interleaved);
   else
     hipLaunchKernelGGL(rope_scatter_kernel<bf16>, grid, block, 0, stream, (bf16*)qkv, row_stride, positions, cos_table,
                        sin_table, slot_mapping, (bf16*)k_pages, (bf16*)v_pages, num_heads, num_kv_heads, head_dim,
-                       block_size, write_kv);
+                       block_size, write_kv, rotary_dim, interleaved);
   PLLM_RETURN_LAST_ERROR();
 }
 
@@ -333,29 +348,5 @@ PLLM_API int pllm_copy_pages(int dtype, void* pages, const int* src, const int* 
     hipLaunchKernelGGL(copy_pages_kernel<float>, grid, block, 0, stream, (float*)pages, src, dst, (size_t)page_elems);
   else
     hipLaunchKernelGGL(copy_pages_kernel<bf16>, grid, block, 0, stream, (bf16*)pages, src, dst, (size_t)page_elems);
-  PLLM_RETURN_LAST_ERROR();
-}
-
-// ---------------------------------------------------------------------------------------------
-// Measurement only: read `bytes` (a multiple of 16) with 16-byte loads, eight under way per thread, and
-// write nothing (the store's condition never holds).  Its time is what streaming a buffer costs here.
-__global__ __launch_bounds__(256) void stream_read_kernel(const float4* __restrict__ src, size_t pieces, float* __restrict__ out) {
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  float s = 0.f;
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + 7 * stride < pieces; i += 8 * stride) {
-    float4 v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = src[i + u * stride];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) s += v[u].x + v[u].y + v[u].z + v[u].w;
-  }
-  for (; i < pieces; i += stride) s += src[i].x;
-  if (s == 12345.678f) out[0] = s;
-}
-
-PLLM_API int pllm_stream_read(const void* src, long bytes, float* out, int blocks, hipStream_t stream) {
-  if (bytes <= 0 || (bytes & 15) || blocks <= 0) return -2;
-  hipLaunchKernelGGL(stream_read_kernel, dim3(blocks), dim3(256), 0, stream, (const float4*)src, (size_t)bytes / 16, out);
   PLLM_RETURN_LAST_ERROR();
 }

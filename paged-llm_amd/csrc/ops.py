@@ -68,7 +68,7 @@ _SIGNATURES = {
     "pllm_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "pllm_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "pllm_rope_scatter": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "pllm_copy_pages": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p],
     "pllm_gemm_nt": [c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "pllm_paged_attention_generic": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
@@ -151,12 +151,15 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
 
 def rope_scatter(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                  num_heads: int, num_kv_heads: int, head_dim: int, slot_mapping: torch.Tensor | None,
-                 k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, block_size: int) -> None:
+                 k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, block_size: int,
+                 rotary_dim: int | None = None, interleaved: bool = False) -> None:
     """Rotate q (in place) and k by the tables' angles at ``positions``; write k and v into pages.
 
     qkv: [T, >= (num_heads + 2 kv_heads) * d] rows (only q columns are needed when nothing is
-    written).  k_pages [P, kv, bs, d], v_pages [P, kv, d, bs].  The caller guarantees
-    positions < cos.shape[0] and slots < P * bs (checked on the host where the batch is built).
+    written).  k_pages [P, kv, bs, d], v_pages [P, kv, d, bs].  ``rotary_dim`` (default: the whole
+    head) is how many leading elements of a head turn; ``interleaved`` pairs (2i, 2i + 1) instead of
+    (i, i + rotary_dim / 2).  The caller guarantees positions < cos.shape[0] and slots < P * bs
+    (checked on the host where the batch is built).
     """
     write_kv = k_pages is not None
     _on_gpu(qkv, positions, cos, sin, slot_mapping, k_pages, v_pages)
@@ -164,9 +167,11 @@ def rope_scatter(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, 
     _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be [T, width] with unit inner stride")
     need_cols = (num_heads + (2 * num_kv_heads if write_kv else 0)) * head_dim
     _need(qkv.shape[1] >= need_cols, f"qkv rows hold {qkv.shape[1]} values, need {need_cols}")
-    _need(head_dim % 2 == 0, "rotary pairing needs an even head size")
+    rotary_dim = head_dim if rotary_dim is None else int(rotary_dim)
+    _need(0 <= rotary_dim <= head_dim and rotary_dim % 2 == 0,
+          f"rotary pairing needs an even width of at most the head size {head_dim}, got {rotary_dim}")
     _need(positions.dtype == torch.int32 and positions.shape == (T,) and positions.is_contiguous(), "positions: int32 [T]")
-    half = head_dim // 2
+    half = rotary_dim // 2
     _need((cos is None) == (sin is None), "cos and sin tables come together")
     for t in (cos, sin):
         if t is None:
@@ -183,8 +188,8 @@ def rope_scatter(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, 
               and v_pages.dtype == qkv.dtype, "v_pages must be contiguous [pages, kv_heads, head_dim, block_size]")
     _check(_fn("elementwise.hip", "pllm_rope_scatter")(
         dtype_code(qkv.dtype), _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
-        _ptr(k_pages), _ptr(v_pages), T, num_heads, num_kv_heads, head_dim, block_size, 1 if write_kv else 0, _stream()),
-        "rope_scatter")
+        _ptr(k_pages), _ptr(v_pages), T, num_heads, num_kv_heads, head_dim, block_size, 1 if write_kv else 0,
+        rotary_dim, 1 if interleaved else 0, _stream()), "rope_scatter")
 
 
 def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
@@ -278,28 +283,13 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     return out
 
 
-def stream_read(buffer: torch.Tensor, blocks: int = 2048) -> None:
-    """Measurement only: read all of ``buffer`` once (what streaming that many bytes costs on this GPU)."""
-    _on_gpu(buffer)
-    nbytes = buffer.numel() * buffer.element_size()
-    _need(buffer.is_contiguous() and nbytes % 16 == 0 and buffer.data_ptr() % 16 == 0, "stream_read takes whole 16-byte pieces")
-    sink = _stream_sink.get(str(buffer.device))
-    if sink is None:
-        sink = _stream_sink[str(buffer.device)] = torch.zeros(1, dtype=torch.float32, device=buffer.device)
-    f = _fn("elementwise.hip", "pllm_stream_read", signature=[c_void_p, c_long, c_void_p, c_int, c_void_p])
-    _check(f(_ptr(buffer), nbytes, _ptr(sink), int(blocks), _stream()), "stream_read")
-
-
-_stream_sink: dict = {}
-
-
 # ------------------------------------------------------------------------------------------- fused decode products
 EPI_BF16, EPI_F32, EPI_GATED, EPI_ROPE_KV = 0, 1, 2, 3
 DECODE_MAX_ROWS = 16          # rows of the fused form with a sum or norm in front
 DECODE_WIDE_MAX_ROWS = 64     # rows of the form for plain rows
 _DECODE_SIG = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
                c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-               c_int, c_void_p]
+               c_void_p]
 _lds_limit: dict = {}
 
 
@@ -345,20 +335,19 @@ def decode_linear_pays(rows: int, N: int, K: int, epi: int, staged: bool) -> boo
 
 def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: torch.Tensor | None = None,
                   norm_weight: torch.Tensor | None = None, eps: float = 0.0, x_out: torch.Tensor | None = None,
-                  row_index: torch.Tensor | None = None, rope: dict | None = None, tune: int = 0) -> torch.Tensor:
+                  row_index: torch.Tensor | None = None, rope: dict | None = None) -> torch.Tensor:
     """rows = x[row_index] (+ delta) -> optional RMS norm -> rows W^T -> epilogue, in one kernel.
 
     epi EPI_BF16 / EPI_F32: [M, N] out.  EPI_GATED: w = [gate; up], out = silu(gate) * up [M, N/2].
     EPI_ROPE_KV: w = [q; k; v] rows; q is rotated and returned [M, heads * d]; k (rotated) and v go
     into the cache pages; ``rope`` = dict(positions, cos, sin, slots, k_pages, v_pages, num_heads,
     num_kv_heads, head_dim, block_size).  ``x_out`` receives x + delta (the new residual).
-    ``tune`` (measurements only) overrides the kernel's choice of work shape.
     """
     _on_gpu(x, w, delta, norm_weight, x_out, row_index)
     M = row_index.numel() if row_index is not None else x.shape[0]
     K = x.shape[1]
     _need(x.dim() == 2 and w.dim() == 2 and w.shape[1] == K, f"decode_linear shapes {tuple(x.shape)} x {tuple(w.shape)}^T")
-    staged = delta is not None or norm_weight is not None or bool(tune & 64)
+    staged = delta is not None or norm_weight is not None
     _need(decode_linear_takes(M, K, x, w, staged),
           "decode_linear takes bfloat16, K a multiple of 8, 1..64 plain rows, or with a sum or norm in front 1..16 rows that fit LDS")
     if delta is not None:
@@ -398,7 +387,7 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
              _ptr(x_out), x_out.stride(0) if x_out is not None else 0, _ptr(row_index), _ptr(w), w.stride(0), _ptr(out),
              out.stride(0), M, N, K, _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")),
              _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)),
-             int(r.get("head_dim", 0)), int(r.get("block_size", 0)), int(tune), _stream()), "decode_linear")
+             int(r.get("head_dim", 0)), int(r.get("block_size", 0)), _stream()), "decode_linear")
     return out
 
 
@@ -418,7 +407,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = 
 
 
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
+             c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]
 _attn_scratch: dict = {}
 _attn_scratch_retired: list = []      # outgrown buffers stay allocated: captured graphs still hold their addresses
 _attn_checked: set = set()
@@ -480,7 +469,7 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
                          cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
                          head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
-                         num_partitions: int = 1, waves: int = 1, column_blocks: int = 0, tune: int = 0,
+                         num_partitions: int = 1, waves: int = 1, column_blocks: int = 0,
                          out: torch.Tensor | None = None, work_list: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
@@ -524,7 +513,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
     _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
              block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
-             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), int(tune), _ptr(work_list),
+             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), _ptr(work_list),
              0 if work_list is None else work_list.shape[0], _stream()),
            "paged_attention_mfma")
     return out

@@ -1,6 +1,5 @@
 from .batch import StepContext, StepEntry
-from .request import Request, RequestStatus, SamplingParams
-from .scheduler import ScheduledRequest, Scheduler, SchedulerOutput
+from .request import EndReason, Request, SamplingParams, Stage
+from .scheduler import Grant, Scheduler, StepPlan
 
-__all__ = ["StepContext", "StepEntry", "Request", "RequestStatus", "SamplingParams", "ScheduledRequest", "Scheduler",
-           "SchedulerOutput"]
+__all__ = ["StepContext", "StepEntry", "Request", "Stage", "EndReason", "SamplingParams", "Grant", "Scheduler", "StepPlan"]

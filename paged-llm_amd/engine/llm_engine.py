@@ -1,4 +1,10 @@
-"""LLMEngine: scheduler + step function + sampler in one loop (pagedllm/engine.py:105-234)."""
+"""LLMEngine: the entry point.  A model folder in, generated tokens out.
+
+The public face is the reference's (pagedllm/engine.py:105-234): ``LLMEngine(model, config, **overrides)``,
+``generate``, ``add_request``, ``step``, ``abort_request``, ``has_unfinished_requests``, ``stats``, and the
+fields of ``RequestOutput`` / ``StepOutput`` / ``EngineStats``.  Behind it one step is: the scheduler's plan
+-> entries for the step function -> logits of the rows to sample from -> the sampler -> the plan committed.
+"""
 
 from __future__ import annotations
 
@@ -7,15 +13,14 @@ import os
 import time
 from dataclasses import dataclass, field
 
-import torch
-
 from ..config.engine_config import EngineConfig
 from ..config.registry import read_config_json
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
 from .loading import build_model, build_runtime, load_model, require_gpu
-from .request import Request, RequestStatus, SamplingParams
-from .scheduler import Scheduler, SchedulerOutput
+from .pool_sizing import pages_that_fit
+from .request import Request, SamplingParams
+from .scheduler import Scheduler, StepPlan
 
 log = logging.getLogger("paged_llm_amd")
 
@@ -46,14 +51,21 @@ class EngineStats:
     num_preemptions: int = 0
     step_times: list = field(default_factory=list)
 
+    def count(self, plan: StepPlan, seconds: float) -> None:
+        self.num_steps += 1
+        self.num_prefill_tokens += plan.prompt_tokens
+        self.num_decode_tokens += plan.decode_tokens
+        self.num_preemptions += len(plan.preempted)
+        self.step_times.append(seconds)
 
-def _load_tokenizer(path: str):
-    """tokenizer.json of the model folder, if there is one; token-id prompts need none."""
-    file = os.path.join(path, "tokenizer.json")
-    if not os.path.isfile(file):
+
+def _tokenizer_of(folder: str):
+    """The folder's tokenizer.json, if it has one; prompts given as token ids need none."""
+    path = os.path.join(folder, "tokenizer.json")
+    if not os.path.isfile(path):
         return None
     from tokenizers import Tokenizer
-    return Tokenizer.from_file(file)
+    return Tokenizer.from_file(path)
 
 
 class LLMEngine:
@@ -61,160 +73,138 @@ class LLMEngine:
         """``model``: a folder with config.json and *.safetensors.  ``random_weights=SEED`` among
         the overrides fills the model of that folder's config.json with seeded random weights
         instead of reading tensors."""
-        random_seed = overrides.pop("random_weights", None)
+        seed_for_weights = overrides.pop("random_weights", None)
         self.config = cfg = config or EngineConfig(**overrides)
         self.device = require_gpu(cfg.device)
         if not os.path.isdir(model):
             raise FileNotFoundError(f"{model!r} is no folder (models are not downloaded)")
-        hf_cfg = read_config_json(model)
-        self.tokenizer = _load_tokenizer(model)
-        t0 = time.perf_counter()
-        if random_seed is None:
+        self.tokenizer = _tokenizer_of(model)
+        started = time.perf_counter()
+        if seed_for_weights is None:
             self.model = load_model(model, cfg.dtype, self.device, cfg.max_model_len)
         else:
             from ..weights.random_init import fill_random
-            self.model = build_model(hf_cfg, cfg.dtype, self.device, cfg.max_model_len)
-            fill_random(self.model, int(random_seed))
+            self.model = build_model(read_config_json(model), cfg.dtype, self.device, cfg.max_model_len)
+            fill_random(self.model, int(seed_for_weights))
         self.dtype = self.model.dtype
-        # What runs the attention (the reference reports its backend's name here, pagedllm/engine.py:117-118).
-        self.attention_backend = "hip"
-        log.info("loaded %s in %.1fs (dtype=%s)", model, time.perf_counter() - t0, self.dtype)
+        self.attention_backend = "hip"       # the one there is; shown where the reference shows its backend's name
+        log.info("model %s ready after %.1f s, computing in %s", model, time.perf_counter() - started, self.dtype)
 
-        num_pages = cfg.num_gpu_blocks or self._profile_num_pages()
+        pages = cfg.num_gpu_blocks or pages_that_fit(self.model, cfg)
         self.cache_manager, self.kv_cache, self.runner = build_runtime(
-            self.model, cfg.block_size, num_pages, cfg.max_num_seqs, cfg.enable_prefix_caching,
-            use_graphs=cfg.enable_hip_graphs)
+            self.model, cfg.block_size, pages, cfg.max_num_seqs, cfg.enable_prefix_caching, use_graphs=cfg.enable_hip_graphs)
         self.groups = list(self.cache_manager.groups)
-        eos = self.model.spec.eos_token_id
-        self.scheduler = Scheduler(cfg, self.cache_manager, eos)
+        self.scheduler = Scheduler(cfg, self.cache_manager, self.model.spec.eos_token_id)
         self.sampler = Sampler(cfg.seed, self.device)
         self.stats = EngineStats()
-        self._requests: dict[int, Request] = {}
-        log.info("KV cache: %d pages x %d tokens = %d tokens (%.2f GiB)", num_pages, cfg.block_size,
-                 num_pages * cfg.block_size, self.kv_cache.total_bytes() / 2**30)
-
-    # ------------------------------------------------------------------ sizing the page pool
-    def _bytes_per_page(self) -> int:
-        return sum(g.bytes_per_page(self.config.block_size, self.model.dtype) for g in self.model.cache_groups().values())
-
-    def _dummy_forward(self, n_tok: int) -> None:
-        """One forward of n_tok tokens against a throw-away cache, to measure the activation peak
-        (pagedllm/engine.py:141-159).  Positions stay inside the model's range."""
-        cfg = self.config
-        n_tok = min(n_tok, self.model.max_positions)
-        pages = (n_tok + cfg.block_size - 1) // cfg.block_size
-        manager, storage, runner = build_runtime(self.model, cfg.block_size, pages, 1, False)
-        assert manager.allocate("probe", 0, n_tok)
-        entry = StepEntry("probe", [0] * n_tok, 0, {g: manager.block_table("probe", g) for g in manager.groups},
-                          manager.state_slot("probe"), list(range(min(n_tok, cfg.max_num_seqs))))
-        runner.step([entry])
-        torch.cuda.synchronize(self.device)
-
-    def _profile_num_pages(self) -> int:
-        cfg = self.config
-        torch.cuda.empty_cache()
-        torch.cuda.reset_peak_memory_stats(self.device)
-        before = torch.cuda.memory_allocated(self.device)
-        self._dummy_forward(cfg.max_num_batched_tokens)
-        peak = torch.cuda.max_memory_allocated(self.device)
-        torch.cuda.empty_cache()
-        free, total = torch.cuda.mem_get_info(self.device)
-        held = torch.cuda.memory_allocated(self.device)
-        used_by_others = total - free - held
-        activation = max(0, peak - before)
-        budget = int(total * cfg.gpu_memory_utilization) - used_by_others - held - activation
-        pages = budget // max(1, self._bytes_per_page())
-        # No request can use more than max_model_len positions; cap what max_num_seqs could ever hold.
-        pages = min(pages, cfg.max_num_seqs * ((cfg.max_model_len + cfg.block_size - 1) // cfg.block_size))
-        if pages < 16:
-            raise RuntimeError(f"not enough GPU memory for the KV cache ({pages} pages); lower "
-                               "max_num_batched_tokens or raise gpu_memory_utilization")
-        return int(pages)
+        self._live: dict[int, Request] = {}          # requests that have not ended
+        # Called, if set, before every sampling with (requests, logits): the requests whose next token is about
+        # to be drawn, in the order of the float logits' rows [n, vocab]; row i is the distribution behind
+        # position len(requests[i].tokens) - 1.  The tensor is only valid during the call.
+        self.on_logits = None
+        log.info("cache: %d pages of %d positions per group (%d positions, %.2f GiB)", pages, cfg.block_size,
+                 pages * cfg.block_size, self.kv_cache.total_bytes() / 2**30)
 
     # ------------------------------------------------------------------ requests
-    def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> int:
+    def _token_ids(self, prompt) -> list:
         if isinstance(prompt, str):
             if self.tokenizer is None:
                 raise ValueError("text prompts need a tokenizer.json in the model folder; pass token ids instead")
-            ids = self.tokenizer.encode(prompt).ids
-        else:
-            ids = [int(t) for t in prompt]
+            return self.tokenizer.encode(prompt).ids
+        ids = [int(t) for t in prompt]
         vocab = self.model.spec.vocab_size
-        if any(t < 0 or t >= vocab for t in ids):
+        if any(not 0 <= t < vocab for t in ids):
             raise ValueError(f"prompt holds a token id outside [0, {vocab})")
-        req = Request(ids, sampling_params or SamplingParams())
-        self.scheduler.add(req)
-        self._requests[req.request_id] = req
-        return req.request_id
+        return ids
+
+    def _new_request(self, prompt, sampling_params: SamplingParams | None) -> Request:
+        request = Request(self._token_ids(prompt), sampling_params)
+        self.scheduler.submit(request)
+        self._live[request.id] = request
+        return request
+
+    def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> int:
+        return self._new_request(prompt, sampling_params).id
 
     def abort_request(self, seq_id: int) -> None:
-        self.scheduler.abort(seq_id)
+        if self.scheduler.cancel(seq_id) is not None:
+            self._live.pop(seq_id, None)
 
     @property
     def has_unfinished_requests(self) -> bool:
-        return self.scheduler.has_unfinished
+        return not self.scheduler.idle
 
     # ------------------------------------------------------------------ one step
-    def _run(self, out: SchedulerOutput) -> dict:
-        entries, sampled_items = [], []
-        for item in out.scheduled:
-            req, n = item.request, item.num_new_tokens
-            start = req.num_computed_tokens
-            entries.append(StepEntry(
-                req.request_id, req.token_ids[start:start + n], start,
-                {g: self.cache_manager.block_table(req.request_id, g) for g in self.groups},
-                self.cache_manager.state_slot(req.request_id), [n - 1] if item.needs_sampling else [],
-                self.cache_manager.table_version(req.request_id)))
-            if item.needs_sampling:
-                sampled_items.append(req)
-        logits = self.runner.step(entries, self.cache_manager.take_pending_copies(), borrow=True)    # sampled from at once
-        if not sampled_items:
+    def _entry(self, grant) -> StepEntry:
+        request, cm = grant.request, self.cache_manager
+        first = request.computed
+        return StepEntry(request.id, request.tokens[first:first + grant.count], first,
+                         {g: cm.block_table(request.id, g) for g in self.groups}, cm.state_slot(request.id),
+                         [grant.count - 1] if grant.samples else [], cm.table_version(request.id))
+
+    def _sample(self, logits, grants: list) -> dict:
+        """request id -> token, for the grants whose last row was asked for (in the order of the rows)."""
+        chosen = [g.request for g in grants if g.samples]
+        if not chosen:
             return {}
-        tokens = self.sampler.sample(logits, [r.sampling_params for r in sampled_items],
-                                     [r.request_id for r in sampled_items],
-                                     [r.num_generated_tokens for r in sampled_items])
-        return {r.request_id: t for r, t in zip(sampled_items, tokens)}
+        if self.on_logits is not None:
+            self.on_logits(chosen, logits[: len(chosen)])
+        tokens = self.sampler.sample(logits, [r.params for r in chosen], [r.id for r in chosen], [r.num_generated for r in chosen])
+        return {r.id: t for r, t in zip(chosen, tokens)}
+
+    def _advance(self):
+        """Runs one step.  (plan, sampled tokens by request id, requests that ended); the plan is empty
+        when there is nothing to do."""
+        started = time.perf_counter()
+        plan = self.scheduler.plan()
+        if not plan:
+            if not self.scheduler.idle:
+                raise RuntimeError("no request can run: " + self.scheduler.why_stuck())
+            return plan, {}, []
+        cm = self.cache_manager
+        state_copies = cm.take_pending_state_copies() if cm.uses_state else None
+        # The sampler runs at once, so the step may hand out its graph's own logits buffer.
+        logits = self.runner.step([self._entry(g) for g in plan.grants], cm.take_pending_copies(), borrow=True,
+                                  state_copies=state_copies)
+        sampled = self._sample(logits, plan.grants)
+        ended = self.scheduler.commit(plan, sampled)
+        for request in ended:
+            self._live.pop(request.id, None)
+        self.stats.count(plan, time.perf_counter() - started)
+        return plan, sampled, ended
 
     def step(self) -> list:
-        t0 = time.perf_counter()
-        out = self.scheduler.schedule()
-        if out.is_empty:
-            if self.scheduler.has_unfinished:
-                raise RuntimeError("nothing can be scheduled: the page pool is too small for the oldest request")
-            return []
-        sampled = self._run(out)
-        finished = {r.request_id for r in self.scheduler.update(out, sampled)}
-        st = self.stats
-        st.num_steps += 1
-        st.num_prefill_tokens += out.num_prefill_tokens
-        st.num_decode_tokens += out.num_decode_tokens
-        st.num_preemptions += len(out.preempted)
-        st.step_times.append(time.perf_counter() - t0)
-        return [StepOutput(i.request.request_id, sampled.get(i.request.request_id), i.request.request_id in finished)
-                for i in out.scheduled]
+        plan, sampled, ended = self._advance()
+        done = {r.id for r in ended}
+        return [StepOutput(g.request.id, sampled.get(g.request.id), g.request.id in done) for g in plan.grants]
 
-    def _to_output(self, req: Request) -> RequestOutput:
-        reason = {RequestStatus.FINISHED_STOPPED: "stop", RequestStatus.FINISHED_LENGTH: "length",
-                  RequestStatus.FINISHED_ABORTED: "abort"}[req.status]
-        text = ""
-        if self.tokenizer is not None:
-            text = self.tokenizer.decode(req.output_token_ids, skip_special_tokens=True)
-        return RequestOutput(req.request_id, req.prompt_token_ids, req.output_token_ids, text, reason,
-                             req.num_cached_tokens, req.num_preemptions)
+    # ------------------------------------------------------------------ whole requests
+    def _output(self, request: Request) -> RequestOutput:
+        generated = request.generated
+        text = self.tokenizer.decode(generated, skip_special_tokens=True) if self.tokenizer is not None else ""
+        return RequestOutput(request.id, request.prompt, generated, text, request.end_reason.value, request.reused_prefix,
+                             request.times_preempted)
 
     def generate(self, prompts: list, sampling_params=None, use_tqdm: bool = False) -> list:
-        """Outputs in the order of the prompts (pagedllm/engine.py:219-234)."""
-        if not isinstance(sampling_params, list):
-            sampling_params = [sampling_params or SamplingParams()] * len(prompts)
-        ids = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
-        bar = None
+        """Runs the prompts to their ends; outputs in the order of the prompts."""
+        if isinstance(sampling_params, list):
+            if len(sampling_params) != len(prompts):
+                raise ValueError(f"{len(sampling_params)} sampling_params for {len(prompts)} prompts")
+            per_prompt = sampling_params
+        else:
+            per_prompt = [sampling_params or SamplingParams()] * len(prompts)
+        mine = [self._new_request(p, sp) for p, sp in zip(prompts, per_prompt)]
+        waiting_for = {r.id for r in mine}
+        progress = None
         if use_tqdm:
             from tqdm import tqdm
-            bar = tqdm(total=len(ids), desc="requests")
-        while self.has_unfinished_requests:
-            for o in self.step():
-                if o.finished and bar:
-                    bar.update(1)
-        if bar:
-            bar.close()
-        return [self._to_output(self._requests.pop(i)) for i in ids]
+            progress = tqdm(total=len(mine), desc="requests")
+        while waiting_for:
+            _, _, ended = self._advance()
+            mine_ended = sum(1 for r in ended if r.id in waiting_for)
+            waiting_for.difference_update(r.id for r in ended)
+            if progress is not None and mine_ended:
+                progress.update(mine_ended)
+        if progress is not None:
+            progress.close()
+        return [self._output(r) for r in mine]

@@ -18,16 +18,19 @@ import numpy as np
 from .batch import StepEntry
 from .loading import build_runtime, load_model
 
-REPLAY_BLOCK_SIZE = 16
+DEFAULT_BLOCK_SIZE = 16
 MAX_LIVE_REQUESTS = 16
 
 
 class ReplaySession:
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, out_dir: str | None, device="cuda"):
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, out_dir: str | None, device="cuda",
+                 block_size: int = DEFAULT_BLOCK_SIZE):
         # A request may hold up to max_tokens positions: the position tables reach that far even where the
         # configuration names fewer (as max(max_position_embeddings, max_model_len) in pagedllm/model/loader.py:42-44).
         self.model = load_model(model_dir, dtype, device, max_model_len=max_tokens)
-        bs = REPLAY_BLOCK_SIZE
+        bs = int(block_size)
+        if bs <= 0 or bs & (bs - 1):
+            raise ValueError(f"block size must be a power of two, got {block_size}")
         num_pages = max(1, (max_tokens + bs - 1) // bs)
         self.manager, self.storage, self.runner = build_runtime(
             self.model, bs, num_pages, MAX_LIVE_REQUESTS, enable_prefix_caching=False, use_graphs=True)
@@ -71,8 +74,9 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True, help="tokens the cache pool is made for")
+    ap.add_argument("--block-size", type=int, default=DEFAULT_BLOCK_SIZE, help="positions per cache page (a power of two)")
     args = ap.parse_args(argv)
-    session = ReplaySession(args.model, args.dtype, args.max_tokens, args.out)
+    session = ReplaySession(args.model, args.dtype, args.max_tokens, args.out, block_size=args.block_size)
     for line in sys.stdin:
         line = line.strip()
         if not line:

@@ -34,9 +34,12 @@ class ModelRunner:
         self.device = model.device
         self.block_size = kv_storage.block_size
         self.group_specs = {name: g.spec for name, g in kv_storage.groups.items()}
-        # Fixed-size per-request state: one tensor [slots, *shape] per schedule step that has any.
-        self.states = {pos: torch.zeros((max(num_state_slots, 1), *ss.shape), dtype=ss.dtype, device=self.device)
+        # Fixed-size per-request state: one tensor [slots + 1, *shape] per schedule step that has any.  The
+        # last slot belongs to no request: the empty rows that pad a replayed batch point at it, so that a
+        # mixer may update "their" state without touching anybody's.
+        self.states = {pos: torch.zeros((num_state_slots + 1, *ss.shape), dtype=ss.dtype, device=self.device)
                        for pos, ss in model.state_specs().items()}
+        self.spare_state_slot = num_state_slots if self.states else -1
 
     # ------------------------------------------------------------------ batch -> device tensors
     def _stage(self, entries: list, fixed_blocks: int | None = None):
@@ -176,7 +179,7 @@ class ModelRunner:
         number of rows, of wanted rows, and a bound on the context length.  Rows and wanted rows are
         rounded up to a few sizes, so that a batch that shrinks by one request at a time does not
         capture a graph per size; the extra rows are empty requests that read one key, write nothing
-        and whose logits nobody sees (only for models without per-request state)."""
+        and whose logits nobody sees (their state slot, if the model keeps state, is the spare one)."""
         if not self.use_graphs or len(entries) > self.max_graph_batch:
             return None
         if any(len(e.tokens) != 1 for e in entries):
@@ -184,11 +187,9 @@ class ModelRunner:
         longest = max(e.start + 1 for e in entries)
         bound = ((longest + 511) // 512) * 512 if longest <= 8192 else 1 << (longest - 1).bit_length()
         bound = min(bound, max(self.model.max_positions, longest))
-        rows, wanted = len(entries), sum(len(e.want) for e in entries)
-        if not self.states:
-            rows = self._bucket(rows)
-            wanted = min(self._bucket(wanted), rows) if wanted else 0
-            wanted = max(wanted, sum(len(e.want) for e in entries))
+        asked = sum(len(e.want) for e in entries)
+        rows = self._bucket(len(entries))
+        wanted = max(min(self._bucket(asked), rows), asked) if asked else 0
         return (rows, wanted, bound)
 
     def _decode_layout(self, S: int, n_want: int, fixed: int):
@@ -213,16 +214,24 @@ class ModelRunner:
         if pinned is None:
             pinned = torch.zeros(max(total, 1), dtype=torch.int32, pin_memory=on_gpu)
         view = pinned.numpy()
+        view[:] = 0                                               # token 0 at position 0, page 0, logits of row 0
         view[offsets[2]: offsets[2] + S + 1] = np.arange(S + 1)
+        view[offsets[3]: offsets[3] + S] = 1                      # one key
+        view[offsets[4]: offsets[4] + S] = self.spare_state_slot
+        for gi in range(len(self.group_specs)):
+            view[offsets[8 + 2 * gi]: offsets[8 + 2 * gi] + S] = -1   # no slot to write to
         return dict(key=key, pinned=pinned, view=view, offsets=offsets, sizes=sizes, table_shapes=table_shapes,
-                    static=torch.zeros(max(total, 1), dtype=torch.int32, device=self.device), staged_rows=[None] * S,
-                    table_lens={name: [0] * S for name in self.group_specs}, last_page={name: [None] * S for name in self.group_specs},
+                    static=torch.zeros(max(total, 1), dtype=torch.int32, device=self.device), staged_rows=["empty"] * S,
+                    table_lens={name: [1] * S for name in self.group_specs}, last_page={name: [None] * S for name in self.group_specs},
                     copied=torch.cuda.Event() if on_gpu else None)
 
     def _capture(self, entry: dict) -> None:
+        """Warm-up and capture on the all-empty batch the entry was made with: no page is written and the only
+        state that moves is the spare slot's, so a step that is captured and then replayed runs its rows once."""
         S, n_want, bound = entry["key"]
         entry["static"].copy_(entry["pinned"])
-        host = dict(T=S, S=S, q_lens=[1] * S, k_lens=[bound] * S, slots_state=[-1] * S, table_shapes=entry["table_shapes"])
+        host = dict(T=S, S=S, q_lens=[1] * S, k_lens=[bound] * S, slots_state=[self.spare_state_slot] * S,
+                    table_shapes=entry["table_shapes"])
         ctx = self._context(entry["static"], entry["offsets"], entry["sizes"], host, max_k_len=bound, capturing=True)
         stream = torch.cuda.Stream(device=self.device)
         stream.wait_stream(torch.cuda.current_stream(self.device))
@@ -280,7 +289,7 @@ class ModelRunner:
 
         starts_padded = starts + [0] * pad
         put(0, ids + [0] * pad); put(1, starts_padded); put(3, [k + 1 for k in starts] + [1] * pad)
-        put(4, slots_state + [-1] * pad); put(5, starts_padded); put(6, logits_idx)
+        put(4, slots_state + [self.spare_state_slot] * pad); put(5, starts_padded); put(6, logits_idx)
         for gi, (name, cs) in enumerate(self.group_specs.items()):
             num_pages = self.kv.num_pages[name]
             fixed = entry["table_shapes"][name][1]
@@ -325,14 +334,12 @@ class ModelRunner:
 
     def _graph_step(self, key, entries: list, borrow: bool = False) -> torch.Tensor:
         entry = self._graphs.get(key)
-        fresh = entry is None
-        if fresh:
+        if entry is None:
             entry = self._new_graph_entry(key)
+            self._capture(entry)                           # before the live rows are staged
         else:
             entry["copied"].synchronize()                  # the last step's copy has left the pinned buffer
         n_want = self._restage_decode(entry, entries)
-        if fresh:
-            self._capture(entry)
         entry["static"].copy_(entry["pinned"], non_blocking=True)
         entry["copied"].record()
         entry["graph"].replay()
@@ -341,12 +348,17 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ run
     @torch.no_grad()
-    def step(self, entries: list, copies: dict | None = None, borrow: bool = False) -> torch.Tensor:
+    def step(self, entries: list, copies: dict | None = None, borrow: bool = False, state_copies: list | None = None) -> torch.Tensor:
         """Float logits [wanted rows, vocab], in the order of the entries and of their ``want``.
+        ``copies``: page copies per cache group, ``state_copies``: state slots to copy (both as the cache
+        manager hands them out after a fork), done before anything is computed.
         ``borrow``: the caller is done with the logits before its next step (a sampler that runs at once): a
         replayed step then hands out its graph's own buffer, which the next replay overwrites, without a copy."""
         if copies:
             self.kv.apply_copies(copies)
+        for c in state_copies or ():
+            for state in self.states.values():
+                state[c.dst].copy_(state[c.src])
         key = self._graph_key(entries)
         if key is not None:
             return self._graph_step(key, entries, borrow)

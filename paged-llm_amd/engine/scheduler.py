@@ -1,19 +1,24 @@
-"""Continuous batching with a token budget, prompt portions and recompute preemption.
+"""Continuous batching: which requests run how many tokens in the next step.
 
-The decisions follow pagedllm/scheduler.py:53-187:
+The policy is the reference's (pagedllm/scheduler.py:53-187); the shape is this engine's: a step's plan
+is made in two passes over one token budget, each pass a method of its own, and committed after the
+forward pass.
 
-* One step has ``max_num_batched_tokens`` tokens to give.  Running requests come first, in the
-  order they were admitted: a decoding request takes one token, a request in the middle of its
-  prompt takes as much of the rest as the budget allows (if portions are enabled; otherwise it
-  waits for a step with room).
-* **When pages run out** for a running request, the request admitted last is preempted: its
-  pages and state slot are given back, its generated tokens are kept, and it returns to the
-  head of the waiting queue to be recomputed as a longer prompt.  Victims are always at or
-  behind the current request, so nothing already scheduled in this step is undone.  If the
-  victim is the request itself, it simply does not run this step.
-* Then waiting requests are admitted first-in first-out while budget, request slots and pages
-  last; a reusable prefix is looked up first.  The first request that does not fit stops
-  admission (no skipping ahead).
+1. **Active requests**, in the order they were admitted.  A decoding request asks for one token, a
+   request inside its prompt for the rest of it; a request that asks for more than the budget has
+   left takes what is left (a *portion*) if portions are enabled, else it sits this step out.
+2. **Queued requests**, first in first out, while budget, request slots, pages and state slots last.
+   The prefix index is asked first, so a request may start behind tokens that are already cached.
+   The first request that does not fit ends the pass: nobody overtakes it.
+
+**When pages run out** for an active request, the request admitted last gives up everything it holds
+and goes back to the *front* of the queue with its generated tokens kept; it is recomputed later as a
+longer prompt.  Victims are at or behind the asking request in admission order, so nothing planned
+earlier in the same step is undone; a request that is its own victim just does not run this step.
+
+A preempted request may have grown beyond the whole budget of a step.  With portions disabled it could
+then never run again, so a request that exceeds the *whole* budget is always split, whatever the option
+says (the option still keeps every prompt that fits in one step in one step).
 """
 
 from __future__ import annotations
@@ -23,168 +28,190 @@ from dataclasses import dataclass, field
 
 from ..cache.block_manager import CacheManager
 from ..config.engine_config import EngineConfig
-from .request import Request, RequestStatus
+from .request import EndReason, Request, Stage
 
 
 @dataclass
-class ScheduledRequest:
+class Grant:
+    """One request's share of a step: its next ``count`` tokens."""
     request: Request
-    num_new_tokens: int
-    # Decided when scheduled: this step computes the last known token, so its logits are sampled.
-    needs_sampling: bool = field(init=False)
-
-    def __post_init__(self) -> None:
-        self.needs_sampling = self.request.num_computed_tokens + self.num_new_tokens == self.request.num_tokens
-
-    @property
-    def seq(self) -> Request:        # the reference's name
-        return self.request
+    count: int
+    # Known when granted: the step reaches the request's last known token, so its logits are sampled from.
+    samples: bool
 
 
 @dataclass
-class SchedulerOutput:
-    scheduled: list = field(default_factory=list)
+class StepPlan:
+    grants: list = field(default_factory=list)
     preempted: list = field(default_factory=list)
-    num_prefill_tokens: int = 0
-    num_decode_tokens: int = 0
+    prompt_tokens: int = 0
+    decode_tokens: int = 0
 
-    @property
-    def is_empty(self) -> bool:
-        return not self.scheduled
+    def __bool__(self) -> bool:
+        return bool(self.grants)
 
-    @property
-    def total_tokens(self) -> int:
-        return self.num_prefill_tokens + self.num_decode_tokens
+    def add(self, request: Request, count: int) -> None:
+        self.grants.append(Grant(request, count, request.computed + count == len(request.tokens)))
+        if request.decoding:
+            self.decode_tokens += count
+        else:
+            self.prompt_tokens += count
+
+
+def _as_id_set(eos) -> frozenset:
+    if eos is None:
+        return frozenset()
+    if isinstance(eos, (list, tuple, set, frozenset)):
+        return frozenset(int(t) for t in eos)
+    return frozenset((int(eos),))
 
 
 class Scheduler:
-    def __init__(self, config: EngineConfig, cache_manager: CacheManager, eos_token_id=None):
-        self.config = config
-        self.cm = cache_manager
-        if eos_token_id is None:
-            self.eos_ids: frozenset = frozenset()
-        elif isinstance(eos_token_id, (list, tuple, set, frozenset)):
-            self.eos_ids = frozenset(int(t) for t in eos_token_id)
-        else:
-            self.eos_ids = frozenset([int(eos_token_id)])
-        self.waiting: deque = deque()
-        self.running: list = []
-        self.finished: list = []
+    def __init__(self, config: EngineConfig, cache: CacheManager, eos_token_id=None):
+        self.step_budget = config.max_num_batched_tokens
+        self.max_active = config.max_num_seqs
+        self.max_positions = config.max_model_len
+        self.portions = config.enable_chunked_prefill
+        self.cache = cache
+        self.eos_ids = _as_id_set(eos_token_id)
+        self.queue: deque = deque()          # Stage.QUEUED, the next to admit at the left
+        self.active: list = []               # Stage.ACTIVE, in admission order
         self.num_preemptions = 0
 
-    # ------------------------------------------------------------------ queues
-    def add(self, req: Request) -> None:
-        cfg = self.config
-        if req.num_prompt_tokens >= cfg.max_model_len:
-            raise ValueError(f"prompt has {req.num_prompt_tokens} tokens, max_model_len={cfg.max_model_len}")
-        if not cfg.enable_chunked_prefill and req.num_prompt_tokens > cfg.max_num_batched_tokens:
-            raise ValueError("prompt longer than max_num_batched_tokens; enable chunked prefill")
-        if req.num_prompt_tokens + req.max_tokens > cfg.max_model_len:
-            req.max_tokens = max(1, cfg.max_model_len - req.num_prompt_tokens)
-        req.status = RequestStatus.WAITING
-        self.waiting.append(req)
+    # ------------------------------------------------------------------ arrivals and departures
+    def submit(self, request: Request) -> None:
+        """Checks a new request against the engine's limits and queues it."""
+        if request.prompt_len >= self.max_positions:
+            raise ValueError(f"a prompt of {request.prompt_len} tokens leaves no room to generate within "
+                             f"max_model_len={self.max_positions}")
+        if not self.portions and request.prompt_len > self.step_budget:
+            raise ValueError(f"a prompt of {request.prompt_len} tokens does not fit one step of max_num_batched_tokens="
+                             f"{self.step_budget}, and enable_chunked_prefill is off")
+        room = self.max_positions - request.prompt_len
+        if request.new_token_limit > room:
+            request.new_token_limit = max(1, room)
+        request.stage = Stage.QUEUED
+        self.queue.append(request)
 
-    def abort(self, request_id: int) -> None:
-        for queue in (self.waiting, self.running):
-            for req in list(queue):
-                if req.request_id == request_id:
-                    queue.remove(req)
-                    self.cm.free(req.request_id)
-                    req.status = RequestStatus.FINISHED_ABORTED
-                    self.finished.append(req)
-                    return
-
-    @property
-    def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+    def cancel(self, request_id) -> Request | None:
+        """Ends a queued or active request at once; returns it, or None if it is not here."""
+        for request in (*self.queue, *self.active):
+            if request.id == request_id:
+                (self.queue if request.stage is Stage.QUEUED else self.active).remove(request)
+                self._retire(request, EndReason.ABORT)
+                return request
+        return None
 
     @property
-    def num_unfinished(self) -> int:
-        return len(self.waiting) + len(self.running)
+    def idle(self) -> bool:
+        return not self.queue and not self.active
 
-    # ------------------------------------------------------------------ one step's plan
-    def _preempt(self, victim: Request, out: SchedulerOutput) -> None:
-        self.running.remove(victim)
-        self.cm.free(victim.request_id)
-        victim.reset_for_recompute()
-        self.waiting.appendleft(victim)
-        out.preempted.append(victim)
-        self.num_preemptions += 1
+    def __len__(self) -> int:
+        return len(self.queue) + len(self.active)
 
-    def schedule(self) -> SchedulerOutput:
-        out = SchedulerOutput()
-        budget = self.config.max_num_batched_tokens
-        portions = self.config.enable_chunked_prefill
+    def _retire(self, request: Request, reason: EndReason) -> None:
+        self.cache.free(request.id)
+        request.end(reason)
 
-        for req in list(self.running):
-            if budget == 0:
+    # ------------------------------------------------------------------ planning a step
+    def plan(self) -> StepPlan:
+        plan = StepPlan()
+        left = self._serve_active(plan, self.step_budget)
+        self._admit_queued(plan, left)
+        return plan
+
+    def _share(self, wanted: int, left: int) -> int:
+        """How many of ``wanted`` tokens a request gets from a budget with ``left`` tokens: all of
+        them, a portion, or none (0)."""
+        if wanted <= left:
+            return wanted
+        if self.portions or wanted > self.step_budget:
+            return left
+        return 0
+
+    def _serve_active(self, plan: StepPlan, left: int) -> int:
+        for request in list(self.active):
+            if left == 0:
                 break
-            if req.status is not RequestStatus.RUNNING:      # preempted earlier in this step
+            if request.stage is not Stage.ACTIVE:            # gave way to an earlier request in this pass
                 continue
-            n = req.num_uncomputed_tokens
-            assert n >= 1
-            if n > budget:
-                if not portions:
-                    continue
-                n = budget
-            while not self.cm.allocate(req.request_id, req.num_computed_tokens, n):
-                victim = self.running[-1]
-                self._preempt(victim, out)
-                if victim is req:
-                    break
-            if req.status is not RequestStatus.RUNNING:
+            count = self._share(request.backlog, left)
+            if count == 0:
                 continue
-            budget -= n
-            out.scheduled.append(ScheduledRequest(req, n))
-            if req.is_prefill_done:
-                out.num_decode_tokens += n
-            else:
-                out.num_prefill_tokens += n
+            if not self._pages_or_preempt(request, count, plan):
+                continue
+            left -= count
+            plan.add(request, count)
+        return left
 
-        while self.waiting and budget > 0 and len(self.running) < self.config.max_num_seqs:
-            req = self.waiting[0]
-            hits, num_cached = self.cm.find_cached_prefix(req.token_ids)
-            n = req.num_tokens - num_cached
-            assert n >= 1
-            if n > budget:
-                if not portions:
-                    break
-                n = budget
-            if not self.cm.allocate(req.request_id, num_cached, n, hits):
+    def _pages_or_preempt(self, request: Request, count: int, plan: StepPlan) -> bool:
+        """Pages for the request's next ``count`` tokens, taken from the requests admitted last if need
+        be.  False when the request itself had to give way."""
+        while not self.cache.allocate(request.id, request.computed, count):
+            victim = self.active.pop()
+            self.cache.free(victim.id)
+            victim.back_to_queue()
+            self.queue.appendleft(victim)
+            plan.preempted.append(victim)
+            self.num_preemptions += 1
+            if victim is request:
+                return False
+        return True
+
+    def _admit_queued(self, plan: StepPlan, left: int) -> int:
+        while self.queue and left > 0 and len(self.active) < self.max_active:
+            request = self.queue[0]
+            pages, reused = self.cache.find_cached_prefix(request.tokens)
+            count = self._share(len(request.tokens) - reused, left)
+            if count == 0 or not self.cache.allocate(request.id, reused, count, pages):
                 break
-            self.waiting.popleft()
-            req.num_computed_tokens = num_cached
-            req.num_cached_tokens = num_cached
-            req.status = RequestStatus.RUNNING
-            self.running.append(req)
-            budget -= n
-            out.scheduled.append(ScheduledRequest(req, n))
-            out.num_prefill_tokens += n
-        return out
+            self.queue.popleft()
+            request.admit(reused)
+            self.active.append(request)
+            left -= count
+            plan.add(request, count)
+        return left
+
+    def why_stuck(self) -> str:
+        """Says why an empty plan came out although requests remain (for the caller's error)."""
+        if not self.queue:
+            return "no request is queued"
+        request = self.queue[0]
+        need = self.cache.pages_for(min(len(request.tokens), self.step_budget))
+        have = self.cache.num_pages()
+        if need > have:
+            return (f"request {request.id} needs {need} pages of {self.cache.block_size} positions for its next "
+                    f"{min(len(request.tokens), self.step_budget)} tokens, the pool holds {have}")
+        if self.cache.uses_state and self.cache.slots.num_slots == 0:
+            return "the model keeps per-request state and there are no state slots"
+        return (f"request {request.id} ({len(request.tokens)} tokens) cannot be admitted with {self.cache.num_free_pages()} "
+                f"free pages of {have} and {len(self.active)} active requests")
 
     # ------------------------------------------------------------------ after the forward pass
-    def update(self, out: SchedulerOutput, sampled: dict) -> list:
-        """Advance what is computed, append sampled tokens, retire finished requests
-        (pagedllm/scheduler.py:161-187).  ``sampled`` maps request id -> token for every
-        scheduled request with ``needs_sampling``."""
-        done = []
-        for item in out.scheduled:
-            req = item.request
-            before = req.num_computed_tokens
-            req.num_computed_tokens += item.num_new_tokens
-            self.cm.note_computed(req.request_id, req.token_ids, before, req.num_computed_tokens)
-            if not item.needs_sampling:
+    def commit(self, plan: StepPlan, sampled: dict) -> list:
+        """Counts the step's tokens as computed, appends the sampled tokens (``sampled``: request id ->
+        token for every grant with ``samples``) and ends the requests that are done; returns those."""
+        ended = []
+        for grant in plan.grants:
+            request = grant.request
+            before = request.computed
+            request.computed = before + grant.count
+            self.cache.note_computed(request.id, request.tokens, before, request.computed)
+            if not grant.samples:
                 continue
-            token = int(sampled[req.request_id])
-            req.token_ids.append(token)
-            sp = req.sampling_params
-            if (not sp.ignore_eos and token in self.eos_ids) or token in sp.stop_token_ids:
-                req.status = RequestStatus.FINISHED_STOPPED
-            elif req.num_generated_tokens >= req.max_tokens or req.num_tokens >= self.config.max_model_len:
-                req.status = RequestStatus.FINISHED_LENGTH
-            if req.is_finished:
-                self.running.remove(req)
-                self.cm.free(req.request_id)
-                done.append(req)
-        self.finished.extend(done)
-        return done
+            token = int(sampled[request.id])
+            request.tokens.append(token)
+            reason = self._end_reason(request, token)
+            if reason is not None:
+                self.active.remove(request)
+                self._retire(request, reason)
+                ended.append(request)
+        return ended
+
+    def _end_reason(self, request: Request, token: int) -> EndReason | None:
+        params = request.params
+        if token in params.stop_token_ids or (token in self.eos_ids and not params.ignore_eos):
+            return EndReason.STOP
+        if request.num_generated >= request.new_token_limit or len(request.tokens) >= self.max_positions:
+            return EndReason.LENGTH
+        return None

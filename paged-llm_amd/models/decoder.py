@@ -23,9 +23,7 @@ class DecoderModel:
         self.blocks = []
         for layer in spec.layers:
             block = registry.build("block", layer.block, env)
-            block.attach(registry.build("norm", layer.mixer_norm, env), registry.build("mixer", layer.mixer, env),
-                         registry.build("norm", layer.feed_forward_norm, env),
-                         registry.build("feed_forward", layer.feed_forward, env))
+            block.build_parts(layer.parts, env)
             self.blocks.append(block)
         self.final_norm = registry.build("norm", spec.final_norm, env)
         self.head = registry.build("head", spec.head, env)
@@ -75,7 +73,7 @@ class DecoderModel:
         for pos, step in enumerate(self.spec.schedule):
             if step.cache_from is not None:
                 continue
-            cs = self.blocks[step.layer].mixer.cache_spec()
+            cs = self.blocks[step.layer].cache_spec()
             if cs is None:
                 continue
             name = cs.group_name()
@@ -86,16 +84,15 @@ class DecoderModel:
         """Schedule step -> StateSpec for mixers with per-request state of fixed size."""
         out = {}
         for pos, step in enumerate(self.spec.schedule):
-            ss = self.blocks[step.layer].mixer.state_spec()
+            ss = self.blocks[step.layer].state_spec()
             if ss is not None:
                 out[pos] = ss
         return out
 
     def graph_capturable(self) -> bool:
-        """True when every mixer and feed-forward only launches kernels (no host reads of device
-        data, no Python-side state): a decode step can then be captured into a HIP graph."""
-        return all(getattr(b.mixer, "graph_capturable", False) and getattr(b.parts["feed_forward"], "graph_capturable", False)
-                   for b in self.blocks)
+        """True when every layer's parts only launch kernels (no host reads of device data, no Python-side
+        state): a decode step can then be captured into a HIP graph."""
+        return all(b.graph_capturable() for b in self.blocks)
 
     # ------------------------------------------------------------------ compute
     def forward(self, ctx, kv_storage, states: dict) -> torch.Tensor:
@@ -107,7 +104,7 @@ class DecoderModel:
         for pos, step in enumerate(self.spec.schedule):
             block = self.blocks[step.layer]
             cache = None
-            if block.mixer.cache_spec() is not None:
+            if block.cache_spec() is not None:
                 owner = pos if step.cache_from is None else step.cache_from
                 cache = kv_storage.for_step(owner, writable=step.cache_from is None)
             x, delta = block.forward(x, delta, ctx, cache, states.get(pos))

@@ -18,13 +18,15 @@ def build_spec(cfg: LlamaConfig) -> ModelSpec:
     ffn = PartSpec("gated_mlp", {"intermediate_size": cfg.intermediate_size, "activation": "silu"})
     block = PartSpec("prenorm", {"mixer_norm": "input_layernorm", "mixer": "self_attn",
                                  "feed_forward_norm": "post_attention_layernorm", "feed_forward": "mlp"})
-    layers = [LayerSpec(f"model.layers.{i}", block, mixer, ffn, norm, norm) for i in range(cfg.num_hidden_layers)]
+    parts = {"mixer_norm": norm, "mixer": mixer, "feed_forward_norm": norm, "feed_forward": ffn}
+    layers = [LayerSpec(f"model.layers.{i}", block, parts) for i in range(cfg.num_hidden_layers)]
     return ModelSpec(
         hidden_size=cfg.hidden_size, vocab_size=cfg.vocab_size,
         embedding=PartSpec("token_embedding", {"vocab_size": cfg.vocab_size}),
         layers=layers, final_norm=norm,
         head=PartSpec("lm_head", {"vocab_size": cfg.vocab_size, "tied": cfg.tie_word_embeddings}),
         embedding_name="model.embed_tokens", final_norm_name="model.norm", head_name="lm_head",
+        ignored_suffixes=("rotary_emb.inv_freq",),
         max_positions=cfg.max_position_embeddings, eos_token_id=cfg.eos_token_id, stored_dtype=cfg.torch_dtype)
 
 

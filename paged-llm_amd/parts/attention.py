@@ -32,8 +32,9 @@ class PagedAttention(Mixer):
         self.kv_proj = bool(params.get("kv_proj", True))
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"{self.num_heads} heads are no multiple of {self.num_kv_heads} kv heads")
-        if self.head_dim % 16 or not 16 <= self.head_dim <= 256:
-            raise ValueError(f"attention kernels take head sizes 16..256 in steps of 16, got {self.head_dim}")
+        if not 1 <= self.head_dim <= ops.MAX_HEAD_DIM_GENERIC:
+            raise ValueError(f"attention kernels take head sizes 1..{ops.MAX_HEAD_DIM_GENERIC} (the matrix-core kernels "
+                             f"multiples of 16, the plain kernel the others), got {self.head_dim}")
         pos = params.get("position")
         self.position = env.position_encoding(PartSpec(**pos) if isinstance(pos, dict) else pos) if pos else None
         self.dtype, self.device = env.dtype, env.device
@@ -74,10 +75,7 @@ class PagedAttention(Mixer):
         if write and not self.kv_proj:
             raise RuntimeError("this attention layer has no k/v projections and must read another layer's cache")
         w_in = self.w_qkv if write or not self.kv_proj else self.w_qkv[: nh * d]
-        cos = sin = None
-        if self.position is not None:
-            cos, sin = self.position.cos, self.position.sin
-        qkv = qkv_rotary_cache(h, w_in, ctx.positions, cos, sin, nh, nkv, d, view.slot_mapping if write else None,
+        qkv = qkv_rotary_cache(h, w_in, ctx.positions, self.position, nh, nkv, d, view.slot_mapping if write else None,
                                cache.k_pages if write else None, cache.v_pages if write else None, cache.block_size)
         o = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
                                 nh, nkv, d, self.scale, self.window, ctx)

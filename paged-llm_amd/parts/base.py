@@ -11,8 +11,8 @@ batch was cut.
                       cache (it then names a ``CacheSpec``: pages of keys and values) and/or a
                       state of fixed size per request (``StateSpec``: a slot in a state tensor).
 * ``FeedForward``     rows -> rows, no mixing between tokens.
-* ``Block``           the arrangement of two norms, a mixer and a feed-forward around the
-                      residual stream.
+* ``Block``           the arrangement of a layer's parts around the residual stream; the kind
+                      names its roles (two norms, a mixer and a feed-forward for the pre-norm block).
 """
 
 from __future__ import annotations
@@ -91,6 +91,16 @@ class _ComputedNorm:
 
 
 class PositionEncoding(Part):
+    """Tables that a mixer's kernel applies to its queries and keys.
+
+    A rotary encoding has ``cos`` and ``sin`` (float [positions, rotary_dim / 2]) and says how they are
+    applied: ``rotary_dim`` leading elements of a head turn (the rest pass), in pairs (i, i + rotary_dim / 2)
+    or, with ``interleaved``, (2i, 2i + 1)."""
+    cos = None
+    sin = None
+    rotary_dim: int | None = None     # None: the whole head
+    interleaved: bool = False
+
     def prepare(self, max_positions: int) -> None:
         """Make tables for positions below ``max_positions``."""
 
@@ -116,11 +126,60 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """Arrangement of the parts around the residual stream.
+    """Arrangement of a layer's parts around the residual stream.
+
+    A block kind declares its roles in ``ROLES`` (role -> family of the part registry: "norm", "mixer",
+    "feed_forward", ...) and computes in ``forward``; building the parts from the layer's specs, their
+    tensor names (``params[role]`` is the role's prefix inside the layer, default the role's name) and
+    what the model asks about the layer's cache and state are common to all kinds and live here.
 
     The stream is handed on as a pair (x, delta): delta is the last branch output that has not
     been added yet, so that the next norm can add it in the same kernel.
     """
+    ROLES: dict = {}
+    # The role whose part owns the layer's cache and state (None: the layer keeps nothing).
+    MIXER_ROLE: str | None = "mixer"
+
+    def __init__(self, params: dict, env):
+        self.names = {role: params.get(role, role) for role in self.ROLES}
+        self.parts: dict = {}
+
+    def build_parts(self, specs: dict, env) -> None:
+        from . import registry
+        missing, unknown = sorted(set(self.ROLES) - set(specs)), sorted(set(specs) - set(self.ROLES))
+        if missing or unknown:
+            raise ValueError(f"block {type(self).__name__} has the roles {sorted(self.ROLES)}: "
+                             f"missing {missing}, unknown {unknown}")
+        self.parts = {role: registry.build(family, specs[role], env) for role, family in self.ROLES.items()}
+
+    @property
+    def mixer(self):
+        return self.parts[self.MIXER_ROLE] if self.MIXER_ROLE else None
+
+    def cache_spec(self):
+        return self.mixer.cache_spec() if self.mixer is not None else None
+
+    def state_spec(self):
+        return self.mixer.state_spec() if self.mixer is not None else None
+
+    def graph_capturable(self) -> bool:
+        """True when every part that computes only launches kernels on the current stream."""
+        return all(getattr(p, "graph_capturable", False) for role, p in self.parts.items() if self.ROLES[role] != "norm")
+
+    def weight_specs(self):
+        return {f"{self.names[role]}.{name}": spec for role, part in self.parts.items()
+                for name, spec in part.weight_specs().items()}
+
+    def assign(self, name, tensor):
+        for role, part in self.parts.items():
+            prefix = self.names[role] + "."
+            if name.startswith(prefix):
+                return part.assign(name[len(prefix):], tensor)
+        raise KeyError(name)
+
+    def finalize(self):
+        for part in self.parts.values():
+            part.finalize()
 
     def forward(self, x: torch.Tensor, delta: torch.Tensor | None, ctx, cache, state):
         raise NotImplementedError

@@ -55,13 +55,23 @@ def gated_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
     return ops.silu_mul(linear(x, w_gate_up))
 
 
-def qkv_rotary_cache(x, w_qkv: torch.Tensor, positions: torch.Tensor, cos, sin, num_heads: int, num_kv_heads: int,
+def qkv_rotary_cache(x, w_qkv: torch.Tensor, positions: torch.Tensor, position_encoding, num_heads: int, num_kv_heads: int,
                      head_dim: int, slot_mapping, k_pages, v_pages, block_size: int) -> torch.Tensor:
     """q, k, v projections, rotation of q and k, and the write of k and v into the cache pages.
     Returns q as rows of a matrix whose first num_heads * head_dim columns hold the rotated heads
-    (the row stride may be larger).  With k_pages None only q is projected and rotated."""
+    (the row stride may be larger).  With k_pages None only q is projected and rotated.
+    ``position_encoding``: a part with ``cos``/``sin`` tables, ``rotary_dim`` and ``interleaved``, or None.
+    The fused kernel pairs element i with i + d/2 over the whole head; another rotated width or pairing
+    goes through the product and the rotary kernel apart."""
     write = k_pages is not None
-    if write and w_qkv.dtype == torch.bfloat16 and head_dim % 16 == 0:
+    cos = sin = None
+    rotary_dim, interleaved = 0, False                      # no position encoding: nothing turns
+    if position_encoding is not None:
+        cos, sin = position_encoding.cos, position_encoding.sin
+        rotary_dim = position_encoding.rotary_dim or head_dim
+        interleaved = bool(position_encoding.interleaved)
+    whole_head_halves = position_encoding is None or (rotary_dim == head_dim and not interleaved)
+    if write and w_qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and whole_head_halves:
         rope = dict(positions=positions, cos=cos, sin=sin, slots=slot_mapping, k_pages=k_pages, v_pages=v_pages,
                     num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size)
         q = _fused(x, w_qkv, ops.EPI_ROPE_KV, rope)
@@ -69,5 +79,5 @@ def qkv_rotary_cache(x, w_qkv: torch.Tensor, positions: torch.Tensor, cos, sin, 
             return q
     qkv = linear(x, w_qkv)
     ops.rope_scatter(qkv, positions, cos, sin, num_heads, num_kv_heads, head_dim, slot_mapping if write else None,
-                     k_pages, v_pages, block_size)
+                     k_pages, v_pages, block_size, rotary_dim, interleaved)
     return qkv

@@ -1,9 +1,10 @@
-"""Rotary position encoding: float tables of cos and sin per position, half-split pairing.
+"""Rotary position encoding: float tables of cos and sin per position.
 
-inv_freq[i] = 1 / theta^(2i/d); optional "llama3" rescale of the low frequencies; angle[p, i] =
-p * inv_freq[i] in float (pagedllm/model/llama.py:86-128).  The tables hold d/2 columns (the
-reference's cat[freqs, freqs] repeats them).  The rotation itself is done by the mixer's kernel,
-fused with the cache write.
+inv_freq[i] = 1 / theta^(2i/r) over the r rotated elements of a head; optional "llama3" rescale of the
+low frequencies; angle[p, i] = p * inv_freq[i] in float (pagedllm/model/llama.py:86-128).  The tables
+hold r/2 columns (the reference's cat[freqs, freqs] repeats them).  The rotation itself is done by the
+mixer's kernel, fused with the cache write; this part says how: ``rotary_dim`` = r (default: the whole
+head, as in the reference) and ``interleaved`` (pairs (2i, 2i+1) instead of the reference's (i, i + r/2)).
 """
 
 from __future__ import annotations
@@ -19,7 +20,8 @@ from .registry import BuildEnv, register_position_encoding
 def llama3_rescale(inv_freq: torch.Tensor, factor: float, low_freq_factor: float, high_freq_factor: float,
                    original_max_position_embeddings: int) -> torch.Tensor:
     """Waves longer than orig/low are slowed by `factor`, shorter than orig/high stay, those in
-    between are blended (pagedllm/model/llama.py:86-97)."""
+    between are blended.  The formula is taken from pagedllm/model/llama.py:86-97 as it stands there
+    (it is the published llama3 rule; there is one way to write it)."""
     wavelen = 2 * math.pi / inv_freq
     low_wl = original_max_position_embeddings / low_freq_factor
     high_wl = original_max_position_embeddings / high_freq_factor
@@ -35,8 +37,11 @@ class RotaryEncoding(PositionEncoding):
         self.head_dim = int(params["head_dim"])
         self.theta = float(params["theta"])
         self.scaling = params.get("scaling")
-        if self.head_dim % 2:
-            raise ValueError(f"rotary encoding pairs element i with i + d/2: head size {self.head_dim} is odd")
+        self.rotary_dim = int(params.get("rotary_dim") or self.head_dim)
+        self.interleaved = bool(params.get("interleaved", False))
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
+            raise ValueError(f"rotary encoding turns pairs of elements: the rotated width must be even and at most the head "
+                             f"size {self.head_dim}, got {self.rotary_dim}")
         if self.scaling:
             kind = self.scaling.get("rope_type", self.scaling.get("type"))
             if kind != "llama3":
@@ -47,7 +52,7 @@ class RotaryEncoding(PositionEncoding):
         self.num_positions = 0
 
     def inverse_frequencies(self) -> torch.Tensor:
-        d = self.head_dim
+        d = self.rotary_dim
         inv_freq = 1.0 / (self.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
         if self.scaling:
             s = self.scaling
@@ -60,7 +65,7 @@ class RotaryEncoding(PositionEncoding):
         if max_positions <= self.num_positions:
             return
         t = torch.arange(max_positions, dtype=torch.float32)
-        angles = torch.outer(t, self.inverse_frequencies())          # [P, d/2], float
+        angles = torch.outer(t, self.inverse_frequencies())          # [P, rotary_dim/2], float
         self.cos = angles.cos().to(self.device).contiguous()
         self.sin = angles.sin().to(self.device).contiguous()
         self.num_positions = max_positions

@@ -38,13 +38,14 @@ class WeightSpec:
 
 @dataclass
 class LayerSpec:
-    """One decoder layer: how its parts are arranged (block) and which parts they are."""
+    """One decoder layer: the arrangement (``block``) and the parts it arranges, by role.
+
+    Which roles there are, and which family of parts fills each, is the block kind's business: the
+    pre-norm block has "mixer_norm", "mixer", "feed_forward_norm" and "feed_forward"; a block with one
+    shared norm, with norms behind its branches or without a feed-forward names other roles."""
     name: str                       # prefix of its tensor names, e.g. "model.layers.3"
     block: PartSpec
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: dict = field(default_factory=dict)      # role -> PartSpec
 
 
 @dataclass
@@ -68,17 +69,21 @@ class ModelSpec:
     head: PartSpec
     # The order in which layers run; empty = every layer once, in order.
     schedule: list[ScheduleStep] = field(default_factory=list)
-    # Prefixes of the tensor names of the parts outside the layers.
-    embedding_name: str = "model.embed_tokens"
-    final_norm_name: str = "model.norm"
-    head_name: str = "lm_head"
+    # Prefixes of the tensor names of the parts outside the layers (the architecture says them: "" is no default
+    # that fits any family of checkpoints).
+    embedding_name: str = ""
+    final_norm_name: str = ""
+    head_name: str = ""
     # Tensor names that may be present in a checkpoint and are ignored (suffix match).
-    ignored_suffixes: tuple = ("rotary_emb.inv_freq",)
+    ignored_suffixes: tuple = ()
     max_positions: int = 4096
     eos_token_id: Any = None
     stored_dtype: str = "bfloat16"
 
     def __post_init__(self) -> None:
+        for what in ("embedding_name", "final_norm_name", "head_name"):
+            if not getattr(self, what):
+                raise ValueError(f"a ModelSpec needs {what}: the prefix of that part's tensor names in the checkpoint")
         if not self.schedule:
             self.schedule = [ScheduleStep(i) for i in range(len(self.layers))]
         self.schedule = [s if isinstance(s, ScheduleStep) else ScheduleStep(int(s)) for s in self.schedule]

@@ -260,3 +260,34 @@ def test_random_orders_lose_nothing(seed, groups):
         m.free(rid)
     m.check_invariants()
     assert all(m.num_free_pages(g) == 24 for g in m.groups) and m.slots.num_free == 5
+
+
+def test_no_prefix_reuse_for_models_with_state_slots():
+    """A state of fixed size exists only as of the last token run: a request that entered behind a cached
+    prefix would start from a state that never saw those tokens.  With state slots in use the prefix index
+    is off, whatever the option says."""
+    m = CacheManager([GroupSpec("full")], 16, 4, True, num_state_slots=4)
+    assert not m.prefix_caching
+    tokens = list(range(100, 120))
+    assert m.allocate("a", 0, len(tokens))
+    m.note_computed("a", tokens, 0, len(tokens))
+    m.free("a")
+    hits, cached = m.find_cached_prefix(tokens + [1, 2])
+    assert cached == 0 and hits == {"full": []} and m.num_cached_pages() == 0
+    m.check_invariants()
+    # the same without state slots finds the prefix again
+    plain = CacheManager([GroupSpec("full")], 16, 4, True)
+    assert plain.allocate("a", 0, len(tokens))
+    plain.note_computed("a", tokens, 0, len(tokens))
+    plain.free("a")
+    assert plain.find_cached_prefix(tokens + [1, 2])[1] == 20
+
+
+def test_a_fork_hands_the_parents_state_to_the_child():
+    m = CacheManager([GroupSpec("full")], 16, 4, False, num_state_slots=3)
+    assert m.allocate("parent", 0, 6)
+    m.fork("parent", "child")
+    copies = m.take_pending_state_copies()
+    assert [(c.src, c.dst) for c in copies] == [(m.state_slot("parent"), m.state_slot("child"))]
+    assert m.state_slot("parent") != m.state_slot("child") and m.take_pending_state_copies() == []
+    m.check_invariants()

@@ -60,7 +60,7 @@ def test_registry_chooses_by_architecture_name():
     assert arch.name == "LlamaForCausalLM"
     spec = arch.build_spec(arch.read_config(TINY_B))
     assert len(spec.layers) == 3 and [s.layer for s in spec.schedule] == [0, 1, 2]
-    assert spec.layers[0].mixer.params["num_kv_heads"] == 1 and spec.head.params["tied"] is True
+    assert spec.layers[0].parts["mixer"].params["num_kv_heads"] == 1 and spec.head.params["tied"] is True
     with pytest.raises(ValueError, match="unsupported architecture"):
         lookup_architecture({"architectures": ["GPT2LMHeadModel"]})
     with pytest.raises(ValueError):
@@ -70,10 +70,10 @@ def test_registry_chooses_by_architecture_name():
 def test_no_size_of_the_config_is_a_constant_in_the_spec():
     arch = lookup_architecture(TINY_C)
     spec = arch.build_spec(arch.read_config(TINY_C))
-    m = spec.layers[0].mixer.params
+    m = spec.layers[0].parts["mixer"].params
     assert (m["num_heads"], m["num_kv_heads"], m["head_dim"]) == (5, 1, 48) and abs(m["scale"] - 48 ** -0.5) < 1e-12
-    assert spec.layers[0].feed_forward.params["intermediate_size"] == 100
-    assert spec.layers[0].mixer_norm.params["eps"] == 1e-4 and spec.vocab_size == 131 and spec.hidden_size == 80
+    assert spec.layers[0].parts["feed_forward"].params["intermediate_size"] == 100
+    assert spec.layers[0].parts["mixer_norm"].params["eps"] == 1e-4 and spec.vocab_size == 131 and spec.hidden_size == 80
     assert m["position"]["params"]["theta"] == 1000.0
 
 

@@ -597,12 +597,3 @@ def test_decode_linear_rotary_and_cache_write(heads, kv_heads, d, bs, m):
         return qkv[:, :heads * d], kp, vp
     for a, b in zip(run_fused(), run_apart()):
         assert torch.equal(a.cpu(), b.cpu())
-
-
-def test_stream_read_runs_and_refuses_odd_sizes():
-    x = torch.zeros(1 << 20, dtype=torch.bfloat16, device="cuda")
-    ops().stream_read(x)
-    ops().stream_read(x[: 8 * 1001])                                   # not a multiple of the unrolled stride
-    torch.cuda.synchronize()
-    with pytest.raises(Exception, match="16-byte"):
-        ops().stream_read(x[:5])

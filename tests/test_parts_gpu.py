@@ -198,10 +198,59 @@ def test_attention_part_whole_in_portions_and_token_by_token(dtype, tol, options
 
 def test_attention_part_refuses_sizes_its_kernels_do_not_take():
     env = env_for("bfloat16")
-    with pytest.raises(ValueError, match="steps of 16"):
-        build("mixer", "paged_attention", {"num_heads": 4, "num_kv_heads": 2, "head_dim": 24}, env)
+    with pytest.raises(ValueError, match="head sizes 1..256"):
+        build("mixer", "paged_attention", {"num_heads": 4, "num_kv_heads": 2, "head_dim": 272}, env)
     with pytest.raises(ValueError, match="multiple"):
         build("mixer", "paged_attention", {"num_heads": 5, "num_kv_heads": 2, "head_dim": 32}, env)
+    with pytest.raises(ValueError, match="even"):
+        build("mixer", "paged_attention", {"num_heads": 4, "num_kv_heads": 2, "head_dim": 23,
+                                           "position": {"kind": "rotary", "params": {"head_dim": 23, "theta": THETA}}}, env)
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("head_dim,rotary_dim,interleaved", [(24, 24, False), (32, 12, False), (32, 32, True), (20, 8, True), (7, 0, False)])
+def test_attention_part_other_head_sizes_rotated_widths_and_pairings(dtype, tol, head_dim, rotary_dim, interleaved):
+    """Head sizes that are no multiple of 16 (the plain attention kernel takes them, the matrix-core one and the
+    fused rotary epilogue do not), a rotation over only the first elements of a head, and interleaved pairs:
+    whole, and as a portion followed by single tokens."""
+    env = env_for(dtype)
+    heads, kv_heads = 4, 2
+    params = {"num_heads": heads, "num_kv_heads": kv_heads, "head_dim": head_dim}
+    if rotary_dim:
+        params["position"] = {"kind": "rotary", "params": {"head_dim": head_dim, "theta": THETA, "rotary_dim": rotary_dim,
+                                                           "interleaved": interleaved}}
+    mixer = build("mixer", "paged_attention", params, env)
+    w = give_weights(mixer, 21, dtype)
+    group = mixer.cache_spec().group_name()
+    L = 41
+    x = rows(L, 22, dtype)
+
+    def turn(t):
+        if not rotary_dim:
+            return t
+        ang = plain.rotary_angles(torch.arange(L), plain.inverse_frequencies(rotary_dim, THETA, None))
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        out = t.clone()
+        if interleaved:
+            a, b = t[..., 0:rotary_dim:2], t[..., 1:rotary_dim:2]
+            out[..., 0:rotary_dim:2], out[..., 1:rotary_dim:2] = a * cos - b * sin, b * cos + a * sin
+        else:
+            a, b = t[..., :rotary_dim // 2], t[..., rotary_dim // 2:rotary_dim]
+            out[..., :rotary_dim // 2], out[..., rotary_dim // 2:rotary_dim] = a * cos - b * sin, b * cos + a * sin
+        return out
+
+    xf = x.float()
+    q = turn((xf @ w["q_proj.weight"].T).view(L, heads, head_dim))
+    k = turn((xf @ w["k_proj.weight"].T).view(L, kv_heads, head_dim))
+    v = (xf @ w["v_proj.weight"].T).view(L, kv_heads, head_dim)
+    want = plain.causal_attention(q, k, v, head_dim ** -0.5, None).reshape(L, heads * head_dim) @ w["o_proj.weight"].T
+    table = [3, 0, 2]
+    got = mixer.forward(x.cuda(), step_context([(0, L)], [table], group, dtype), layer_cache(mixer, dtype, 4), None)
+    assert rel(got, want) <= tol, "whole"
+    cache, out = layer_cache(mixer, dtype, 4), []
+    for start, n in [(0, 19), (19, 2)] + [(p, 1) for p in range(21, L)]:
+        out.append(mixer.forward(x[start:start + n].cuda(), step_context([(start, n)], [table], group, dtype), cache, None))
+    assert rel(torch.cat(out), want) <= tol, "portions and single tokens"
 
 
 # ----------------------------------------------------------------------------------- feed-forward
@@ -234,11 +283,16 @@ def test_block_part(dtype, tol, num_rows):
     env = env_for(dtype)
     block = build("block", "prenorm", {"mixer_norm": "input_layernorm", "mixer": "self_attn",
                                        "feed_forward_norm": "post_attention_layernorm", "feed_forward": "mlp"}, env)
-    mixer = build("mixer", "paged_attention", {
-        "num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM,
-        "position": {"kind": "rotary", "params": {"head_dim": HEAD_DIM, "theta": THETA, "scaling": None}}}, env)
-    block.attach(build("norm", "rmsnorm", {"eps": EPS}, env), mixer, build("norm", "rmsnorm", {"eps": 2 * EPS}, env),
-                 build("feed_forward", "gated_mlp", {"intermediate_size": INTER}, env))
+    from paged_llm_amd.parts import PartSpec
+    with pytest.raises(ValueError, match="missing"):
+        block.build_parts({"mixer": PartSpec("paged_attention", {})}, env)
+    block.build_parts({
+        "mixer_norm": PartSpec("rmsnorm", {"eps": EPS}), "feed_forward_norm": PartSpec("rmsnorm", {"eps": 2 * EPS}),
+        "mixer": PartSpec("paged_attention", {
+            "num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM,
+            "position": {"kind": "rotary", "params": {"head_dim": HEAD_DIM, "theta": THETA, "scaling": None}}}),
+        "feed_forward": PartSpec("gated_mlp", {"intermediate_size": INTER})}, env)
+    mixer = block.mixer
     names = set(block.weight_specs())
     assert {"input_layernorm.weight", "self_attn.q_proj.weight", "mlp.down_proj.weight",
             "post_attention_layernorm.weight"} <= names and len(names) == 9

@@ -31,9 +31,9 @@ def folders(tmp_path_factory):
     return out
 
 
-def session_for(folder, dtype, max_tokens):
+def session_for(folder, dtype, max_tokens, block_size=16):
     from paged_llm_amd.engine.replay import ReplaySession
-    return ReplaySession(folder, dtype, max_tokens, None)
+    return ReplaySession(folder, dtype, max_tokens, None, block_size=block_size)
 
 
 def requests_for(name):
@@ -213,3 +213,42 @@ def test_request_longer_than_the_configured_positions(folders, dtype):
     got = helpers.replay_in_process(session_for(folder, dtype, 192), trace)
     assert len(got) == 32
     check(got, folder, {"long": toks}, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("block_size", [8, 32])
+def test_every_mode_at_other_page_sizes(folders, dtype, block_size):
+    """Configuration B with pages of 8 positions (the matrix-core attention kernel needs 16: bfloat16 then takes
+    the plain attention kernel behind the fused rotary epilogue and cache write) and of 32: whole, the last 32
+    tokens one by one, portions of changing size, and mixed with pages used again."""
+    folder = folders["B", "float32" if dtype == "float32" else "bfloat16"]
+    reqs = requests_for("B")
+    longest = rounded(max(len(t) for t in reqs.values()))
+    whole, tail, portions = TraceBuilder(), TraceBuilder(), TraceBuilder()
+    sizes = itertools.cycle([3, 2, 11, 1, 8, 2, 17, 5])
+    for rid, toks in reqs.items():
+        whole.step([(rid, toks, "all")], end=[rid])
+        if len(toks) > 34:
+            cut = len(toks) - 32
+            tail.step([(rid, toks[:cut], "last")])
+            for i in range(cut, len(toks)):
+                tail.step([(rid, toks[i:i + 1], "all")], end=[rid] if i == len(toks) - 1 else [])
+        at = 0
+        while at < len(toks):
+            n = min(next(sizes), len(toks) - at)
+            portions.step([(rid, toks[at:at + n], "all")], end=[rid] if at + n == len(toks) else [])
+            at += n
+    for trace in (whole, tail, portions):
+        session = session_for(folder, dtype, longest, block_size)
+        assert session.manager.block_size == block_size
+        check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+    twice = dict(reqs)
+    for i, (rid, toks) in enumerate(reqs.items()):
+        twice[rid + "x"] = helpers.random_tokens(len(toks), TINY_B["vocab_size"], seed=950 + i)
+    trace, peak = mixed_trace(twice, max_live=4, seed=6)
+    session = session_for(folder, dtype, peak, block_size)
+    got = helpers.replay_in_process(session, trace)
+    assert len(got) == sum(len(t) for t in twice.values())
+    check(got, folder, twice, dtype)
+    session.manager.check_invariants()
+    assert session.manager.num_free_pages() == session.manager.num_pages()

@@ -5,7 +5,7 @@ import pytest
 
 from paged_llm_amd import EngineConfig, SamplingParams
 from paged_llm_amd.cache import CacheManager, GroupSpec
-from paged_llm_amd.engine import Request, RequestStatus, Scheduler
+from paged_llm_amd.engine import EndReason, Request, Scheduler, Stage
 
 EOS = 2
 
@@ -19,85 +19,85 @@ def make(num_blocks=64, block_size=4, budget=32, max_seqs=8, chunked=True, prefi
 
 
 def run_step(sched, next_token=7):
-    out = sched.schedule()
-    sampled = {s.request.request_id: next_token for s in out.scheduled if s.needs_sampling}
-    finished = sched.update(out, sampled)
-    sched.cm.check_invariants()
-    return out, finished
+    plan = sched.plan()
+    sampled = {g.request.id: next_token for g in plan.grants if g.samples}
+    ended = sched.commit(plan, sampled)
+    sched.cache.check_invariants()
+    return plan, ended
 
 
 def test_prefill_then_decode_then_finish():
     _, _, sched = make()
     req = Request(list(range(10, 20)), SamplingParams(max_tokens=3))
-    sched.add(req)
+    sched.submit(req)
     out, _ = run_step(sched)
-    assert out.num_prefill_tokens == 10 and out.num_decode_tokens == 0
-    assert req.status is RequestStatus.RUNNING and req.num_generated_tokens == 1
+    assert out.prompt_tokens == 10 and out.decode_tokens == 0
+    assert req.stage is Stage.ACTIVE and req.num_generated == 1
     out, _ = run_step(sched)
-    assert out.num_decode_tokens == 1
+    assert out.decode_tokens == 1
     out, finished = run_step(sched)
-    assert finished == [req] and req.status is RequestStatus.FINISHED_LENGTH
-    assert req.output_token_ids == [7, 7, 7] and not sched.has_unfinished
+    assert finished == [req] and req.end_reason is EndReason.LENGTH
+    assert req.generated == [7, 7, 7] and sched.idle
 
 
 def test_eos_and_stop_tokens():
     _, cm, sched = make()
     req = Request([5, 6, 7], SamplingParams(max_tokens=10))
-    sched.add(req)
-    sched.update(out := sched.schedule(), {req.request_id: EOS})
-    assert req.status is RequestStatus.FINISHED_STOPPED and cm.num_free_pages() == 64
-    assert req.output_token_ids == [EOS]                        # the stop token stays in the output
+    sched.submit(req)
+    sched.commit(out := sched.plan(), {req.id: EOS})
+    assert req.end_reason is EndReason.STOP and cm.num_free_pages() == 64
+    assert req.generated == [EOS]                        # the stop token stays in the output
     ignoring = Request([5, 6, 7], SamplingParams(max_tokens=2, ignore_eos=True))
-    sched.add(ignoring)
-    sched.update(out := sched.schedule(), {ignoring.request_id: EOS})
-    assert ignoring.status is RequestStatus.RUNNING
+    sched.submit(ignoring)
+    sched.commit(out := sched.plan(), {ignoring.id: EOS})
+    assert ignoring.stage is Stage.ACTIVE
     stopper = Request([5, 6, 7], SamplingParams(max_tokens=9, stop_token_ids=(42,)))
-    sched.add(stopper)
-    out = sched.schedule()
-    sched.update(out, {ignoring.request_id: 1, stopper.request_id: 42})
-    assert stopper.status is RequestStatus.FINISHED_STOPPED and ignoring.status is RequestStatus.FINISHED_LENGTH
+    sched.submit(stopper)
+    out = sched.plan()
+    sched.commit(out, {ignoring.id: 1, stopper.id: 42})
+    assert stopper.end_reason is EndReason.STOP and ignoring.end_reason is EndReason.LENGTH
 
 
 def test_several_eos_ids_from_config_json():
     _, _, sched = make(eos=[2, 9])
     req = Request([5], SamplingParams(max_tokens=10))
-    sched.add(req)
-    sched.update(out := sched.schedule(), {req.request_id: 9})
-    assert req.status is RequestStatus.FINISHED_STOPPED
+    sched.submit(req)
+    sched.commit(out := sched.plan(), {req.id: 9})
+    assert req.end_reason is EndReason.STOP
 
 
 def test_prompt_portions_respect_the_budget():
     _, _, sched = make(budget=8)
     req = Request(list(range(100, 120)), SamplingParams(max_tokens=2))
-    sched.add(req)
+    sched.submit(req)
     out, _ = run_step(sched)
-    assert out.scheduled[0].num_new_tokens == 8 and req.num_computed_tokens == 8
-    assert req.num_generated_tokens == 0 and not out.scheduled[0].needs_sampling
+    assert out.grants[0].count == 8 and req.computed == 8
+    assert req.num_generated == 0 and not out.grants[0].samples
     run_step(sched)
-    assert req.num_computed_tokens == 16
+    assert req.computed == 16
     run_step(sched)
-    assert req.num_computed_tokens == 20 and req.num_generated_tokens == 1
+    assert req.computed == 20 and req.num_generated == 1
 
 
 def test_decode_and_prompt_portion_share_a_step():
     _, _, sched = make(budget=16)
     a = Request(list(range(4)), SamplingParams(max_tokens=10))
-    sched.add(a)
+    sched.submit(a)
     run_step(sched)
     b = Request(list(range(40)), SamplingParams(max_tokens=10))
-    sched.add(b)
+    sched.submit(b)
     out, _ = run_step(sched)
-    assert out.num_decode_tokens == 1 and out.num_prefill_tokens == 15
-    assert [s.request for s in out.scheduled] == [a, b]
+    assert out.decode_tokens == 1 and out.prompt_tokens == 15
+    assert [g.request for g in out.grants] == [a, b]
 
 
 def test_first_in_first_out_and_max_num_seqs():
     _, _, sched = make(max_seqs=2, budget=1000)
     reqs = [Request([1, 2, 3], SamplingParams(max_tokens=5)) for _ in range(3)]
     for r in reqs:
-        sched.add(r)
+        sched.submit(r)
     out, _ = run_step(sched)
-    assert [x.request for x in out.scheduled] == reqs[:2] and reqs[2].status is RequestStatus.WAITING
+    assert [g.request for g in out.grants] == reqs[:2] and reqs[2].stage is Stage.QUEUED
 
 
 def test_when_pages_run_out_the_last_admitted_is_preempted_and_recomputed():
@@ -105,8 +105,8 @@ def test_when_pages_run_out_the_last_admitted_is_preempted_and_recomputed():
     _, cm, sched = make(num_blocks=6, block_size=4, budget=1000)
     a = Request(list(range(8)), SamplingParams(max_tokens=8))
     b = Request(list(range(8, 16)), SamplingParams(max_tokens=8))
-    sched.add(a)
-    sched.add(b)
+    sched.submit(a)
+    sched.submit(b)
     run_step(sched)
     assert cm.num_free_pages() == 2
     run_step(sched)
@@ -115,35 +115,35 @@ def test_when_pages_run_out_the_last_admitted_is_preempted_and_recomputed():
         out, _ = run_step(sched)
     assert cm.num_free_pages() == 0 and not out.preempted
     out, _ = run_step(sched)
-    assert b in out.preempted and b.status is RequestStatus.WAITING and not cm.holds(b.request_id)
-    assert a.status is RequestStatus.RUNNING and sched.num_preemptions >= 1 and sched.waiting[0] is b
-    generated_before = b.num_generated_tokens
-    while a.status is RequestStatus.RUNNING:
+    assert b in out.preempted and b.stage is Stage.QUEUED and not cm.holds(b.id)
+    assert a.stage is Stage.ACTIVE and sched.num_preemptions >= 1 and sched.queue[0] is b
+    generated_before = b.num_generated
+    while a.stage is Stage.ACTIVE:
         run_step(sched)
-    assert a.output_token_ids == [7] * 8
-    while sched.has_unfinished:
+    assert a.generated == [7] * 8
+    while not sched.idle:
         run_step(sched)
-    assert b.status is RequestStatus.FINISHED_LENGTH and b.num_generated_tokens == 8
-    assert b.num_preemptions >= 1 and generated_before >= 1 and cm.num_free_pages() == 6
+    assert b.end_reason is EndReason.LENGTH and b.num_generated == 8
+    assert b.times_preempted >= 1 and generated_before >= 1 and cm.num_free_pages() == 6
 
 
 def test_a_request_that_cannot_get_a_page_alone_just_waits_this_step():
     # one running request needs a page that does not exist: it is its own victim and returns to waiting
     _, cm, sched = make(num_blocks=2, block_size=4, budget=1000, prefix=False)
     a = Request(list(range(8)), SamplingParams(max_tokens=4))
-    sched.add(a)
+    sched.submit(a)
     run_step(sched)                                             # 8 tokens fill both pages
-    out = sched.schedule()
-    assert out.is_empty and out.preempted == [a] and a.status is RequestStatus.WAITING and cm.num_free_pages() == 2
+    out = sched.plan()
+    assert not out and out.preempted == [a] and a.stage is Stage.QUEUED and cm.num_free_pages() == 2
 
 
 def test_admission_stops_at_the_first_request_that_does_not_fit():
     _, cm, sched = make(num_blocks=4, block_size=4, budget=1000)
     big, small = Request(list(range(30)), SamplingParams()), Request([1, 2], SamplingParams())
-    sched.add(big)
-    sched.add(small)
-    out = sched.schedule()
-    assert out.is_empty and list(sched.waiting) == [big, small]    # no skipping ahead
+    sched.submit(big)
+    sched.submit(small)
+    out = sched.plan()
+    assert not out and list(sched.queue) == [big, small]    # no skipping ahead
     assert cm.num_free_pages() == 4
 
 
@@ -151,57 +151,92 @@ def test_prefix_reuse_across_requests():
     _, cm, sched = make(block_size=4, budget=1000)
     shared = list(range(50, 66))
     a = Request(shared + [1, 2], SamplingParams(max_tokens=1))
-    sched.add(a)
-    while sched.has_unfinished:
+    sched.submit(a)
+    while not sched.idle:
         run_step(sched)
     b = Request(shared + [3, 4, 5], SamplingParams(max_tokens=1))
-    sched.add(b)
+    sched.submit(b)
     out, _ = run_step(sched)
-    assert b.num_cached_tokens == 16 and out.scheduled[0].num_new_tokens == 3 and cm.num_cache_hits == 1
+    assert b.reused_prefix == 16 and out.grants[0].count == 3 and cm.num_cache_hits == 1
 
 
 def test_no_portions_when_disabled():
     _, _, sched = make(budget=8, chunked=False)
     small = Request(list(range(8)), SamplingParams(max_tokens=1))
-    sched.add(small)
+    sched.submit(small)
     out, _ = run_step(sched)
-    assert out.scheduled[0].num_new_tokens == 8
-    with pytest.raises(ValueError, match="chunked"):
-        sched.add(Request(list(range(9)), SamplingParams()))
+    assert out.grants[0].count == 8
+    with pytest.raises(ValueError, match="enable_chunked_prefill"):
+        sched.submit(Request(list(range(9)), SamplingParams()))
 
 
 def test_length_checks_and_clamp_do_not_touch_shared_params():
     _, _, sched = make(max_len=32)
     with pytest.raises(ValueError, match="max_model_len"):
-        sched.add(Request(list(range(32)), SamplingParams()))
+        sched.submit(Request(list(range(32)), SamplingParams()))
     shared = SamplingParams(max_tokens=100)
     a, b = Request(list(range(20)), shared), Request(list(range(5)), shared)
-    sched.add(a)
-    sched.add(b)
-    assert a.max_tokens == 12 and b.max_tokens == 27 and shared.max_tokens == 100
-    with pytest.raises(ValueError, match="empty"):
+    sched.submit(a)
+    sched.submit(b)
+    assert a.new_token_limit == 12 and b.new_token_limit == 27 and shared.max_tokens == 100
+    with pytest.raises(ValueError, match="at least one prompt token"):
         Request([], SamplingParams())
 
 
 def test_abort_gives_everything_back():
     _, cm, sched = make()
     a, b = Request(list(range(9)), SamplingParams()), Request(list(range(5)), SamplingParams())
-    sched.add(a)
+    sched.submit(a)
     run_step(sched)
-    sched.add(b)
-    sched.abort(a.request_id)
-    sched.abort(b.request_id)
-    assert a.status is b.status is RequestStatus.FINISHED_ABORTED and not sched.has_unfinished
+    sched.submit(b)
+    sched.cancel(a.id)
+    sched.cancel(b.id)
+    assert a.end_reason is b.end_reason is EndReason.ABORT and sched.idle
     assert cm.num_free_pages() == 64
 
 
 def test_state_slots_limit_admission():
     _, cm, sched = make(state_slots=1, budget=1000)
     a, b = Request([1, 2, 3], SamplingParams(max_tokens=2)), Request([4, 5], SamplingParams(max_tokens=2))
-    sched.add(a)
-    sched.add(b)
+    sched.submit(a)
+    sched.submit(b)
     out, _ = run_step(sched)
-    assert [s.request for s in out.scheduled] == [a] and b.status is RequestStatus.WAITING
+    assert [g.request for g in out.grants] == [a] and b.stage is Stage.QUEUED
     run_step(sched)                                             # a finishes, its slot comes back
     out, _ = run_step(sched)
-    assert [s.request for s in out.scheduled] == [b] and cm.state_slot(b.request_id) == 0
+    assert [g.request for g in out.grants] == [b] and cm.state_slot(b.id) == 0
+
+
+def test_a_preempted_request_beyond_the_whole_budget_is_recomputed_in_portions_even_when_portions_are_off():
+    """Portions disabled, budget 8: a request admitted with 8 tokens grows, loses its pages to an earlier
+    request, and is then longer than any step may hold.  It must still come back (in portions), not
+    block the queue for ever."""
+    _, cm, sched = make(num_blocks=5, block_size=4, budget=8, chunked=False, prefix=False)
+    a, b = Request(list(range(4)), SamplingParams(max_tokens=10)), Request(list(range(8, 12)), SamplingParams(max_tokens=10))
+    sched.submit(a)
+    sched.submit(b)
+    steps, longest_backlog = 0, 0
+    while not sched.idle:
+        plan, _ = run_step(sched)
+        assert plan or sched.idle, "an empty plan although requests remain"
+        longest_backlog = max([longest_backlog] + [len(r.tokens) for r in plan.preempted])
+        steps += 1
+        assert steps < 200
+    assert b.times_preempted >= 1 and longest_backlog > 8          # it came back longer than a step's whole budget
+    assert a.end_reason is b.end_reason is EndReason.LENGTH
+    assert a.generated == b.generated == [7] * 10 and cm.num_free_pages() == 5
+
+
+def test_why_stuck_names_the_pool_when_one_request_cannot_fit():
+    _, _, sched = make(num_blocks=2, block_size=4, budget=1000)
+    sched.submit(Request(list(range(30)), SamplingParams()))
+    assert not sched.plan()
+    assert "pages" in sched.why_stuck() and "the pool holds 2" in sched.why_stuck()
+
+
+def test_a_finished_request_is_no_longer_held_by_the_scheduler():
+    _, _, sched = make()
+    req = Request([1, 2, 3], SamplingParams(max_tokens=1))
+    sched.submit(req)
+    _, ended = run_step(sched)
+    assert ended == [req] and sched.idle and len(sched) == 0

@@ -1,9 +1,11 @@
 """The framework's generality, shown with toy parts that are defined here and registered without a
-change to the framework's files: a mixer with per-request state of fixed size, a layer that runs
-twice, a layer that reads another layer's cache, a windowed attention layer with pages of its
-own, a feed-forward with a router and experts, and another position encoding (rotation angles on a
-linear grid of frequencies).  The toy model is replayed whole, in portions and mixed, and compared
-with a plain implementation written here."""
+change to the framework's files: a mixer with per-request state of fixed size (which also runs inside
+replayed HIP graphs), a layer that runs twice, a layer that reads another layer's cache, a windowed
+attention layer with pages of its own whose rotary encoding turns only half of each head in interleaved
+pairs, a feed-forward with a router and experts, another position encoding (rotation angles on a
+linear grid of frequencies), and a block of another arrangement (one norm shared by a mixer and a
+feed-forward that run side by side).  The toy model is replayed whole, in portions and mixed, generated
+from through the entry point, and compared with a plain implementation written here."""
 
 import numpy as np
 import pytest
@@ -18,14 +20,16 @@ pytestmark = pytest.mark.gpu
 TOY = {"architectures": ["ToyHybridForCausalLM"], "vocab_size": 120, "hidden_size": 48, "intermediate_size": 72,
        "heads": 3, "kv_heads": 1, "head_dim": 16, "decay": 0.8, "window": 7, "eps": 1e-5, "theta": 100.0,
        "experts": 3, "expert_size": 24, "linear_base": 0.37, "max_position_embeddings": 256}
-# step -> (layer, cache_from): layer 1 (the stateful mixer) runs twice, step 2 reads the cache of step 0
-SCHEDULE = [(0, None), (1, None), (2, 0), (3, None), (1, None)]
+# step -> (layer, cache_from): layer 1 (the stateful mixer) runs twice, step 2 reads the cache of step 0,
+# layer 4 is the block with one shared norm
+SCHEDULE = [(0, None), (1, None), (2, 0), (3, None), (1, None), (4, None)]
+PARTIAL_ROTARY = 8          # of 16 elements of a head, in interleaved pairs (layer 3)
 
 
 def register_toy():
     from paged_llm_amd.config.registry import ARCHITECTURES, Architecture, register_architecture
-    from paged_llm_amd.parts import (FeedForward, LayerSpec, Mixer, ModelSpec, PartSpec, PositionEncoding, ScheduleStep,
-                                     StateSpec, WeightSpec, register_feed_forward, register_mixer,
+    from paged_llm_amd.parts import (Block, FeedForward, LayerSpec, Mixer, ModelSpec, PartSpec, PositionEncoding, ScheduleStep,
+                                     StateSpec, WeightSpec, register_block, register_feed_forward, register_mixer,
                                      register_position_encoding)
     from paged_llm_amd.parts.linear import gated_linear, linear
     from paged_llm_amd.parts.norm import rows_of
@@ -33,7 +37,10 @@ def register_toy():
         return
 
     class DecayMixer(Mixer):
-        """s_t = decay * s_{t-1} + W x_t, output s_t; the state is one float vector per request."""
+        """s_t = decay * s_{t-1} + W x_t, output s_t; the state is one float vector per request.  A step of
+        single tokens touches device tensors only (slots and starts as the context holds them), so it may
+        be captured into a graph; prompt portions walk the host lists."""
+        graph_capturable = True
 
         def __init__(self, params, env):
             self.hidden, self.decay = env.hidden_size, float(params["decay"])
@@ -51,10 +58,16 @@ def register_toy():
 
         def forward(self, h, ctx, cache, state):
             u = linear(h, self.w).float()
+            if ctx.decode_only:
+                slots = ctx.state_slots.long()
+                carried = state.index_select(0, slots) * (ctx.seq_starts > 0).unsqueeze(1)    # a fresh request starts at zero
+                new = self.decay * carried + u
+                state.index_copy_(0, slots, new)
+                return new.to(h.dtype)
             out = torch.empty_like(u)
             at = 0
             for n, k_len, slot in zip(ctx.q_lens, ctx.k_lens, ctx.state_slot_list):
-                s0 = state[slot] if k_len - n > 0 else torch.zeros_like(state[slot])     # a fresh request starts at zero
+                s0 = state[slot] if k_len - n > 0 else torch.zeros_like(state[slot])
                 i = torch.arange(n, device=u.device, dtype=torch.float32)
                 powers = torch.tril(self.decay ** (i[:, None] - i[None, :]).clamp_min(0))
                 seg = powers @ u[at:at + n] + (self.decay ** (i + 1))[:, None] * s0
@@ -69,6 +82,7 @@ def register_toy():
         """A router (logits and softmax in float, its matrix kept in float) and gated experts; the output is
         the experts' outputs weighted by the router's probabilities.  Every expert sees every row here, so that
         rounding cannot flip a choice in the comparison; a top-k choice would gather its rows in the same place."""
+        graph_capturable = True
 
         def __init__(self, params, env):
             self.hidden, self.experts, self.inter = env.hidden_size, int(params["experts"]), int(params["expert_size"])
@@ -117,6 +131,19 @@ def register_toy():
 
     register_position_encoding("toy_linear_rotary", LinearRotary)
 
+    class SharedNormBlock(Block):
+        """x += mixer(norm(x)) + feed_forward(norm(x)): one norm, two branches side by side."""
+        ROLES = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+
+        def forward(self, x, delta, ctx, cache, state):
+            p = self.parts
+            h = p["norm"].pending(x, delta)
+            rows = rows_of(h)                               # both branches read the same normed rows
+            x = h.residual()
+            return x, p["mixer"].forward(rows, ctx, cache, state) + p["feed_forward"].forward(rows, ctx)
+
+    register_block("toy_shared_norm", SharedNormBlock)
+
     def build_spec(c):
         norm = PartSpec("rmsnorm", {"eps": c["eps"]})
         rotary = {"kind": "rotary", "params": {"head_dim": c["head_dim"], "theta": c["theta"], "scaling": None}}
@@ -127,10 +154,20 @@ def register_toy():
         ffn = PartSpec("gated_mlp", {"intermediate_size": c["intermediate_size"]})
         routed = PartSpec("toy_soft_experts", {"experts": c["experts"], "expert_size": c["expert_size"]})
         block = PartSpec("prenorm", {"mixer_norm": "norm1", "mixer": "mixer", "feed_forward_norm": "norm2", "feed_forward": "ffn"})
-        # layers 0 and 2 share a cache, so they share the position encoding too (the linear grid); layer 3 has the experts
+        shared = PartSpec("toy_shared_norm", {"norm": "norm1", "mixer": "mixer", "feed_forward": "ffn"})
+        partial = {"kind": "rotary", "params": {"head_dim": c["head_dim"], "theta": c["theta"], "scaling": None,
+                                                "rotary_dim": PARTIAL_ROTARY, "interleaved": True}}
+        # layers 0 and 2 share a cache, so they share the position encoding too (the linear grid); layer 3 has the
+        # experts, a window and the partial interleaved rotation; layer 4 is the other arrangement
         mixers = [attention(linear_grid), PartSpec("toy_decay", {"decay": c["decay"]}), attention(linear_grid, kv_proj=False),
-                  attention(window=c["window"])]
-        layers = [LayerSpec(f"layers.{i}", block, m, routed if i == 3 else ffn, norm, norm) for i, m in enumerate(mixers)]
+                  attention(partial, window=c["window"]), attention()]
+        layers = []
+        for i, m in enumerate(mixers):
+            if i == 4:
+                layers.append(LayerSpec(f"layers.{i}", shared, {"norm": norm, "mixer": m, "feed_forward": ffn}))
+            else:
+                layers.append(LayerSpec(f"layers.{i}", block, {"mixer_norm": norm, "mixer": m, "feed_forward_norm": norm,
+                                                               "feed_forward": routed if i == 3 else ffn}))
         return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"],
                          embedding=PartSpec("token_embedding", {"vocab_size": c["vocab_size"]}), layers=layers, final_norm=norm,
                          head=PartSpec("lm_head", {"vocab_size": c["vocab_size"], "tied": False}),
@@ -140,11 +177,27 @@ def register_toy():
     register_architecture(Architecture("ToyHybridForCausalLM", lambda raw: dict(raw), build_spec))
 
 
+def rotate_some(x, angles, width, interleaved):
+    """The first ``width`` elements of each head turn by ``angles`` [T, width/2], in pairs (i, i + width/2) or
+    (2i, 2i + 1); the others pass."""
+    out = x.clone()
+    cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]
+    if interleaved:
+        a, b = x[..., 0:width:2], x[..., 1:width:2]
+        out[..., 0:width:2], out[..., 1:width:2] = a * cos - b * sin, b * cos + a * sin
+    else:
+        a, b = x[..., :width // 2], x[..., width // 2:width]
+        out[..., :width // 2], out[..., width // 2:width] = a * cos - b * sin, b * cos + a * sin
+    return out
+
+
 def plain_toy(folder, tokens):
     c, w = TOY, {k: v.float() for k, v in plain.load_weights(folder).items()}
     T, nh, nkv, d = len(tokens), c["heads"], c["kv_heads"], c["head_dim"]
-    ang_usual = plain.rotary_angles(torch.arange(T), plain.inverse_frequencies(d, c["theta"], None))
-    ang_linear = plain.rotary_angles(torch.arange(T), c["linear_base"] * (torch.arange(d // 2, dtype=torch.float32) + 1) / (d // 2))
+    pos = torch.arange(T)
+    ang_usual = plain.rotary_angles(pos, plain.inverse_frequencies(d, c["theta"], None))
+    ang_linear = plain.rotary_angles(pos, c["linear_base"] * (torch.arange(d // 2, dtype=torch.float32) + 1) / (d // 2))
+    ang_partial = plain.rotary_angles(pos, plain.inverse_frequencies(PARTIAL_ROTARY, c["theta"], None))
     x = w["embed.weight"][torch.tensor(tokens)]
     kept = {}
     for step, (layer, cache_from) in enumerate(SCHEDULE):
@@ -157,16 +210,23 @@ def plain_toy(folder, tokens):
                 rows.append(s)
             a = torch.stack(rows)
         else:
-            ang = ang_linear if layer in (0, 2) else ang_usual
-            q = plain.apply_rotary((h @ w[p + "mixer.q_proj.weight"].T).view(T, nh, d), ang)
+            if layer == 3:
+                turn = lambda t: rotate_some(t, ang_partial, PARTIAL_ROTARY, True)
+            else:
+                ang = ang_linear if layer in (0, 2) else ang_usual
+                turn = lambda t: plain.apply_rotary(t, ang)
+            q = turn((h @ w[p + "mixer.q_proj.weight"].T).view(T, nh, d))
             if cache_from is None:
-                k = plain.apply_rotary((h @ w[p + "mixer.k_proj.weight"].T).view(T, nkv, d), ang)
+                k = turn((h @ w[p + "mixer.k_proj.weight"].T).view(T, nkv, d))
                 v = (h @ w[p + "mixer.v_proj.weight"].T).view(T, nkv, d)
                 kept[step] = (k, v)
             else:
                 k, v = kept[cache_from]
             o = plain.causal_attention(q, k, v, d ** -0.5, c["window"] if layer == 3 else None)
             a = o.reshape(T, nh * d) @ w[p + "mixer.o_proj.weight"].T
+        if layer == 4:                                       # one norm, both branches from the same rows
+            x = x + a + plain.swiglu(h, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+            continue
         x = x + a
         h = plain.rms_norm(x, w[p + "norm2.weight"], c["eps"])
         if layer == 3:
@@ -189,7 +249,8 @@ def test_toy_model_is_built_from_registered_parts(toy_folder):
     s = ReplaySession(toy_folder, "float32", 256, None)
     groups = s.model.cache_groups()
     assert sorted(groups) == ["full_kv1x16", "window7_kv1x16"]
-    assert groups["full_kv1x16"].owners == [0] and groups["window7_kv1x16"].owners == [3]      # step 2 owns no pages
+    assert groups["full_kv1x16"].owners == [0, 5] and groups["window7_kv1x16"].owners == [3]   # step 2 owns no pages
+    assert "layers.4.norm2.weight" not in s.model.weight_specs() and "layers.4.norm1.weight" in s.model.weight_specs()
     assert sorted(s.model.state_specs()) == [1, 4]                                             # one state per step, not per layer
     assert "layers.2.mixer.k_proj.weight" not in s.model.weight_specs()
     assert s.manager.uses_state and set(s.runner.states) == {1, 4}
@@ -229,3 +290,50 @@ def test_toy_model_whole_in_portions_and_mixed(toy_folder, dtype, tol):
     assert session.manager.slots.num_free == session.manager.slots.num_slots
     # the windowed group gave pages back while requests were still running
     assert all(session.manager.num_free_pages(g) == session.manager.num_pages(g) for g in session.manager.groups)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 5e-2)])
+def test_toy_state_inside_replayed_graphs(toy_folder, dtype, tol):
+    """Single-token steps of the toy model are replayed from HIP graphs: the state of every request must move
+    once per token, also in the step that captures a graph, and the empty rows that pad a batch must not
+    touch anybody's state."""
+    from paged_llm_amd.engine.replay import ReplaySession
+    reqs = {f"g{i}": helpers.random_tokens(40 + i, TOY["vocab_size"], seed=260 + i) for i in range(5)}
+    want = {rid: plain_toy(toy_folder, toks) for rid, toks in reqs.items()}
+    session = ReplaySession(toy_folder, dtype, 64 * 5, None)
+    assert session.runner.use_graphs and session.runner.states
+    trace = TraceBuilder()
+    trace.step([(rid, toks[:9], "last") for rid, toks in reqs.items()])
+    at = {rid: 9 for rid in reqs}
+    for step in range(36):
+        chosen = list(reqs)[:3] if step % 5 == 0 else list(reqs)       # five rows run as six, three as three
+        chosen = [rid for rid in chosen if at[rid] < len(reqs[rid])]
+        trace.step([(rid, reqs[rid][at[rid]:at[rid] + 1], "all") for rid in chosen])
+        for rid in chosen:
+            at[rid] += 1
+    got = helpers.replay_in_process(session, trace)
+    assert len(session.runner._graphs) >= 2
+    for (rid, pos), row in got.items():
+        err = helpers.worst(row, want[rid][pos])
+        assert err <= tol, f"{rid} position {pos}: {err:.3g}"
+
+
+def test_toy_model_generates_through_the_entry_point_with_default_settings(toy_folder):
+    """Prefix reuse is on by default; a model that keeps state of fixed size cannot re-enter a cached prefix
+    (its state never saw it), so the cache manager must switch reuse off by itself: two requests with a
+    long common beginning still give the plain implementation's greedy tokens."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    engine = LLMEngine(toy_folder, EngineConfig(dtype="float32", num_gpu_blocks=48, max_model_len=128, max_num_seqs=4))
+    assert engine.config.enable_prefix_caching and not engine.cache_manager.prefix_caching
+    shared = helpers.random_tokens(40, TOY["vocab_size"], seed=290)
+    prompts = [shared + [3, 4], shared + [5, 6, 7], helpers.random_tokens(11, TOY["vocab_size"], seed=291)]
+    sp = SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=True)
+    outs = engine.generate(prompts[:1], sp) + engine.generate(prompts[1:], sp)
+    for prompt, out in zip(prompts, outs):
+        toks = list(prompt)
+        for _ in range(9):
+            toks.append(int(np.argmax(plain_toy(toy_folder, toks)[-1])))
+        assert out.token_ids == toks[len(prompt):] and out.num_cached_tokens == 0
+    assert all(engine.cache_manager.num_free_pages(g) == engine.cache_manager.num_pages(g) for g in engine.cache_manager.groups)
+    engine.cache_manager.check_invariants()
