@@ -95,13 +95,15 @@ def apply_rotary(x: torch.Tensor, angles: torch.Tensor) -> torch.Tensor:
 
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
-                     window: int | None = None) -> torch.Tensor:
+                     window: int | None = None, r=lambda t: t) -> torch.Tensor:
     """Dense causal attention of one whole sequence with grouped heads.
 
     q: [L, nh, d], k, v: [L, nkv, d].  Query head j reads KV head j // (nh // nkv); the scale
     multiplies the finished dot product; key n is hidden from query i when n > i
     (pagedllm/attention/reference.py:33-55).  ``window`` (not a Llama option; the cache
     manager's windowed groups are tested with it) also hides keys with n <= i - window.
+    ``r`` rounds the probabilities before they meet the values, as the reference's kernel does when the
+    model is stored in a 16-bit type (pagedllm/attention/triton_kernel.py:88); the identity otherwise.
     """
     L, nh, d = q.shape
     group = nh // k.shape[1]
@@ -116,40 +118,50 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
             hidden = hidden | (n_idx <= i_idx - window)
         scores = scores.masked_fill(hidden, float("-inf"))
         probs = torch.softmax(scores, dim=-1)
-        out[:, j, :] = probs @ vj
+        out[:, j, :] = r(probs) @ vj
     return out
 
 
-def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
-    """down(silu(gate(x)) * up(x)), silu(z) = z * sigmoid(z), no bias (pagedllm/model/llama.py:163-171)."""
-    g = x @ w_gate.T
-    u = x @ w_up.T
-    return ((g * torch.sigmoid(g)) * u) @ w_down.T
+def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, r=lambda t: t) -> torch.Tensor:
+    """down(silu(gate(x)) * up(x)), silu(z) = z * sigmoid(z), no bias (pagedllm/model/llama.py:163-171).
+    ``r``: see ``forward``."""
+    g = r(x @ w_gate.T)
+    u = r(x @ w_up.T)
+    return r(r(r(g * torch.sigmoid(g)) * u) @ w_down.T)
 
 
 def attention_block(h: torch.Tensor, positions: torch.Tensor, w: dict, prefix: str, cfg: dict,
-                    inv_freq: torch.Tensor, window: int | None = None) -> torch.Tensor:
+                    inv_freq: torch.Tensor, window: int | None = None, r=lambda t: t) -> torch.Tensor:
     """q/k/v projections, rotation of q and k only, attention, output projection
-    (pagedllm/model/llama.py:146-160)."""
+    (pagedllm/model/llama.py:146-160).  ``r``: see ``forward``."""
     T = h.shape[0]
     nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-    q = (h @ w[prefix + "q_proj.weight"].T).view(T, nh, d)
-    k = (h @ w[prefix + "k_proj.weight"].T).view(T, nkv, d)
-    v = (h @ w[prefix + "v_proj.weight"].T).view(T, nkv, d)
+    q = r(h @ w[prefix + "q_proj.weight"].T).view(T, nh, d)
+    k = r(h @ w[prefix + "k_proj.weight"].T).view(T, nkv, d)
+    v = r(h @ w[prefix + "v_proj.weight"].T).view(T, nkv, d)
     angles = rotary_angles(positions, inv_freq)
-    q, k = apply_rotary(q, angles), apply_rotary(k, angles)
-    o = causal_attention(q, k, v, d ** -0.5, window)
-    return o.reshape(T, nh * d) @ w[prefix + "o_proj.weight"].T
+    q, k = r(apply_rotary(q, angles)), r(apply_rotary(k, angles))
+    o = r(causal_attention(q, k, v, d ** -0.5, window, r))
+    return r(o.reshape(T, nh * d) @ w[prefix + "o_proj.weight"].T)
 
 
 def forward(cfg: dict, weights: dict, tokens: list[int], dtype=torch.float32,
-            first_position: int = 0) -> torch.Tensor:
+            first_position: int = 0, stored: torch.dtype | None = None) -> torch.Tensor:
     """Logits [L, vocab] at every position of one whole sequence (pagedllm/model/llama.py:182-216).
 
     ``first_position`` shifts all positions together; only distances count, so the logits
     must not change (used as an invariant test, not by the engine).
+
+    ``stored``: a narrower type (bfloat16) in which the reference's model would keep its tensors.  Every
+    value that its modules hand on in that type is rounded to it here: the output of each norm (computed in
+    float, pagedllm/model/llama.py:80-83), of each projection, of the rotation (:120-128), of the
+    attention, of the activation and its product with the up branch (:171), each residual sum (:183-184)
+    and the logits (:216).  The arithmetic in between stays in ``dtype``.  This gives the size of the
+    rounding noise that the reference's own order of operations has at these sizes: a yardstick for the
+    engine's bfloat16 error, not a second oracle.
     """
     w = {k: v.to(dtype) for k, v in weights.items()}
+    r = (lambda t: t.to(stored).to(dtype)) if stored is not None else (lambda t: t)
     eps = cfg["rms_norm_eps"]
     ids = torch.tensor(tokens, dtype=torch.long)
     positions = torch.arange(first_position, first_position + len(tokens))
@@ -157,14 +169,14 @@ def forward(cfg: dict, weights: dict, tokens: list[int], dtype=torch.float32,
     x = w["model.embed_tokens.weight"][ids]                                   # llama.py:197
     for layer in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{layer}."
-        h = rms_norm(x, w[p + "input_layernorm.weight"], eps)
-        x = x + attention_block(h, positions, w, p + "self_attn.", cfg, inv_freq)   # llama.py:183
-        h = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
-        x = x + swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                       w[p + "mlp.down_proj.weight"])                          # llama.py:184
-    x = rms_norm(x, w["model.norm.weight"], eps)                               # llama.py:200
+        h = r(rms_norm(x, w[p + "input_layernorm.weight"], eps))
+        x = r(x + attention_block(h, positions, w, p + "self_attn.", cfg, inv_freq, r=r))   # llama.py:183
+        h = r(rms_norm(x, w[p + "post_attention_layernorm.weight"], eps))
+        x = r(x + swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                         w[p + "mlp.down_proj.weight"], r))                    # llama.py:184
+    x = r(rms_norm(x, w["model.norm.weight"], eps))                            # llama.py:200
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
-    return x @ head.T                                                          # llama.py:216
+    return r(x @ head.T)                                                       # llama.py:216
 
 
 def load_weights(model_dir: str) -> dict:

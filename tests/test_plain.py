@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 from tests.plain import llama_plain as plain
-from tests.tiny_configs import TINY_A, TINY_B
+from tests.tiny_configs import TINY_A, TINY_B, TINY_C
 
 
 def rnd(*shape, seed=0):
@@ -86,6 +86,33 @@ def test_llama3_rescale():
         plain.inverse_frequencies(d, theta, {"rope_type": "yarn", "factor": 2.0})
 
 
+def test_llama3_middle_band_joins_both_sides_without_a_jump():
+    """Across the band the slow-down goes from none (at wavelength orig/high, where the untouched short
+    waves end) to the full factor (at orig/low, where the slowed long waves begin), steadily.  With the
+    blend weight and its complement swapped the band would meet each side with a jump of the whole factor."""
+    factor, low, high, orig = 8.0, 1.0, 4.0, 64
+    sc = {"rope_type": "llama3", "factor": factor, "low_freq_factor": low, "high_freq_factor": high,
+          "original_max_position_embeddings": orig}
+    d, theta = 4096, 1.0e4                                   # 2048 frequencies: a fine grid across the band
+    base = plain.inverse_frequencies(d, theta, None, dtype=torch.float64)
+    scaled = plain.inverse_frequencies(d, theta, sc, dtype=torch.float64)
+    wavelen = 2 * math.pi / base
+    ratio = scaled / base                                     # 1 = untouched, 1/factor = fully slowed
+    mid = (wavelen >= orig / high) & (wavelen <= orig / low)
+    idx = mid.nonzero().flatten()
+    assert idx.numel() > 100
+    first, last = int(idx[0]), int(idx[-1])                   # shortest and longest wave inside the band
+    assert abs(float(ratio[first]) - 1.0) < 0.02 and abs(float(ratio[first - 1]) - 1.0) < 1e-12
+    assert abs(float(ratio[last]) - 1.0 / factor) < 0.02 and abs(float(ratio[last + 1]) - 1.0 / factor) < 1e-12
+    inside = ratio[first:last + 1]
+    assert (inside[1:] < inside[:-1]).all()                   # the longer the wave, the slower
+    # the blend is linear in the frequency: halfway between the edges' frequencies lies halfway between the effects
+    f_short, f_long = 2 * math.pi / (orig / high), 2 * math.pi / (orig / low)
+    f_half = 0.5 * (f_short + f_long)
+    near = int((base - f_half).abs().argmin())
+    assert abs(float(ratio[near]) - 0.5 * (1.0 + 1.0 / factor)) < 0.02
+
+
 def test_attention_is_the_library_routine():
     L, nh, nkv, d = 19, 4, 2, 16
     q, k, v = rnd(L, nh, d, seed=6), rnd(L, nkv, d, seed=7), rnd(L, nkv, d, seed=8)
@@ -156,6 +183,93 @@ def test_forward_invariants(cfg):
     l2 = plain.forward(c, w, other)
     torch.testing.assert_close(l2[:15], logits[:15])
     assert not torch.allclose(l2[15:], logits[15:], atol=1e-4)
+
+
+def library_forward(c, w, toks):
+    """The same model put together from the tensor library's own routines, in other formulations than the plain
+    implementation's: rotation as a multiplication of complex numbers (element i is the real and element i + d/2
+    the imaginary part), attention through the library's fused routine with its own causal mask and the kv heads
+    repeated, norm and activation as the library defines them."""
+    L, nh, nkv, d = len(toks), c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"]
+    eps = c["rms_norm_eps"]
+    inv = plain.inverse_frequencies(d, c["rope_theta"], c["rope_scaling"])
+    turn = torch.polar(torch.ones(L, d // 2), torch.arange(L, dtype=torch.float32)[:, None] * inv[None, :])[:, None, :]
+    def rotate(t):                                                       # [L, heads, d]
+        z = torch.complex(t[..., : d // 2], t[..., d // 2:]) * turn
+        return torch.cat([z.real, z.imag], dim=-1)
+    x = F.embedding(torch.tensor(toks), w["model.embed_tokens.weight"])
+    for l in range(c["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        h = F.rms_norm(x, (x.shape[-1],), w[p + "input_layernorm.weight"], eps)
+        q = rotate(F.linear(h, w[p + "self_attn.q_proj.weight"]).view(L, nh, d)).transpose(0, 1)
+        k = rotate(F.linear(h, w[p + "self_attn.k_proj.weight"]).view(L, nkv, d)).transpose(0, 1)
+        v = F.linear(h, w[p + "self_attn.v_proj.weight"]).view(L, nkv, d).transpose(0, 1)
+        o = F.scaled_dot_product_attention(q, k.repeat_interleave(nh // nkv, 0), v.repeat_interleave(nh // nkv, 0), is_causal=True)
+        x = x + F.linear(o.transpose(0, 1).reshape(L, nh * d), w[p + "self_attn.o_proj.weight"])
+        h = F.rms_norm(x, (x.shape[-1],), w[p + "post_attention_layernorm.weight"], eps)
+        x = x + F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                         w[p + "mlp.down_proj.weight"])
+    head = w["model.embed_tokens.weight"] if c["tie_word_embeddings"] else w["lm_head.weight"]
+    return F.linear(F.rms_norm(x, (x.shape[-1],), w["model.norm.weight"], eps), head)
+
+
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B, TINY_C])
+def test_forward_is_the_composition_of_library_routines(cfg):
+    """Whole forward, 100 positions (configuration B beyond its original 64 positions, with one frequency inside
+    the llama3 band; configuration C with a head size that is not hidden / heads)."""
+    c, w = random_weights(cfg, seed=3)
+    toks = torch.randint(0, c["vocab_size"], (100,), generator=torch.Generator().manual_seed(2)).tolist()
+    got, want = plain.forward(c, w, toks), library_forward(c, w, toks)
+    assert float((got - want).abs().max() / want.abs().max()) <= 1e-5
+
+
+def silence(w, c, which):
+    """A copy of the weights in which the named branch's last projection is zero in every layer."""
+    out = dict(w)
+    for l in range(c["num_hidden_layers"]):
+        for name in which:
+            key = f"model.layers.{l}.{name}.weight"
+            out[key] = torch.zeros_like(w[key])
+    return out
+
+
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B])
+def test_wiring_of_the_layer(cfg):
+    """What fixes where the norms and the residual sums stand, beside the reference's text:
+
+    * Both branches silent (output and down projections zero): every layer hands its input on untouched, so the
+      logits are norm(embedding) x head, a library routine.  A norm behind the sum (post-norm), or a residual
+      taken from the normed rows, would norm the stream once per layer and fail this.
+    * One branch silent, one layer deep: the stream is the embedding plus that one branch of the normed
+      embedding, each with its own norm weights (the two norms of a layer carry different weights here, so
+      feeding a branch from the other norm fails), and the feed-forward sees the stream after the attention's sum.
+    """
+    c, w = random_weights(cfg, seed=4)
+    eps, H = c["rms_norm_eps"], c["hidden_size"]
+    toks = torch.randint(0, c["vocab_size"], (23,), generator=torch.Generator().manual_seed(5)).tolist()
+    head = w["model.embed_tokens.weight"] if c["tie_word_embeddings"] else w["lm_head.weight"]
+    emb = F.embedding(torch.tensor(toks), w["model.embed_tokens.weight"])
+    last = lambda x: F.linear(F.rms_norm(x, (H,), w["model.norm.weight"], eps), head)
+    close = lambda a, b: torch.testing.assert_close(a, b, atol=2e-5, rtol=1e-4)
+
+    both_silent = silence(w, c, ["self_attn.o_proj", "mlp.down_proj"])
+    close(plain.forward(c, both_silent, toks), last(emb))
+
+    one = dict(c, num_hidden_layers=1)
+    p = "model.layers.0."
+    mlp = lambda h: F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                             w[p + "mlp.down_proj.weight"])
+    no_attention = silence(w, one, ["self_attn.o_proj"])
+    close(plain.forward(one, no_attention, toks), last(emb + mlp(F.rms_norm(emb, (H,), w[p + "post_attention_layernorm.weight"], eps))))
+
+    inv = plain.inverse_frequencies(c["head_dim"], c["rope_theta"], c["rope_scaling"])
+    attn = plain.attention_block(F.rms_norm(emb, (H,), w[p + "input_layernorm.weight"], eps), torch.arange(len(toks)), w,
+                                 p + "self_attn.", c, inv)
+    no_mlp = silence(w, one, ["mlp.down_proj"])
+    close(plain.forward(one, no_mlp, toks), last(emb + attn))
+    # both branches on: the feed-forward reads the stream after the attention has been added
+    after = emb + attn
+    close(plain.forward(one, w, toks), last(after + mlp(F.rms_norm(after, (H,), w[p + "post_attention_layernorm.weight"], eps))))
 
 
 def test_tied_head_uses_the_embedding_table():

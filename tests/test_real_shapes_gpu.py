@@ -5,8 +5,10 @@ tokens decoded one by one, and a second request fed in portions beside them; in 
 bfloat16 against the plain implementation."""
 
 import pytest
+import torch
 
 from tests import helpers
+from tests.plain import llama_plain
 from tests.helpers import TraceBuilder
 
 pytestmark = pytest.mark.gpu
@@ -38,17 +40,28 @@ SHAPES = {
 # on every row that sits inside that tail passes or fails by the choice of positions, so the bound of 4e-2
 # is held by the median of the rows (a systematic loss of precision moves all rows) and a single row may
 # reach 1.5 times that (a fault at one position, a wrong key or page, shows as 0.3 and more).
+# Beside that fixed bound the median is held against a yardstick of its own depth: the error that the plain
+# implementation itself shows when it rounds to bfloat16 wherever the reference's model hands a tensor on
+# (``forward(stored=bfloat16)``).  The engine rounds in fewer places than that (its fused kernels keep the
+# normed rows, the gate and the logits in float), so its median must not exceed the yardstick's: one more
+# rounding or a lossier order than the reference's in any kernel shows here long before it reaches 4e-2.
 TOL = {"float32": 2e-5, "bfloat16": 4e-2}
 ROW_FACTOR = {"float32": 1.0, "bfloat16": 1.5}
+YARDSTICK_FACTOR = 1.0
 
 
-def check_rows(got: dict, want: dict, dtype: str) -> None:
+def check_rows(got: dict, want: dict, dtype: str, yardstick: dict | None = None) -> None:
     errs = {key: helpers.worst(row, want[key[0]][key[1]]) for key, row in got.items()}
     for (rid, pos), err in errs.items():
         bound = TOL[dtype] * ROW_FACTOR[dtype]
         assert err <= bound, f"request {rid} position {pos}: relative error {err:.3g} > {bound}"
     median = sorted(errs.values())[len(errs) // 2]
     assert median <= TOL[dtype], f"median relative error of {len(errs)} rows {median:.3g} > {TOL[dtype]}"
+    if yardstick is not None:
+        ref = sorted(helpers.worst(yardstick[rid][pos], want[rid][pos]) for rid, pos in got)[len(errs) // 2]
+        print(f"median relative error: engine {median:.4f}, plain implementation with the reference's roundings {ref:.4f}")
+        assert median <= YARDSTICK_FACTOR * ref, (f"median relative error {median:.3g} against {ref:.3g} of the plain "
+                                                  "implementation rounding where the reference's model does")
 
 
 @pytest.fixture(scope="module", params=list(SHAPES))
@@ -58,13 +71,15 @@ def case(request, tmp_path_factory):
     vocab = cfg["vocab_size"]
     reqs = {"p": helpers.random_tokens(308, vocab, seed=1), "q": helpers.random_tokens(90, vocab, seed=2)}
     want = {rid: helpers.plain_logits(folder, toks) for rid, toks in reqs.items()}
-    return folder, reqs, want
+    cfg_plain, weights = llama_plain.read_config(folder), llama_plain.load_weights(folder)
+    yardstick = {rid: llama_plain.forward(cfg_plain, weights, toks, stored=torch.bfloat16).numpy() for rid, toks in reqs.items()}
+    return folder, reqs, want, yardstick
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_prompt_decoding_and_portions_at_real_sizes(case, dtype):
     from paged_llm_amd.engine.replay import ReplaySession
-    folder, reqs, want = case
+    folder, reqs, want, yardstick = case
     p, q = reqs["p"], reqs["q"]
     session = ReplaySession(folder, dtype, 320 + 128, None)
     trace = TraceBuilder()
@@ -78,7 +93,7 @@ def test_prompt_decoding_and_portions_at_real_sizes(case, dtype):
         trace.step(entries)
     got = helpers.replay_in_process(session, trace)
     assert len(got) == 5 + 8 + 3
-    check_rows(got, want, dtype)
+    check_rows(got, want, dtype, yardstick if dtype == "bfloat16" else None)
 
 
 def test_graph_replays_with_library_products_equal_eager_steps(tmp_path):
