@@ -172,6 +172,8 @@ E2E_CASES = [
 
 
 def e2e_prompts(num_prompts: int, input_len: int, output_len: int, shared_prefix: float, var_len: bool, vocab: int, seed: int = 0):
+    """The reference's workload generator, taken as it stands (benchmarks/bench.py:27-45 there, minus the tokenizer): the
+    same draws in the same order give the same prompts and lengths, and so the same numbers of engine steps."""
     import torch
     g = torch.Generator().manual_seed(seed)
     shared_len = int(input_len * shared_prefix)
@@ -288,6 +290,211 @@ def run_attention_cases() -> dict:
     return out
 
 
+def time_mixed_step(engine, decode_requests: int, context: int, portion: int, seed: int, repeats: int = 6) -> dict:
+    """One step that holds `decode_requests` decoded tokens at contexts near `context` beside a prompt portion of
+    `portion` tokens (what continuous batching runs whenever a request arrives): wall time of the step, and the
+    GPU's own time for it between two events (what is left is the host's share that the GPU waits for)."""
+    import torch
+    from paged_llm_amd import SamplingParams
+    vocab = engine.model.spec.vocab_size
+    sp = SamplingParams(temperature=0.0, max_tokens=repeats * 4 + 40, ignore_eos=True)
+    for p in random_prompts(decode_requests, context - repeats * 4 - 8, vocab, seed):
+        engine.add_request(p, sp)
+    while any(not r.decoding for r in engine.scheduler.active) or engine.scheduler.queue:
+        engine.step()
+    for _ in range(3):
+        engine.step()
+    best = None
+    for r in range(repeats):
+        prompt = random_prompts(1, portion, vocab, seed + 100 + r)[0]
+        rid = engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record()
+        out = engine.step()
+        end.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        assert len(out) == decode_requests + 1, "the step did not hold the decoded tokens and the portion"
+        gpu = start.elapsed_time(end) * 1e-3
+        if r >= 2 and (best is None or wall < best[0]):        # the shape is captured at its second sighting
+            best = (wall, gpu)
+        engine.step()                                          # a plain decode step in between
+    for r in list(engine.scheduler.active):
+        engine.abort_request(r.id)
+    wall, gpu = best
+    tokens = decode_requests + portion
+    return {"tokens": tokens, "ms": round(wall * 1e3, 3), "tokens_per_s": round(tokens / wall, 1)}
+
+
+def run_ragged64(cfg: dict, dtype: str, model_name: str, num_requests: int = 64, min_in: int = 64, max_in: int = 2048,
+                 out_len: int = 256, max_num_batched_tokens: int = 8192) -> dict:
+    """64 requests at once with prompts of `min_in`..`max_in` seeded random tokens (uniform) and `out_len` generated
+    tokens each, greedy, end-of-sequence ignored, max_num_seqs = 64: output tokens / wall time of generate(),
+    prompts included.  The roofline beside it is the decode step's at 64 requests of the mean final context."""
+    import torch
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    block = 16
+    pages = num_requests * ((max_in + out_len + block - 1) // block + 1) + 64
+    results = {}
+    with tempfile.TemporaryDirectory() as folder:
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        engine = LLMEngine(folder, EngineConfig(block_size=block, num_gpu_blocks=pages, max_num_seqs=num_requests,
+                                                max_num_batched_tokens=max_num_batched_tokens, max_model_len=max_in + out_len + 1,
+                                                dtype=dtype, seed=0, enable_prefix_caching=True), random_weights=0)
+        vocab = min(cfg["vocab_size"], 32000)
+        for seed in (1, 0):                                    # other prompts first: that pass captures the graphs
+            g = torch.Generator().manual_seed(seed)
+            lens = torch.randint(min_in, max_in + 1, (num_requests,), generator=g).tolist()
+            prompts = [torch.randint(100, vocab, (n,), generator=g).tolist() for n in lens]
+            steps0, pre0 = engine.stats.num_steps, engine.stats.num_preemptions
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=out_len, ignore_eos=True))
+            torch.cuda.synchronize()
+            elapsed = time.perf_counter() - t0
+        assert all(len(o.token_ids) == out_len for o in outs)
+        numbers = model_numbers(cfg, 2)
+        mean_context = sum(lens) / len(lens) + out_len / 2
+        step_bytes = numbers["weight_bytes"] + num_requests * mean_context * numbers["kv_bytes_per_token"]
+        roof = num_requests / (step_bytes / (PEAK_HBM_GBS * 1e9))
+        out_tokens = num_requests * out_len
+        results = {"output_tok_per_s": round(out_tokens / elapsed, 1), "elapsed_s": round(elapsed, 3),
+                   "total_tok_per_s": round((sum(lens) + out_tokens) / elapsed, 1), "prompt_tokens": sum(lens),
+                   "steps": engine.stats.num_steps - steps0, "preemptions": engine.stats.num_preemptions - pre0,
+                   "decode_roofline_tok_per_s": round(roof, 1), "frac_of_decode_roofline": round(out_tokens / elapsed / roof, 4)}
+    return results
+
+
+def run_prompt_sweep(cfg: dict, dtype: str, lengths: list) -> dict:
+    """Prefill of one prompt of each length in one step: tokens/s, milliseconds and the fraction of the matrix peak."""
+    short = "bf16" if dtype == "bfloat16" else "fp32"
+    out = {}
+    with tempfile.TemporaryDirectory() as folder:
+        engine = make_engine(cfg, folder, dtype, 4, max(lengths))
+        for n in lengths:
+            sec = time_prefill(engine, n, seed=200 + n)
+            out[str(n)] = {"tokens_per_s": round(n / sec, 1), "ms": round(sec * 1e3, 3),
+                           "frac": round(prefill_flops(cfg, n, 1) / sec / PEAK_FLOPS[short], 4)}
+    return out
+
+
+def run_context_sweep(cfg: dict, dtype: str, batch: int, contexts: list, steps: int, warmup: int) -> dict:
+    """Decode at `batch` requests for each context length, and the prefill of a prompt that long, each with its fraction."""
+    short = "bf16" if dtype == "bfloat16" else "fp32"
+    numbers = model_numbers(cfg, 2 if short == "bf16" else 4)
+    out = {}
+    for context in contexts:
+        with tempfile.TemporaryDirectory() as folder:
+            engine = make_engine(cfg, folder, dtype, max(batch, 4), context)
+            sec, mean_context = time_decode(engine, batch, context, steps, warmup, seed=3)
+            step_bytes = numbers["weight_bytes"] + batch * mean_context * numbers["kv_bytes_per_token"]
+            row = {"decode_tok_per_s": round(batch / sec, 1), "decode_ms": round(sec * 1e3, 4),
+                   "decode_frac_of_hbm": round(step_bytes / sec / 1e9 / PEAK_HBM_GBS, 4)}
+            if context <= 8192:
+                psec = time_prefill(engine, context, seed=300)
+                row.update(prefill_tok_per_s=round(context / psec, 1), prefill_ms=round(psec * 1e3, 3),
+                           prefill_frac=round(prefill_flops(cfg, context, 1) / psec / PEAK_FLOPS[short], 4))
+            out[str(context)] = row
+            del engine
+            import torch
+            torch.cuda.empty_cache()
+    return out
+
+
+def run_kernel_cases(cfg: dict, batch: int, context: int, prefill_tokens: int) -> dict:
+    """Every kernel of a decode step (`batch` requests at `context`) and of a prompt step (`prefill_tokens` tokens) on
+    its own, at the model's sizes: microseconds per call (replays of a HIP graph that holds calls on several copies of
+    the weights or pages, so that no call finds its operands in a cache) and its own roofline fraction: bytes it has to
+    read / time / 8 TB/s for the decode kernels, flops / time / 2.5 PFLOP/s for the prompt step's."""
+    import types
+    import torch
+    from paged_llm_amd.csrc import ops
+    from paged_llm_amd.parts.linear import gated_linear, linear
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    bs, dev, bf = 16, "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = lambda *shape: torch.randn(*shape, device=dev, dtype=bf, generator=g)
+
+    def per_call(fn, copies, calls_per_graph=None):
+        calls = calls_per_graph or 2 * copies
+        fn(0)
+        torch.cuda.synchronize()
+        stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(calls):
+                fn(i % copies)
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / (5 * calls) * 1e6
+
+    def weights(n, k):
+        copies = max(2, min(8, int(6.0e8 // (n * k * 2))))
+        return [rnd(n, k) * 0.02 for _ in range(copies)]
+
+    out = {}
+    for label, T, S, ctx_len in (("decode", batch, batch, context), ("prefill", prefill_tokens, 1, prefill_tokens)):
+        q_len = T // S
+        x, delta, nw = rnd(T, H), rnd(T, H), torch.ones(H, device=dev)
+        pages_per = (ctx_len + bs - 1) // bs
+        P = S * pages_per
+        kv_copies = max(2, min(6, int(6.0e8 // (S * ctx_len * nkv * d * 4))))
+        kps = [rnd(P, nkv, bs, d) for _ in range(kv_copies)]
+        vps = [rnd(P, nkv, d, bs) for _ in range(kv_copies)]
+        tables = torch.randperm(P, device=dev, generator=g).to(torch.int32).view(S, pages_per)
+        cu = torch.arange(0, T + 1, q_len, device=dev, dtype=torch.int32)
+        sl = torch.full((S,), ctx_len, device=dev, dtype=torch.int32)
+        positions = torch.cat([torch.arange(ctx_len - q_len, ctx_len, device=dev, dtype=torch.int32) for _ in range(S)])
+        slots = torch.cat([tables[s, (positions[s * q_len:(s + 1) * q_len] // bs).long()] * bs + positions[s * q_len:(s + 1) * q_len] % bs
+                           for s in range(S)]).to(torch.int32)
+        inv = 1.0 / (cfg["rope_theta"] ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        ang = torch.outer(torch.arange(ctx_len, dtype=torch.float32), inv)
+        rope = types.SimpleNamespace(cos=ang.cos().to(dev).contiguous(), sin=ang.sin().to(dev).contiguous(), rotary_dim=d, interleaved=False)
+        ctx = types.SimpleNamespace(num_seqs=S, max_q_len=q_len, max_k_len=ctx_len, q_lens=[q_len] * S, k_lens=[ctx_len] * S, capturing=False,
+                                    device=torch.device(dev), launch_cache={}, graph_layout=None)
+        from paged_llm_amd.parts.linear import qkv_rotary_cache
+        from paged_llm_amd.parts.norm import PendingNorm
+        w_qkv, w_o, w_gu, w_down, w_head = weights((nh + 2 * nkv) * d, H), weights(H, nh * d), weights(2 * I, H), weights(H, I), weights(V, H)
+        attn_in, act, last = rnd(T, (nh + 2 * nkv) * d), rnd(T, I), rnd(min(T, S), H)
+        pend = lambda rows=None: PendingNorm(nw, 1e-5, x.clone() if rows is None else rows, delta if rows is None else None)
+        cases = {
+            "qkv product (norm in front, rotary and cache write behind)": (
+                lambda i: qkv_rotary_cache(pend(), w_qkv[i % len(w_qkv)], positions, rope, nh, nkv, d, slots, kps[i % kv_copies], vps[i % kv_copies], bs),
+                len(w_qkv), w_qkv[0].numel() * 2, 2.0 * T * w_qkv[0].numel()),
+            "attention over the cache": (
+                lambda i: ops.paged_attention(attn_in, kps[i % kv_copies], vps[i % kv_copies], tables, cu, sl, nh, nkv, d, d ** -0.5, 0, ctx),
+                kv_copies, S * ctx_len * nkv * d * 4, 4.0 * nh * d * S * sum(ctx_len - q_len + j + 1 for j in range(q_len))),
+            "output product": (lambda i: linear(attn_in[:, :nh * d], w_o[i % len(w_o)]), len(w_o), w_o[0].numel() * 2, 2.0 * T * w_o[0].numel()),
+            "gate/up product (norm in front, SiLU gating behind)": (
+                lambda i: gated_linear(pend(), w_gu[i % len(w_gu)]), len(w_gu), w_gu[0].numel() * 2, 2.0 * T * w_gu[0].numel()),
+            "down product": (lambda i: linear(act, w_down[i % len(w_down)]), len(w_down), w_down[0].numel() * 2, 2.0 * T * w_down[0].numel()),
+            "head product (last norm in front, float logits)": (
+                lambda i: linear(pend(last), w_head[i % len(w_head)], out_dtype=torch.float32), len(w_head), w_head[0].numel() * 2,
+                2.0 * last.shape[0] * w_head[0].numel()),
+        }
+        rows = {}
+        for name, (fn, copies, nbytes, flops) in cases.items():
+            us = per_call(fn, copies)
+            row = {"us": round(us, 2)}
+            if label == "decode":
+                row.update(mb=round(nbytes / 1e6, 2), gb_per_s=round(nbytes / us / 1e3, 1), frac_of_hbm=round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4))
+            else:
+                row.update(tflops=round(flops / us / 1e6, 1), frac_of_matrix_peak=round(flops / us * 1e6 / PEAK_FLOPS["bf16"], 4))
+            rows[name] = row
+        out[f"{label}_{'b%d_ctx%d' % (batch, context) if label == 'decode' else 'tokens%d' % prefill_tokens}"] = rows
+        del kps, vps, w_qkv, w_o, w_gu, w_down, w_head
+        torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -312,6 +519,11 @@ def main() -> int:
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--max-num-batched-tokens", type=int, default=4096)
     ap.add_argument("--no-prefix-caching", action="store_true")
+    ap.add_argument("--workload", choices=["ragged64"], default=None, help="ragged64: 64 requests at once, prompts of 64-2048 tokens, "
+                    "256 generated tokens each (use with --model llama-3.1-8b)")
+    ap.add_argument("--prompt-sweep", default=None, metavar="N,N,...", help="prefill of one prompt of each of these lengths")
+    ap.add_argument("--context-sweep", default=None, metavar="N,N,...", help="decode at --batch requests (and prefill up to 8192) at each of these contexts")
+    ap.add_argument("--kernels", action="store_true", help="every kernel of a decode step and of a prompt step on its own, with its fraction")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -328,6 +540,24 @@ def main() -> int:
     nbytes = 2 if short == "bf16" else 4
     numbers = model_numbers(cfg, nbytes)
 
+    if args.workload == "ragged64":
+        print(json.dumps({"metric": f"output tokens/s, 64 ragged requests at once, prompts 64-2048 tokens, 256 generated each ({model_name}, random weights)",
+                          "dtype": short, "unit": "tokens/s", "result": run_ragged64(cfg, args.dtype, model_name)}))
+        return 0
+    if args.prompt_sweep:
+        lengths = [int(n) for n in args.prompt_sweep.split(",")]
+        print(json.dumps({"metric": f"prefill of one prompt in one step ({model_name}, random weights)", "dtype": short,
+                          "lengths": run_prompt_sweep(cfg, args.dtype, lengths)}))
+        return 0
+    if args.context_sweep:
+        contexts = [int(n) for n in args.context_sweep.split(",")]
+        print(json.dumps({"metric": f"decode at batch {args.batch} and prefill by context length ({model_name}, random weights)", "dtype": short,
+                          "contexts": run_context_sweep(cfg, args.dtype, args.batch, contexts, max(16, args.steps // 2), max(4, args.warmup // 2))}))
+        return 0
+    if args.kernels:
+        print(json.dumps({"metric": f"kernels of one layer and the head on their own ({model_name}, bf16)",
+                          "cases": run_kernel_cases(cfg, args.batch, args.context, PREFILL_TOKENS)}))
+        return 0
     if args.attention:
         print(json.dumps({"metric": "attention op, microseconds per call (bf16, pages of 16 positions)", "cases": run_attention_cases()}))
         return 0
@@ -370,15 +600,22 @@ def main() -> int:
             for b in (1, 64):
                 s, _ = time_decode(engine, b, args.context, max(16, args.steps // 2), max(4, args.warmup // 2), seed=10 + b)
                 points[f"decode_b{b}"] = round(b / s, 1)
+            # a step of continuous batching: the batch's decoded tokens beside a prompt portion of 256 tokens
+            mixed = time_mixed_step(engine, args.batch, args.context, 256, seed=50)
+            points[f"mixed_b{args.batch}_p256"] = mixed["tokens_per_s"]
+            record["mixed_step"] = mixed
             record["points"] = points
             psec = time_prefill(engine, PREFILL_TOKENS, seed=100)
             flops = prefill_flops(cfg, PREFILL_TOKENS, 1)
             record["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3),
                                  "frac": round(flops / psec / PEAK_FLOPS[short], 4)}
+            del engine
+            torch.cuda.empty_cache()
+            # the reference's end-to-end workload at 8 and 64 requests at a time (64 requests, 256 in / 128 out): output tokens/s
+            e2e = run_e2e(cfg, args.dtype, [c for c in E2E_CASES if c["name"] in ("256in_128out_b8", "256in_128out_b64")])
+            record["e2e"] = {name: row["output_tok_per_s"] for name, row in e2e.items()}
             if short == "bf16":
-                # the same two fractions against what the GPU gives to a plain large read and a plain large product
-                del engine
-                torch.cuda.empty_cache()
+                # the same two fractions against what the GPU gives to a plain large copy and a plain large product
                 peaks = measured_peaks()
                 record["measured_peaks"] = dict(peaks, decode_frac=round(achieved / peaks["hbm_copy_gbs"], 4),
                                                 prefill_frac=round(flops / psec / (peaks["bf16_product_tflops"] * 1e12), 4))

@@ -17,8 +17,9 @@ class EngineConfig:
     max_model_len: int = 4096
     enable_prefix_caching: bool = True
     enable_chunked_prefill: bool = True
-    # "auto" | "hip": this engine's own kernels (there is one implementation; the reference's "triton",
-    # "flash" and "torch" are refused).
+    # Inert: it selects nothing.  The reference's command line and configuration carry this option
+    # (pagedllm/config.py), so a caller's "auto" is accepted, as is "hip" (this engine's own kernels, the one
+    # implementation there is); the reference's "triton", "flash" and "torch" are refused.
     attention_backend: str = "auto"
     dtype: str = "auto"            # "auto" | "bfloat16" | "float32"
     device: str = "cuda"

@@ -22,6 +22,13 @@ def resolve_dtype(requested: str, stored: str) -> torch.dtype:
     return _DTYPES[requested]
 
 
+def _rotary_keys(cfg: dict) -> tuple:
+    """(theta, the other rotary keys) from either spelling (pagedllm/model/llama.py:40-45)."""
+    rope = dict(cfg.get("rope_parameters") or cfg.get("rope_scaling") or {})
+    theta = rope.pop("rope_theta", None) or cfg.get("rope_theta", 10000.0)
+    return theta, rope
+
+
 @dataclass
 class LlamaConfig:
     vocab_size: int
@@ -42,11 +49,11 @@ class LlamaConfig:
 
     @classmethod
     def from_hf(cls, cfg: dict) -> "LlamaConfig":
-        """Both spellings of the rotary keys: {"rope_parameters": {...}} of newer exporters, or
-        "rope_theta" + "rope_scaling" (pagedllm/model/llama.py:40-45)."""
+        """From the keys of a Llama config.json.  Which keys there are, their defaults and the two spellings
+        of the rotary keys ({"rope_parameters": {...}} of newer exporters, or "rope_theta" + "rope_scaling") are
+        a file format, taken as the reference reads it (pagedllm/model/llama.py:37-60)."""
         heads = cfg["num_attention_heads"]
-        rope = dict(cfg.get("rope_parameters") or cfg.get("rope_scaling") or {})
-        rope_theta = rope.pop("rope_theta", None) or cfg.get("rope_theta", 10000.0)
+        rope_theta, rope = _rotary_keys(cfg)
         rope_type = rope.get("rope_type", rope.get("type", "default"))
         out = cls(
             vocab_size=int(cfg["vocab_size"]),

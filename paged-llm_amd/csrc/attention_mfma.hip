@@ -404,6 +404,7 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
     kvh = blockIdx.x;
     seq = work[2 * blockIdx.y];
     listed_tile = work[2 * blockIdx.y + 1];
+    if (seq < 0) return;                                          // an unused entry of a list of fixed length
   } else {
     seq = blockIdx.x / num_kv_heads;
     kvh = blockIdx.x - seq * num_kv_heads;

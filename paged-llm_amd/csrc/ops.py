@@ -542,36 +542,49 @@ def _upload_ints(values: np.ndarray, device) -> torch.Tensor:
     return out
 
 
+def prompt_tiles(q_lens: list, k_lens: list, first_seq: int, group: int, capacity: int | None = None) -> np.ndarray | None:
+    """Host side of the prompt kernel's work list for the sequences from ``first_seq`` on: int32 [n, 2] pairs
+    (sequence counted from ``first_seq``, tile of PROMPT_TILE_COLUMNS query columns), the tiles that see the most
+    keys first.  Without ``capacity``: None when the sequences are all alike (the kernel's own grid then does the
+    same).  With ``capacity``: always a list, of exactly that many pairs, the unused ones (-1, -1)."""
+    counts = [-(-n * group // PROMPT_TILE_COLUMNS) for n in q_lens[first_seq:]]
+    if capacity is None and len(set(counts)) == 1 and len(set(k_lens[first_seq:])) == 1:
+        return None
+    seqs, tiles, keys = [], [], []
+    for i, n in enumerate(counts):
+        s = first_seq + i
+        t = np.arange(n, dtype=np.int64)
+        seqs.append(np.full(n, i, dtype=np.int64))
+        tiles.append(t)
+        keys.append(k_lens[s] - q_lens[s] + (t + 1) * PROMPT_TILE_COLUMNS // group)
+    seqs, tiles, keys = np.concatenate(seqs), np.concatenate(tiles), np.concatenate(keys)
+    order = np.argsort(-keys, kind="stable")
+    pairs = np.stack([seqs[order], tiles[order]], axis=1).astype(np.int32)
+    if capacity is not None:
+        _need(pairs.shape[0] <= capacity, f"{pairs.shape[0]} prompt tiles for a list of {capacity}")
+        pairs = np.concatenate([pairs, np.full((capacity - pairs.shape[0], 2), -1, dtype=np.int32)])
+    return pairs
+
+
+def prompt_tiles_capacity(num_sequences: int, tokens: int, group: int) -> int:
+    """Most pairs ``prompt_tiles`` can give for ``num_sequences`` sequences that share ``tokens`` tokens."""
+    return -(-tokens * group // PROMPT_TILE_COLUMNS) + num_sequences
+
+
 def prompt_work_list(ctx, first_seq: int, group: int) -> torch.Tensor | None:
-    """The prompt kernel's work for the sequences from ``first_seq`` on: int32 [n, 2] pairs (sequence counted
-    from ``first_seq``, tile), the tiles that see the most keys first.  Workgroups take them in that order, so
-    long pieces start first and none is launched for a tile that a shorter sequence does not have (with one
-    long and many short sequences most of a rectangular grid is empty, and handing out empty workgroups was
-    measured at 80 us for 3,800 of them).  Built from the host lengths once per step and kept in the context;
-    None when the sequences are all alike and the kernel's own grid does the same."""
+    """The prompt kernel's work for the sequences from ``first_seq`` on (``prompt_tiles``) on the device.
+    Workgroups take the pairs in order, so long pieces start first and none is launched for a tile that a shorter
+    sequence does not have (with one long and many short sequences most of a rectangular grid is empty, and
+    handing out empty workgroups was measured at 80 us for 3,800 of them).  Built from the host lengths once per
+    step and kept in the context; None when the sequences are all alike and the kernel's own grid does the same."""
     cache = getattr(ctx, "launch_cache", None)
     key = ("prompt_tiles", first_seq, group)
     if cache is not None and key in cache:
         return cache[key]
-    counts = {-(-n * group // PROMPT_TILE_COLUMNS) for n in ctx.q_lens[first_seq:]}
-    if len(counts) == 1 and len(set(ctx.k_lens[first_seq:])) == 1:
-        # every sequence has the same tiles with the same keys: the kernel's own grid (sequence x kv head, tiles
-        # from the last one down) has no empty workgroup and hands the work out in the same order
-        if cache is not None:
-            cache[key] = None
-        return None
-    seqs, tiles, keys = [], [], []
-    for s in range(first_seq, len(ctx.q_lens)):
-        n = -(-ctx.q_lens[s] * group // PROMPT_TILE_COLUMNS)
-        t = np.arange(n, dtype=np.int64)
-        seqs.append(np.full(n, s - first_seq, dtype=np.int64))
-        tiles.append(t)
-        keys.append(ctx.k_lens[s] - ctx.q_lens[s] + (t + 1) * PROMPT_TILE_COLUMNS // group)
-    seqs, tiles, keys = np.concatenate(seqs), np.concatenate(tiles), np.concatenate(keys)
+    pairs = prompt_tiles(ctx.q_lens, ctx.k_lens, first_seq, group)
     work = None
-    if 0 < seqs.size <= 65535:
-        order = np.argsort(-keys, kind="stable")
-        work = _upload_ints(np.stack([seqs[order], tiles[order]], axis=1), ctx.device)
+    if pairs is not None and 0 < pairs.shape[0] <= 65535:
+        work = _upload_ints(pairs, ctx.device)
     if cache is not None:
         cache[key] = work
     return work
@@ -596,6 +609,25 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
     if mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs) and q.stride(0) % 8 == 0:
         group = num_heads // num_kv_heads
         lds = _max_lds_bytes(q.device)
+        layout = getattr(ctx, "graph_layout", None)
+        if ctx.capturing and layout is not None:
+            # A step with prompt portions that is replayed from a graph: the launches depend on the layout's counts
+            # and the context bound only.  The single-token rows go to the kernel that cuts their keys into
+            # partitions, the portions to the prompt kernel with the work list the step function has put there.
+            few = layout.num_single_rows
+            work = ctx.launch_cache.get(("prompt_tiles", few, group))
+            _need(work is not None, "a replayed step with prompt portions needs the prompt kernel's work list in the context")
+            work = work.view(-1, 2)
+            out = torch.empty((q.shape[0], num_heads * head_dim), dtype=q.dtype, device=q.device)
+            if few:
+                waves, size, parts = attention_plan(few, num_kv_heads, 1, ctx.max_k_len, group, head_dim, lds)
+                paged_attention_mfma(q[:few], k_pages, v_pages, block_tables[:few], cu_seqlens_q[:few + 1], seq_lens_k[:few],
+                                     num_heads, num_kv_heads, head_dim, scale, window, 1, size, parts, waves,
+                                     2 if waves == 1 else 0, out=out[:few])
+            prompt_q = max(layout.portion_tokens, FEW_QUERY_COLUMNS // group + 1)     # enough columns for the prompt kernel's form
+            paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
+                                 num_kv_heads, head_dim, scale, window, prompt_q, 0, 1, 1, 2, out=out, work_list=work)
+            return out
         q_lens, k_lens = ctx.q_lens, ctx.k_lens
         few = 0
         while few < len(q_lens) and q_lens[few] * group <= FEW_QUERY_COLUMNS:

@@ -59,8 +59,11 @@ class StepContext:
     # num_tokens/num_seqs only, and `max_k_len` is an upper bound, not the batch's own maximum.
     capturing: bool = False
     # Device arrays that a part derives from the host lengths, kept for the other layers of the step
-    # (the list of prompt tiles the attention kernel works through, for one).
+    # (the list of prompt tiles the attention kernel works through, for one).  When a step with prompt
+    # portions is replayed from a graph, the step function fills them in beforehand (see
+    # ``parts.base.Part.graph_step_arrays``) and ``graph_layout`` says how the batch is laid out.
     launch_cache: dict = field(default_factory=dict)
+    graph_layout: object = None
 
     @property
     def decode_only(self) -> bool:

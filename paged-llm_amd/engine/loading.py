@@ -47,7 +47,7 @@ def random_model(hf_config: dict, seed: int = 0, dtype: str = "auto", device="cu
 
 
 def build_runtime(model: DecoderModel, block_size: int, num_pages: int | dict, num_state_slots: int,
-                  enable_prefix_caching: bool, use_graphs: bool = False):
+                  enable_prefix_caching: bool, use_graphs: bool = False, **runner_options):
     """(CacheManager, KVCacheStorage, ModelRunner) for a model: one page pool per cache group,
     one state slot pool when a mixer keeps per-request state."""
     groups = model.cache_groups()
@@ -56,5 +56,5 @@ def build_runtime(model: DecoderModel, block_size: int, num_pages: int | dict, n
     manager = CacheManager(specs, num_pages, block_size, enable_prefix_caching,
                            num_state_slots=num_state_slots if uses_state else 0)
     storage = KVCacheStorage(groups, num_pages, block_size, model.dtype, model.device)
-    runner = ModelRunner(model, storage, num_state_slots if uses_state else 0, use_graphs=use_graphs)
+    runner = ModelRunner(model, storage, num_state_slots if uses_state else 0, use_graphs=use_graphs, **runner_options)
     return manager, storage, runner

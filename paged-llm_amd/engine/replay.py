@@ -33,7 +33,8 @@ class ReplaySession:
             raise ValueError(f"block size must be a power of two, got {block_size}")
         num_pages = max(1, (max_tokens + bs - 1) // bs)
         self.manager, self.storage, self.runner = build_runtime(
-            self.model, bs, num_pages, MAX_LIVE_REQUESTS, enable_prefix_caching=False, use_graphs=True)
+            self.model, bs, num_pages, MAX_LIVE_REQUESTS, enable_prefix_caching=False, use_graphs=True,
+            graph_after_sightings=1)
         self.groups = list(self.manager.groups)
         self.computed: dict = {}
         self.out_dir = out_dir

@@ -23,13 +23,22 @@ class StepError(ValueError):
 
 class ModelRunner:
     def __init__(self, model, kv_storage: KVCacheStorage, num_state_slots: int = 0, use_graphs: bool = False,
-                 max_graph_batch: int = 256):
+                 max_graph_batch: int = 256, max_graph_tokens: int = 1024, graph_after_sightings: int = 2):
         self.model = model
         # Graph replay needs every part of the model to do nothing but launch kernels on the
-        # current stream; parts say so with ``graph_capturable``.
+        # current stream; parts say so with ``graph_capturable`` (steps of single tokens) and
+        # ``graph_capturable_prompts`` (steps that hold prompt portions as well).
         self.use_graphs = bool(use_graphs) and model.graph_capturable()
+        self.prompt_graphs = self.use_graphs and model.graph_capturable(prompts=True)
         self.max_graph_batch = max_graph_batch
+        # Steps with prompt portions are replayed from graphs up to this many portion tokens (beyond it the
+        # GPU's time hides the host's), and once their shape has been seen this often (a capture costs
+        # several steps' time; shapes that never come back are not worth one).
+        self.max_graph_tokens = max_graph_tokens
+        self.graph_after_sightings = max(1, graph_after_sightings)
+        self._sightings: dict = {}
         self._graphs: dict = {}
+        self._graph_pool = None               # one memory pool for the activations of all prompt-step graphs
         self.kv = kv_storage
         self.device = model.device
         self.block_size = kv_storage.block_size
@@ -332,6 +341,194 @@ class ModelRunner:
             staged[s] = "empty"
         return n_want
 
+    # ------------------------------------------------------------------ steps with prompt portions as HIP graphs
+    MAX_GRAPH_PORTIONS = 4
+
+    @staticmethod
+    def _token_bucket(n: int) -> int:
+        """Portion tokens a graph is captured for: steps of 32 up to 128, of 64 up to 512, of 128 up to 1024, of 256 beyond."""
+        for limit, step in ((128, 32), (512, 64), (1024, 128)):
+            if n <= limit:
+                return -(-n // step) * step
+        return -(-n // 256) * 256
+
+    def _prompt_graph_key(self, entries: list):
+        """A step that holds prompt portions (entries of two or more tokens), alone or beside single tokens, can be
+        replayed from a graph whose launch shapes depend on: the number of single-token rows (rounded up as for
+        decode steps), the number of portions (at most four), the portions' tokens together (rounded up to a
+        bucket; a sequence of padding tokens that writes nothing fills the rest, at least one), the wanted rows and
+        a bound on the context lengths.  None when the step is not of that kind or too large to be worth it."""
+        if not self.prompt_graphs:
+            return None
+        singles = portions = portion_tokens = asked = longest = 0
+        for e in entries:
+            n = len(e.tokens)
+            if n == 1:
+                singles += 1
+            else:
+                portions += 1
+                portion_tokens += n
+            asked += len(e.want)
+            longest = max(longest, e.start + n)
+        if portions == 0 or portions > self.MAX_GRAPH_PORTIONS or singles > self.max_graph_batch:
+            return None
+        bucket = self._token_bucket(portion_tokens + 1)
+        bound = ((longest + 511) // 512) * 512 if longest <= 8192 else 1 << (longest - 1).bit_length()
+        bound = min(bound, max(self.model.max_positions, longest))
+        if bucket > min(self.max_graph_tokens, bound):      # (the padding sequence's positions stay below the bound)
+            return None
+        rows = self._bucket(singles) if singles else 0
+        wanted = max(self._bucket(asked), asked) if asked else 0
+        return ("prompt", rows, portions, bucket, wanted, bound)
+
+    def _prompt_layout(self, key):
+        _, rows, portions, bucket, wanted, bound = key
+        T, S = rows + bucket, rows + portions + 1
+        fixed = (bound + self.block_size - 1) // self.block_size
+        sizes = [T, T, S + 1, S, S, S, wanted]
+        table_shapes = {}
+        for name in self.group_specs:
+            sizes += [S * fixed, T]
+            table_shapes[name] = (S, fixed)
+        from ..parts.base import GraphLayout
+        layout = GraphLayout(num_single_rows=rows, num_portions=portions + 1, portion_tokens=bucket)
+        arrays = self.model.graph_step_arrays(layout)            # key -> (capacity in int32, fill(q_lens, k_lens) -> array)
+        array_keys = list(arrays)
+        sizes += [arrays[k][0] for k in array_keys]
+        offsets, cursor = [], 0
+        for n in sizes:
+            offsets.append(cursor)
+            cursor += n + (-n) % 4
+        return dict(T=T, S=S, fixed=fixed, sizes=sizes, offsets=offsets, total=cursor, table_shapes=table_shapes,
+                    arrays=arrays, array_keys=array_keys, layout=layout)
+
+    def _stage_prompt_graph(self, entry: dict, entries: list) -> int:
+        """Checks the batch (as ``_stage`` does) and lays it out in the fixed shape of the graph: single-token rows,
+        empty rows up to their bucket, the portions in ascending order of their lengths, the padding sequence."""
+        _, rows, portions, bucket, wanted, bound = entry["key"]
+        lay = entry["layout"]
+        T, S, fixed, offsets, sizes = lay["T"], lay["S"], lay["fixed"], lay["offsets"], lay["sizes"]
+        buf, off, siz, host = self._stage(entries, fixed_blocks=fixed)
+        piece = lambda i: buf[off[i]: off[i] + siz[i]]
+        q_real, k_real = host["q_lens"], host["k_lens"]
+        ones = sum(1 for n in q_real if n == 1)
+        tp = host["T"] - ones
+        pad_rows, pad_tokens = rows - ones, bucket - tp
+        view = entry["view"]
+        def put(i, values):
+            view[offsets[i]: offsets[i] + sizes[i]] = values
+        def spread(values, fill_rows, fill_tail, dtype=np.int32):
+            """per-token array of the real batch -> the fixed batch"""
+            values = np.asarray(values, dtype=dtype)
+            return np.concatenate([values[:ones], fill_rows, values[ones:], fill_tail])
+        zeros_rows, spare = np.zeros(pad_rows, dtype=np.int32), self.spare_state_slot
+        put(0, spread(piece(0), zeros_rows, np.zeros(pad_tokens, dtype=np.int32)))
+        put(1, spread(piece(1), zeros_rows, np.arange(pad_tokens, dtype=np.int32)))
+        q_fixed = [1] * rows + q_real[ones:] + [pad_tokens]
+        k_fixed = k_real[:ones] + [1] * pad_rows + k_real[ones:] + [pad_tokens]
+        put(2, np.concatenate([[0], np.cumsum(q_fixed)]).astype(np.int32))
+        put(3, k_fixed)
+        per_seq = lambda values, fill: np.concatenate([values[:ones], np.full(pad_rows, fill, dtype=np.int32), values[ones:], [fill]])
+        put(4, per_seq(piece(4), spare))
+        put(5, per_seq(piece(5), 0))
+        want_rows = piece(6)
+        n_want = int(want_rows.size)
+        shifted = np.where(want_rows >= ones, want_rows + pad_rows, want_rows)
+        put(6, np.concatenate([shifted, np.zeros(sizes[6] - n_want, dtype=np.int32)]))
+        for gi, name in enumerate(self.group_specs):
+            tables = piece(7 + 2 * gi).reshape(host["S"], fixed)
+            out = view[offsets[7 + 2 * gi]: offsets[7 + 2 * gi] + S * fixed].reshape(S, fixed)
+            out[:ones] = tables[:ones]
+            out[ones:rows] = 0
+            out[rows:rows + portions] = tables[ones:]
+            out[rows + portions] = 0
+            put(8 + 2 * gi, spread(piece(8 + 2 * gi), np.full(pad_rows, -1, dtype=np.int32), np.full(pad_tokens, -1, dtype=np.int32)))
+        base = 7 + 2 * len(self.group_specs)
+        for j, akey in enumerate(lay["array_keys"]):
+            capacity, fill = lay["arrays"][akey]
+            values = np.asarray(fill(q_fixed, k_fixed), dtype=np.int32).reshape(-1)
+            assert values.size == capacity, f"step array {akey!r}: {values.size} values for a capacity of {capacity}"
+            put(base + j, values)
+        return n_want
+
+    def _new_prompt_graph(self, key) -> dict:
+        lay = self._prompt_layout(key)
+        on_gpu = self.device.type == "cuda"
+        pinned = torch.zeros(max(lay["total"], 1), dtype=torch.int32, pin_memory=on_gpu)
+        return dict(key=key, layout=lay, pinned=pinned, view=pinned.numpy(),
+                    static=torch.zeros(max(lay["total"], 1), dtype=torch.int32, device=self.device),
+                    copied=torch.cuda.Event() if on_gpu else None)
+
+    def _prompt_context(self, entry: dict) -> StepContext:
+        _, rows, portions, bucket, wanted, bound = entry["key"]
+        lay = entry["layout"]
+        S = lay["S"]
+        host = dict(T=lay["T"], S=S, q_lens=[1] * rows + [bucket] * (portions + 1), k_lens=[bound] * S,
+                    slots_state=[self.spare_state_slot] * S, table_shapes=lay["table_shapes"])
+        ctx = self._context(entry["static"], lay["offsets"], lay["sizes"], host, max_k_len=bound, capturing=True)
+        ctx.graph_layout = lay["layout"]
+        base = 7 + 2 * len(self.group_specs)
+        for j, akey in enumerate(lay["array_keys"]):
+            ctx.launch_cache[akey] = entry["static"][lay["offsets"][base + j]: lay["offsets"][base + j] + lay["sizes"][base + j]]
+        return ctx
+
+    def _capture_prompt_graph(self, entry: dict) -> None:
+        """Warm-up and capture on a batch of the graph's shape that writes nothing: empty single-token rows and
+        portions that are all padding."""
+        _, rows, portions, bucket, wanted, bound = entry["key"]
+        lay = entry["layout"]
+        view, offsets, sizes, S, T = entry["view"], lay["offsets"], lay["sizes"], lay["S"], lay["T"]
+        view[:] = 0
+        each = [bucket // (portions + 1)] * (portions + 1)
+        each[-1] += bucket - sum(each)
+        q_lens = [1] * rows + each
+        view[offsets[1]: offsets[1] + T] = np.concatenate([np.zeros(rows, dtype=np.int32)] + [np.arange(n, dtype=np.int32) for n in each])
+        view[offsets[2]: offsets[2] + S + 1] = np.concatenate([[0], np.cumsum(q_lens)])
+        view[offsets[3]: offsets[3] + S] = q_lens
+        view[offsets[4]: offsets[4] + S] = self.spare_state_slot
+        base = 7 + 2 * len(self.group_specs)
+        for gi in range(len(self.group_specs)):
+            view[offsets[8 + 2 * gi]: offsets[8 + 2 * gi] + T] = -1
+        for j, akey in enumerate(lay["array_keys"]):
+            capacity, fill = lay["arrays"][akey]
+            view[offsets[base + j]: offsets[base + j] + capacity] = np.asarray(fill(q_lens, q_lens), dtype=np.int32).reshape(-1)
+        entry["static"].copy_(entry["pinned"])
+        ctx = self._prompt_context(entry)
+        stream = torch.cuda.Stream(device=self.device)
+        stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(stream):
+            self.model.forward(ctx, self.kv, self.states)
+        torch.cuda.current_stream(self.device).wait_stream(stream)
+        torch.cuda.synchronize(self.device)
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream, pool=self._graph_pool):
+            logits = self.model.forward(ctx, self.kv, self.states)
+        entry.update(graph=graph, logits=logits, ctx=ctx)
+        if len(self._graphs) >= 64:
+            self._graphs.pop(next(iter(self._graphs)))
+        self._graphs[entry["key"]] = entry
+
+    def _prompt_graph_step(self, key, entries: list, borrow: bool) -> torch.Tensor | None:
+        entry = self._graphs.get(key)
+        if entry is None:
+            seen = self._sightings[key] = self._sightings.get(key, 0) + 1
+            if seen < self.graph_after_sightings:
+                if len(self._sightings) > 4096:
+                    self._sightings.clear()
+                return None                                 # run it eagerly this time
+            entry = self._new_prompt_graph(key)
+            self._capture_prompt_graph(entry)
+        else:
+            entry["copied"].synchronize()
+        n_want = self._stage_prompt_graph(entry, entries)
+        entry["static"].copy_(entry["pinned"], non_blocking=True)
+        entry["copied"].record()
+        entry["graph"].replay()
+        logits = entry["logits"][:n_want]
+        return logits if borrow else logits.clone()
+
     def _graph_step(self, key, entries: list, borrow: bool = False) -> torch.Tensor:
         entry = self._graphs.get(key)
         if entry is None:
@@ -362,5 +559,10 @@ class ModelRunner:
         key = self._graph_key(entries)
         if key is not None:
             return self._graph_step(key, entries, borrow)
+        key = self._prompt_graph_key(entries)
+        if key is not None:
+            logits = self._prompt_graph_step(key, entries, borrow)
+            if logits is not None:
+                return logits
         ctx = self.build_context(entries)
         return self.model.forward(ctx, self.kv, self.states)

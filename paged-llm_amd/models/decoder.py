@@ -89,10 +89,17 @@ class DecoderModel:
                 out[pos] = ss
         return out
 
-    def graph_capturable(self) -> bool:
+    def graph_capturable(self, prompts: bool = False) -> bool:
         """True when every layer's parts only launch kernels (no host reads of device data, no Python-side
-        state): a decode step can then be captured into a HIP graph."""
-        return all(b.graph_capturable() for b in self.blocks)
+        state): a decode step (``prompts``: also a step with prompt portions) can then be captured into a HIP graph."""
+        return all(b.graph_capturable(prompts) for b in self.blocks)
+
+    def graph_step_arrays(self, layout) -> dict:
+        """Host-made integer arrays the layers' parts need for a replayed step of that layout (equal keys are one array)."""
+        out = {}
+        for b in self.blocks:
+            out.update(b.graph_step_arrays(layout))
+        return out
 
     # ------------------------------------------------------------------ compute
     def forward(self, ctx, kv_storage, states: dict) -> torch.Tensor:

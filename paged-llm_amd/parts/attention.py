@@ -20,6 +20,7 @@ from .spec import PartSpec, WeightSpec
 
 class PagedAttention(Mixer):
     graph_capturable = True
+    graph_capturable_prompts = True
 
     def __init__(self, params: dict, env: BuildEnv):
         self.hidden = env.hidden_size
@@ -66,6 +67,13 @@ class PagedAttention(Mixer):
     def cache_spec(self):
         kind = "window" if self.window > 0 else "full"
         return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
+
+    def graph_step_arrays(self, layout):
+        """The prompt kernel's work list (pairs of sequence and tile, most keys first) for a replayed step."""
+        group = self.num_heads // self.num_kv_heads
+        first = layout.num_single_rows
+        pairs = ops.prompt_tiles_capacity(layout.num_portions, layout.portion_tokens, group)
+        return {("prompt_tiles", first, group): (2 * pairs, lambda q_lens, k_lens: ops.prompt_tiles(q_lens, k_lens, first, group, pairs))}
 
     # ---- compute
     def forward(self, h, ctx, cache, state):

@@ -44,8 +44,28 @@ class StateSpec:
     dtype: torch.dtype = torch.float32
 
 
+@dataclass(frozen=True)
+class GraphLayout:
+    """Shape of a step with prompt portions that is replayed from a captured graph.  The batch holds
+    ``num_single_rows`` sequences of one token each (decoded tokens; some may be empty rows) followed by
+    ``num_portions`` sequences that share ``portion_tokens`` tokens between them in any way (prompt portions;
+    the last one is padding).  Launch shapes may depend on these three numbers, on ``StepContext.max_k_len``
+    (a bound) and on nothing else of the batch."""
+    num_single_rows: int
+    num_portions: int
+    portion_tokens: int
+
+
 class Part:
     """Common ground: declared weights, assignment, and a hook once all weights are there."""
+
+    def graph_step_arrays(self, layout: GraphLayout) -> dict:
+        """Integer arrays that this part's kernels need and that are made on the host from the step's lengths
+        (a work list, say), for steps replayed from a graph: key -> (capacity, fill), where
+        ``fill(q_lens, k_lens)`` returns exactly ``capacity`` int32 values for the step's sequences.  The step
+        function calls ``fill`` before every replay and hands the device copy to the part in
+        ``StepContext.launch_cache[key]``."""
+        return {}
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {}
@@ -162,9 +182,18 @@ class Block(Part):
     def state_spec(self):
         return self.mixer.state_spec() if self.mixer is not None else None
 
-    def graph_capturable(self) -> bool:
-        """True when every part that computes only launches kernels on the current stream."""
-        return all(getattr(p, "graph_capturable", False) for role, p in self.parts.items() if self.ROLES[role] != "norm")
+    def graph_capturable(self, prompts: bool = False) -> bool:
+        """True when every part that computes only launches kernels on the current stream and takes its launch
+        shapes from the batch's counts alone: ``graph_capturable`` on a part says so for steps of single tokens,
+        ``graph_capturable_prompts`` for steps with prompt portions (see ``GraphLayout``)."""
+        flag = "graph_capturable_prompts" if prompts else "graph_capturable"
+        return all(getattr(p, flag, False) for role, p in self.parts.items() if self.ROLES[role] != "norm")
+
+    def graph_step_arrays(self, layout) -> dict:
+        out = {}
+        for part in self.parts.values():
+            out.update(part.graph_step_arrays(layout))
+        return out
 
     def weight_specs(self):
         return {f"{self.names[role]}.{name}": spec for role, part in self.parts.items()

@@ -15,6 +15,7 @@ from .spec import WeightSpec
 
 class GatedMLP(FeedForward):
     graph_capturable = True
+    graph_capturable_prompts = True
 
     def __init__(self, params: dict, env: BuildEnv):
         self.hidden = env.hidden_size

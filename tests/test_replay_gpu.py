@@ -147,6 +147,9 @@ def test_mixed_batches_with_pages_used_again(folders, name, dtype):
     check(got, folder, reqs, dtype)
     session.manager.check_invariants()
     assert session.manager.num_free_pages() == session.manager.num_pages()
+    # the steps of this trace were replayed from graphs of both kinds (single tokens only; with prompt portions)
+    kinds = {"prompt" if key[0] == "prompt" else "decode" for key in session.runner._graphs}
+    assert kinds == {"prompt", "decode"}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

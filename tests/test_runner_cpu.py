@@ -201,3 +201,44 @@ def test_replayed_decode_steps_refuse_bad_batches_too(runtime):
     with pytest.raises(StepError, match="wanted row"):
         runner._restage_decode(runner._new_graph_entry((1, 1, 64)), [StepEntry("x", [1], 0, {g: [0]}, None, [1])])
     manager.free("ok2")
+
+
+def test_layout_of_a_step_with_portions_replayed_from_a_graph():
+    """Single tokens first (rounded up with empty rows), then the portions in ascending order, then a padding
+    sequence that fills the token bucket; the attention's work list is made for exactly these sequences."""
+    model = build_model(TINY_A, "bfloat16", "cpu")
+    fill_random(model, seed=0)
+    manager, storage, runner = build_runtime(model, 16, 40, 4, enable_prefix_caching=False)
+    runner.use_graphs = runner.prompt_graphs = True              # (no GPU here: only the host side is exercised)
+    g = next(iter(manager.groups))
+    def make(rid, tokens, start, want=()):
+        assert manager.allocate(rid, start, len(tokens))
+        return StepEntry(rid, list(tokens), start, {g: manager.block_table(rid, g)}, None, list(want))
+    manager.allocate("c", 0, 17)
+    manager.allocate("d", 0, 40)
+    entries = [make("a", [5, 6, 7, 8, 9], 0, [4]), make("b", list(range(20)), 0), make("c", [3], 17, [0]), make("d", [4], 40, [0]),
+               make("e", [2], 0, [0])]
+    key = runner._prompt_graph_key(entries)
+    assert key == ("prompt", 3, 2, 32, 4, 256)                  # 3 single rows, 2 portions of 25 tokens -> bucket 32, bound = the model's 256 positions
+    entry = runner._new_prompt_graph(key)
+    n_want = runner._stage_prompt_graph(entry, entries)
+    lay, view = entry["layout"], entry["view"]
+    piece = lambda i: view[lay["offsets"][i]: lay["offsets"][i] + lay["sizes"][i]]
+    assert n_want == 4 and lay["T"] == 35 and lay["S"] == 6
+    assert piece(0).tolist() == [3, 4, 2] + [5, 6, 7, 8, 9] + list(range(20)) + [0] * 7
+    assert piece(1).tolist() == [17, 40, 0] + list(range(5)) + list(range(20)) + list(range(7))
+    assert piece(2).tolist() == [0, 1, 2, 3, 8, 28, 35] and piece(3).tolist() == [18, 41, 1, 5, 20, 7]
+    assert piece(6).tolist() == [7, 0, 1, 2]                     # in the callers' order: a's last row (3 + 4), c's, d's, e's
+    slots = piece(8)
+    assert slots[3] == manager.block_table("a", g)[0] * 16 and (slots[28:] == -1).all()
+    tables = piece(7).reshape(6, 16)
+    assert tables[1, :3].tolist() == manager.block_table("d", g)[:3] and not tables[5].any()
+    # the work list: pairs (sequence counted from the first portion, tile), the rest unused
+    (akey, (capacity, fill)), = lay["arrays"].items()
+    assert akey == ("prompt_tiles", 3, 2)
+    pairs = piece(9).reshape(-1, 2).tolist()
+    assert pairs[:3] == [[0, 0], [1, 0], [2, 0]] and all(p == [-1, -1] for p in pairs[3:]) and len(pairs) * 2 == capacity
+    # too many portions, or too many tokens: no graph
+    assert runner._prompt_graph_key([make(f"p{i}", [1, 2], 0) for i in range(5)]) is None
+    runner.max_graph_tokens = 16
+    assert runner._prompt_graph_key(entries) is None
