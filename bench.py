@@ -464,7 +464,7 @@ def run_kernel_cases(cfg: dict, batch: int, context: int, prefill_tokens: int) -
         from paged_llm_amd.parts.norm import PendingNorm
         w_qkv, w_o, w_gu, w_down, w_head = weights((nh + 2 * nkv) * d, H), weights(H, nh * d), weights(2 * I, H), weights(H, I), weights(V, H)
         attn_in, act, last = rnd(T, (nh + 2 * nkv) * d), rnd(T, I), rnd(min(T, S), H)
-        pend = lambda rows=None: PendingNorm(nw, 1e-5, x.clone() if rows is None else rows, delta if rows is None else None)
+        pend = lambda rows=None: PendingNorm(nw, 1e-5, x if rows is None else rows, delta if rows is None else None)
         cases = {
             "qkv product (norm in front, rotary and cache write behind)": (
                 lambda i: qkv_rotary_cache(pend(), w_qkv[i % len(w_qkv)], positions, rope, nh, nkv, d, slots, kps[i % kv_copies], vps[i % kv_copies], bs),

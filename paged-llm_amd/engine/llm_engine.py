@@ -102,6 +102,7 @@ class LLMEngine:
         # to be drawn, in the order of the float logits' rows [n, vocab]; row i is the distribution behind
         # position len(requests[i].tokens) - 1.  The tensor is only valid during the call.
         self.on_logits = None
+        self._ahead = None                           # the next step, planned and staged while this one ran (or None)
         log.info("cache: %d pages of %d positions per group (%d positions, %.2f GiB)", pages, cfg.block_size,
                  pages * cfg.block_size, self.kv_cache.total_bytes() / 2**30)
 
@@ -142,31 +143,56 @@ class LLMEngine:
                          {g: cm.block_table(request.id, g) for g in self.groups}, cm.state_slot(request.id),
                          [grant.count - 1] if grant.samples else [], cm.table_version(request.id))
 
-    def _sample(self, logits, grants: list) -> dict:
-        """request id -> token, for the grants whose last row was asked for (in the order of the rows)."""
+    def _sample(self, logits, grants: list):
+        """Queues the sampling of the grants whose last row was asked for; (requests in the order of the rows, pending tokens)."""
         chosen = [g.request for g in grants if g.samples]
-        if not chosen:
-            return {}
-        if self.on_logits is not None:
+        if self.on_logits is not None and chosen:
             self.on_logits(chosen, logits[: len(chosen)])
-        tokens = self.sampler.sample(logits, [r.params for r in chosen], [r.id for r in chosen], [r.num_generated for r in chosen])
-        return {r.id: t for r, t in zip(chosen, tokens)}
+        pending = self.sampler.launch(logits[: len(chosen)], [r.params for r in chosen], [r.id for r in chosen],
+                                      [r.num_generated for r in chosen])
+        return chosen, pending
+
+    def _stage_ahead(self, plan: StepPlan):
+        """While the GPU runs ``plan``: the next step's plan and, where its graph exists, its staging, all but the token
+        ids (see ``Scheduler.plan_ahead``).  (epoch the prediction holds for, next plan, staged step or None)."""
+        if self.cache_manager.uses_state:
+            return None
+        ahead = self.scheduler.plan_ahead(plan)
+        if ahead is None:
+            return None
+        cm = self.cache_manager
+        entries = []
+        for now, then in zip(plan.grants, ahead.grants):
+            request = then.request
+            entries.append(StepEntry(request.id, [0], request.computed + now.count, {g: cm.block_table(request.id, g) for g in self.groups},
+                                     None, [0], cm.table_version(request.id)))
+        return self.scheduler.epoch, ahead, self.runner.prepare(entries)
 
     def _advance(self):
         """Runs one step.  (plan, sampled tokens by request id, requests that ended); the plan is empty
         when there is nothing to do."""
         started = time.perf_counter()
-        plan = self.scheduler.plan()
+        cm = self.cache_manager
+        ahead, self._ahead = self._ahead, None
+        staged = None
+        if ahead is not None and ahead[0] == self.scheduler.epoch:
+            _, plan, staged = ahead                          # made while the step before ran; nothing has moved since
+        else:
+            plan = self.scheduler.plan()
         if not plan:
             if not self.scheduler.idle:
                 raise RuntimeError("no request can run: " + self.scheduler.why_stuck())
             return plan, {}, []
-        cm = self.cache_manager
-        state_copies = cm.take_pending_state_copies() if cm.uses_state else None
         # The sampler runs at once, so the step may hand out its graph's own logits buffer.
-        logits = self.runner.step([self._entry(g) for g in plan.grants], cm.take_pending_copies(), borrow=True,
-                                  state_copies=state_copies)
-        sampled = self._sample(logits, plan.grants)
+        if staged is not None:
+            logits = self.runner.run_prepared(staged, [g.request.tokens[-1] for g in plan.grants], cm.take_pending_copies(), borrow=True)
+        else:
+            state_copies = cm.take_pending_state_copies() if cm.uses_state else None
+            logits = self.runner.step([self._entry(g) for g in plan.grants], cm.take_pending_copies(), borrow=True,
+                                      state_copies=state_copies)
+        chosen, pending = self._sample(logits, plan.grants)
+        self._ahead = self._stage_ahead(plan)                # host work while the GPU computes
+        sampled = {r.id: t for r, t in zip(chosen, pending.result())}
         ended = self.scheduler.commit(plan, sampled)
         for request in ended:
             self._live.pop(request.id, None)

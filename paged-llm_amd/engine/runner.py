@@ -543,6 +543,37 @@ class ModelRunner:
         logits = entry["logits"][:n_want]
         return logits if borrow else logits.clone()
 
+    # ------------------------------------------------------------------ a decode step staged ahead of its token ids
+    def prepare(self, entries: list):
+        """Stages a step of single tokens whose token ids are not known yet (the entries carry any valid id) into the
+        buffer of its graph, if that graph exists already: everything but the ids.  Returns a handle for
+        ``run_prepared``, or None when the step is not of that kind (the caller then runs it through ``step``)."""
+        key = self._graph_key(entries)
+        entry = self._graphs.get(key) if key is not None else None
+        if entry is None:
+            return None                                     # no capture here: it would wait for the GPU
+        entry["copied"].synchronize()
+        return entry, self._restage_decode(entry, entries), len(entries)
+
+    @torch.no_grad()
+    def run_prepared(self, handle, token_ids: list, copies: dict | None = None, borrow: bool = False) -> torch.Tensor:
+        """Runs a step staged by ``prepare`` with the token ids of its entries, in their order."""
+        entry, n_want, rows = handle
+        if len(token_ids) != rows:
+            raise StepError(f"{len(token_ids)} token ids for a prepared step of {rows} entries")
+        vocab = self.model.spec.vocab_size
+        if min(token_ids) < 0 or max(token_ids) >= vocab:
+            raise StepError(f"token id outside [0, {vocab})")
+        if copies:
+            self.kv.apply_copies(copies)
+        at = entry["offsets"][0]
+        entry["view"][at: at + rows] = token_ids
+        entry["static"].copy_(entry["pinned"], non_blocking=True)
+        entry["copied"].record()
+        entry["graph"].replay()
+        logits = entry["logits"][:n_want]
+        return logits if borrow else logits.clone()
+
     # ------------------------------------------------------------------ run
     @torch.no_grad()
     def step(self, entries: list, copies: dict | None = None, borrow: bool = False, state_copies: list | None = None) -> torch.Tensor:

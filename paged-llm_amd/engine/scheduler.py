@@ -77,6 +77,9 @@ class Scheduler:
         self.queue: deque = deque()          # Stage.QUEUED, the next to admit at the left
         self.active: list = []               # Stage.ACTIVE, in admission order
         self.num_preemptions = 0
+        # Counts everything that changes who runs next apart from every active request taking its next token: arrivals,
+        # cancellations, ends, preemptions.  A plan made ahead (``plan_ahead``) holds only while this number stands.
+        self.epoch = 0
 
     # ------------------------------------------------------------------ arrivals and departures
     def submit(self, request: Request) -> None:
@@ -92,6 +95,7 @@ class Scheduler:
             request.new_token_limit = max(1, room)
         request.stage = Stage.QUEUED
         self.queue.append(request)
+        self.epoch += 1
 
     def cancel(self, request_id) -> Request | None:
         """Ends a queued or active request at once; returns it, or None if it is not here."""
@@ -112,6 +116,7 @@ class Scheduler:
     def _retire(self, request: Request, reason: EndReason) -> None:
         self.cache.free(request.id)
         request.end(reason)
+        self.epoch += 1
 
     # ------------------------------------------------------------------ planning a step
     def plan(self) -> StepPlan:
@@ -154,6 +159,7 @@ class Scheduler:
             self.queue.appendleft(victim)
             plan.preempted.append(victim)
             self.num_preemptions += 1
+            self.epoch += 1
             if victim is request:
                 return False
         return True
@@ -171,6 +177,29 @@ class Scheduler:
             left -= count
             plan.add(request, count)
         return left
+
+    def plan_ahead(self, plan: StepPlan) -> StepPlan | None:
+        """The plan of the step after ``plan``, made while ``plan`` still runs (its sampled tokens are not known yet), so
+        that the host's work for the next step overlaps the GPU's work for this one.  Only the steady state is
+        predicted: every active request is in ``plan`` and reaches its last known token there, nobody waits in the
+        queue, nobody can end by length in this step, and a page for everybody's next token is there without taking
+        anybody's.  Then the next plan is one token for each of them, in the same order.  None otherwise.  The caller
+        uses what it gets only while ``epoch`` stands (an end-of-sequence token in this step moves it)."""
+        if self.queue or plan.preempted or len(plan.grants) != len(self.active) or len(self.active) > self.step_budget:
+            return None
+        for grant in plan.grants:
+            request = grant.request
+            if (not grant.samples or request.num_generated + 1 >= request.new_token_limit
+                    or len(request.tokens) + 1 >= self.max_positions):
+                return None
+        ahead = StepPlan()
+        for grant in plan.grants:
+            request = grant.request
+            if not self.cache.allocate(request.id, request.computed + grant.count, 1):
+                return None                   # (pages taken for the others so far are the ones their next step takes anyway)
+            ahead.grants.append(Grant(request, 1, True))
+        ahead.decode_tokens = len(ahead.grants)
+        return ahead
 
     def why_stuck(self) -> str:
         """Says why an empty plan came out although requests remain (for the caller's error)."""
