@@ -507,6 +507,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time only the 2048-token prefill (for profiling)")
+    ap.add_argument("--mixed-only", action="store_true", help="time only the step of --batch decoded tokens beside a 256-token portion (for profiling)")
     ap.add_argument("--attention", action="store_true", help="the reference's attention micro-benchmark cases instead")
     ap.add_argument("--e2e", action="store_true", help="the reference's end-to-end workload (64 requests, 256 in / 128 out) instead: "
                     "its published cases, or one case given by the options below (names as in the reference's benchmarks/bench.py)")
@@ -578,6 +579,9 @@ def main() -> int:
             psec = time_prefill(engine, PREFILL_TOKENS, seed=100)
             print(json.dumps({"prefill_ms": round(psec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / psec, 1),
                               "frac": round(prefill_flops(cfg, PREFILL_TOKENS, 1) / psec / PEAK_FLOPS[short], 4)}))
+            return 0
+        if args.mixed_only:
+            print(json.dumps(time_mixed_step(engine, args.batch, args.context, 256, seed=50, repeats=12)))
             return 0
         sec, mean_context = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
         value = args.batch / sec
