@@ -49,13 +49,33 @@ __device__ __forceinline__ bf16x8 zero8() {
 // v_exp_f32: 2^x, with 2^-inf = 0 and tiny results flushed to zero (harmless in a softmax).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ float group_max(float v) {      // over the 4 lanes that mirror a column
-  v = fmaxf(v, __shfl_xor(v, 16, 64));
-  return fmaxf(v, __shfl_xor(v, 32, 64));
+// The four lanes that mirror a column are 16 lanes apart.  v_permlane16_swap exchanges the odd rows (of 16 lanes)
+// of one register with the even rows of another, v_permlane32_swap the upper half of one with the lower half of
+// the other; applied to two copies of a value they leave every lane with its own row's (half's) value in one
+// register and the neighbour row's (half's) in the other, without a trip through the LDS crossbar.
+__device__ __forceinline__ void rows_swapped(float v, float& mine_or_left, float& right_or_mine) {
+  const auto t = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  mine_or_left = __uint_as_float(t[0]);
+  right_or_mine = __uint_as_float(t[1]);
 }
-__device__ __forceinline__ float group_sum(float v) {
-  v += __shfl_xor(v, 16, 64);
-  return v + __shfl_xor(v, 32, 64);
+__device__ __forceinline__ void halves_swapped(float v, float& lower, float& upper) {
+  const auto t = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  lower = __uint_as_float(t[0]);
+  upper = __uint_as_float(t[1]);
+}
+__device__ __forceinline__ float group_max(float v) {      // over the 4 lanes that mirror a column
+  float a, b;
+  rows_swapped(v, a, b);
+  v = fmaxf(a, b);
+  halves_swapped(v, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float group_sum(float v) {      // the same four terms in the same order in every lane
+  float a, b;
+  rows_swapped(v, a, b);
+  v = a + b;
+  halves_swapped(v, a, b);
+  return a + b;
 }
 
 // Partials of one (token, head, partition): [m (log2 units), l, acc[D]].
@@ -67,7 +87,10 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
     int block_size, float scale, int window, int partition_size, int num_partitions, float* __restrict__ partials) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  // The wavefront's index is the same in all its lanes; saying so keeps everything derived from it (key ranges,
+  // page-table entries, page addresses) in scalar registers.
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = lane & 15, g = lane >> 4;
+  const int bs_shift = __builtin_ctz(block_size);              // pages hold a power of two of positions
   const int seq = blockIdx.z;
   const int kvh = blockIdx.y / num_partitions, part = blockIdx.y - kvh * num_partitions;
   const int G = num_heads / num_kv_heads;
@@ -139,7 +162,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
       const int nk = n0 + kt * 16;
       blk.on[kt] = nk < k_hi;                                   // uniform; tiles past the range: table entries stay unread
       if (!blk.on[kt]) continue;
-      const int page = bt[nk / block_size];
+      const int page = bt[nk >> bs_shift];
       const int off = nk & (block_size - 1);
       const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
       const bf16* krow = k_pages + base + (size_t)(off + r) * D;
@@ -380,11 +403,12 @@ struct MaskedTag { static constexpr bool value = true; };
 struct PlainTag { static constexpr bool value = false; };
 
 template <int NCB, int KG>
-__global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
+__global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
-    int block_size, float scale, int window, const int* __restrict__ work) {
+    int block_size, float scale, int window, const int* __restrict__ work, int partition_size, int num_partitions,
+    float* __restrict__ partials) {
   extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
   constexpr int kKTile = 64 * kKRow, kVTile = D * kVRow;         // elements of one group's keys / values of a step
   // keys [2 buffers][KG][64 rows][kKRow], then values [2 buffers][KG][D rows][kVRow].  Addresses are formed
@@ -394,6 +418,11 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
 #define PLLM_V_TILE(buf, group) (reinterpret_cast<bf16*>(prefill_lds) + 2 * KG * kKTile + ((buf) * KG + (group)) * kVTile)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int cw = wave & 3, kg = wave >> 2;                      // column share and key group of this wavefront
+  // The wavefront's index is the same in all its lanes; saying so keeps what the fetches derive from it (the tile's
+  // page-table entry and page address) in scalar registers.  (Used for the fetches only: with the column share
+  // and key group declared uniform as well the compiler needs more vector registers than large heads leave.)
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int bs_shift = __builtin_ctz(block_size);
   // Workgroups are handed out x first.  With a work list (pairs of sequence and tile, those with the most keys
   // first): blockIdx.x = kv head, blockIdx.y = entry of the list, so the longest pieces of work of all sequences
   // start first and no workgroup is launched for nothing.  Without one: blockIdx.x = (sequence, kv head),
@@ -422,8 +451,16 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
   // key range of the whole workgroup
   const int wg_last = min(wg_col0 + kWgCols, num_cols) - 1;
   const int wg_qmin = pos0 + wg_col0 / G, wg_qmax = pos0 + wg_last / G;
-  const int k_hi = wg_qmax + 1;
-  const int k_lo = ((window > 0 && wg_qmin - window + 1 > 0) ? wg_qmin - window + 1 : 0) & ~63;
+  int k_hi = wg_qmax + 1;
+  int k_lo = ((window > 0 && wg_qmin - window + 1 > 0) ? wg_qmin - window + 1 : 0) & ~63;
+  // With partitions (few tiles, long contexts: too few workgroups to fill the GPU otherwise) blockIdx.z takes one
+  // aligned partition of the keys and leaves a partial result for the merge kernel.
+  const int part = blockIdx.z;
+  if (partition_size > 0) {
+    k_lo = max(k_lo, part * partition_size);
+    k_hi = min(k_hi, (part + 1) * partition_size);
+    if (k_lo >= k_hi) return;                                   // nothing of this partition is visible to the tile
+  }
   // this wavefront's columns
   const int col0 = wg_col0 + cw * 16 * NCB;
   const bool wave_on = col0 < num_cols;
@@ -465,31 +502,31 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
   const size_t page_elems = (size_t)block_size * D;
   const size_t page_stride = page_elems * num_kv_heads;
 
-  // ---- fetch of one tile (16 keys) per wavefront: wavefront w fetches tile w of the block
+  // ---- fetch of one tile (16 keys) per wavefront: wavefront w fetches tile w of the step.  Everything but the
+  //      lane's own offset is uniform (page-table entry, page address), so it stays in scalar registers.  A tile
+  //      past the range is fetched as the range's last tile again: the loads are unconditional (the count of loads
+  //      in flight is then known at every wait), no table entry past the context is read, and what lands in LDS
+  //      for keys past the range is never used (the masked version drops scores and values by position).
   struct Fetched {
     bf16x8 k[kKPerLane], v[kVPerLane];
   };
-  auto fetch = [&](Fetched& f, int n0) {
-    const int nk = n0 + wave * 16;
-    const bool on = nk < k_hi;                                   // past the range: table entry unread, zeros stored
-    const bf16* kbase = k_pages;
-    const bf16* vbase = v_pages;
-    if (on) {
-      const int page = bt[nk / block_size];
-      const int off = nk & (block_size - 1);
-      const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
-      kbase = k_pages + base + (size_t)off * D;                  // 16 rows of D, contiguous
-      vbase = v_pages + base + off;                              // + channel * block_size + key
-    }
+  const int last_tile = (k_hi - 1) & ~15;
+  auto page_of = [&](int n0) -> int { return bt[min(n0 + wave_u * 16, last_tile) >> bs_shift]; };
+  auto fetch = [&](Fetched& f, int n0, int page) {
+    const int nk = min(n0 + wave_u * 16, last_tile);
+    const int off = nk & (block_size - 1);
+    const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
+    const bf16* kbase = k_pages + base + (size_t)off * D;        // 16 rows of D, contiguous
+    const bf16* vbase = v_pages + base + off;                    // + channel * block_size + key
 #pragma unroll
     for (int i = 0; i < kKPerLane; ++i) {
       const int c = lane + i * 64;
-      f.k[i] = (on && c < kKChunks) ? *reinterpret_cast<const bf16x8*>(kbase + (size_t)c * 8) : zero8();
+      f.k[i] = (c < kKChunks) ? *reinterpret_cast<const bf16x8*>(kbase + c * 8) : zero8();
     }
 #pragma unroll
     for (int i = 0; i < kVPerLane; ++i) {
       const int c = lane + i * 64;                                // c = channel * 2 + half
-      f.v[i] = (on && c < kVChunks) ? *reinterpret_cast<const bf16x8*>(vbase + (size_t)(c >> 1) * block_size + (c & 1) * 8) : zero8();
+      f.v[i] = (c < kVChunks) ? *reinterpret_cast<const bf16x8*>(vbase + (c >> 1) * block_size + (c & 1) * 8) : zero8();
     }
   };
   auto stash = [&](const Fetched& f, int buf) {
@@ -629,28 +666,47 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
   };
   const int full_from = window > 0 ? max(qpos_max - window + 1, 0) : 0;   // blocks from here on are inside every column's window
 
-  // ---- the steps.  Step i is computed from LDS while step i + 1 sits in registers (requested one step
-  //      earlier); after the computation it is written to the other LDS buffer and step i + 2 is requested
-  //      into the same registers: a fetch has a whole step to arrive.
+  // ---- the steps.  Step i is computed from LDS while the next steps are on their way in registers: two sets
+  //      of them (steps i + 1 and i + 2) for head sizes up to 64, one set (step i + 1) where a second would not
+  //      fit.  After the computation step i + 1 is written to the other LDS buffer and the registers it leaves take
+  //      the request for the step after those in flight, with the page-table entry that was looked up a step
+  //      earlier: with two sets a fetch has two steps to arrive, and it never waits for its table entry.  Fetches
+  //      and stashes past the last step repeat the last tile into a buffer nobody reads.
   constexpr int kStepKeys = 64 * KG;
-  Fetched regs;
-  auto step = [&](int n0, int buf) {
+  constexpr bool kTwoSets = D <= 64;
+  constexpr int kAhead = kTwoSets ? 3 : 2;                        // the fetch issued in step i is for step i + kAhead
+  Fetched set_a, set_b;
+  int page_next;
+  auto step = [&](int n0, int buf, Fetched& next) {               // `next` holds step n0 + kStepKeys
     const int mine = n0 + kg * 64;                                // this group's 64 keys of the step
-    if (wave_on && mine < vis_hi && mine + 64 > vis_lo) {
+    if (wave_on && mine < vis_hi && mine < k_hi && mine + 64 > vis_lo) {   // (k_hi: a partition's end, a multiple of 64)
       if (mine + 63 <= qpos_min && mine >= full_from) compute(buf, mine, PlainTag{});
       else compute(buf, mine, MaskedTag{});
     }
-    if (n0 + kStepKeys < k_hi) stash(regs, buf ^ 1);
-    if (n0 + 2 * kStepKeys < k_hi) fetch(regs, n0 + 2 * kStepKeys);
+    // (the compiler may not move the requests up into the computation: their registers are free only here)
+    __builtin_amdgcn_sched_barrier(0);
+    stash(next, buf ^ 1);
+    fetch(next, n0 + kAhead * kStepKeys, page_next);
+    page_next = page_of(n0 + (kAhead + 1) * kStepKeys);
     __syncthreads();
   };
-  fetch(regs, k_lo);
-  stash(regs, 0);
-  if (k_lo + kStepKeys < k_hi) fetch(regs, k_lo + kStepKeys);
+  fetch(set_a, k_lo, page_of(k_lo));
+  if constexpr (kTwoSets) fetch(set_b, k_lo + kStepKeys, page_of(k_lo + kStepKeys));
+  page_next = page_of(k_lo + (kAhead - 1) * kStepKeys);
+  stash(set_a, 0);
+  fetch(set_a, k_lo + (kAhead - 1) * kStepKeys, page_next);
+  page_next = page_of(k_lo + kAhead * kStepKeys);
   __syncthreads();
-  for (int n0 = k_lo; n0 < k_hi; n0 += 2 * kStepKeys) {
-    step(n0, 0);
-    if (n0 + kStepKeys < k_hi) step(n0 + kStepKeys, 1);
+  // (the loop is left from between the two steps, not around the second one: on every way back to its head the
+  //  set that was requested first is the one that is stashed next, so the wait before a stash can leave the
+  //  younger set's loads in flight)
+  for (int n0 = k_lo;;) {
+    if constexpr (kTwoSets) step(n0, 0, set_b); else step(n0, 0, set_a);
+    n0 += kStepKeys;
+    if (n0 >= k_hi) break;
+    step(n0, 1, set_a);
+    n0 += kStepKeys;
+    if (n0 >= k_hi) break;
   }
 
   if (KG == 2) {
@@ -679,6 +735,7 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
         const float a_mine = fast_exp2(m_run[cb] - m_safe), a_other = fast_exp2(m_other - m_safe);   // 2^-inf = 0: an empty half adds nothing
         l_run[cb] = l_run[cb] * a_mine + l_other * a_other;
+        m_run[cb] = m_new;
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
@@ -689,8 +746,20 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_prefill_kernel(
 
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb) {
-    const float inv = 1.f / group_sum(l_run[cb]);                 // every lane takes part in the exchange
+    const float l_tot = group_sum(l_run[cb]);                     // every lane takes part in the exchange
+    const float inv = 1.f / l_tot;
     if (!my_valid[cb] || kg != 0) continue;
+    if (partition_size > 0) {                                     // unnormalised sum, maximum and weight of this partition
+      const int c = col0 + cb * 16 + r;
+      const int tok = c / G, hg = c - tok * G;
+      float* dst = partials + (((size_t)(q_begin + tok) * num_heads + (kvh * G + hg)) * num_partitions + part) * kPartialFloats;
+      if (g == 0) { dst[0] = m_run[cb]; dst[1] = l_tot; }
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[2 + db * 16 + g * 4 + i] = acc[cb][db][i];
+      continue;
+    }
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) {
       bf16x4 o;
@@ -732,6 +801,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     seq = lo;
     q_begin = cu_seqlens_q[lo];
     num_q = cu_seqlens_q[lo + 1] - q_begin;
+    if (tok < q_begin || tok >= q_begin + num_q) return;           // a row of none of this launch's sequences
   }
   const int qpos = seq_lens_k[seq] - num_q + (tok - q_begin);
   const int first_key = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
@@ -838,7 +908,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   if (num_kv_heads * num_partitions > 65535 || num_seqs > 65535) return -2;
   if (waves != 1 && waves != 4 && waves != 8) return -2;
   if (waves > 1 && (long)merge_lds_bytes(ncb, waves) > pllm_max_lds()) return -2;
-  if (waves == 1 && partition_size == 0 && max_cols > 64 && column_blocks != 1 && column_blocks != 4) {
+  if (waves == 1 && max_cols > 64 && column_blocks != 1 && column_blocks != 4) {
     // prompt portions: workgroups of four wavefronts that share every block of keys through LDS
     constexpr int kCols = 4 * 16 * 2;
     const int ptiles = (max_cols + kCols - 1) / kCols;
@@ -847,8 +917,9 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // units evenly loaded for any number and length of prompts (pairing far and near tiles in one workgroup
     // was 5 % faster when the pairs filled the compute units exactly and up to 40 % slower just past that).
     if (ptiles > 65535 || num_work > 65535 || (work_list && num_work <= 0)) return -2;
-    dim3 pgrid(num_kv_heads * num_seqs, ptiles, 1);
-    if (work_list) pgrid = dim3(num_kv_heads, num_work, 1);
+    if (num_partitions > 65535) return -2;
+    dim3 pgrid(num_kv_heads * num_seqs, ptiles, num_partitions);
+    if (work_list) pgrid = dim3(num_kv_heads, num_work, num_partitions);
     // Two key groups (eight wavefronts, one workgroup per compute unit) for the head sizes that then still fit
     // into registers and LDS (up to 128): always where a wavefront of the four-wavefront kind needs more than half
     // of a SIMD's registers (head sizes above 96: two groups are then the only way to two wavefronts per SIMD,
@@ -858,7 +929,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     constexpr bool two_fits = D <= 128 && prefill_lds_bytes(2) <= 160 * 1024;
     // (workgroups that find work: a sequence has as many tiles as its own queries need, the grid as many slots
     // as the longest)
-    const long busy = work_list ? (long)num_work * num_kv_heads : ((long)total_q * G / kCols + num_seqs) * num_kv_heads;
+    const long busy = (work_list ? (long)num_work * num_kv_heads : ((long)total_q * G / kCols + num_seqs) * num_kv_heads) * num_partitions;
     const bool two = two_fits && (D > 96 || 2L * busy <= 5L * num_compute_units());
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
     if ((long)lds > pllm_max_lds()) return -2;
@@ -872,7 +943,11 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     }
     hipLaunchKernelGGL(kern, pgrid, dim3(two ? 512 : 256), lds, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q,
-                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, work_list);
+                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, work_list, partition_size, num_partitions, partials);
+    int perr = (int)hipGetLastError();
+    if (perr || partition_size == 0) return perr;
+    hipLaunchKernelGGL(attention_merge_kernel<false>, dim3((total_q * num_heads + 3) / 4), dim3(256), 0, stream, partials, (bf16*)out,
+                       out_stride, cu_seqlens_q, seq_lens_k, num_seqs, total_q, num_heads, window, partition_size, num_partitions);
     return (int)hipGetLastError();
   }
   dim3 grid(tiles, num_kv_heads * num_partitions, num_seqs), block(64 * waves);

@@ -473,7 +473,8 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                          out: torch.Tensor | None = None, work_list: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
-    work item into aligned partitions that a second kernel merges; ``waves`` > 1 shares the keys
+    work item into aligned partitions that a second kernel merges (best a multiple of 128 for prompt portions, whose
+    workgroups walk the keys in steps of up to 128); ``waves`` > 1 shares the keys
     of a work item between the wavefronts of one workgroup (few queries per sequence only).  ``work_list``
     (prompt portions): int32 [n, 2] pairs of (sequence, tile of 128 query columns), the order in which the
     kernel's workgroups take them (``prompt_work_list``)."""
@@ -590,6 +591,37 @@ def prompt_work_list(ctx, first_seq: int, group: int) -> torch.Tensor | None:
     return work
 
 
+_compute_units: dict = {}
+
+
+def _num_compute_units(device) -> int:
+    key = str(device)
+    if key not in _compute_units:
+        _compute_units[key] = torch.cuda.get_device_properties(device).multi_processor_count
+    return _compute_units[key]
+
+
+PROMPT_PARTITION_MIN_KEYS = 512   # a partition of the prompt kernel holds at least this many keys (four steps of 128)
+
+
+def prompt_partitions(num_tiles: int, num_kv_heads: int, max_k_len: int, compute_units: int) -> tuple[int, int]:
+    """(partition_size, num_partitions) for a launch of the prompt kernel with ``num_tiles`` tiles of query columns
+    (all sequences together) whose longest context is ``max_k_len``; (0, 1): no partitions.
+
+    A workgroup walks its tile's keys one step of 128 after the other (about 1.9 us a step at head size 64), so a
+    prompt portion of a few hundred tokens behind a long context is a few dozen workgroups that run for a long time
+    on a GPU of 256 compute units: 256 tokens at context 2048 took 30 us.  The keys are then cut into as many
+    aligned partitions as it takes to give every compute unit a workgroup, each at least PROMPT_PARTITION_MIN_KEYS
+    long, and a second kernel merges the partitions (about 5 us)."""
+    workgroups = max(1, num_tiles * num_kv_heads)
+    parts = min(compute_units // workgroups, max_k_len // PROMPT_PARTITION_MIN_KEYS)
+    if parts < 2:
+        return 0, 1
+    size = -(-max_k_len // parts)
+    size = (size + 127) // 128 * 128
+    return size, -(-max_k_len // size)
+
+
 FEW_QUERY_COLUMNS = 64      # queries x heads per kv head that one tile of the decode kernel holds
 SPLIT_FROM_CONTEXT_TIMES_HEAD = 160_000   # context x head size of a few-query sequence from which two launches pay
 
@@ -625,8 +657,9 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                                      num_heads, num_kv_heads, head_dim, scale, window, 1, size, parts, waves,
                                      2 if waves == 1 else 0, out=out[:few])
             prompt_q = max(layout.portion_tokens, FEW_QUERY_COLUMNS // group + 1)     # enough columns for the prompt kernel's form
+            psize, pparts = prompt_partitions(work.shape[0], num_kv_heads, ctx.max_k_len, _num_compute_units(q.device))
             paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
-                                 num_kv_heads, head_dim, scale, window, prompt_q, 0, 1, 1, 2, out=out, work_list=work)
+                                 num_kv_heads, head_dim, scale, window, prompt_q, psize, pparts, 1, 2, out=out, work_list=work)
             return out
         q_lens, k_lens = ctx.q_lens, ctx.k_lens
         few = 0
@@ -642,14 +675,19 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                                  num_heads, num_kv_heads, head_dim, scale, window, max_q, size, parts, waves,
                                  2 if waves == 1 else 0, out=out[:rows])
             # the portions: rows, cu_seqlens_q and the output stay absolute, the per-sequence arrays start at `few`
+            psize, pparts = prompt_partitions(sum(-(-n * group // PROMPT_TILE_COLUMNS) for n in q_lens[few:]), num_kv_heads,
+                                              max(k_lens[few:]), _num_compute_units(q.device))
             paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
-                                 num_kv_heads, head_dim, scale, window, max(q_lens[few:]), 0, 1, 1, 2, out=out,
+                                 num_kv_heads, head_dim, scale, window, max(q_lens[few:]), psize, pparts, 1, 2, out=out,
                                  work_list=prompt_work_list(ctx, few, group))
             return out
         waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, group, head_dim, lds)
         # Prompt portions: 32 columns per wavefront leave registers for two wavefronts per SIMD
         # (measured faster than 64 columns at one).
         prompt = waves == 1 and ctx.max_q_len * group > FEW_QUERY_COLUMNS and not ctx.capturing
+        if prompt:
+            size, parts = prompt_partitions(sum(-(-n * group // PROMPT_TILE_COLUMNS) for n in q_lens), num_kv_heads, ctx.max_k_len,
+                                            _num_compute_units(q.device))
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
                                     head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0,
                                     work_list=prompt_work_list(ctx, 0, group) if prompt else None)

@@ -496,6 +496,39 @@ def test_decoded_tokens_beside_prompt_portions(heads, kv_heads, d):
     assert rel_err(back, want) <= 1.6e-2
 
 
+@pytest.mark.parametrize("heads,kv_heads,d", [(32, 4, 64), (8, 2, 128), (6, 1, 96), (4, 4, 32)])
+@pytest.mark.parametrize("window", [0, 700])
+def test_prompt_portions_with_key_partitions(heads, kv_heads, d, window):
+    """Prompt portions behind long contexts with their keys cut into partitions that the merge kernel joins: partitions
+    that end inside, at and beyond a sequence's context, a sequence that starts at position 0, a window, one query
+    that looks at a single far key, and stale slots full of NaN behind a context's end."""
+    bs = 16
+    group = heads // kv_heads
+    q_lens, k_lens = [200, 64 // group + 3, 130], [2300, 1024, 130]
+    q, kp, vp, tables, cu, sl = paged_case(k_lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16, seed=13)
+    n, row, head = 777 if window == 0 else 2100, 150, 1 % heads           # row 150 of sequence 0 (position 2250) sees key n only
+    page, off = int(tables[0, n // bs]), n % bs
+    kp[page, head // group, off, :] = (q[row, head * d:(head + 1) * d].float() * 40).to(torch.bfloat16)
+    stale = int(tables[2, 130 // bs])                                   # the slots behind sequence 2's 130 keys
+    kp[stale, :, 130 % bs:, :], vp[stale, :, :, 130 % bs:] = float("nan"), float("nan")
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, 1.0, window or None)
+    for size in (128, 512, 640, 4096):
+        parts = (max(k_lens) + size - 1) // size
+        got = ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, 1.0,
+                                         window, max(q_lens), size, parts, 1, 2).cpu().float()
+        assert torch.allclose(got[row, head * d:(head + 1) * d], vp[page, head // group, :, off].float(), atol=2e-2), f"partition {size}"
+        assert rel_err(got, want) <= 1.6e-2, f"partition {size}"
+
+
+def test_prompt_partitions_are_chosen_to_fill_the_gpu():
+    pp = ops().prompt_partitions
+    assert pp(512, 4, 2048, 256) == (0, 1)                              # a whole prompt: tiles enough
+    assert pp(16, 4, 2048, 256) == (512, 4)                             # 256 tokens behind 2048: 64 workgroups -> 256
+    assert pp(16, 4, 600, 256) == (0, 1)                                # too short to cut
+    size, parts = pp(2, 8, 100_000, 256)
+    assert size % 128 == 0 and size >= 512 and (parts - 1) * size < 100_000 <= parts * size and parts <= 16
+
+
 def test_decode_attention_kernel_leaves_room_for_two_workgroups():
     """At head size 64 the decode kernel keeps two blocks of keys and values in registers; two of its workgroups of
     four wavefronts share a compute unit only while it takes at most 256 registers per lane, vector and accumulation
