@@ -31,9 +31,9 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and model.graph_capturable()
         self.prompt_graphs = self.use_graphs and model.graph_capturable(prompts=True)
         self.max_graph_batch = max_graph_batch
-        # Steps with prompt portions are replayed from graphs up to this many portion tokens (beyond it the
-        # GPU's time hides the host's), and once their shape has been seen this often (a capture costs
-        # several steps' time; shapes that never come back are not worth one).
+        # Steps with prompt portions are replayed from graphs up to this many portion tokens (eight times as many
+        # when no padding is needed), and once their shape has been seen this often (a capture costs several
+        # steps' time; shapes that never come back are not worth one).
         self.max_graph_tokens = max_graph_tokens
         self.graph_after_sightings = max(1, graph_after_sightings)
         self._sightings: dict = {}
@@ -356,7 +356,8 @@ class ModelRunner:
         """A step that holds prompt portions (entries of two or more tokens), alone or beside single tokens, can be
         replayed from a graph whose launch shapes depend on: the number of single-token rows (rounded up as for
         decode steps), the number of portions (at most four), the portions' tokens together (rounded up to a
-        bucket; a sequence of padding tokens that writes nothing fills the rest, at least one), the wanted rows and
+        bucket; a sequence of padding tokens that writes nothing fills the rest, none when the portions fill the bucket
+        exactly, as the portions of a long prompt under a token budget do step after step), the wanted rows and
         a bound on the context lengths.  None when the step is not of that kind or too large to be worth it."""
         if not self.prompt_graphs:
             return None
@@ -372,10 +373,13 @@ class ModelRunner:
             longest = max(longest, e.start + n)
         if portions == 0 or portions > self.MAX_GRAPH_PORTIONS or singles > self.max_graph_batch:
             return None
-        bucket = self._token_bucket(portion_tokens + 1)
+        bucket = self._token_bucket(portion_tokens)
         bound = ((longest + 511) // 512) * 512 if longest <= 8192 else 1 << (longest - 1).bit_length()
         bound = min(bound, max(self.model.max_positions, longest))
-        if bucket > min(self.max_graph_tokens, bound):      # (the padding sequence's positions stay below the bound)
+        # Padded steps up to max_graph_tokens (beyond it the padding's work costs more than the host's launches); steps
+        # that fill their bucket exactly (the portions of a long prompt under a token budget) up to eight times that.
+        limit = self.max_graph_tokens * (8 if bucket == portion_tokens else 1)
+        if bucket > min(limit, bound):                      # (the padding sequence's positions stay below the bound)
             return None
         rows = self._bucket(singles) if singles else 0
         wanted = max(self._bucket(asked), asked) if asked else 0

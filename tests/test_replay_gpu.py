@@ -101,6 +101,27 @@ def test_portions_of_changing_size(folders, name, dtype):
     check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_that_fill_their_graph_bucket(folders, dtype):
+    """Portions of 32, 64 and 96 tokens are exactly the token counts that graphs of steps with prompt portions are
+    captured for: the padding sequence of such a step is empty.  Each size comes twice, so the second is a replay."""
+    name = "B"
+    folder = folders[name, "float32" if dtype == "float32" else "bfloat16"]
+    vocab = CONFIGS[name]["vocab_size"]
+    reqs = {f"f{i}": helpers.random_tokens(2 * (32 + 64 + 96), vocab, seed=300 + i) for i in range(2)}
+    session = session_for(folder, dtype, 2 * rounded(2 * (32 + 64 + 96)))
+    trace = TraceBuilder()
+    for rid, toks in reqs.items():
+        at = 0
+        for n in (32, 64, 96, 96, 64, 32):
+            trace.step([(rid, toks[at:at + n], [0, n // 2, n - 1])], end=[rid] if at + n == len(toks) else [])
+            at += n
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+    if dtype == "bfloat16":
+        buckets = {key[3] for key in session.runner._graphs if key[0] == "prompt"}
+        assert {32, 64, 96} <= buckets, buckets
+
+
 def mixed_trace(reqs: dict, max_live: int, seed: int):
     """Portions of some requests beside decoded tokens of others, up to ``max_live`` at a time.
     Returns the trace and the largest number of tokens (rounded up per request to 64) live at once."""
