@@ -413,7 +413,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
 // MT tiles of 16 input rows side by side.  A weight slab is loaded once per wavefront and multiplied with
 // each tile's rows, which come straight from memory (cache hits) beside it; there is no sum or norm in
 // front of this form (the caller runs the norm on its own) and no LDS for the rows.
-template <int EPI, int MT>
+// XFIXED (K of at most PRE slabs per wavefront, 2048): a wavefront's share of the rows is the same for every
+// unit, so it is loaded once and stays in registers; a workgroup with several units (the gate/up product) then
+// reads the rows once instead of once per unit, which otherwise is four times what it streams of weights.
+template <int EPI, int MT, bool XFIXED>
 __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLinearParams p, int num_units) {
   constexpr int WAVES = 8, PRE = 2;
   asm volatile("" ::"s"(p.x), "s"(p.row_index), "s"(p.W), "s"(p.ldx), "s"(p.ldw), "s"(p.M), "s"(p.K), "s"(p.N), "s"(num_units));
@@ -512,10 +515,10 @@ __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLin
         }
         const int ahead = nth + PRE;
         if (ahead < padded_slabs) {
-          load_x(ahead, xbuf[s]);
+          if (!XFIXED) load_x(ahead, xbuf[s]);
           load_w(wrow, ahead, wbuf[s]);
         } else if (next < num_units) {
-          load_x(ahead - padded_slabs, xbuf[s]);
+          if (!XFIXED) load_x(ahead - padded_slabs, xbuf[s]);
           load_w(wrow_next, ahead - padded_slabs, wbuf[s]);
         }
       }
@@ -568,12 +571,19 @@ template <int EPI>
 static int launch_wide(const DecodeLinearParams& p, int units, int blocks, hipStream_t stream) {
   const int tiles = (p.M + 15) / 16;
   const size_t lds = (size_t)8 * tiles * 256 * sizeof(float);
+  const bool fixed = (p.K + kSlab - 1) / kSlab <= 2 * 8;      // at most PRE slabs for each of the 8 wavefronts
+#define PLLM_WIDE(MT_)                                                                                                              \
+  do {                                                                                                                              \
+    if (fixed) hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, MT_, true>), dim3(blocks), dim3(512), lds, stream, p, units);     \
+    else hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, MT_, false>), dim3(blocks), dim3(512), lds, stream, p, units);          \
+  } while (0)
   switch (tiles) {
-    case 2: hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, 2>), dim3(blocks), dim3(512), lds, stream, p, units); break;
-    case 3: hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, 3>), dim3(blocks), dim3(512), lds, stream, p, units); break;
-    case 4: hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, 4>), dim3(blocks), dim3(512), lds, stream, p, units); break;
+    case 2: PLLM_WIDE(2); break;
+    case 3: PLLM_WIDE(3); break;
+    case 4: PLLM_WIDE(4); break;
     default: return -2;
   }
+#undef PLLM_WIDE
   return (int)hipGetLastError();
 }
 
