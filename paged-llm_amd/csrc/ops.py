@@ -662,7 +662,7 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                                      num_heads, num_kv_heads, head_dim, scale, window, 1, size, parts, waves,
                                      2 if waves == 1 else 0, out=out[:few])
             prompt_q = max(layout.portion_tokens, FEW_QUERY_COLUMNS // group + 1)     # enough columns for the prompt kernel's form
-            psize, pparts = prompt_partitions(work.shape[0], num_kv_heads, ctx.max_k_len, _num_compute_units(q.device))
+            psize, pparts = prompt_partitions(work.shape[0], num_kv_heads, layout.portion_context, _num_compute_units(q.device))
             paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
                                  num_kv_heads, head_dim, scale, window, prompt_q, psize, pparts, 1, 2, out=out, work_list=work)
             return out

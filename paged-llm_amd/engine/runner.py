@@ -361,7 +361,7 @@ class ModelRunner:
         a bound on the context lengths.  None when the step is not of that kind or too large to be worth it."""
         if not self.prompt_graphs:
             return None
-        singles = portions = portion_tokens = asked = longest = 0
+        singles = portions = portion_tokens = asked = longest = longest_portion = 0
         for e in entries:
             n = len(e.tokens)
             if n == 1:
@@ -369,6 +369,7 @@ class ModelRunner:
             else:
                 portions += 1
                 portion_tokens += n
+                longest_portion = max(longest_portion, e.start + n)
             asked += len(e.want)
             longest = max(longest, e.start + n)
         if portions == 0 or portions > self.MAX_GRAPH_PORTIONS or singles > self.max_graph_batch:
@@ -383,10 +384,13 @@ class ModelRunner:
             return None
         rows = self._bucket(singles) if singles else 0
         wanted = max(self._bucket(asked), asked) if asked else 0
-        return ("prompt", rows, portions, bucket, wanted, bound)
+        # The portions' own contexts, as far as the attention's launch depends on them: nothing below 1024 (no
+        # partitions of keys there), else a power of two.
+        portion_context = 0 if longest_portion < 1024 else min(bound, 1 << (longest_portion - 1).bit_length())
+        return ("prompt", rows, portions, bucket, wanted, bound, portion_context)
 
     def _prompt_layout(self, key):
-        _, rows, portions, bucket, wanted, bound = key
+        _, rows, portions, bucket, wanted, bound, portion_context = key
         T, S = rows + bucket, rows + portions + 1
         fixed = (bound + self.block_size - 1) // self.block_size
         sizes = [T, T, S + 1, S, S, S, wanted]
@@ -395,7 +399,7 @@ class ModelRunner:
             sizes += [S * fixed, T]
             table_shapes[name] = (S, fixed)
         from ..parts.base import GraphLayout
-        layout = GraphLayout(num_single_rows=rows, num_portions=portions + 1, portion_tokens=bucket)
+        layout = GraphLayout(num_single_rows=rows, num_portions=portions + 1, portion_tokens=bucket, portion_context=portion_context)
         arrays = self.model.graph_step_arrays(layout)            # key -> (capacity in int32, fill(q_lens, k_lens) -> array)
         array_keys = list(arrays)
         sizes += [arrays[k][0] for k in array_keys]
@@ -409,7 +413,7 @@ class ModelRunner:
     def _stage_prompt_graph(self, entry: dict, entries: list) -> int:
         """Checks the batch (as ``_stage`` does) and lays it out in the fixed shape of the graph: single-token rows,
         empty rows up to their bucket, the portions in ascending order of their lengths, the padding sequence."""
-        _, rows, portions, bucket, wanted, bound = entry["key"]
+        _, rows, portions, bucket, wanted, bound, _ = entry["key"]
         lay = entry["layout"]
         T, S, fixed, offsets, sizes = lay["T"], lay["S"], lay["fixed"], lay["offsets"], lay["sizes"]
         buf, off, siz, host = self._stage(entries, fixed_blocks=fixed)
@@ -464,7 +468,7 @@ class ModelRunner:
                     copied=torch.cuda.Event() if on_gpu else None)
 
     def _prompt_context(self, entry: dict) -> StepContext:
-        _, rows, portions, bucket, wanted, bound = entry["key"]
+        _, rows, portions, bucket, wanted, bound, _ = entry["key"]
         lay = entry["layout"]
         S = lay["S"]
         host = dict(T=lay["T"], S=S, q_lens=[1] * rows + [bucket] * (portions + 1), k_lens=[bound] * S,
@@ -479,7 +483,7 @@ class ModelRunner:
     def _capture_prompt_graph(self, entry: dict) -> None:
         """Warm-up and capture on a batch of the graph's shape that writes nothing: empty single-token rows and
         portions that are all padding."""
-        _, rows, portions, bucket, wanted, bound = entry["key"]
+        _, rows, portions, bucket, wanted, bound, _ = entry["key"]
         lay = entry["layout"]
         view, offsets, sizes, S, T = entry["view"], lay["offsets"], lay["sizes"], lay["S"], lay["T"]
         view[:] = 0

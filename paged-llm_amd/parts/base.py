@@ -49,11 +49,13 @@ class GraphLayout:
     """Shape of a step with prompt portions that is replayed from a captured graph.  The batch holds
     ``num_single_rows`` sequences of one token each (decoded tokens; some may be empty rows) followed by
     ``num_portions`` sequences that share ``portion_tokens`` tokens between them in any way (prompt portions;
-    the last one is padding).  Launch shapes may depend on these three numbers, on ``StepContext.max_k_len``
-    (a bound) and on nothing else of the batch."""
+    the last one is padding).  ``portion_context`` bounds the contexts that the portions end at (0: below the
+    length from which it pays to cut a portion's keys into partitions).  Launch shapes may depend on these
+    numbers, on ``StepContext.max_k_len`` (a bound over all sequences) and on nothing else of the batch."""
     num_single_rows: int
     num_portions: int
     portion_tokens: int
+    portion_context: int = 0
 
 
 class Part:

@@ -122,6 +122,29 @@ def test_portions_that_fill_their_graph_bucket(folders, dtype):
         assert {32, 64, 96} <= buckets, buckets
 
 
+def test_portions_behind_a_long_context(folders):
+    """Portions of 64 tokens behind more than a thousand cached positions, beside a decoding request: such a step's
+    graph cuts the portion's keys into partitions that a second kernel merges (few tiles, many keys).  Rows from
+    before and behind the length at which the partitions begin are compared with the plain implementation."""
+    name, dtype = "B", "bfloat16"
+    folder = folders[name, "bfloat16"]
+    vocab = CONFIGS[name]["vocab_size"]
+    reqs = {"long": helpers.random_tokens(1216, vocab, seed=400), "side": helpers.random_tokens(40, vocab, seed=401)}
+    session = session_for(folder, dtype, rounded(1216) + 64)
+    trace = TraceBuilder()
+    trace.step([("side", reqs["side"][:20], "last")])
+    side_at = 20
+    for at in range(0, 1216, 64):
+        entries = [("long", reqs["long"][at:at + 64], [0, 63] if at >= 896 else [])]
+        if side_at < 40:
+            entries.insert(0, ("side", reqs["side"][side_at:side_at + 1], "all"))
+            side_at += 1
+        trace.step(entries, end=["long"] if at + 64 == 1216 else [])
+    check(helpers.replay_in_process(session, trace), folder, reqs, dtype)
+    contexts = {key[6] for key in session.runner._graphs if key[0] == "prompt"}
+    assert 0 in contexts and max(contexts) >= 1024, contexts
+
+
 def mixed_trace(reqs: dict, max_live: int, seed: int):
     """Portions of some requests beside decoded tokens of others, up to ``max_live`` at a time.
     Returns the trace and the largest number of tokens (rounded up per request to 64) live at once."""

@@ -219,7 +219,7 @@ def test_layout_of_a_step_with_portions_replayed_from_a_graph():
     entries = [make("a", [5, 6, 7, 8, 9], 0, [4]), make("b", list(range(20)), 0), make("c", [3], 17, [0]), make("d", [4], 40, [0]),
                make("e", [2], 0, [0])]
     key = runner._prompt_graph_key(entries)
-    assert key == ("prompt", 3, 2, 32, 4, 256)                  # 3 single rows, 2 portions of 25 tokens -> bucket 32, bound = the model's 256 positions
+    assert key == ("prompt", 3, 2, 32, 4, 256, 0)                  # 3 single rows, 2 portions of 25 tokens -> bucket 32, bound = the model's 256 positions
     entry = runner._new_prompt_graph(key)
     n_want = runner._stage_prompt_graph(entry, entries)
     lay, view = entry["layout"], entry["view"]
