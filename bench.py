@@ -298,7 +298,7 @@ def time_mixed_step(engine, decode_requests: int, context: int, portion: int, se
     from paged_llm_amd import SamplingParams
     vocab = engine.model.spec.vocab_size
     sp = SamplingParams(temperature=0.0, max_tokens=repeats * 4 + 40, ignore_eos=True)
-    for p in random_prompts(decode_requests, context - repeats * 4 - 8, vocab, seed):
+    for p in random_prompts(decode_requests, context - repeats * 3 - 8, vocab, seed):
         engine.add_request(p, sp)
     while any(not r.decoding for r in engine.scheduler.active) or engine.scheduler.queue:
         engine.step()
@@ -308,6 +308,8 @@ def time_mixed_step(engine, decode_requests: int, context: int, portion: int, se
     for r in range(repeats):
         prompt = random_prompts(1, portion, vocab, seed + 100 + r)[0]
         rid = engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
+        if engine.step_in_flight:                              # the decode step that was under way when the request arrived
+            assert len(engine.step()) == decode_requests
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()

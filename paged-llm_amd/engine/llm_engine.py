@@ -102,7 +102,10 @@ class LLMEngine:
         # to be drawn, in the order of the float logits' rows [n, vocab]; row i is the distribution behind
         # position len(requests[i].tokens) - 1.  The tensor is only valid during the call.
         self.on_logits = None
-        self._ahead = None                           # the next step, planned and staged while this one ran (or None)
+        # A step that is launched and sampled but not committed yet: (plan, requests of the sampled rows, pending tokens).
+        self._flight = None
+        # Launch the step after the one under way before waiting for its tokens (see ``_advance``); off: one step at a time.
+        self.run_ahead = True
         log.info("cache: %d pages of %d positions per group (%d positions, %.2f GiB)", pages, cfg.block_size,
                  pages * cfg.block_size, self.kv_cache.total_bytes() / 2**30)
 
@@ -135,6 +138,12 @@ class LLMEngine:
     def has_unfinished_requests(self) -> bool:
         return not self.scheduler.idle
 
+    @property
+    def step_in_flight(self) -> bool:
+        """A step has been launched beyond the last committed one (see ``_advance``): the next ``step()`` commits it,
+        whatever has arrived or been cancelled since."""
+        return self._flight is not None and not all(g.request.ended for g in self._flight[0].grants)
+
     # ------------------------------------------------------------------ one step
     def _entry(self, grant) -> StepEntry:
         request, cm = grant.request, self.cache_manager
@@ -144,18 +153,32 @@ class LLMEngine:
                          [grant.count - 1] if grant.samples else [], cm.table_version(request.id))
 
     def _sample(self, logits, grants: list):
-        """Queues the sampling of the grants whose last row was asked for; (requests in the order of the rows, pending tokens)."""
+        """Queues the sampling of the grants whose last row was asked for; (requests in the order of the rows, pending
+        tokens).  Rows of requests that ended while the step was already running are sampled with the others and
+        dropped when the step is committed; the ``on_logits`` hook does not see them."""
         chosen = [g.request for g in grants if g.samples]
+        rows = logits[: len(chosen)]
         if self.on_logits is not None and chosen:
-            self.on_logits(chosen, logits[: len(chosen)])
-        pending = self.sampler.launch(logits[: len(chosen)], [r.params for r in chosen], [r.id for r in chosen],
-                                      [r.num_generated for r in chosen])
+            live = [i for i, r in enumerate(chosen) if not r.ended]
+            if len(live) == len(chosen):
+                self.on_logits(chosen, rows)
+            elif live:
+                self.on_logits([chosen[i] for i in live], rows[live])
+        pending = self.sampler.launch(rows, [r.params for r in chosen], [r.id for r in chosen], [r.num_generated for r in chosen])
         return chosen, pending
 
-    def _stage_ahead(self, plan: StepPlan):
-        """While the GPU runs ``plan``: the next step's plan and, where its graph exists, its staging, all but the token
-        ids (see ``Scheduler.plan_ahead``).  (epoch the prediction holds for, next plan, staged step or None)."""
-        if self.cache_manager.uses_state:
+    def _launch(self, plan: StepPlan):
+        """Queues the step of ``plan`` from the tokens the requests hold; the step's logits."""
+        cm = self.cache_manager
+        state_copies = cm.take_pending_state_copies() if cm.uses_state else None
+        return self.runner.step([self._entry(g) for g in plan.grants], cm.take_pending_copies(), borrow=True, state_copies=state_copies)
+
+    def _launch_ahead(self, plan: StepPlan, pending):
+        """While the GPU runs ``plan`` and its sampling: the step after it, queued behind them with the sampled ids
+        taken where the sampling kernel leaves them on the GPU, so that the GPU goes from one step into the next
+        without waiting for the host to see the tokens (see ``Scheduler.plan_ahead`` for when that is possible;
+        the step's graph must exist already).  (the next plan, its logits), or None."""
+        if not self.run_ahead or self.cache_manager.uses_state or pending.on_device is None:
             return None
         ahead = self.scheduler.plan_ahead(plan)
         if ahead is None:
@@ -166,43 +189,50 @@ class LLMEngine:
             request = then.request
             entries.append(StepEntry(request.id, [0], request.computed + now.count, {g: cm.block_table(request.id, g) for g in self.groups},
                                      None, [0], cm.table_version(request.id)))
-        return self.scheduler.epoch, ahead, self.runner.prepare(entries)
+        staged = self.runner.prepare(entries)
+        if staged is None:
+            return None                                      # (the pages taken for the next tokens stay with their requests)
+        return ahead, self.runner.run_prepared(staged, pending.on_device, cm.take_pending_copies(), borrow=True)
 
     def _advance(self):
-        """Runs one step.  (plan, sampled tokens by request id, requests that ended); the plan is empty
-        when there is nothing to do."""
+        """Commits one step.  (the grants it commits, sampled tokens by request id, requests that ended); no grants
+        when there is nothing to do.
+
+        One step may be under way beyond the committed one: a step is launched together with its sampling, and
+        before the host waits for the sampled ids it launches the step after, if that one can be foreseen.  When the
+        ids arrive the step is committed; a request that ends there (an end-of-sequence token, a cancellation) is
+        dropped from the step that is already running, whose other rows are as good as ever."""
         started = time.perf_counter()
-        cm = self.cache_manager
-        ahead, self._ahead = self._ahead, None
-        staged = None
-        if ahead is not None and ahead[0] == self.scheduler.epoch:
-            _, plan, staged = ahead                          # made while the step before ran; nothing has moved since
-        else:
+        flight, self._flight = self._flight, None
+        if flight is not None and all(g.request.ended for g in flight[0].grants):
+            flight = None                                    # everybody in it was cancelled meanwhile: nothing to commit
+        if flight is None:
             plan = self.scheduler.plan()
-        if not plan:
-            if not self.scheduler.idle:
-                raise RuntimeError("no request can run: " + self.scheduler.why_stuck())
-            return plan, {}, []
-        # The sampler runs at once, so the step may hand out its graph's own logits buffer.
-        if staged is not None:
-            logits = self.runner.run_prepared(staged, [g.request.tokens[-1] for g in plan.grants], cm.take_pending_copies(), borrow=True)
+            if not plan:
+                if not self.scheduler.idle:
+                    raise RuntimeError("no request can run: " + self.scheduler.why_stuck())
+                return [], {}, []
+            # The sampler runs at once, so the step may hand out its graph's own logits buffer.
+            chosen, pending = self._sample(self._launch(plan), plan.grants)
         else:
-            state_copies = cm.take_pending_state_copies() if cm.uses_state else None
-            logits = self.runner.step([self._entry(g) for g in plan.grants], cm.take_pending_copies(), borrow=True,
-                                      state_copies=state_copies)
-        chosen, pending = self._sample(logits, plan.grants)
-        self._ahead = self._stage_ahead(plan)                # host work while the GPU computes
+            plan, chosen, pending = flight
+        ahead = self._launch_ahead(plan, pending)            # the GPU's next millisecond, queued before the host waits
         sampled = {r.id: t for r, t in zip(chosen, pending.result())}
+        committed = [g for g in plan.grants if not g.request.ended]      # (the others ended while this step already ran)
         ended = self.scheduler.commit(plan, sampled)
         for request in ended:
             self._live.pop(request.id, None)
+        if ahead is not None:
+            next_plan, logits = ahead
+            if any(not g.request.ended for g in next_plan.grants):
+                self._flight = (next_plan, *self._sample(logits, next_plan.grants))
         self.stats.count(plan, time.perf_counter() - started)
-        return plan, sampled, ended
+        return committed, sampled, ended
 
     def step(self) -> list:
-        plan, sampled, ended = self._advance()
+        grants, sampled, ended = self._advance()
         done = {r.id for r in ended}
-        return [StepOutput(g.request.id, sampled.get(g.request.id), g.request.id in done) for g in plan.grants]
+        return [StepOutput(g.request.id, sampled.get(g.request.id) if g.samples else None, g.request.id in done) for g in grants]
 
     # ------------------------------------------------------------------ whole requests
     def _output(self, request: Request) -> RequestOutput:

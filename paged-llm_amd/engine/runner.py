@@ -564,20 +564,30 @@ class ModelRunner:
         return entry, self._restage_decode(entry, entries), len(entries)
 
     @torch.no_grad()
-    def run_prepared(self, handle, token_ids: list, copies: dict | None = None, borrow: bool = False) -> torch.Tensor:
-        """Runs a step staged by ``prepare`` with the token ids of its entries, in their order."""
+    def run_prepared(self, handle, token_ids, copies: dict | None = None, borrow: bool = False) -> torch.Tensor:
+        """Runs a step staged by ``prepare`` with the token ids of its entries, in their order: a list, or an int32
+        tensor on the GPU as the sampling kernel left it (the host need not have seen the ids: the step is queued
+        behind the kernel that writes them)."""
         entry, n_want, rows = handle
-        if len(token_ids) != rows:
-            raise StepError(f"{len(token_ids)} token ids for a prepared step of {rows} entries")
-        vocab = self.model.spec.vocab_size
-        if min(token_ids) < 0 or max(token_ids) >= vocab:
-            raise StepError(f"token id outside [0, {vocab})")
+        on_device = isinstance(token_ids, torch.Tensor)
+        if (token_ids.numel() if on_device else len(token_ids)) != rows:
+            raise StepError(f"{token_ids.numel() if on_device else len(token_ids)} token ids for a prepared step of {rows} entries")
+        if on_device:
+            if token_ids.dtype != torch.int32 or token_ids.device.type != self.device.type or token_ids.dim() != 1:
+                raise StepError("token ids on the device: an int32 vector on the model's GPU")
+        else:
+            vocab = self.model.spec.vocab_size
+            if min(token_ids) < 0 or max(token_ids) >= vocab:
+                raise StepError(f"token id outside [0, {vocab})")
         if copies:
             self.kv.apply_copies(copies)
         at = entry["offsets"][0]
-        entry["view"][at: at + rows] = token_ids
+        if not on_device:
+            entry["view"][at: at + rows] = token_ids
         entry["static"].copy_(entry["pinned"], non_blocking=True)
         entry["copied"].record()
+        if on_device:
+            entry["static"][at: at + rows].copy_(token_ids)       # (a sampled id is a valid id)
         entry["graph"].replay()
         logits = entry["logits"][:n_want]
         return logits if borrow else logits.clone()

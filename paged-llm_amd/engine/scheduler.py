@@ -77,9 +77,6 @@ class Scheduler:
         self.queue: deque = deque()          # Stage.QUEUED, the next to admit at the left
         self.active: list = []               # Stage.ACTIVE, in admission order
         self.num_preemptions = 0
-        # Counts everything that changes who runs next apart from every active request taking its next token: arrivals,
-        # cancellations, ends, preemptions.  A plan made ahead (``plan_ahead``) holds only while this number stands.
-        self.epoch = 0
 
     # ------------------------------------------------------------------ arrivals and departures
     def submit(self, request: Request) -> None:
@@ -95,7 +92,6 @@ class Scheduler:
             request.new_token_limit = max(1, room)
         request.stage = Stage.QUEUED
         self.queue.append(request)
-        self.epoch += 1
 
     def cancel(self, request_id) -> Request | None:
         """Ends a queued or active request at once; returns it, or None if it is not here."""
@@ -116,7 +112,6 @@ class Scheduler:
     def _retire(self, request: Request, reason: EndReason) -> None:
         self.cache.free(request.id)
         request.end(reason)
-        self.epoch += 1
 
     # ------------------------------------------------------------------ planning a step
     def plan(self) -> StepPlan:
@@ -159,7 +154,6 @@ class Scheduler:
             self.queue.appendleft(victim)
             plan.preempted.append(victim)
             self.num_preemptions += 1
-            self.epoch += 1
             if victim is request:
                 return False
         return True
@@ -183,8 +177,8 @@ class Scheduler:
         that the host's work for the next step overlaps the GPU's work for this one.  Only the steady state is
         predicted: every active request is in ``plan`` and reaches its last known token there, nobody waits in the
         queue, nobody can end by length in this step, and a page for everybody's next token is there without taking
-        anybody's.  Then the next plan is one token for each of them, in the same order.  None otherwise.  The caller
-        uses what it gets only while ``epoch`` stands (an end-of-sequence token in this step moves it)."""
+        anybody's.  Then the next plan is one token for each of them, in the same order.  None otherwise.  A request
+        that ends in ``plan`` after all (an end-of-sequence token) is passed over when the plan made here is committed."""
         if self.queue or plan.preempted or len(plan.grants) != len(self.active) or len(self.active) > self.step_budget:
             return None
         for grant in plan.grants:
@@ -219,10 +213,14 @@ class Scheduler:
     # ------------------------------------------------------------------ after the forward pass
     def commit(self, plan: StepPlan, sampled: dict) -> list:
         """Counts the step's tokens as computed, appends the sampled tokens (``sampled``: request id ->
-        token for every grant with ``samples``) and ends the requests that are done; returns those."""
+        token for every grant with ``samples``) and ends the requests that are done; returns those.  A grant
+        whose request is no longer active (it ended in the step before, which was still running when this one
+        was launched, or it was cancelled) is passed over: what the step computed for it is dropped."""
         ended = []
         for grant in plan.grants:
             request = grant.request
+            if request.stage is not Stage.ACTIVE:               # ended or cancelled after the step was launched
+                continue
             before = request.computed
             request.computed = before + grant.count
             self.cache.note_computed(request.id, request.tokens, before, request.computed)

@@ -16,8 +16,11 @@ class PendingTokens:
     """Token ids on their way from the GPU: the kernel and the copy to pinned host memory are queued, ``result()``
     waits for them.  Host work done between the two overlaps the GPU's."""
 
-    def __init__(self, staged: torch.Tensor | None, count: int, copied):
+    def __init__(self, staged: torch.Tensor | None, count: int, copied, on_device: torch.Tensor | None = None):
         self._staged, self._count, self._copied = staged, count, copied
+        # The same ids as the sampling kernel left them on the GPU (int32 [count]): a step that is launched before
+        # the host has seen them takes them from here.
+        self.on_device = on_device
 
     def result(self) -> list:
         if self._count == 0:
@@ -41,7 +44,7 @@ class Sampler:
             self._copied = torch.cuda.Event()
         self._pinned[:n].copy_(tokens, non_blocking=True)
         self._copied.record()
-        return PendingTokens(self._pinned, n, self._copied)
+        return PendingTokens(self._pinned, n, self._copied, tokens)
 
     @torch.no_grad()
     def launch(self, logits: torch.Tensor, params: list, request_keys: list, steps: list) -> PendingTokens:

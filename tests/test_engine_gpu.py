@@ -202,6 +202,57 @@ def test_step_api_and_abort(folder_a):
         engine.add_request("text")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_requests_that_stop_while_the_next_step_already_runs(folder_a, dtype):
+    """Decode steps are launched one ahead of the tokens the host has seen.  Requests stop on tokens of their own at
+    different steps (the plain implementation's greedy token at steps 6, 9 and 13), one is cancelled by hand and one
+    runs to its length: whoever goes on must get the logits of its own sequence, whoever stops must stop on its stop
+    token, and nothing of the step that was already running for it may show."""
+    from paged_llm_amd import SamplingParams
+    prompts = [helpers.random_tokens(n, 256, seed=60 + n) for n in (7, 12, 21, 9, 15)]
+    stops = []
+    for p, k in zip(prompts[:3], (6, 9, 13)):
+        greedy = plain_greedy(folder_a, p, 20)
+        stops.append(next(t for i, t in enumerate(greedy) if i >= k and t not in greedy[:i]))   # first new token from step k on
+    engine = engine_for(folder_a, dtype=dtype, max_num_batched_tokens=64)
+    assert engine.run_ahead
+    observed = Observed(engine)
+    params = [SamplingParams(temperature=0.0, max_tokens=20, stop_token_ids=[t]) for t in stops] + \
+             [SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)] * 2
+    ids = [engine.add_request(p, sp) for p, sp in zip(prompts, params)]
+    finished, steps = {}, 0
+    while engine.has_unfinished_requests:
+        for out in engine.step():
+            assert out.seq_id not in finished, "a finished request showed up again"
+            if out.finished:
+                finished[out.seq_id] = steps
+        steps += 1
+        if steps == 8:
+            engine.abort_request(ids[3])                        # while a step with its row is under way
+    assert ids[3] not in finished and not engine.step_in_flight
+    assert engine.cache_manager.num_free_pages() == 64
+    engine.cache_manager.check_invariants()
+    if dtype == "float32":
+        assert len({finished[i] for i in ids[:3]}) == 3         # they stopped at three different steps
+    for i, (rid, p) in enumerate(zip(ids, prompts)):
+        rows = sorted(pos for (r, pos) in observed.rows if r == rid)
+        assert rows == list(range(len(p) - 1, len(p) - 1 + len(rows))), "a position is missing or came twice"
+        tokens = list(p)
+        for pos in rows:                                        # the sequence the engine went along, from its own rows
+            want = helpers.plain_logits(folder_a, tokens)[pos]
+            assert helpers.worst(observed.rows[(rid, pos)], want) <= TOL[dtype], (rid, pos)
+            tokens.append(int(np.argmax(observed.rows[(rid, pos)])))
+        generated = tokens[len(p):]
+        if i < 3:
+            if dtype == "float32":
+                assert generated == plain_greedy(folder_a, p, len(generated)) and generated[-1] == stops[i]
+            # (in bfloat16 the engine may go another way than the plain implementation and never meet the token)
+            assert (generated[-1] == stops[i] and stops[i] not in generated[:-1]) or (stops[i] not in generated and len(generated) == 20)
+        elif i == 4:
+            assert len(generated) == 20
+    assert any(key[0] != "prompt" for key in engine.runner._graphs), "no decode step was replayed, so none ran ahead"
+
+
 def test_command_line(folder_a):
     cmd = [sys.executable, os.path.join(ROOT, "examples", "generate.py"), "--model", folder_a, "--max-tokens", "6",
            "--dtype", "float32", "--num-gpu-blocks", "32", "--max-model-len", "128", "--ignore-eos",

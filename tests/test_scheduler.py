@@ -240,3 +240,65 @@ def test_a_finished_request_is_no_longer_held_by_the_scheduler():
     sched.submit(req)
     _, ended = run_step(sched)
     assert ended == [req] and sched.idle and len(sched) == 0
+
+
+def test_the_step_after_can_be_planned_while_this_one_runs_only_in_the_steady_state():
+    """``plan_ahead`` foresees one more token for everybody, in the same order, and nothing else: not while somebody
+    waits in the queue, is still inside its prompt, may end by length in the step under way, or would need
+    somebody else's pages."""
+    _, cm, sched = make(num_blocks=12, block_size=4, budget=16)
+    a, b = Request([1] * 6, SamplingParams(max_tokens=5, ignore_eos=True)), Request([2] * 3, SamplingParams(max_tokens=9, ignore_eos=True))
+    sched.submit(a), sched.submit(b)
+    plan = sched.plan()                                              # both prompts whole
+    ahead = sched.plan_ahead(plan)
+    assert [g.request for g in ahead.grants] == [a, b] and all(g.count == 1 and g.samples for g in ahead.grants) and ahead.decode_tokens == 2
+    sched.commit(plan, {a.id: 7, b.id: 7})
+    after = sched.plan_ahead(ahead)                                  # and the one after that, from the plan that is under way
+    assert [g.request for g in after.grants] == [a, b]
+    sched.commit(ahead, {a.id: 7, b.id: 7})
+    sched.commit(after, {a.id: 7, b.id: 7})
+    cm.check_invariants()
+    assert a.num_generated == 3 and a.computed == 8 and len(cm.block_table(a.id, "full")) == 2
+    plan = sched.plan()                                              # a's fourth token of five
+    sched.commit(plan, {a.id: 7, b.id: 7})
+    plan = sched.plan()                                              # a's fifth: it ends by length in this step
+    assert sched.plan_ahead(plan) is None                            # so the step after is not one token for each of the two
+    sched.commit(plan, {a.id: 7, b.id: 7})
+    assert a.ended and not b.ended
+    late = Request([3] * 40, SamplingParams(max_tokens=2))
+    sched.submit(late)
+    plan = sched.plan()                                              # a portion of the newcomer beside b
+    assert len(plan.grants) == 2 and not plan.grants[1].samples and sched.plan_ahead(plan) is None
+    sched.cancel(late.id)
+    sched.commit(plan, {b.id: 7})                                    # (the cancelled request's grant is passed over)
+    plan = sched.plan()
+    assert [g.request for g in plan.grants] == [b] and sched.plan_ahead(plan) is not None
+    cm.check_invariants()
+
+
+def test_a_request_that_ended_is_passed_over_by_the_step_that_already_ran_for_it():
+    _, cm, sched = make()
+    a, b = Request([1] * 5, SamplingParams(max_tokens=9, stop_token_ids=(42,))), Request([2] * 5, SamplingParams(max_tokens=9, ignore_eos=True))
+    sched.submit(a), sched.submit(b)
+    sched.commit(sched.plan(), {a.id: 7, b.id: 7})
+    plan = sched.plan()
+    ahead = sched.plan_ahead(plan)
+    assert sched.commit(plan, {a.id: 42, b.id: 7}) == [a]            # a stops; the step after is under way with a row for it
+    free = cm.num_free_pages()
+    assert sched.commit(ahead, {a.id: 9, b.id: 8}) == []
+    assert a.generated == [7, 42] and b.generated == [7, 7, 8] and cm.num_free_pages() == free
+    assert sched.plan_ahead(ahead) is None                           # two grants, one active request: plan afresh
+    cm.check_invariants()
+
+
+def test_no_plan_ahead_when_the_next_token_needs_a_page_that_somebody_would_have_to_give():
+    _, cm, sched = make(num_blocks=4, block_size=4, budget=16)
+    a, b = Request([1] * 8, SamplingParams(max_tokens=9, ignore_eos=True)), Request([2] * 7, SamplingParams(max_tokens=9, ignore_eos=True))
+    sched.submit(a), sched.submit(b)
+    plan = sched.plan()                                              # 2 + 2 pages: the pool is full
+    assert cm.num_free_pages() == 0 and len(plan.grants) == 2
+    assert sched.plan_ahead(plan) is None                            # a's next token needs a third page
+    sched.commit(plan, {a.id: 7, b.id: 7})
+    plan = sched.plan()                                              # decided the ordinary way: the last admitted gives way
+    assert plan.preempted == [b] and [g.request for g in plan.grants] == [a]
+    cm.check_invariants()
