@@ -687,8 +687,12 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   const bool two = 2 * lds <= (size_t)pllm_lds_bytes_per_cu() && busiest2 <= busiest1;
   const int per_block = two ? per_block2 : busiest1;
   const int blocks = ceil_div(units, per_block);
+  // Slabs in flight per wavefront: two, or three when a wavefront of a workgroup with plain rows has three slabs of a
+  // unit (the down projection: K = 5632 is 22 slabs of 256 for 8 wavefronts), so that all of them travel at once.
 #define GO(EPI_, HALF_)                                                                                                   \
   do {                                                                                                                    \
+    const int step = (HALF_) ? 2 * kSlab : kSlab, most = ((K + step - 1) / step + waves - 1) / waves;                     \
+    if (direct && most == 3) return launch<EPI_, waves, HALF_, true, 3>(p, units, blocks, lds, stream);                   \
     if (direct) return launch<EPI_, waves, HALF_, true, 2>(p, units, blocks, lds, stream);                                \
     return launch<EPI_, waves, HALF_, false, 2>(p, units, blocks, lds, stream);                                           \
   } while (0)
