@@ -51,10 +51,11 @@ class EngineStats:
     num_preemptions: int = 0
     step_times: list = field(default_factory=list)
 
-    def count(self, plan: StepPlan, seconds: float) -> None:
+    def count(self, plan: StepPlan, seconds: float, dropped: int = 0) -> None:
+        """``dropped``: decoded tokens of the plan that were computed for requests that had ended meanwhile."""
         self.num_steps += 1
         self.num_prefill_tokens += plan.prompt_tokens
-        self.num_decode_tokens += plan.decode_tokens
+        self.num_decode_tokens += plan.decode_tokens - dropped
         self.num_preemptions += len(plan.preempted)
         self.step_times.append(seconds)
 
@@ -226,7 +227,7 @@ class LLMEngine:
             next_plan, logits = ahead
             if any(not g.request.ended for g in next_plan.grants):
                 self._flight = (next_plan, *self._sample(logits, next_plan.grants))
-        self.stats.count(plan, time.perf_counter() - started)
+        self.stats.count(plan, time.perf_counter() - started, dropped=len(plan.grants) - len(committed))
         return committed, sampled, ended
 
     def step(self) -> list:

@@ -220,10 +220,11 @@ def test_requests_that_stop_while_the_next_step_already_runs(folder_a, dtype):
     params = [SamplingParams(temperature=0.0, max_tokens=20, stop_token_ids=[t]) for t in stops] + \
              [SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)] * 2
     ids = [engine.add_request(p, sp) for p, sp in zip(prompts, params)]
-    finished, steps = {}, 0
+    finished, steps, shown = {}, 0, {}
     while engine.has_unfinished_requests:
         for out in engine.step():
             assert out.seq_id not in finished, "a finished request showed up again"
+            shown[out.seq_id] = shown.get(out.seq_id, 0) + (out.new_token is not None)
             if out.finished:
                 finished[out.seq_id] = steps
         steps += 1
@@ -232,6 +233,8 @@ def test_requests_that_stop_while_the_next_step_already_runs(folder_a, dtype):
     assert ids[3] not in finished and not engine.step_in_flight
     assert engine.cache_manager.num_free_pages() == 64
     engine.cache_manager.check_invariants()
+    # every token a step handed out is counted once (the first of a request with its prompt), the dropped rows are not
+    assert engine.stats.num_decode_tokens == sum(n - 1 for n in shown.values()) and engine.stats.num_prefill_tokens == sum(map(len, prompts))
     if dtype == "float32":
         assert len({finished[i] for i in ids[:3]}) == 3         # they stopped at three different steps
     for i, (rid, p) in enumerate(zip(ids, prompts)):
