@@ -49,6 +49,7 @@ class EngineStats:
     num_prefill_tokens: int = 0
     num_decode_tokens: int = 0
     num_preemptions: int = 0
+    num_dropped_tokens: int = 0        # computed in a step that ran ahead for requests that had ended meanwhile
     step_times: list = field(default_factory=list)
 
     def count(self, plan: StepPlan, seconds: float, dropped: int = 0) -> None:
@@ -56,6 +57,7 @@ class EngineStats:
         self.num_steps += 1
         self.num_prefill_tokens += plan.prompt_tokens
         self.num_decode_tokens += plan.decode_tokens - dropped
+        self.num_dropped_tokens += dropped
         self.num_preemptions += len(plan.preempted)
         self.step_times.append(seconds)
 

@@ -237,6 +237,7 @@ def test_requests_that_stop_while_the_next_step_already_runs(folder_a, dtype):
     assert engine.stats.num_decode_tokens == sum(n - 1 for n in shown.values()) and engine.stats.num_prefill_tokens == sum(map(len, prompts))
     if dtype == "float32":
         assert len({finished[i] for i in ids[:3]}) == 3         # they stopped at three different steps
+        assert engine.stats.num_dropped_tokens >= 3             # each time with the step after already under way
     for i, (rid, p) in enumerate(zip(ids, prompts)):
         rows = sorted(pos for (r, pos) in observed.rows if r == rid)
         assert rows == list(range(len(p) - 1, len(p) - 1 + len(rows))), "a position is missing or came twice"
