@@ -187,15 +187,19 @@ class LLMEngine:
         if ahead is None:
             return None
         cm = self.cache_manager
-        entries = []
-        for now, then in zip(plan.grants, ahead.grants):
+        row_of = {g.request.id: (i, g.count) for i, g in enumerate(plan.grants)}       # every grant of ``plan`` samples: row i
+        entries, rows = [], []
+        for then in ahead.grants:
             request = then.request
-            entries.append(StepEntry(request.id, [0], request.computed + now.count, {g: cm.block_table(request.id, g) for g in self.groups},
+            row, count = row_of[request.id]
+            rows.append(row)
+            entries.append(StepEntry(request.id, [0], request.computed + count, {g: cm.block_table(request.id, g) for g in self.groups},
                                      None, [0], cm.table_version(request.id)))
         staged = self.runner.prepare(entries)
         if staged is None:
             return None                                      # (the pages taken for the next tokens stay with their requests)
-        return ahead, self.runner.run_prepared(staged, pending.on_device, cm.take_pending_copies(), borrow=True)
+        take = None if len(rows) == len(plan.grants) else rows    # (some reach their limit in ``plan``: their rows are left out)
+        return ahead, self.runner.run_prepared(staged, pending.on_device, cm.take_pending_copies(), borrow=True, take=take)
 
     def _advance(self):
         """Commits one step.  (the grants it commits, sampled tokens by request id, requests that ended); no grants

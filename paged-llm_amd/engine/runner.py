@@ -564,12 +564,17 @@ class ModelRunner:
         return entry, self._restage_decode(entry, entries), len(entries)
 
     @torch.no_grad()
-    def run_prepared(self, handle, token_ids, copies: dict | None = None, borrow: bool = False) -> torch.Tensor:
+    def run_prepared(self, handle, token_ids, copies: dict | None = None, borrow: bool = False, take: list | None = None) -> torch.Tensor:
         """Runs a step staged by ``prepare`` with the token ids of its entries, in their order: a list, or an int32
         tensor on the GPU as the sampling kernel left it (the host need not have seen the ids: the step is queued
-        behind the kernel that writes them)."""
+        behind the kernel that writes them).  ``take``: the entries' ids are these elements of ``token_ids``."""
         entry, n_want, rows = handle
         on_device = isinstance(token_ids, torch.Tensor)
+        if take is not None:
+            if on_device:
+                token_ids = token_ids.index_select(0, torch.tensor(take, dtype=torch.int64).to(token_ids.device, non_blocking=True))
+            else:
+                token_ids = [token_ids[i] for i in take]
         if (token_ids.numel() if on_device else len(token_ids)) != rows:
             raise StepError(f"{token_ids.numel() if on_device else len(token_ids)} token ids for a prepared step of {rows} entries")
         if on_device:

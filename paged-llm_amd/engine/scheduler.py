@@ -174,26 +174,26 @@ class Scheduler:
 
     def plan_ahead(self, plan: StepPlan) -> StepPlan | None:
         """The plan of the step after ``plan``, made while ``plan`` still runs (its sampled tokens are not known yet), so
-        that the host's work for the next step overlaps the GPU's work for this one.  Only the steady state is
-        predicted: every active request is in ``plan`` and reaches its last known token there, nobody waits in the
-        queue, nobody can end by length in this step, and a page for everybody's next token is there without taking
-        anybody's.  Then the next plan is one token for each of them, in the same order.  None otherwise.  A request
-        that ends in ``plan`` after all (an end-of-sequence token) is passed over when the plan made here is committed."""
+        that the step after can be launched before the host has seen them.  Only the steady state is foreseen: every
+        active request is in ``plan`` and reaches its last known token there, nobody waits in the queue, and a page
+        for everybody's next token is there without taking anybody's.  Then the next plan is one token for each of
+        them, in the same order, but for those that reach their limit of new tokens or of positions in ``plan``: they
+        end there, whatever they sample.  None otherwise, or when nobody is left.  A request that ends in ``plan`` for
+        another reason (an end-of-sequence token) is passed over when the plan made here is committed."""
         if self.queue or plan.preempted or len(plan.grants) != len(self.active) or len(self.active) > self.step_budget:
             return None
-        for grant in plan.grants:
-            request = grant.request
-            if (not grant.samples or request.num_generated + 1 >= request.new_token_limit
-                    or len(request.tokens) + 1 >= self.max_positions):
-                return None
+        if not all(grant.samples for grant in plan.grants):
+            return None
         ahead = StepPlan()
         for grant in plan.grants:
             request = grant.request
+            if request.num_generated + 1 >= request.new_token_limit or len(request.tokens) + 1 >= self.max_positions:
+                continue                      # its last token comes from ``plan``
             if not self.cache.allocate(request.id, request.computed + grant.count, 1):
                 return None                   # (pages taken for the others so far are the ones their next step takes anyway)
             ahead.grants.append(Grant(request, 1, True))
         ahead.decode_tokens = len(ahead.grants)
-        return ahead
+        return ahead if ahead.grants else None
 
     def why_stuck(self) -> str:
         """Says why an empty plan came out although requests remain (for the caller's error)."""

@@ -93,8 +93,10 @@ class StandInRunner:
             return None                                        # no graph for this many rows yet
         return list(entries)
 
-    def run_prepared(self, handle, token_ids, copies=None, borrow=False):
+    def run_prepared(self, handle, token_ids, copies=None, borrow=False, take=None):
         self._copy(copies)
+        if take is not None:
+            token_ids = [token_ids[i] for i in take]
         assert len(token_ids) == len(handle)
         self.prepared += 1
         return self._run(handle, [[t] for t in token_ids])

@@ -243,11 +243,11 @@ def test_a_finished_request_is_no_longer_held_by_the_scheduler():
 
 
 def test_the_step_after_can_be_planned_while_this_one_runs_only_in_the_steady_state():
-    """``plan_ahead`` foresees one more token for everybody, in the same order, and nothing else: not while somebody
-    waits in the queue, is still inside its prompt, may end by length in the step under way, or would need
+    """``plan_ahead`` foresees one more token for everybody who does not reach a limit in the step under way, in the
+    same order, and nothing else: not while somebody waits in the queue, is still inside its prompt, or would need
     somebody else's pages."""
     _, cm, sched = make(num_blocks=12, block_size=4, budget=16)
-    a, b = Request([1] * 6, SamplingParams(max_tokens=5, ignore_eos=True)), Request([2] * 3, SamplingParams(max_tokens=9, ignore_eos=True))
+    a, b = Request([1] * 6, SamplingParams(max_tokens=5, ignore_eos=True)), Request([2] * 3, SamplingParams(max_tokens=19, ignore_eos=True))
     sched.submit(a), sched.submit(b)
     plan = sched.plan()                                              # both prompts whole
     ahead = sched.plan_ahead(plan)
@@ -261,10 +261,18 @@ def test_the_step_after_can_be_planned_while_this_one_runs_only_in_the_steady_st
     assert a.num_generated == 3 and a.computed == 8 and len(cm.block_table(a.id, "full")) == 2
     plan = sched.plan()                                              # a's fourth token of five
     sched.commit(plan, {a.id: 7, b.id: 7})
-    plan = sched.plan()                                              # a's fifth: it ends by length in this step
-    assert sched.plan_ahead(plan) is None                            # so the step after is not one token for each of the two
+    plan = sched.plan()                                              # a's fifth: it ends by length in this step, whatever it samples
+    ahead = sched.plan_ahead(plan)
+    assert [g.request for g in ahead.grants] == [b]                  # so the step after is foreseen without it
     sched.commit(plan, {a.id: 7, b.id: 7})
     assert a.ended and not b.ended
+    sched.commit(ahead, {b.id: 7})
+    only = Request([9] * 3, SamplingParams(max_tokens=1))
+    sched.submit(only)
+    plan = sched.plan()
+    assert len(plan.grants) == 2 and sched.plan_ahead(plan).grants[0].request is b and len(sched.plan_ahead(plan).grants) == 1
+    sched.commit(plan, {b.id: 7, only.id: 7})
+    assert only.ended
     late = Request([3] * 40, SamplingParams(max_tokens=2))
     sched.submit(late)
     plan = sched.plan()                                              # a portion of the newcomer beside b
