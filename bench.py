@@ -292,8 +292,8 @@ def run_attention_cases() -> dict:
 
 def time_mixed_step(engine, decode_requests: int, context: int, portion: int, seed: int, repeats: int = 6) -> dict:
     """One step that holds `decode_requests` decoded tokens at contexts near `context` beside a prompt portion of
-    `portion` tokens (what continuous batching runs whenever a request arrives): wall time of the step, and the
-    GPU's own time for it between two events (what is left is the host's share that the GPU waits for)."""
+    `portion` tokens (what continuous batching runs whenever a request arrives): wall time from the call of the step
+    to the arrival of its sampled tokens on the host."""
     import torch
     from paged_llm_amd import SamplingParams
     vocab = engine.model.spec.vocab_size
@@ -310,22 +310,18 @@ def time_mixed_step(engine, decode_requests: int, context: int, portion: int, se
         rid = engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
         if engine.step_in_flight:                              # the decode step that was under way when the request arrived
             assert len(engine.step()) == decode_requests
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        start.record()
-        out = engine.step()
-        end.record()
-        torch.cuda.synchronize()
+        out = engine.step()                                    # returns when the step's sampled tokens are on the host ...
         wall = time.perf_counter() - t0
+        torch.cuda.synchronize()                               # ... (the decode step after it may already be under way: not this step's time)
         assert len(out) == decode_requests + 1, "the step did not hold the decoded tokens and the portion"
-        gpu = start.elapsed_time(end) * 1e-3
-        if r >= 2 and (best is None or wall < best[0]):        # the shape is captured at its second sighting
-            best = (wall, gpu)
+        if r >= 2 and (best is None or wall < best):           # the shape is captured at its second sighting
+            best = wall
         engine.step()                                          # a plain decode step in between
     for r in list(engine.scheduler.active):
         engine.abort_request(r.id)
-    wall, gpu = best
+    wall = best
     tokens = decode_requests + portion
     return {"tokens": tokens, "ms": round(wall * 1e3, 3), "tokens_per_s": round(tokens / wall, 1)}
 
