@@ -520,6 +520,20 @@ def test_prompt_portions_with_key_partitions(heads, kv_heads, d, window):
         assert rel_err(got, want) <= 1.6e-2, f"partition {size}"
 
 
+def test_prompt_portion_with_more_partitions_than_a_wavefront_has_lanes():
+    """A portion behind 9,000 cached positions in 71 partitions of 128 keys: the merge walks them 64 at a time."""
+    heads, kv_heads, d, bs = 4, 1, 32, 16
+    q, kp, vp, tables, cu, sl = paged_case([9000], [80], heads, kv_heads, d, bs, torch.bfloat16, seed=14)
+    n, row, head = 8321, 40, 2                                         # one query looks at a key in the 66th partition only
+    page, off = int(tables[0, n // bs]), n % bs
+    kp[page, 0, off, :] = (q[row, head * d:(head + 1) * d].float() * 40).to(torch.bfloat16)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, 1.0)
+    got = ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, 1.0,
+                                     0, 80, 128, 71, 1, 2).cpu().float()
+    assert torch.allclose(got[row, head * d:(head + 1) * d], vp[page, 0, :, off].float(), atol=2e-2)
+    assert rel_err(got, want) <= 1.6e-2
+
+
 def test_prompt_partitions_are_chosen_to_fill_the_gpu():
     pp = ops().prompt_partitions
     assert pp(512, 4, 2048, 256) == (0, 1)                              # a whole prompt: tiles enough
