@@ -175,19 +175,25 @@ class Scheduler:
     def plan_ahead(self, plan: StepPlan) -> StepPlan | None:
         """The plan of the step after ``plan``, made while ``plan`` still runs (its sampled tokens are not known yet), so
         that the step after can be launched before the host has seen them.  Only the steady state is foreseen: every
-        active request is in ``plan`` and reaches its last known token there, nobody waits in the queue, and a page
-        for everybody's next token is there without taking anybody's.  Then the next plan is one token for each of
+        active request is in ``plan`` and reaches its last known token there, nobody waits in the queue (or every
+        place stays taken, so that nobody can be admitted: a place that an end-of-sequence token frees in ``plan``
+        is then filled one step later than it could be), and a page for everybody's next token is there without
+        taking anybody's.  Then the next plan is one token for each of
         them, in the same order, but for those that reach their limit of new tokens or of positions in ``plan``: they
         end there, whatever they sample.  None otherwise, or when nobody is left.  A request that ends in ``plan`` for
         another reason (an end-of-sequence token) is passed over when the plan made here is committed."""
-        if self.queue or plan.preempted or len(plan.grants) != len(self.active) or len(self.active) > self.step_budget:
+        if plan.preempted or len(plan.grants) != len(self.active) or len(self.active) > self.step_budget:
             return None
         if not all(grant.samples for grant in plan.grants):
             return None
+        at_limit = lambda r: r.num_generated + 1 >= r.new_token_limit or len(r.tokens) + 1 >= self.max_positions
+        staying = sum(1 for grant in plan.grants if not at_limit(grant.request))
+        if self.queue and staying < self.max_active:
+            return None                       # a place comes free (or is free): the next plan may admit somebody
         ahead = StepPlan()
         for grant in plan.grants:
             request = grant.request
-            if request.num_generated + 1 >= request.new_token_limit or len(request.tokens) + 1 >= self.max_positions:
+            if at_limit(request):
                 continue                      # its last token comes from ``plan``
             if not self.cache.allocate(request.id, request.computed + grant.count, 1):
                 return None                   # (pages taken for the others so far are the ones their next step takes anyway)

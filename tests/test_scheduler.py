@@ -310,3 +310,24 @@ def test_no_plan_ahead_when_the_next_token_needs_a_page_that_somebody_would_have
     plan = sched.plan()                                              # decided the ordinary way: the last admitted gives way
     assert plan.preempted == [b] and [g.request for g in plan.grants] == [a]
     cm.check_invariants()
+
+
+def test_plan_ahead_goes_on_while_others_wait_for_a_place_that_stays_taken():
+    _, cm, sched = make(max_seqs=2)
+    a, b = Request([1] * 4, SamplingParams(max_tokens=3, ignore_eos=True)), Request([2] * 4, SamplingParams(max_tokens=9, ignore_eos=True))
+    waiting = Request([3] * 4, SamplingParams(max_tokens=2))
+    for r in (a, b, waiting):
+        sched.submit(r)
+    plan = sched.plan()
+    assert [g.request for g in plan.grants] == [a, b] and len(sched.queue) == 1
+    ahead = sched.plan_ahead(plan)                                   # both stay: nobody can be admitted in the step after
+    assert [g.request for g in ahead.grants] == [a, b]
+    sched.commit(plan, {a.id: 7, b.id: 7})
+    sched.commit(ahead, {a.id: 7, b.id: 7})
+    plan = sched.plan()                                              # a's third token, its last
+    assert sched.plan_ahead(plan) is None                            # its place comes free: the step after may admit the one that waits
+    sched.commit(plan, {a.id: 7, b.id: 7})
+    assert a.ended
+    plan = sched.plan()
+    assert [g.request for g in plan.grants] == [b, waiting]
+    cm.check_invariants()
