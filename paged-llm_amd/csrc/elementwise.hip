@@ -232,7 +232,37 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
                                     const float* __restrict__ cos_table, const float* __restrict__ sin_table,
                                     const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                     int num_heads, int num_kv_heads, int head_dim, int block_size, int write_kv,
-                                    int rotary_dim, int interleaved) {
+                                    int rotary_dim, int interleaved, int num_tokens, int value_groups) {
+  // With value_groups > 0 the workgroups past the first num_tokens write the values: one for 16 tokens in a row.
+  // Values sit transposed in a page ([channel][position]), so a token alone writes single elements a page's
+  // width apart; 16 tokens whose slots follow each other inside one page (a prompt portion) fill whole rows of
+  // 16 positions, written in 16-byte pieces.
+  if (value_groups > 0 && (int)blockIdx.x >= num_tokens) {
+    const int t0 = ((int)blockIdx.x - num_tokens) * 16, n = min(16, num_tokens - t0);
+    const int s0 = slot_mapping[t0];
+    bool in_a_row = n == 16 && s0 >= 0 && (s0 & (block_size - 1)) + 16 <= block_size && ((s0 * sizeof(T)) & 15) == 0 &&
+                    ((uintptr_t)v_pages & 15) == 0 && ((block_size * sizeof(T)) & 15) == 0;
+    for (int i = 1; i < 16 && in_a_row; ++i) in_a_row = slot_mapping[t0 + i] == s0 + i;      // (uniform in the workgroup)
+    const size_t v_at = (size_t)(num_heads + num_kv_heads) * head_dim;
+    for (int w = threadIdx.x; w < num_kv_heads * head_dim; w += blockDim.x) {
+      const int kvh = w / head_dim, i = w - kvh * head_dim;
+      if (in_a_row) {
+        const int page = s0 / block_size, off = s0 - page * block_size;
+        struct alignas(16) Row { T v[16]; } out;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) out.v[j] = qkv[(size_t)(t0 + j) * row_stride + v_at + w];
+        *reinterpret_cast<Row*>(v_pages + (((size_t)page * num_kv_heads + kvh) * head_dim + i) * block_size + off) = out;
+      } else {
+        for (int j = 0; j < n; ++j) {
+          const int slot = slot_mapping[t0 + j];
+          if (slot < 0) continue;
+          const int page = slot / block_size, off = slot - page * block_size;
+          v_pages[(((size_t)page * num_kv_heads + kvh) * head_dim + i) * block_size + off] = qkv[(size_t)(t0 + j) * row_stride + v_at + w];
+        }
+      }
+    }
+    return;
+  }
   const int t = blockIdx.x;
   const int half = rotary_dim >> 1;                      // pairs per head, and the tables' row length
   const int pos = positions[t];
@@ -299,7 +329,7 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
       }
     }
   }
-  if (slot >= 0) {
+  if (slot >= 0 && value_groups == 0) {
     const T* v = row + (size_t)(num_heads + num_kv_heads) * head_dim;
     for (int w = threadIdx.x; w < num_kv_heads * head_dim; w += blockDim.x) {
       const int kvh = w / head_dim, i = w - kvh * head_dim;
@@ -316,15 +346,18 @@ PLLM_API int pllm_rope_scatter(int dtype, void* qkv, int row_stride, const int* 
                                int write_kv, int rotary_dim, int interleaved, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (rotary_dim < 0 || rotary_dim > head_dim || (rotary_dim & 1)) return -2;
-  dim3 grid(num_tokens), block(256);
+  // Many tokens (prompt portions) and pages that hold 16 positions of a row: the values are written by workgroups of
+  // their own, 16 tokens each.
+  const int value_groups = (write_kv && num_tokens >= 64 && block_size >= 16) ? (num_tokens + 15) / 16 : 0;
+  dim3 grid(num_tokens + value_groups), block(256);
   if (dtype == PLLM_F32)
     hipLaunchKernelGGL(rope_scatter_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, positions, cos_table,
                        sin_table, slot_mapping, (float*)k_pages, (float*)v_pages, num_heads, num_kv_heads, head_dim,
-                       block_size, write_kv, rotary_dim, interleaved);
+                       block_size, write_kv, rotary_dim, interleaved, num_tokens, value_groups);
   else
     hipLaunchKernelGGL(rope_scatter_kernel<bf16>, grid, block, 0, stream, (bf16*)qkv, row_stride, positions, cos_table,
                        sin_table, slot_mapping, (bf16*)k_pages, (bf16*)v_pages, num_heads, num_kv_heads, head_dim,
-                       block_size, write_kv, rotary_dim, interleaved);
+                       block_size, write_kv, rotary_dim, interleaved, num_tokens, value_groups);
   PLLM_RETURN_LAST_ERROR();
 }
 

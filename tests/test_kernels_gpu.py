@@ -85,10 +85,12 @@ def test_silu_mul(dtype):
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 16, 16), (3, 1, 48, 8), (8, 8, 128, 32)])
 def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs, slots):
     """``runs``: the slots of prompt portions (consecutive positions): a portion from a page's start, one that
-    starts 3 slots into a page, and between them a token that writes nothing."""
+    starts 3 slots into a page, and between them a token that writes nothing.  Enough tokens for the form that
+    writes the values of 16 tokens at a time: whole rows where their slots follow each other inside a page, single
+    elements where they do not (shuffled slots, a portion that starts inside a page, the token without a slot)."""
     from paged_llm_amd.parts.registry import BuildEnv
     from paged_llm_amd.parts.rope import RotaryEncoding
-    T, pages = (23, 9) if slots == "shuffled" else (61, 12)
+    T, pages = (71, 9) if slots == "shuffled" else (93, 12)
     rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, dtype, torch.device("cuda"), 512, {}))
     rope.prepare(512)
     width = (heads + 2 * kv_heads) * d
@@ -100,7 +102,7 @@ def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs, slots):
         def portion(first_page, start, n):                       # n consecutive positions from `start` of a request
             table = order[first_page:]
             return [table[(start + i) // bs] * bs + (start + i) % bs for i in range(n)]
-        perm = torch.tensor(portion(0, 0, 32) + [-1] + portion(6, 3, 28), dtype=torch.int32)
+        perm = torch.tensor(portion(0, 0, 48) + [-1] + portion(6, 3, 44), dtype=torch.int32)
         assert perm.numel() == T
     k_pages = torch.zeros(pages, kv_heads, bs, d, dtype=dtype).cuda()
     v_pages = torch.zeros(pages, kv_heads, d, bs, dtype=dtype).cuda()
