@@ -102,11 +102,17 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed:
         engine.step()
     torch.cuda.synchronize()
     before = sum(len(r.tokens) for r in engine.scheduler.active)
+    returns = []
     t0 = time.perf_counter()
     for _ in range(steps):
         out = engine.step()
+        returns.append(time.perf_counter())          # a step returns when its tokens are on the host: no extra waiting
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    # How even the steps are: the time between the returns of consecutive steps (the first one has no predecessor).
+    gaps = sorted(b - a for a, b in zip(returns, returns[1:]))
+    time_decode.spread = ({"min_ms": round(gaps[0] * 1e3, 4), "median_ms": round(gaps[len(gaps) // 2] * 1e3, 4),
+                           "max_ms": round(gaps[-1] * 1e3, 4)} if gaps else {})
     assert len(out) == batch
     after = sum(len(r.tokens) for r in engine.scheduler.active)
     assert max(len(r.tokens) for r in engine.scheduler.active) <= context + 1, "a context passed the one asked for"
@@ -582,6 +588,7 @@ def main() -> int:
             print(json.dumps(time_mixed_step(engine, args.batch, args.context, 256, seed=50, repeats=12)))
             return 0
         sec, mean_context = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
+        spread = time_decode.spread
         value = args.batch / sec
         decode_bytes = numbers["weight_bytes"] + args.batch * mean_context * numbers["kv_bytes_per_token"]
         achieved = decode_bytes / sec / 1e9
@@ -596,6 +603,7 @@ def main() -> int:
                        "parallelism": "single GPU"},
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(achieved / PEAK_HBM_GBS, 4)},
+            "step_spread": spread,
         }
         if not args.no_points:
             points = {}
