@@ -239,10 +239,13 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
   // 16 positions, written in 16-byte pieces.
   if (value_groups > 0 && (int)blockIdx.x >= num_tokens) {
     const int t0 = ((int)blockIdx.x - num_tokens) * 16, n = min(16, num_tokens - t0);
-    const int s0 = slot_mapping[t0];
-    bool in_a_row = n == 16 && s0 >= 0 && (s0 & (block_size - 1)) + 16 <= block_size && ((s0 * sizeof(T)) & 15) == 0 &&
-                    ((uintptr_t)v_pages & 15) == 0 && ((block_size * sizeof(T)) & 15) == 0;
-    for (int i = 1; i < 16 && in_a_row; ++i) in_a_row = slot_mapping[t0 + i] == s0 + i;      // (uniform in the workgroup)
+    // The 16 slots with one load (lane j of every wavefront holds token j's), not one after the other.
+    const int lane = threadIdx.x & 63;
+    const int my_slot = lane < n ? slot_mapping[t0 + lane] : -1;
+    const int s0 = __builtin_amdgcn_readlane(my_slot, 0);
+    const bool in_a_row = __all(lane >= 16 || my_slot == s0 + lane) && n == 16 && s0 >= 0 &&      // (uniform in the workgroup)
+                          (s0 & (block_size - 1)) + 16 <= block_size && ((s0 * sizeof(T)) & 15) == 0 &&
+                          ((uintptr_t)v_pages & 15) == 0 && ((block_size * sizeof(T)) & 15) == 0;
     const size_t v_at = (size_t)(num_heads + num_kv_heads) * head_dim;
     for (int w = threadIdx.x; w < num_kv_heads * head_dim; w += blockDim.x) {
       const int kvh = w / head_dim, i = w - kvh * head_dim;
@@ -253,8 +256,9 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
         for (int j = 0; j < 16; ++j) out.v[j] = qkv[(size_t)(t0 + j) * row_stride + v_at + w];
         *reinterpret_cast<Row*>(v_pages + (((size_t)page * num_kv_heads + kvh) * head_dim + i) * block_size + off) = out;
       } else {
-        for (int j = 0; j < n; ++j) {
-          const int slot = slot_mapping[t0 + j];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {                           // (tokens past the last one hold -1)
+          const int slot = __builtin_amdgcn_readlane(my_slot, j);
           if (slot < 0) continue;
           const int page = slot / block_size, off = slot - page * block_size;
           v_pages[(((size_t)page * num_kv_heads + kvh) * head_dim + i) * block_size + off] = qkv[(size_t)(t0 + j) * row_stride + v_at + w];
@@ -347,8 +351,9 @@ PLLM_API int pllm_rope_scatter(int dtype, void* qkv, int row_stride, const int* 
   if (num_tokens <= 0) return 0;
   if (rotary_dim < 0 || rotary_dim > head_dim || (rotary_dim & 1)) return -2;
   // Many tokens (prompt portions) and pages that hold 16 positions of a row: the values are written by workgroups of
-  // their own, 16 tokens each.
-  const int value_groups = (write_kv && num_tokens >= 64 && block_size >= 16) ? (num_tokens + 15) / 16 : 0;
+  // their own, 16 tokens each.  (A few hundred tokens are done sooner without: the kernel then ends with its longest
+  // workgroup, and one that gathers 16 tokens is longer than one that scatters a single token.)
+  const int value_groups = (write_kv && num_tokens >= 512 && block_size >= 16) ? (num_tokens + 15) / 16 : 0;
   dim3 grid(num_tokens + value_groups), block(256);
   if (dtype == PLLM_F32)
     hipLaunchKernelGGL(rope_scatter_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, positions, cos_table,

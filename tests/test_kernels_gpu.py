@@ -90,7 +90,9 @@ def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs, slots):
     elements where they do not (shuffled slots, a portion that starts inside a page, the token without a slot)."""
     from paged_llm_amd.parts.registry import BuildEnv
     from paged_llm_amd.parts.rope import RotaryEncoding
-    T, pages = (71, 9) if slots == "shuffled" else (93, 12)
+    n1, n2 = 272, 270                                            # (the 16-at-a-time form is taken from 512 tokens on)
+    second = (n1 + bs - 1) // bs                                 # the second portion's first page
+    T, pages = (531, (531 + bs - 1) // bs + 2) if slots == "shuffled" else (n1 + 1 + n2, second + (3 + n2 + bs - 1) // bs + 1)
     rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, dtype, torch.device("cuda"), 512, {}))
     rope.prepare(512)
     width = (heads + 2 * kv_heads) * d
@@ -102,7 +104,7 @@ def test_rope_and_cache_write(dtype, heads, kv_heads, d, bs, slots):
         def portion(first_page, start, n):                       # n consecutive positions from `start` of a request
             table = order[first_page:]
             return [table[(start + i) // bs] * bs + (start + i) % bs for i in range(n)]
-        perm = torch.tensor(portion(0, 0, 48) + [-1] + portion(6, 3, 44), dtype=torch.int32)
+        perm = torch.tensor(portion(0, 0, n1) + [-1] + portion(second, 3, n2), dtype=torch.int32)
         assert perm.numel() == T
     k_pages = torch.zeros(pages, kv_heads, bs, d, dtype=dtype).cuda()
     v_pages = torch.zeros(pages, kv_heads, d, bs, dtype=dtype).cuda()
