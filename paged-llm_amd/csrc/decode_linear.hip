@@ -430,10 +430,11 @@ __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLin
   const int my_slabs = wave < num_slabs ? (num_slabs - wave + WAVES - 1) / WAVES : 0;
   const int padded_slabs = max(PRE, (my_slabs + PRE - 1) / PRE * PRE);
   bf16x8 wbuf[PRE][4], xbuf[PRE][MT][4];
+  const int row0 = blockIdx.y * (MT * 16);                      // (a second line of workgroups takes the rows after the first MT tiles)
   const bf16* xsrc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {                                // tile columns past M read row M - 1; never stored
-    const int row = min(t * 16 + r, M - 1);
+    const int row = min(row0 + t * 16 + r, M - 1);
     xsrc[t] = p.x + (size_t)(p.row_index ? p.row_index[row] : row) * p.ldx;
   }
   auto load_w = [&](const bf16* wrow, int nth, bf16x8 (&dst)[4]) {      // unconditional, as in the kernel above
@@ -466,9 +467,9 @@ __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLin
   for (int t = 0; t < MT; ++t) {
     rope_pos[t] = 0;
     rope_slot[t] = -1;
-    if (EPI == EPI_ROPE_KV && tid < 256 && t * 16 + r < M) {
-      rope_pos[t] = p.cos_t ? p.positions[t * 16 + r] : 0;
-      rope_slot[t] = p.slots[t * 16 + r];
+    if (EPI == EPI_ROPE_KV && tid < 256 && row0 + t * 16 + r < M) {
+      rope_pos[t] = p.cos_t ? p.positions[row0 + t * 16 + r] : 0;
+      rope_slot[t] = p.slots[row0 + t * 16 + r];
     }
   }
 #pragma unroll
@@ -493,7 +494,7 @@ __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLin
       if (row < 8 && head < p.num_heads + p.num_kv_heads) {
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-          if (t * 16 + r < M) {
+          if (row0 + t * 16 + r < M) {
             rope_cs[t] = p.cos_t[(size_t)rope_pos[t] * half + ri];
             rope_sn[t] = p.sin_t[(size_t)rope_pos[t] * half + ri];
           }
@@ -541,7 +542,7 @@ __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLin
           for (int w = 0; w < WAVES; ++w) s += part[(w * MT + t) * 256 + i * 64 + ln];
           return s;
         };
-        const int m = t * 16 + r;
+        const int m = row0 + t * 16 + r;
         if (m >= M) continue;
         if (EPI == EPI_BF16 || EPI == EPI_F32) {
           const int n = unit * 16 + row;
@@ -568,16 +569,32 @@ __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLin
 }
 
 template <int EPI>
-static int launch_wide(const DecodeLinearParams& p, int units, int blocks, hipStream_t stream) {
-  const int tiles = (p.M + 15) / 16;
+static int launch_wide(const DecodeLinearParams& p, int units, int blocks, int cus, hipStream_t stream) {
+  int tiles = (p.M + 15) / 16, lines = 1;
+  // A matrix with so few units that one workgroup each leaves compute units idle (the output and q/k/v products of a
+  // 2048-wide model): two lines of workgroups, each with half of the row tiles, all resident at once (half of the compute
+  // units per line).  Every unit's weights are then read by two workgroups (with a number of workgroups per line that
+  // is a multiple of the L2s' number both sit behind the same L2, and the second read is a hit), each of which fetches
+  // half the rows and finishes half the sums.  2048 x 2048: 11.5 -> 7.9 us at 64 rows, 7.8 -> 6.1 us at 32 rows;
+  // 2560 x 2048 (160 units, so some workgroups take two): 11.7 -> 10.2 us at 64 rows.  More workgroups than compute
+  // units lose: four lines of one tile at 64 rows 9.6 us, 160 units in two full lines 13.0 us.
+  if (tiles >= 3 && units <= cus) {
+    tiles = 2;
+    lines = 2;
+    blocks = min(blocks, cus / 2);
+  } else if (tiles == 2 && 2 * units <= cus) {
+    tiles = 1;
+    lines = 2;
+  }
   const size_t lds = (size_t)8 * tiles * 256 * sizeof(float);
   const bool fixed = (p.K + kSlab - 1) / kSlab <= 2 * 8;      // at most PRE slabs for each of the 8 wavefronts
-#define PLLM_WIDE(MT_)                                                                                                              \
-  do {                                                                                                                              \
-    if (fixed) hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, MT_, true>), dim3(blocks), dim3(512), lds, stream, p, units);     \
-    else hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, MT_, false>), dim3(blocks), dim3(512), lds, stream, p, units);          \
+#define PLLM_WIDE(MT_)                                                                                                                     \
+  do {                                                                                                                                     \
+    if (fixed) hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, MT_, true>), dim3(blocks, lines), dim3(512), lds, stream, p, units);     \
+    else hipLaunchKernelGGL((decode_linear_wide_kernel<EPI, MT_, false>), dim3(blocks, lines), dim3(512), lds, stream, p, units);          \
   } while (0)
   switch (tiles) {
+    case 1: PLLM_WIDE(1); break;
     case 2: PLLM_WIDE(2); break;
     case 3: PLLM_WIDE(3); break;
     case 4: PLLM_WIDE(4); break;
@@ -668,10 +685,10 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   if (M > 16) {                                                 // tiles of 16 rows side by side, one workgroup per compute unit
     const int per_block = (units + cus - 1) / cus, blocks = (units + per_block - 1) / per_block;
     switch (epi) {
-      case EPI_BF16: return launch_wide<EPI_BF16>(p, units, blocks, stream);
-      case EPI_F32: return launch_wide<EPI_F32>(p, units, blocks, stream);
-      case EPI_GATED: return launch_wide<EPI_GATED>(p, units, blocks, stream);
-      case EPI_ROPE_KV: return launch_wide<EPI_ROPE_KV>(p, units, blocks, stream);
+      case EPI_BF16: return launch_wide<EPI_BF16>(p, units, blocks, cus, stream);
+      case EPI_F32: return launch_wide<EPI_F32>(p, units, blocks, cus, stream);
+      case EPI_GATED: return launch_wide<EPI_GATED>(p, units, blocks, cus, stream);
+      case EPI_ROPE_KV: return launch_wide<EPI_ROPE_KV>(p, units, blocks, cus, stream);
     }
     return -3;
   }

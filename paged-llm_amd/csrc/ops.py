@@ -324,7 +324,8 @@ def decode_linear_pays(rows: int, N: int, K: int, epi: int, staged: bool) -> boo
     product; by sizes only).  Every unit of 16 weight rows rereads all rows from the cache: beyond 8 rows
     that is as much as it streams of weights, and the library wins for long rows (K = 5632, 14336); beyond
     16 rows it wins for all but small matrices (q/k/v and output projections of 2048-wide models), where
-    the fused kernel still fills the chip better; beyond 32 rows only the saved rotary kernel pays.  The gate/up
+    the fused kernel still fills the chip better; beyond 32 rows only the saved rotary kernel pays, and matrices of
+    at most 2048 rows, whose units leave half of the GPU free for a second line of workgroups.  The gate/up
     product of a 2048-wide model is the exception: with K <= 2048 a wavefront keeps its share of the rows in
     registers for all units of its workgroup, and with the SiLU kernel saved the fused form wins up to 48 rows
     (11264 x 2048: 15.3 against 17.2 us at 32 rows, 18.0 against 18.8 at 48, 20.2 against 18.7 at 64)."""
@@ -335,6 +336,8 @@ def decode_linear_pays(rows: int, N: int, K: int, epi: int, staged: bool) -> boo
     if epi == EPI_GATED and K <= 2048 and rows <= 48:
         return True
     small = N * K <= (1 << 23)
+    if small and N <= 2048:
+        return True          # (at most 128 units: two lines of workgroups with half the rows each, 7.9 against 9.0 us at 64 rows)
     return small and (rows <= 32 or epi == EPI_ROPE_KV)
 
 
