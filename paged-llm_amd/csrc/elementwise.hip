@@ -115,11 +115,20 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
   const int pieces = hidden / V;
   const Piece* xr = reinterpret_cast<const Piece*>(x + src * hidden);
   Piece px[P], pd[P];
+  // The norm's weights are requested with the row (for rows of up to 8 pieces per lane, which leaves registers for
+  // them): asked for where they are used, behind the sum, they would cost a second wait for memory.
+  constexpr bool kWeightsEarly = P <= 8;
+  struct alignas(16) Weights { float v[V]; };
+  Weights pw[kWeightsEarly ? P : 1];
 #pragma unroll
   for (int i = 0; i < P; ++i) {
     const int c = min(lane + i * 64, pieces - 1);                // inside the row; what lies past it is not used
     px[i] = xr[c];
     if (delta) pd[i] = reinterpret_cast<const Piece*>(delta + src * hidden)[c];
+  }
+  if constexpr (kWeightsEarly) {
+#pragma unroll
+    for (int i = 0; i < P; ++i) pw[i] = reinterpret_cast<const Weights*>(w)[min(lane + i * 64, pieces - 1)];
   }
   float acc = 0.f;
 #pragma unroll
@@ -142,7 +151,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
     if (c >= pieces) continue;
     Piece po;
 #pragma unroll
-    for (int j = 0; j < V; ++j) po.v[j] = from_f32<T>((to_f32(px[i].v[j]) * inv) * w[c * V + j]);
+    for (int j = 0; j < V; ++j) po.v[j] = from_f32<T>((to_f32(px[i].v[j]) * inv) * (kWeightsEarly ? pw[i].v[j] : w[c * V + j]));
     o[c] = po;
   }
 }
