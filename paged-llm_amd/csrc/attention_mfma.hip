@@ -791,6 +791,19 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
   // maxima of up to 64 partitions at a time, one per lane, requested at once
   float m_mine = -INFINITY;
   if (lane < num_partitions) m_mine = base[(size_t)lane * kPartialFloats];
+  // ... and behind them, before anything is waited for, the partial results of the first kEarly partitions (all there
+  // are, for most contexts): a loop over a number of partitions that is known only at run time would request
+  // them after the maxima and the lengths have arrived, four at a time, each time with a wait of its own.
+  constexpr int kEarly = 8, kPerLane = (D + 63) / 64;
+  float early_m[kEarly], early_l[kEarly], early_a[kEarly][kPerLane];
+#pragma unroll
+  for (int p = 0; p < kEarly; ++p) {
+    const float* pp = base + (size_t)min(p, num_partitions - 1) * kPartialFloats;
+    early_m[p] = pp[0];
+    early_l[p] = pp[1];
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) early_a[p][j] = pp[2 + min(lane + j * 64, D - 1)];
+  }
   int seq = tok, q_begin = tok, num_q = 1;
   if (!ONE_QUERY) {
     int lo = 0, hi = num_seqs - 1;
@@ -814,8 +827,16 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
   float o[(D + 63) / 64];
 #pragma unroll
   for (int j = 0; j < (D + 63) / 64; ++j) o[j] = 0.f;
+#pragma unroll
+  for (int p = 0; p < kEarly; ++p) {                             // (in partition order, as below)
+    const bool counts = p < num_partitions && p >= p_lo && p <= p_hi;
+    const float w = counts ? fast_exp2(early_m[p] - M) : 0.f;
+    l += counts ? w * early_l[p] : 0.f;
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) o[j] += counts ? w * early_a[p][j] : 0.f;
+  }
 #pragma unroll 4
-  for (int p = 0; p < num_partitions; ++p) {                     // all of them: the loads wait for nothing
+  for (int p = kEarly; p < num_partitions; ++p) {                // all of them: the loads wait for nothing
     const float* pp = base + (size_t)p * kPartialFloats;
     const bool counts = p >= p_lo && p <= p_hi;
     const float m_p = pp[0], l_p = pp[1];
