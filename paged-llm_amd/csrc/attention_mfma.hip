@@ -34,6 +34,13 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
+// Lengths and page tables are read through the constant address space: what a launch is given there does not change
+// while it runs, and a load from that address space at an address that is the same in all lanes is a scalar load
+// whatever else the kernel does (the compiler otherwise makes vector loads of them as soon as anything it cannot see
+// through stands in front, and a vector load's result arrives only behind every vector load requested before it).
+typedef const int __attribute__((address_space(4))) * ConstantInts;
+__device__ __forceinline__ ConstantInts as_constant(const int* p) { return (ConstantInts)p; }
+
 constexpr int D = HEAD_DIM;
 constexpr int KSTEPS = (D + 31) / 32;   // MFMA steps over the head dimension for Q K^T
 constexpr int DBLOCKS = D / 16;          // 16-channel blocks of the output
@@ -87,6 +94,11 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
     int block_size, float scale, int window, int partition_size, int num_partitions, float* __restrict__ partials) {
+  // Fetch all arguments in one go (left alone, the compiler fetches each where it is first used, and every fetch is
+  // a wait of its own in the chain lengths -> page table -> keys).
+  asm volatile("" ::"s"(q), "s"(q_stride), "s"(k_pages), "s"(v_pages), "s"(out), "s"(out_stride), "s"(block_tables), "s"(bt_stride),
+               "s"(cu_seqlens_q), "s"(seq_lens_k), "s"(num_heads), "s"(num_kv_heads), "s"(block_size), "s"(scale), "s"(window),
+               "s"(partition_size), "s"(num_partitions), "s"(partials));
   // The wavefront's index is the same in all its lanes; saying so keeps everything derived from it (key ranges,
   // page-table entries, page addresses) in scalar registers.
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = lane & 15, g = lane >> 4;
@@ -94,8 +106,9 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   const int seq = blockIdx.z;
   const int kvh = blockIdx.y / num_partitions, part = blockIdx.y - kvh * num_partitions;
   const int G = num_heads / num_kv_heads;
-  const int q_begin = cu_seqlens_q[seq], num_q = cu_seqlens_q[seq + 1] - q_begin;
-  const int len_k = seq_lens_k[seq];
+  const int q_begin = as_constant(cu_seqlens_q)[seq], num_q = as_constant(cu_seqlens_q)[seq + 1] - q_begin;
+  const int len_k = as_constant(seq_lens_k)[seq];
+  asm volatile("" ::"s"(q_begin), "s"(num_q), "s"(len_k));       // (all three requested here, with one wait)
   const int num_cols = num_q * G;
   const int col0 = blockIdx.x * 16 * NCB;
   if (col0 >= num_cols) return;
@@ -143,7 +156,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     for (int db = 0; db < DBLOCKS; ++db) acc[cb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
   const float sl2 = scale * kLog2e;
-  const int* bt = block_tables + (size_t)seq * bt_stride;
+  ConstantInts bt = as_constant(block_tables) + (size_t)seq * bt_stride;
   const size_t page_elems = (size_t)block_size * D;             // one kv head's part of a page
   const size_t page_stride = page_elems * num_kv_heads;
 
@@ -156,13 +169,20 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     bf16x4 v[4][DBLOCKS];
     bool on[4];
   };
+  const int last_tile = (k_hi - 1) & ~15;
   auto load_block = [&](KVBlock& blk, int n0) {
+    // The four tiles' page-table entries first, together (a tile past the range looks the range's last tile up
+    // again, so no entry past the context is read): one wait, not one per tile.
+    int pages[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) pages[kt] = bt[min(n0 + kt * 16, last_tile) >> bs_shift];
+    asm volatile("" ::"s"(pages[0]), "s"(pages[1]), "s"(pages[2]), "s"(pages[3]));   // (here, not each where its tile begins)
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
       const int nk = n0 + kt * 16;
-      blk.on[kt] = nk < k_hi;                                   // uniform; tiles past the range: table entries stay unread
+      blk.on[kt] = nk < k_hi;                                   // uniform
       if (!blk.on[kt]) continue;
-      const int page = bt[nk >> bs_shift];
+      const int page = pages[kt];
       const int off = nk & (block_size - 1);
       const size_t base = (size_t)page * page_stride + (size_t)kvh * page_elems;
       const bf16* krow = k_pages + base + (size_t)(off + r) * D;
