@@ -96,9 +96,11 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     int block_size, float scale, int window, int partition_size, int num_partitions, float* __restrict__ partials) {
   // Fetch all arguments in one go (left alone, the compiler fetches each where it is first used, and every fetch is
   // a wait of its own in the chain lengths -> page table -> keys).
-  asm volatile("" ::"s"(q), "s"(q_stride), "s"(k_pages), "s"(v_pages), "s"(out), "s"(out_stride), "s"(block_tables), "s"(bt_stride),
-               "s"(cu_seqlens_q), "s"(seq_lens_k), "s"(num_heads), "s"(num_kv_heads), "s"(block_size), "s"(scale), "s"(window),
-               "s"(partition_size), "s"(num_partitions), "s"(partials));
+  constexpr bool kLookupsTogether = D <= 64;
+  if constexpr (kLookupsTogether)
+    asm volatile("" ::"s"(q), "s"(q_stride), "s"(k_pages), "s"(v_pages), "s"(out), "s"(out_stride), "s"(block_tables), "s"(bt_stride),
+                 "s"(cu_seqlens_q), "s"(seq_lens_k), "s"(num_heads), "s"(num_kv_heads), "s"(block_size), "s"(scale), "s"(window),
+                 "s"(partition_size), "s"(num_partitions), "s"(partials));
   // The wavefront's index is the same in all its lanes; saying so keeps everything derived from it (key ranges,
   // page-table entries, page addresses) in scalar registers.
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = lane & 15, g = lane >> 4;
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   const int G = num_heads / num_kv_heads;
   const int q_begin = as_constant(cu_seqlens_q)[seq], num_q = as_constant(cu_seqlens_q)[seq + 1] - q_begin;
   const int len_k = as_constant(seq_lens_k)[seq];
-  asm volatile("" ::"s"(q_begin), "s"(num_q), "s"(len_k));       // (all three requested here, with one wait)
+  if constexpr (kLookupsTogether) asm volatile("" ::"s"(q_begin), "s"(num_q), "s"(len_k));       // (all three requested here, with one wait)
   const int num_cols = num_q * G;
   const int col0 = blockIdx.x * 16 * NCB;
   if (col0 >= num_cols) return;
@@ -176,7 +178,10 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     int pages[4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) pages[kt] = bt[min(n0 + kt * 16, last_tile) >> bs_shift];
-    asm volatile("" ::"s"(pages[0]), "s"(pages[1]), "s"(pages[2]), "s"(pages[3]));   // (here, not each where its tile begins)
+    // (here, not each where its tile begins.  Only for the head sizes whose kernels have registers to spare: at 128 the
+    //  form with eight wavefronts takes all 256, and holding it to this order made it spill, 112 -> 125 us for 64 sequences
+    //  of 2048 keys.)
+    if constexpr (kLookupsTogether) asm volatile("" ::"s"(pages[0]), "s"(pages[1]), "s"(pages[2]), "s"(pages[3]));
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
       const int nk = n0 + kt * 16;
@@ -888,6 +893,15 @@ PLLM_API int pllm_attention_decode_registers(int waves) {
                  : waves == 8 ? reinterpret_cast<const void*>(paged_attention_mfma_kernel<1, 8>) : nullptr;
   if (!fn || hipFuncGetAttributes(&attr, fn) != hipSuccess) return -1;
   return attr.numRegs;
+}
+
+// Bytes per lane that the same two forms keep outside registers (spilled registers): 0 as long as they fit.
+PLLM_API int pllm_attention_decode_spill_bytes(int waves) {
+  hipFuncAttributes attr;
+  const void* fn = waves == 4 ? reinterpret_cast<const void*>(paged_attention_mfma_kernel<1, 4>)
+                 : waves == 8 ? reinterpret_cast<const void*>(paged_attention_mfma_kernel<1, 8>) : nullptr;
+  if (!fn || hipFuncGetAttributes(&attr, fn) != hipSuccess) return -1;
+  return (int)attr.localSizeBytes;
 }
 
 static int num_compute_units() {

@@ -431,6 +431,11 @@ def attention_decode_registers(head_dim: int, waves: int) -> int:
     return int(_fn("attention_mfma.hip", "pllm_attention_decode_registers", {"HEAD_DIM": head_dim}, [c_int])(waves))
 
 
+def attention_decode_spill_bytes(head_dim: int, waves: int) -> int:
+    """Bytes per lane that the same kernel keeps outside registers; 0 unless registers were spilled."""
+    return int(_fn("attention_mfma.hip", "pllm_attention_decode_spill_bytes", {"HEAD_DIM": head_dim}, [c_int])(waves))
+
+
 def _merge_lds_bytes(column_blocks: int, waves: int, head_dim: int) -> int:
     """LDS of the attention kernel's several-wavefront variant (as merge_lds_bytes in attention_mfma.hip):
     maximum and weight per column and wavefront, and every wavefront's partial output."""

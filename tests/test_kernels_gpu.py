@@ -555,6 +555,15 @@ def test_decode_attention_kernel_leaves_room_for_two_workgroups():
     assert 0 < ops().attention_decode_registers(64, 4) <= 256
 
 
+@pytest.mark.parametrize("head_dim", [64, 128])
+def test_decode_attention_kernel_spills_no_registers(head_dim):
+    """The forms that decoding uses (16 columns, four or eight wavefronts) must fit their registers: at head size 128
+    the eight-wavefront form takes all 256, and a change that made it spill four of them cost 12 % of its speed
+    at 64 sequences."""
+    for waves in (4, 8):
+        assert ops().attention_decode_spill_bytes(head_dim, waves) == 0, (head_dim, waves)
+
+
 def test_attention_plan():
     plan = ops().attention_plan
     lds = 160 * 1024
