@@ -42,6 +42,10 @@ class ModelRunner:
         self.kv = kv_storage
         self.device = model.device
         self.block_size = kv_storage.block_size
+        if self.device.type == "cuda":
+            # The library kernel that ``run_prepared`` picks rows of sampled ids with: its first use loads its code
+            # (over 100 ms), which belongs here and not into the first step that happens to need it.
+            torch.zeros(2, dtype=torch.int32, device=self.device).index_select(0, torch.tensor([1, 0], device=self.device))
         self.group_specs = {name: g.spec for name, g in kv_storage.groups.items()}
         # Fixed-size per-request state: one tensor [slots + 1, *shape] per schedule step that has any.  The
         # last slot belongs to no request: the empty rows that pad a replayed batch point at it, so that a
