@@ -5,11 +5,13 @@
 // where, as in pagedllm/sampler.py:21-35, a token stays if fewer than top_k tokens have a larger
 // logit and the probability mass of the tokens with a larger logit is at most top_p.  Both tests
 // depend only on the token's own logit, so the kept set is {logit >= threshold}; the threshold is
-// found by bisection over the ordered bit patterns of float (32 passes over the row, which stays
-// in cache), not by a sort.  Tokens with equal logits are kept or dropped together.
+// found by a search over the ordered bit patterns of float that moves from token to token (a few
+// passes over the row, which stays in registers or in cache), not by a sort.  Tokens with equal
+// logits are kept or dropped together.
 //
-// The draw is the inverse CDF in index order with one uniform number per row from Philox4x32-10
-// keyed by (seed, request key, step), so a request's tokens do not depend on its neighbours.
+// The draw is the inverse CDF over the kept tokens in a fixed order (thread by thread) with one uniform
+// number per row from Philox4x32-10 keyed by (seed, request key, step), so a request's tokens do not
+// depend on its neighbours; every sum is taken in an order that depends on the row's length only.
 #include "common.h"
 
 using namespace pllm;
@@ -58,94 +60,292 @@ __device__ ArgMax block_argmax(ArgMax a, ArgMax* scratch) {
   return t;
 }
 
-__global__ __launch_bounds__(kThreads) void sample_kernel(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
-                                                          const int* __restrict__ top_k, const float* __restrict__ top_p,
-                                                          const long long* __restrict__ request_key, const int* __restrict__ step,
-                                                          unsigned long long seed, int* __restrict__ out) {
+// ---------------------------------------------------------------------------------------------
+// The row is walked in passes.  A thread's elements are the same in every pass and come in the same order:
+// with rows of whole 16-byte pieces, piece c * 512 + tid for c = 0, 1, ...; else element c * 512 + tid.
+// The sampling kernel's workgroup has 512 threads (eight wavefronts, so that a thread may hold up to 256 registers): rows of
+// up to 64 elements per thread (32768 logits) are read once and stay in registers; longer rows are read again in each
+// pass (cache hits), eight requests under way at a time.
+constexpr int kSampleThreads = 512;
+constexpr int kSlots = 64;                   // elements per thread that registers hold
+// elements per thread that the end of the search keeps in registers: 16 for a row that is read from memory (each pass
+// before that is long), 8 for a row in registers (which leave no room for more)
+template <bool IN_REGS> constexpr int kWindowSlots = IN_REGS ? 8 : 16;
+
+__device__ __forceinline__ float key_value(uint32_t k) {       // inverse of float_key
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+struct Four { float a, b, c, d; };          // sums / extremes of one pass, reduced over the workgroup together
+__device__ __forceinline__ void block_reduce_pass(float& mass, int& cnt, uint32_t& below, uint32_t& above, int& low_most, int& high_most,
+                                                  float* fs, int* is) {
+  // mass, cnt: sums; below: maximum; above: minimum; low_most / high_most: maxima.  Fixed order: wavefront, then wavefronts.
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mass += __shfl_xor(mass, o, 64);
+    cnt += __shfl_xor(cnt, o, 64);
+    below = max(below, (uint32_t)__shfl_xor((int)below, o, 64));
+    above = min(above, (uint32_t)__shfl_xor((int)above, o, 64));
+    low_most = max(low_most, __shfl_xor(low_most, o, 64));
+    high_most = max(high_most, __shfl_xor(high_most, o, 64));
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) {
+    fs[wave] = mass;
+    is[wave] = cnt; is[16 + wave] = (int)below; is[32 + wave] = (int)above; is[48 + wave] = low_most; is[64 + wave] = high_most;
+  }
+  __syncthreads();
+  mass = fs[0]; cnt = is[0]; below = (uint32_t)is[16]; above = (uint32_t)is[32]; low_most = is[48]; high_most = is[64];
+  for (int w = 1; w < kSampleThreads / 64; ++w) {
+    mass += fs[w]; cnt += is[w];
+    below = max(below, (uint32_t)is[16 + w]); above = min(above, (uint32_t)is[32 + w]);
+    low_most = max(low_most, is[48 + w]); high_most = max(high_most, is[64 + w]);
+  }
+}
+
+// Exclusive prefix of one float per thread in thread order, and the total; fixed order of additions.
+__device__ __forceinline__ float block_exclusive_scan(float v, float* fs, float& total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float incl = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  __syncthreads();
+  if (lane == 63) fs[wave] = incl;
+  __syncthreads();
+  float before = 0.f, all = 0.f;
+  for (int w = 0; w < kSampleThreads / 64; ++w) {
+    if (w < wave) before += fs[w];
+    all += fs[w];
+  }
+  total = all;
+  return before + (incl - v);
+}
+
+// f(value, index) for every element of the calling thread, in its fixed order; the visitor goes in and comes back by
+// value, so that what it gathers stays in registers.
+template <bool IN_REGS, bool VEC, class F>
+__device__ __forceinline__ F for_each_element(const float (&held)[IN_REGS ? kSlots : 1], const float* __restrict__ z, int units, int tid, F f) {
+  constexpr int kPer = VEC ? 4 : 1;
+  constexpr int kFlight = 8;                                     // requests under way per thread in a pass over memory
+  if constexpr (IN_REGS) {
+#pragma unroll
+    for (int s = 0; s < kSlots; ++s) {
+      const int u = (s / kPer) * kSampleThreads + tid, i = u * kPer + (s % kPer);
+      if (u < units) f(held[s], i);
+    }
+  } else {
+    for (int u0 = 0; u0 < units; u0 += kFlight * kSampleThreads) {
+      float v[kFlight][kPer];
+#pragma unroll
+      for (int q = 0; q < kFlight; ++q) {
+        const int u = u0 + q * kSampleThreads + tid;
+        if constexpr (VEC) {
+          const float4 t = u < units ? reinterpret_cast<const float4*>(z)[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+          v[q][0] = t.x; v[q][1] = t.y; v[q][2] = t.z; v[q][3] = t.w;
+        } else {
+          v[q][0] = u < units ? z[u] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kFlight; ++q) {
+        const int u = u0 + q * kSampleThreads + tid;
+        if (u >= units) continue;
+#pragma unroll
+        for (int e = 0; e < kPer; ++e) f(v[q][e], u * kPer + e);
+      }
+    }
+  }
+  return f;
+}
+
+// weight of a token (unnormalised probability): 2^((v - max) / T * log2 e), at most 1
+struct Weigh {
+  float zmax, rate;
+  __device__ __forceinline__ float operator()(float v) const { return __builtin_amdgcn_exp2f((v - zmax) * rate); }
+};
+struct Extremes {                      // the maximum (first index) and the minimum
+  ArgMax best; float lowest;
+  __device__ __forceinline__ void operator()(float v, int i) { ArgMax c; c.v = v; c.i = i; best = better(best, c); lowest = fminf(lowest, v); }
+};
+struct SumOfWeights {
+  Weigh w; float sum;
+  __device__ __forceinline__ void operator()(float v, int) { sum += w(v); }
+};
+struct AroundPivot {                   // what lies above the pivot, and the nearest tokens on both sides inside [lo, hi]
+  Weigh w; uint32_t lo, hi, mid;
+  float mass; int cnt, low_mine, high_mine; uint32_t below, above;
+  __device__ __forceinline__ void look(uint32_t key, float weight) {
+    const bool up = key > mid, in_hi = up && key <= hi, in_lo = !up && key >= lo;
+    cnt += up ? 1 : 0;
+    mass += up ? weight : 0.f;
+    above = in_hi ? min(above, key) : above;
+    below = in_lo ? max(below, key) : below;
+    high_mine += in_hi ? 1 : 0;
+    low_mine += in_lo ? 1 : 0;
+  }
+  __device__ __forceinline__ void operator()(float v, int) {
+    const uint32_t key = float_key(v);
+    // (the weight only where it counts: late passes have their pivot far up, and whole wavefronts skip the exponential)
+    float weight = 0.f;
+    if (key > mid) weight = w(v);
+    look(key, weight);
+  }
+};
+template <int SLOTS>
+struct IntoWindow {                    // this thread's tokens inside [lo, hi] into registers, what lies above summed
+  Weigh w; uint32_t lo, hi;
+  uint32_t key[SLOTS]; float weight[SLOTS];
+  int n, cnt_up; float mass_up;
+  __device__ __forceinline__ void operator()(float v, int) {
+    const uint32_t k = float_key(v);
+    float wt = 0.f;
+    if (k >= lo) wt = w(v);
+    const bool up = k > hi, in = !up && k >= lo;
+    cnt_up += up ? 1 : 0;
+    mass_up += up ? wt : 0.f;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+      const bool here = in && n == s;
+      key[s] = here ? k : key[s];
+      weight[s] = here ? wt : weight[s];
+    }
+    n += in ? 1 : 0;
+  }
+};
+struct KeptSum {
+  Weigh w; uint32_t threshold; float sum;
+  __device__ __forceinline__ void operator()(float v, int) { if (float_key(v) >= threshold) sum += w(v); }
+};
+struct Pick {                          // the first kept token at which the running sum passes the target
+  Weigh w; uint32_t threshold; float run, target; int pick, last;
+  __device__ __forceinline__ void operator()(float v, int i) {
+    if (pick < 0 && float_key(v) >= threshold) {
+      run += w(v);
+      last = i;
+      if (run > target) pick = i;
+    }
+  }
+};
+
+template <bool IN_REGS, bool VEC>
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
+                                                                const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                                const long long* __restrict__ request_key, const int* __restrict__ step,
+                                                                unsigned long long seed, int* __restrict__ out) {
   __shared__ float fscratch[16];
+  __shared__ int iscratch[80];
   __shared__ ArgMax ascratch[16];
-  __shared__ float chunk_sum[kThreads];
   __shared__ int chosen;
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* z = logits + (size_t)row * vocab;
+  const int units = VEC ? vocab >> 2 : vocab;                    // pieces of four, or single elements
+  constexpr int kPer = VEC ? 4 : 1;
 
-  ArgMax best; best.v = -INFINITY; best.i = 0x7fffffff;
-  for (int i = tid; i < vocab; i += kThreads) { ArgMax c; c.v = z[i]; c.i = i; best = better(best, c); }
-  best = block_argmax(best, ascratch);
+  float held[IN_REGS ? kSlots : 1];
+  if constexpr (IN_REGS) {
+#pragma unroll
+    for (int s = 0; s < kSlots; s += kPer) {
+      const int u = (s / kPer) * kSampleThreads + tid;
+      if constexpr (VEC) {
+        const float4 t = u < units ? reinterpret_cast<const float4*>(z)[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+        held[s] = t.x; held[s + 1] = t.y; held[s + 2] = t.z; held[s + 3] = t.w;
+      } else {
+        held[s] = u < units ? z[u] : 0.f;
+      }
+    }
+  }
+#define PLLM_WALK(visitor) for_each_element<IN_REGS, VEC>(held, z, units, tid, visitor)
+
+  Extremes ex; ex.best.v = -INFINITY; ex.best.i = 0x7fffffff; ex.lowest = INFINITY;
+  ex = PLLM_WALK(ex);
+  const ArgMax best = block_argmax(ex.best, ascratch);
   const float temp = temperature[row];
   if (temp < 1e-5f) {
     if (tid == 0) out[row] = best.i;
     return;
   }
-  const float inv_t = 1.f / fmaxf(temp, 1e-5f);
-  const float zmax = best.v;
-  // weight of token i (unnormalised probability)
-  auto weight = [&](float v) { return expf((v - zmax) * inv_t); };
+  Weigh weigh; weigh.zmax = best.v; weigh.rate = 1.4426950408889634f / fmaxf(temp, 1e-5f);
 
-  float part = 0.f;
-  for (int i = tid; i < vocab; i += kThreads) part += weight(z[i]);
-  const float total = block_sum(part, fscratch);
+  SumOfWeights sw; sw.w = weigh; sw.sum = 0.f;
+  sw = PLLM_WALK(sw);
+  const float total = block_sum(sw.sum, fscratch);
 
   int k = top_k[row];
   if (k <= 0 || k > vocab) k = vocab;
   const float p = top_p[row];
-  uint32_t threshold = 0;  // keep tokens whose key >= threshold; 0 keeps all
+  uint32_t threshold = 0;                                        // tokens whose key >= threshold stay; 0 keeps all
   if (k < vocab || p < 1.f) {
-    // Largest key value `c` whose tokens fail neither test is monotone: find the smallest kept key.
-    // kept(v)  <=>  count(key > v) < k  and  mass(key > v) <= p * total.   Bisection on v.
-    uint32_t lo_key = 0, hi_key = float_key(zmax);  // hi_key is always kept (nothing is larger)
-    while (lo_key < hi_key) {
-      const uint32_t mid = lo_key + ((hi_key - lo_key) >> 1);
-      float cnt = 0.f, mass = 0.f;
-      for (int i = tid; i < vocab; i += kThreads) {
-        const float v = z[i];
-        if (float_key(v) > mid) { cnt += 1.f; mass += weight(v); }
+    // kept(c)  <=>  count(key > c) < k  and  mass(key > c) <= p * total  is monotone in c; the threshold is the
+    // smallest key of a token that stays.  [lo, hi]: kept(hi) holds, kept(lo - 1) does not, and both ends are keys of
+    // tokens of the row (at the start its minimum, which cannot stay, and its maximum, which always does).  A pass takes
+    // a pivot between them (the middle of the two values; of the two keys where that gives nothing new), counts and
+    // weighs what lies above it, and moves one end to the nearest token's key on the pivot's side: the interval loses
+    // the pivot's side and all the empty room next to it, so about a dozen passes are left where 32 halvings of all
+    // keys were.  Once every thread has at most kWindowSlots of its tokens inside the interval it keeps those in
+    // registers and the row is not read again.
+    const float lowest = -block_max(-ex.lowest, fscratch);
+    uint32_t lo = float_key(lowest), hi = float_key(best.v);
+    constexpr int kSlotsHere = kWindowSlots<IN_REGS>;
+    IntoWindow<kSlotsHere> win; win.n = 0;
+    bool windowed = false;
+    float mass_above = 0.f;                                      // of the tokens above the interval, once windowed
+    int cnt_above = 0;
+    while (lo < hi) {
+      const float vmid = 0.5f * key_value(lo) + 0.5f * key_value(hi);
+      uint32_t mid = float_key(vmid);
+      if (!(mid >= lo && mid < hi)) mid = lo + ((hi - lo) >> 1);
+      AroundPivot ap; ap.w = weigh; ap.lo = lo; ap.hi = hi; ap.mid = mid;
+      ap.mass = 0.f; ap.cnt = 0; ap.low_mine = 0; ap.high_mine = 0; ap.below = lo; ap.above = hi;
+      if (windowed) {
+#pragma unroll
+        for (int s = 0; s < kSlotsHere; ++s) ap.look(win.key[s], win.weight[s]);     // (unused slots hold key 0: below every interval)
+        ap.cnt += cnt_above; ap.mass += mass_above;
+      } else {
+        ap = PLLM_WALK(ap);
       }
-      cnt = block_sum(cnt, fscratch);
-      mass = block_sum(mass, fscratch);
-      const bool kept = cnt < (float)k && mass <= p * total;
-      if (kept) hi_key = mid; else lo_key = mid + 1;
+      int low_most = ap.low_mine, high_most = ap.high_mine;
+      block_reduce_pass(ap.mass, ap.cnt, ap.below, ap.above, low_most, high_most, fscratch, iscratch);
+      const bool kept = ap.cnt < k && ap.mass <= p * total;
+      if (kept) hi = ap.below; else lo = ap.above;
+      if (!windowed && lo < hi && (kept ? low_most : high_most) <= kSlotsHere) {
+        win.w = weigh; win.lo = lo; win.hi = hi; win.n = 0; win.cnt_up = 0; win.mass_up = 0.f;
+#pragma unroll
+        for (int s = 0; s < kSlotsHere; ++s) { win.key[s] = 0u; win.weight[s] = 0.f; }
+        win = PLLM_WALK(win);
+        mass_above = block_sum(win.mass_up, fscratch);
+        cnt_above = (int)block_sum((float)win.cnt_up, fscratch);       // (exact: below 2^24)
+        windowed = true;
+      }
     }
-    threshold = hi_key;
+    threshold = hi;
   }
 
-  // Inverse CDF in index order over contiguous chunks, one chunk per thread.
-  const int chunk = (vocab + kThreads - 1) / kThreads;
-  const int begin = tid * chunk, end = min(begin + chunk, vocab);
-  float mine = 0.f;
-  for (int i = begin; i < end; ++i) { const float v = z[i]; if (float_key(v) >= threshold) mine += weight(v); }
-  chunk_sum[tid] = mine;
+  // ---- the draw: inverse CDF over the tokens that stay, in the order thread by thread, each thread's tokens in its own order
+  KeptSum ks; ks.w = weigh; ks.threshold = threshold; ks.sum = 0.f;
+  ks = PLLM_WALK(ks);
+  float kept_total;
+  const float before = block_exclusive_scan(ks.sum, fscratch, kept_total);
   if (tid == 0) chosen = -1;
   __syncthreads();
-  if (tid == 0) {
-    const long long key = request_key[row];
-    const uint32_t bits = philox_first_word((uint32_t)step[row], 0u, (uint32_t)key, (uint32_t)(key >> 32),
-                                            (uint32_t)seed, (uint32_t)(seed >> 32));
-    const float u = (float)(bits >> 8) * (1.0f / 16777216.0f);  // [0, 1)
-    float kept_total = 0.f;
-    for (int t = 0; t < kThreads; ++t) kept_total += chunk_sum[t];
-    const float target = u * kept_total;
-    // Find the chunk, then the token inside it.
-    float run = 0.f;
-    int t = 0;
-    for (; t < kThreads - 1; ++t) {
-      if (run + chunk_sum[t] > target) break;
-      run += chunk_sum[t];
-    }
-    int pick = -1, last_kept = -1;
-    const int b = t * chunk, e = min(b + chunk, vocab);
-    for (int i = b; i < e; ++i) {
-      const float v = z[i];
-      if (float_key(v) < threshold) continue;
-      last_kept = i;
-      run += weight(v);
-      if (run > target) { pick = i; break; }
-    }
-    if (pick < 0) pick = last_kept >= 0 ? last_kept : best.i;  // rounding at the very end of the range
-    chosen = pick;
+  const long long rkey = request_key[row];
+  const uint32_t bits = philox_first_word((uint32_t)step[row], 0u, (uint32_t)rkey, (uint32_t)(rkey >> 32),
+                                          (uint32_t)seed, (uint32_t)(seed >> 32));
+  const float u01 = (float)(bits >> 8) * (1.0f / 16777216.0f);   // [0, 1)
+  const float target = u01 * kept_total;
+  // the thread whose share of the line holds the target takes the token there (one thread at most: shares do not overlap)
+  if (ks.sum > 0.f && before <= target && target < before + ks.sum) {
+    Pick pk; pk.w = weigh; pk.threshold = threshold; pk.run = before; pk.target = target; pk.pick = -1; pk.last = -1;
+    pk = PLLM_WALK(pk);
+    chosen = pk.pick >= 0 ? pk.pick : pk.last;
   }
   __syncthreads();
-  if (tid == 0) out[row] = chosen;
+  // (rounding at the very end of the line, or a row without a finite weight: the maximum)
+  if (tid == 0) out[row] = chosen >= 0 ? chosen : best.i;
+#undef PLLM_WALK
 }
 
 PLLM_API int pllm_sample(const float* logits, int rows, int vocab, const float* temperature, const int* top_k,
@@ -153,8 +353,16 @@ PLLM_API int pllm_sample(const float* logits, int rows, int vocab, const float* 
                          int* out, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) return -2;
-  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kThreads), 0, stream, logits, vocab, temperature, top_k, top_p,
-                     request_key, step, seed, out);
+  const bool vec = (vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0;
+  const bool in_regs = vocab <= kSlots * kSampleThreads;
+#define PLLM_SAMPLE(IN_REGS_, VEC_)                                                                                          \
+  hipLaunchKernelGGL((sample_kernel<IN_REGS_, VEC_>), dim3(rows), dim3(kSampleThreads), 0, stream, logits, vocab, temperature, top_k, \
+                     top_p, request_key, step, seed, out)
+  if (in_regs && vec) PLLM_SAMPLE(true, true);
+  else if (in_regs) PLLM_SAMPLE(true, false);
+  else if (vec) PLLM_SAMPLE(false, true);
+  else PLLM_SAMPLE(false, false);
+#undef PLLM_SAMPLE
   PLLM_RETURN_LAST_ERROR();
 }
 

@@ -7,6 +7,7 @@ a generator shared by the batch, so a request draws the same tokens whatever run
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..csrc import ops
@@ -36,6 +37,7 @@ class Sampler:
         self.device = torch.device(device)
         self._pinned = None
         self._copied = None
+        self._rows_pinned = self._rows_device = self._rows_copied = None
 
     def _to_host(self, tokens: torch.Tensor) -> PendingTokens:
         n = tokens.numel()
@@ -56,13 +58,32 @@ class Sampler:
             return PendingTokens(None, 0, None)
         if all(p.temperature < 1e-5 for p in params):
             return self._to_host(ops.argmax(logits))
-        dev = logits.device
-        temperature = torch.tensor([float(p.temperature) for p in params], dtype=torch.float32, device=dev)
-        top_k = torch.tensor([int(p.top_k) for p in params], dtype=torch.int32, device=dev)
-        top_p = torch.tensor([float(p.top_p) for p in params], dtype=torch.float32, device=dev)
-        keys = torch.tensor([int(k) for k in request_keys], dtype=torch.int64, device=dev)
-        step = torch.tensor([int(s) for s in steps], dtype=torch.int32, device=dev)
+        temperature, top_k, top_p, keys, step = self._rows_to_device(params, request_keys, steps, logits.device)
         return self._to_host(ops.sample(logits, temperature, top_k, top_p, keys, step, self.seed))
+
+    def _rows_to_device(self, params: list, request_keys: list, steps: list, device):
+        """The rows' settings as device tensors.  They travel as one piece of pinned memory with one queued copy: five
+        small tensors made from lists would be five copies from pageable memory, each of which the host waits for
+        behind whatever the stream still has to do."""
+        n = len(params)
+        if self._rows_pinned is None or self._rows_pinned.numel() < 6 * n:
+            cap = max(6 * n, 6 * 64)
+            self._rows_pinned = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self._rows_device = torch.empty(cap, dtype=torch.int32, device=device)
+            self._rows_copied = torch.cuda.Event()
+        else:
+            self._rows_copied.synchronize()                    # the copy before has read the pinned piece (long ago)
+        host = self._rows_pinned.numpy()
+        host[:2 * n].view(np.int64)[:] = request_keys          # (first: 8-byte aligned)
+        host[2 * n:3 * n].view(np.float32)[:] = [p.temperature for p in params]
+        host[3 * n:4 * n].view(np.float32)[:] = [p.top_p for p in params]
+        host[4 * n:5 * n] = [p.top_k for p in params]
+        host[5 * n:6 * n] = steps
+        dev = self._rows_device
+        dev[:6 * n].copy_(self._rows_pinned[:6 * n], non_blocking=True)
+        self._rows_copied.record()
+        return (dev[2 * n:3 * n].view(torch.float32), dev[4 * n:5 * n], dev[3 * n:4 * n].view(torch.float32),
+                dev[:2 * n].view(torch.int64), dev[5 * n:6 * n])
 
     def sample(self, logits: torch.Tensor, params: list, request_keys: list, steps: list) -> list:
         """The n token ids, waited for."""

@@ -297,10 +297,19 @@ def test_sampling_same_seed_same_tokens_other_seed_other_tokens():
     assert torch.equal(a, b) and not torch.equal(a, c)
 
 
+@pytest.mark.parametrize("vocab", [24, 40000, 33001])
 @pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, -1, 1.0), (0.7, -1, 1.0), (1.3, 5, 1.0), (1.0, -1, 0.6), (0.9, 8, 0.8)])
-def test_sampling_frequencies_follow_the_filtered_distribution(temperature, top_k, top_p):
-    vocab, draws = 24, 4000
-    z = rnd(1, vocab, seed=17, scale=1.5)
+def test_sampling_frequencies_follow_the_filtered_distribution(temperature, top_k, top_p, vocab):
+    """24 tokens that matter.  In the long rows (which the kernel reads again in every pass instead of holding them in
+    registers: one a multiple of four, read in pieces of 16 bytes, one not) they are spread over the row among tokens
+    whose logits lie 40 to 50 below and share a few values, so that the search for the threshold starts far away."""
+    draws = 4000
+    few = rnd(1, 24, seed=17, scale=1.5)
+    if vocab == 24:
+        z = few
+    else:
+        z = -45.0 + 5.0 * torch.round(rnd(1, vocab, seed=18) * 2).clamp(-2, 2) / 2
+        z[0, (torch.arange(24) * 1663 + 11) % vocab] = few[0]
     probs = plain.filtered_probabilities(z[0], temperature, top_k, top_p).numpy()
     got = sample_rows(z, temperature, top_k, top_p, draws)[:, 0].numpy()
     counts = np.bincount(got, minlength=vocab)
@@ -309,6 +318,51 @@ def test_sampling_frequencies_follow_the_filtered_distribution(temperature, top_
     chi2 = float(((counts[keep] - draws * probs[keep]) ** 2 / (draws * probs[keep])).sum())
     dof = int(keep.sum()) - 1
     assert chi2 < dof + 5 * math.sqrt(2 * max(dof, 1)) + 5, f"chi-square {chi2:.1f} for {dof} degrees of freedom"
+
+
+@pytest.mark.parametrize("vocab", [1000, 32000, 50001, 128256])
+@pytest.mark.parametrize("top_k,top_p", [(50, 1.0), (-1, 0.9), (40, 0.95), (-1, 0.999), (3, 0.2)])
+def test_sampling_draws_only_and_all_of_the_kept_tokens(vocab, top_k, top_p):
+    """Rows of real sizes: every drawn token belongs to the kept set of the plain implementation, and where that set is
+    small all of it is drawn in the end."""
+    z = rnd(3, vocab, seed=19, scale=3.0)
+    z[1] = z[1] * 0.05                                                  # a flat row: the kept set of top-p is most of it
+    draws = 300
+    got = sample_rows(z, 0.8, top_k, top_p, draws)
+    for row in range(3):
+        probs = plain.filtered_probabilities(z[row], 0.8, top_k, top_p)
+        assert bool((probs[got[:, row].long()] > 0).all()), f"row {row}: a filtered token was drawn"
+        kept = int((probs > 0).sum())
+        if kept <= 6:
+            assert set(got[:, row].tolist()) == set(torch.nonzero(probs > 0).flatten().tolist()), f"row {row}"
+
+
+@pytest.mark.parametrize("vocab", [97, 40000])
+def test_sampling_keeps_or_drops_equal_logits_together(vocab):
+    """A token stays if fewer than top_k tokens have a larger logit: with the second and third largest equal and
+    top_k = 2 both stay (one token is larger than each), and the fourth goes."""
+    z = torch.full((1, vocab), -20.0)
+    z[0, 5], z[0, vocab // 2], z[0, vocab - 3], z[0, 70] = 3.0, 2.5, 2.5, 2.0
+    got = set(sample_rows(z, 1.0, 2, 1.0, 200)[:, 0].tolist())
+    assert got == {5, vocab // 2, vocab - 3}
+
+
+def test_sampling_rows_do_not_depend_on_their_neighbours():
+    z = rnd(5, 50001, seed=23, scale=2.0)
+    alone = torch.stack([sample_rows(z[r:r + 1], 0.9, 30, 0.9, 4)[:, 0] for r in range(5)], dim=1)
+    keys = torch.arange(5, dtype=torch.int64)
+    # the same rows in one launch, in another order, with the same request keys
+    order = [3, 0, 4, 1, 2]
+    zg = z[order].cuda()
+    t, k, pp = torch.full((5,), 0.9).cuda(), torch.full((5,), 30, dtype=torch.int32).cuda(), torch.full((5,), 0.9).cuda()
+    for step in range(4):
+        s_ = torch.full((5,), step, dtype=torch.int32).cuda()
+        got = ops().sample(zg, t, k, pp, keys[order].cuda(), s_, 0).cpu()
+        for j, r in enumerate(order):
+            # alone, row r was drawn with request key 0: draw it again in the batch with key r and alone with key r
+            one = ops().sample(z[r:r + 1].cuda(), t[:1], k[:1], pp[:1], keys[r:r + 1].cuda(), s_[:1], 0).cpu()
+            assert int(got[j]) == int(one[0]), (step, r)
+    assert alone.shape == (4, 5)
 
 
 # ----------------------------------------------------------------------------------- bfloat16 products for many rows
