@@ -325,8 +325,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   }
 
   // ---- the draw: inverse CDF over the tokens that stay, in the order thread by thread, each thread's tokens in its own order
-  KeptSum ks; ks.w = weigh; ks.threshold = threshold; ks.sum = 0.f;
-  ks = PLLM_WALK(ks);
+  KeptSum ks; ks.w = weigh; ks.threshold = threshold; ks.sum = sw.sum;
+  if (threshold != 0u) {                                         // (without a threshold every token stays: the sums above)
+    ks.sum = 0.f;
+    ks = PLLM_WALK(ks);
+  }
   float kept_total;
   const float before = block_exclusive_scan(ks.sum, fscratch, kept_total);
   if (tid == 0) chosen = -1;
