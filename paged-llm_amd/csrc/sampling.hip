@@ -189,10 +189,15 @@ struct AroundPivot {                   // what lies above the pivot, and the nea
   }
   __device__ __forceinline__ void operator()(float v, int) {
     const uint32_t key = float_key(v);
-    // (the weight only where it counts: late passes have their pivot far up, and whole wavefronts skip the exponential)
-    float weight = 0.f;
-    if (key > mid) weight = w(v);
-    look(key, weight);
+    // (under branches: late passes have their pivot far up and a narrow interval, and whole wavefronts pass these by)
+    if (key > mid) {
+      cnt += 1;
+      mass += w(v);
+    }
+    if (key - lo <= hi - lo) {                                   // inside [lo, hi]
+      if (key > mid) { above = min(above, key); high_mine += 1; }
+      else { below = max(below, key); low_mine += 1; }
+    }
   }
 };
 template <int SLOTS>
@@ -207,13 +212,15 @@ struct IntoWindow {                    // this thread's tokens inside [lo, hi] i
     const bool up = k > hi, in = !up && k >= lo;
     cnt_up += up ? 1 : 0;
     mass_up += up ? wt : 0.f;
+    if (in) {                                                    // (few tokens are: most wavefronts pass this by)
 #pragma unroll
-    for (int s = 0; s < SLOTS; ++s) {
-      const bool here = in && n == s;
-      key[s] = here ? k : key[s];
-      weight[s] = here ? wt : weight[s];
+      for (int s = 0; s < SLOTS; ++s) {
+        const bool here = n == s;
+        key[s] = here ? k : key[s];
+        weight[s] = here ? wt : weight[s];
+      }
+      n += 1;
     }
-    n += in ? 1 : 0;
   }
 };
 struct KeptSum {
@@ -278,6 +285,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   if (k <= 0 || k > vocab) k = vocab;
   const float p = top_p[row];
   uint32_t threshold = 0;                                        // tokens whose key >= threshold stay; 0 keeps all
+  constexpr int kSlotsHere = kWindowSlots<IN_REGS>;
+  IntoWindow<kSlotsHere> win; win.n = 0; win.mass_up = 0.f;
+  bool windowed = false;
   if (k < vocab || p < 1.f) {
     // kept(c)  <=>  count(key > c) < k  and  mass(key > c) <= p * total  is monotone in c; the threshold is the
     // smallest key of a token that stays.  [lo, hi]: kept(hi) holds, kept(lo - 1) does not, and both ends are keys of
@@ -289,13 +299,14 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
     // registers and the row is not read again.
     const float lowest = -block_max(-ex.lowest, fscratch);
     uint32_t lo = float_key(lowest), hi = float_key(best.v);
-    constexpr int kSlotsHere = kWindowSlots<IN_REGS>;
-    IntoWindow<kSlotsHere> win; win.n = 0;
-    bool windowed = false;
     float mass_above = 0.f;                                      // of the tokens above the interval, once windowed
     int cnt_above = 0;
+    // The first pivot: the logit whose weight is 2^-13 of the largest.  Where a few tokens carry the mass (the usual
+    // row) nearly all of it lies above that pivot, so the first pass already leaves an interval with few tokens in it.
+    bool first = true;
     while (lo < hi) {
-      const float vmid = 0.5f * key_value(lo) + 0.5f * key_value(hi);
+      const float vmid = first ? best.v - 13.f / weigh.rate : 0.5f * key_value(lo) + 0.5f * key_value(hi);
+      first = false;
       uint32_t mid = float_key(vmid);
       if (!(mid >= lo && mid < hi)) mid = lo + ((hi - lo) >> 1);
       AroundPivot ap; ap.w = weigh; ap.lo = lo; ap.hi = hi; ap.mid = mid;
@@ -326,7 +337,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
 
   // ---- the draw: inverse CDF over the tokens that stay, in the order thread by thread, each thread's tokens in its own order
   KeptSum ks; ks.w = weigh; ks.threshold = threshold; ks.sum = sw.sum;
-  if (threshold != 0u) {                                         // (without a threshold every token stays: the sums above)
+  if (windowed) {
+    // (what this thread had above the interval when it took its tokens inside it into registers, and those of them that stay)
+    ks.sum = win.mass_up;
+#pragma unroll
+    for (int s = 0; s < kSlotsHere; ++s) ks.sum += win.key[s] >= threshold ? win.weight[s] : 0.f;
+  } else if (threshold != 0u) {                                  // (without a threshold every token stays: the sums above)
     ks.sum = 0.f;
     ks = PLLM_WALK(ks);
   }
