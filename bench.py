@@ -81,9 +81,9 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
     return [torch.randint(100, vocab, (length,), generator=g).tolist() for _ in range(n)]
 
 
-def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int):
+def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed: int, sampling: dict | None = None):
     """(seconds per decode step, mean context length over the timed steps) at `batch` requests whose
-    contexts end at (or just under) `context` tokens."""
+    contexts end at (or just under) `context` tokens.  ``sampling``: other settings than greedy."""
     import torch
     from paged_llm_amd import SamplingParams
     # Requests whose prompt is done go on decoding while the others' prompts are still computed, so some
@@ -92,7 +92,7 @@ def time_decode(engine, batch: int, context: int, steps: int, warmup: int, seed:
     ahead = batch * context // budget + 1
     prompt_len = context - (steps + warmup) - ahead
     assert prompt_len >= 1, "context too short for this many steps"
-    sp = SamplingParams(temperature=0.0, max_tokens=steps + warmup + ahead + 40, ignore_eos=True)
+    sp = SamplingParams(max_tokens=steps + warmup + ahead + 40, ignore_eos=True, **(sampling or {"temperature": 0.0}))
     for p in random_prompts(batch, prompt_len, engine.model.spec.vocab_size, seed):
         engine.add_request(p, sp)
     while any(not r.decoding for r in engine.scheduler.active) or engine.scheduler.queue:
@@ -613,6 +613,10 @@ def main() -> int:
             for b in (1, 64):
                 s, _ = time_decode(engine, b, args.context, max(16, args.steps // 2), max(4, args.warmup // 2), seed=10 + b)
                 points[f"decode_b{b}"] = round(b / s, 1)
+            # the headline batch with temperature, top-k and top-p instead of greedy choice (the sampling kernel's share)
+            s, _ = time_decode(engine, args.batch, args.context, max(16, args.steps // 2), max(4, args.warmup // 2), seed=30,
+                               sampling={"temperature": 0.8, "top_k": 50, "top_p": 0.9})
+            points[f"decode_b{args.batch}_sampled"] = round(args.batch / s, 1)
             # a step of continuous batching: the batch's decoded tokens beside a prompt portion of 256 tokens
             mixed = time_mixed_step(engine, args.batch, args.context, 256, seed=50)
             points[f"mixed_b{args.batch}_p256"] = mixed["tokens_per_s"]
