@@ -377,3 +377,36 @@ def test_page_pool_sized_from_free_memory(folder_a):
     assert out.token_ids == plain_greedy(folder_a, out.prompt_token_ids, 5)
     with pytest.raises(RuntimeError, match="not enough GPU memory"):
         engine_for(folder_a, num_gpu_blocks=None, gpu_memory_utilization=1e-6)
+
+
+@pytest.mark.parametrize("requests,hidden,inter,heads,kv_heads,head_dim", [(33, 136, 176, 2, 2, 128), (48, 2048, 64, 8, 2, 32), (64, 256, 704, 4, 1, 16)])
+def test_many_live_requests_in_bfloat16(tmp_path, requests, hidden, inter, heads, kv_heads, head_dim):
+    """Decode steps of 17 to 64 rows take other kernels than small batches do (tiles of 16 rows side by side, small
+    matrices in two lines of workgroups, the library for the large ones): the logits in front of every sampled token, for
+    every request, against the plain implementation of the request alone."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2, "hidden_size": hidden,
+           "num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": head_dim, "intermediate_size": inter,
+           "vocab_size": 1001, "rope_theta": 10000.0, "rope_scaling": None, "tie_word_embeddings": False, "rms_norm_eps": 1e-5,
+           "max_position_embeddings": 256}
+    folder = helpers.make_folder(tmp_path, cfg, seed=requests, stored="bfloat16")
+    rng = np.random.default_rng(requests)
+    prompts = [helpers.random_tokens(int(rng.integers(3, 40)), 1001, seed=100 + i) for i in range(requests)]
+    engine = LLMEngine(folder, EngineConfig(dtype="bfloat16", max_num_seqs=64, num_gpu_blocks=64 * 8, block_size=16, max_model_len=128))
+    seen, rows_of_steps = {}, []
+
+    def keep(live, logits):
+        rows_of_steps.append(len(live))
+        for request, row in zip(live, logits.float().cpu().numpy()):
+            seen[request.id, len(request.tokens)] = row.copy()
+
+    engine.on_logits = keep
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    assert max(rows_of_steps) == requests and sum(1 for n in rows_of_steps if n >= 17) >= 6      # such steps did occur
+    for out, prompt in zip(outs, prompts):
+        whole = prompt + out.token_ids
+        want = helpers.plain_logits(folder, whole)
+        for n in range(len(prompt), len(whole)):
+            err = helpers.worst(seen[out.seq_id, n], want[n - 1])
+            assert err <= 4e-2, f"request {out.seq_id}, {n} tokens: {err:.3g}"
