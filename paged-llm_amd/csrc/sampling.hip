@@ -201,6 +201,30 @@ struct AroundPivot {                   // what lies above the pivot, and the nea
   }
 };
 template <int SLOTS>
+struct FirstLook {                     // the first pass: as AroundPivot, and the tokens above the pivot taken along
+  AroundPivot ap;
+  uint32_t key[SLOTS]; float weight[SLOTS]; int n;
+  __device__ __forceinline__ void operator()(float v, int) {
+    const uint32_t k = float_key(v);
+    if (k > ap.mid) {                                            // (few, in the usual row)
+      const float wt = ap.w(v);
+      ap.cnt += 1;
+      ap.mass += wt;
+#pragma unroll
+      for (int s = 0; s < SLOTS; ++s) {
+        const bool here = n == s;
+        key[s] = here ? k : key[s];
+        weight[s] = here ? wt : weight[s];
+      }
+      n += 1;
+    }
+    if (k - ap.lo <= ap.hi - ap.lo) {
+      if (k > ap.mid) { ap.above = min(ap.above, k); ap.high_mine += 1; }
+      else { ap.below = max(ap.below, k); ap.low_mine += 1; }
+    }
+  }
+};
+template <int SLOTS>
 struct IntoWindow {                    // this thread's tokens inside [lo, hi] into registers, what lies above summed
   Weigh w; uint32_t lo, hi;
   uint32_t key[SLOTS]; float weight[SLOTS];
@@ -303,10 +327,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
     int cnt_above = 0;
     // The first pivot: the logit whose weight is 2^-13 of the largest.  Where a few tokens carry the mass (the usual
     // row) nearly all of it lies above that pivot, so the first pass already leaves an interval with few tokens in it.
+    // That pass also takes the tokens above its pivot along, as many as the registers for the interval's tokens hold:
+    // if the threshold does lie above the pivot they are the interval's tokens, and the pass that would fetch them is saved.
     bool first = true;
     while (lo < hi) {
       const float vmid = first ? best.v - 13.f / weigh.rate : 0.5f * key_value(lo) + 0.5f * key_value(hi);
-      first = false;
       uint32_t mid = float_key(vmid);
       if (!(mid >= lo && mid < hi)) mid = lo + ((hi - lo) >> 1);
       AroundPivot ap; ap.w = weigh; ap.lo = lo; ap.hi = hi; ap.mid = mid;
@@ -315,6 +340,14 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
 #pragma unroll
         for (int s = 0; s < kSlotsHere; ++s) ap.look(win.key[s], win.weight[s]);     // (unused slots hold key 0: below every interval)
         ap.cnt += cnt_above; ap.mass += mass_above;
+      } else if (first) {
+        FirstLook<kSlotsHere> fl; fl.ap = ap; fl.n = 0;
+#pragma unroll
+        for (int s = 0; s < kSlotsHere; ++s) { fl.key[s] = 0u; fl.weight[s] = 0.f; }
+        fl = PLLM_WALK(fl);
+        ap = fl.ap;
+#pragma unroll
+        for (int s = 0; s < kSlotsHere; ++s) { win.key[s] = fl.key[s]; win.weight[s] = fl.weight[s]; }
       } else {
         ap = PLLM_WALK(ap);
       }
@@ -322,6 +355,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
       block_reduce_pass(ap.mass, ap.cnt, ap.below, ap.above, low_most, high_most, fscratch, iscratch);
       const bool kept = ap.cnt < k && ap.mass <= p * total;
       if (kept) hi = ap.below; else lo = ap.above;
+      if (first && !kept && high_most <= kSlotsHere) {
+        // (the interval is what lay above the first pivot: its tokens are in the registers already, nothing lies above it)
+        win.mass_up = 0.f;
+        windowed = true;
+      }
+      first = false;
       if (!windowed && lo < hi && (kept ? low_most : high_most) <= kSlotsHere) {
         win.w = weigh; win.lo = lo; win.hi = hi; win.n = 0; win.cnt_up = 0; win.mass_up = 0.f;
 #pragma unroll
