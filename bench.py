@@ -487,6 +487,20 @@ def run_kernel_cases(cfg: dict, batch: int, context: int, prefill_tokens: int) -
                 lambda i: linear(pend(last), w_head[i % len(w_head)], out_dtype=torch.float32), len(w_head), w_head[0].numel() * 2,
                 2.0 * last.shape[0] * w_head[0].numel()),
         }
+        if label == "decode":
+            # the choice of the next token from the float logits: greedy, and with temperature, top-k and top-p (on rows in
+            # which a few tokens carry the mass, as a model's logits do, and on rows of plain noise)
+            peaked = [torch.randn(S, V, device=dev, generator=g) * 2 for _ in range(4)]
+            for z in peaked:
+                z[:, 100:140] += torch.linspace(6, 16, 40, device=dev)
+            noise = [torch.randn(S, V, device=dev, generator=g) * 3 for _ in range(4)]
+            t_, k_, p_ = torch.full((S,), 0.8, device=dev), torch.full((S,), 50, device=dev, dtype=torch.int32), torch.full((S,), 0.9, device=dev)
+            keys, step0 = torch.arange(S, device=dev, dtype=torch.int64), torch.zeros(S, device=dev, dtype=torch.int32)
+            cases["greedy choice (argmax)"] = (lambda i: ops.argmax(peaked[i % 4]), 4, S * V * 4, 0.0)
+            cases["sampling, temperature 0.8 / top-k 50 / top-p 0.9, peaked rows"] = (
+                lambda i: ops.sample(peaked[i % 4], t_, k_, p_, keys, step0, 0), 4, S * V * 4, 0.0)
+            cases["sampling, temperature 0.8 / top-k 50 / top-p 0.9, rows of noise"] = (
+                lambda i: ops.sample(noise[i % 4], t_, k_, p_, keys, step0, 0), 4, S * V * 4, 0.0)
         rows = {}
         for name, (fn, copies, nbytes, flops) in cases.items():
             us = per_call(fn, copies)
