@@ -327,6 +327,7 @@ def test_sampling_draws_only_and_all_of_the_kept_tokens(vocab, top_k, top_p):
     small all of it is drawn in the end."""
     z = rnd(3, vocab, seed=19, scale=3.0)
     z[1] = z[1] * 0.05                                                  # a flat row: the kept set of top-p is most of it
+    z[2, ::7] = float("-inf")                                           # tokens that are ruled out beforehand
     draws = 300
     got = sample_rows(z, 0.8, top_k, top_p, draws)
     for row in range(3):
