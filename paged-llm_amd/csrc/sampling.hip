@@ -201,13 +201,14 @@ struct AroundPivot {                   // what lies above the pivot, and the nea
   }
 };
 template <int SLOTS>
-struct FirstLook {                     // the first pass: as AroundPivot, and the tokens above the pivot taken along
+struct FirstLook {                     // the first pass: the sum of all weights, as AroundPivot, and the tokens above the pivot taken along
   AroundPivot ap;
-  uint32_t key[SLOTS]; float weight[SLOTS]; int n;
+  uint32_t key[SLOTS]; float weight[SLOTS]; int n; float sum;
   __device__ __forceinline__ void operator()(float v, int) {
     const uint32_t k = float_key(v);
+    const float wt = ap.w(v);
+    sum += wt;
     if (k > ap.mid) {                                            // (few, in the usual row)
-      const float wt = ap.w(v);
       ap.cnt += 1;
       ap.mass += wt;
 #pragma unroll
@@ -301,18 +302,22 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   }
   Weigh weigh; weigh.zmax = best.v; weigh.rate = 1.4426950408889634f / fmaxf(temp, 1e-5f);
 
-  SumOfWeights sw; sw.w = weigh; sw.sum = 0.f;
-  sw = PLLM_WALK(sw);
-  const float total = block_sum(sw.sum, fscratch);
-
   int k = top_k[row];
   if (k <= 0 || k > vocab) k = vocab;
   const float p = top_p[row];
+  const bool filtered = k < vocab || p < 1.f;
+  // The sum of all weights: a pass of its own where nothing is filtered, else part of the search's first pass.
+  SumOfWeights sw; sw.w = weigh; sw.sum = 0.f;
+  float total = 0.f;
+  if (!filtered) {
+    sw = PLLM_WALK(sw);
+    total = block_sum(sw.sum, fscratch);
+  }
   uint32_t threshold = 0;                                        // tokens whose key >= threshold stay; 0 keeps all
   constexpr int kSlotsHere = kWindowSlots<IN_REGS>;
   IntoWindow<kSlotsHere> win; win.n = 0; win.mass_up = 0.f;
   bool windowed = false;
-  if (k < vocab || p < 1.f) {
+  if (filtered) {
     // kept(c)  <=>  count(key > c) < k  and  mass(key > c) <= p * total  is monotone in c; the threshold is the
     // smallest key of a token that stays.  [lo, hi]: kept(hi) holds, kept(lo - 1) does not, and both ends are keys of
     // tokens of the row (at the start its minimum, which cannot stay, and its maximum, which always does).  A pass takes
@@ -341,11 +346,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
         for (int s = 0; s < kSlotsHere; ++s) ap.look(win.key[s], win.weight[s]);     // (unused slots hold key 0: below every interval)
         ap.cnt += cnt_above; ap.mass += mass_above;
       } else if (first) {
-        FirstLook<kSlotsHere> fl; fl.ap = ap; fl.n = 0;
+        FirstLook<kSlotsHere> fl; fl.ap = ap; fl.n = 0; fl.sum = 0.f;
 #pragma unroll
         for (int s = 0; s < kSlotsHere; ++s) { fl.key[s] = 0u; fl.weight[s] = 0.f; }
         fl = PLLM_WALK(fl);
         ap = fl.ap;
+        total = block_sum(fl.sum, fscratch);
 #pragma unroll
         for (int s = 0; s < kSlotsHere; ++s) { win.key[s] = fl.key[s]; win.weight[s] = fl.weight[s]; }
       } else {
