@@ -1,11 +1,12 @@
-"""Minimal usage (options as in the reference's examples/generate.py:10-15; --backend takes "auto" or
-"hip", the one attention implementation there is):
+"""Minimal usage (options as in the reference's examples/generate.py:10-15; --backend is parsed for that command
+line's sake and takes "auto" or "hip", the one attention implementation there is):
 
     python examples/generate.py --model DIR --max-tokens 64 --temperature 0.0
+    python examples/generate.py --model DIR --prompt "Once upon a time" --prompt "The capital of France is"
     python examples/generate.py --model DIR --random-weights 0 --prompt-ids 1,2,3 --prompt-ids 4,5
 
-With a tokenizer.json in the folder the three built-in text prompts are used (two share a prefix,
-to show a cache hit); without one, token-id prompts.
+Without --prompt or --prompt-ids: with a tokenizer.json in the folder the three built-in text prompts are used (two
+share a prefix, to show a cache hit); without one, token-id prompts.  Text prompts need the folder's tokenizer.json.
 """
 import argparse
 import logging
@@ -35,6 +36,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-model-len", type=int, default=4096)
     ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
                     help="ignore the folder's tensors and fill the model of its config.json with seeded random weights")
+    ap.add_argument("--prompt", action="append", default=None, help="a text prompt (needs tokenizer.json in the folder); may be repeated")
     ap.add_argument("--prompt-ids", action="append", default=None, help="comma-separated token ids; may be repeated")
     ap.add_argument("--ignore-eos", action="store_true")
     args = ap.parse_args(argv)
@@ -44,9 +46,11 @@ def main(argv=None) -> int:
         overrides["random_weights"] = args.random_weights
     engine = LLMEngine(args.model, EngineConfig(
         block_size=args.block_size, num_gpu_blocks=args.num_gpu_blocks, max_num_batched_tokens=args.max_num_batched_tokens,
-        max_model_len=args.max_model_len, dtype=args.dtype, seed=args.seed, attention_backend=args.backend), **overrides)
-    if args.prompt_ids:
-        prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
+        max_model_len=args.max_model_len, dtype=args.dtype, seed=args.seed), **overrides)
+    if args.prompt or args.prompt_ids:
+        if args.prompt and engine.tokenizer is None:
+            ap.error(f"--prompt needs a tokenizer.json in {args.model}; give token ids with --prompt-ids instead")
+        prompts = list(args.prompt or []) + [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids or []]
     elif engine.tokenizer is not None:
         prompts = [
             "The three laws of robotics are",

@@ -2,7 +2,8 @@
 a caller of that engine passes; the grouping, the defaults' reasons and the checks are this engine's.
 
 The cache
-    ``block_size``              positions per page of keys and values, a power of two
+    ``block_size``              positions per page of keys and values, a power of two (bfloat16 attention runs on the
+                                matrix cores from 16 positions on; smaller pages take a slower kernel)
     ``num_gpu_blocks``          pages per cache group; None sizes the pool from free device memory at start-up
     ``gpu_memory_utilization``  the share of device memory the process may hold when the pool is sized that way
     ``enable_prefix_caching``   full pages of finished prompts stay findable by content and are shared
@@ -15,8 +16,6 @@ The model and the run
     ``dtype``                   "auto" (what the weights are stored in), "bfloat16" or "float32"
     ``device``, ``seed``
     ``enable_hip_graphs``       steps of known shapes are captured once and replayed
-    ``attention_backend``       inert: "auto" and "hip" both mean this engine's own kernels, the one implementation
-                                there is; the other engine's "triton", "flash" and "torch" are refused
 """
 
 from __future__ import annotations
@@ -45,7 +44,6 @@ class EngineConfig:
     device: str = "cuda"
     seed: int = 0
     enable_hip_graphs: bool = True
-    attention_backend: str = "auto"
 
     def __post_init__(self) -> None:
         problems = []
@@ -55,8 +53,5 @@ class EngineConfig:
             problems.append("max_num_batched_tokens must be >= block_size")
         if self.max_num_seqs <= 0:
             problems.append("max_num_seqs must be positive")
-        if self.attention_backend not in ("auto", "hip"):
-            problems.append(f"attention_backend={self.attention_backend!r}: this engine has one attention implementation, "
-                            "its HIP kernels (\"auto\" or \"hip\")")
         if problems:
             raise ValueError("; ".join(problems))

@@ -3,7 +3,8 @@
 The reference accepts exactly one name (pagedllm/model/loader.py:14,24-30); here the name
 selects an ``Architecture``: how to read the typed configuration, and how to turn it into a
 ``ModelSpec`` (the list of layers and their parts).  Another architecture is one more
-``register_architecture`` call; nothing else in the engine names a model.
+``register_architecture`` call (the modules of ``models/`` make theirs when that package is imported); nothing
+else in the engine names a model.
 """
 
 from __future__ import annotations
@@ -29,7 +30,7 @@ def register_architecture(arch: Architecture) -> None:
 
 
 def lookup_architecture(hf_config: dict) -> Architecture:
-    _ensure_builtin()
+    from .. import models  # noqa: F401  (importing the package registers the architectures it ships)
     names = hf_config.get("architectures") or []
     for n in names:
         if n in ARCHITECTURES:
@@ -43,8 +44,3 @@ def read_config_json(model_dir: str) -> dict:
         raise FileNotFoundError(f"{path} not found: a model folder holds config.json and *.safetensors")
     with open(path) as f:
         return json.load(f)
-
-
-def _ensure_builtin() -> None:
-    if "LlamaForCausalLM" not in ARCHITECTURES:
-        from ..models import llama  # noqa: F401  (registers itself)

@@ -1041,82 +1041,14 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
   return err;
 }
 
-// ---------------------------------------------------------------------------------------------
-// The same partitioned decode attention for callers that cannot allocate (see attention_noalloc.h): the
-// partitions' partial results go to an array of the library itself instead of a workspace argument.
-// In host code the array's name is only a stand-in for the symbol, so its device address is asked
-// for once per device (each GPU holds its own copy at its own address) and only that address is used.
+// What the library that holds the no-allocation entry point needs from this one (see attention_noalloc.h): the head
+// size it was compiled for, the entry point above, and a call that makes the device queries of the launch code now
+// (they are made lazily otherwise, at the first launch, which may be inside a stream capture).
 #include "attention_noalloc.h"
-#include <mutex>
-#include <stdio.h>
 
-static __device__ __align__(256) float scratch[PLLM_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+static int warm_up_device_queries() { return (num_compute_units() > 0 && pllm_max_lds() > 0) ? 0 : -1; }
 
-constexpr int kMaxDevices = 64;
-static float* scratch_of_device[kMaxDevices];
-static std::mutex scratch_lock;
-static thread_local char noalloc_error[256];
-
-// Device address of this GPU's copy of `scratch`, looked up at the first call on the device (which is current).
-static int scratch_address(float** ptr) {
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-    snprintf(noalloc_error, sizeof noalloc_error, "no current device, or device %d beyond the %d this library keeps addresses for", dev, kMaxDevices);
-    return PLLM_NOALLOC_NO_SYMBOL;
-  }
-  std::lock_guard<std::mutex> hold(scratch_lock);
-  if (!scratch_of_device[dev]) {
-    void* address = nullptr;
-    e = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || !address) {
-      snprintf(noalloc_error, sizeof noalloc_error, "hipGetSymbolAddress of the partials array failed on device %d: %s", dev, hipGetErrorString(e));
-      return PLLM_NOALLOC_NO_SYMBOL;
-    }
-    scratch_of_device[dev] = static_cast<float*>(address);
-  }
-  *ptr = scratch_of_device[dev];
-  return 0;
-}
-
-PLLM_API const char* pllm_attention_noalloc_error() { return noalloc_error; }
-
-PLLM_API int pllm_paged_attention_decode_noalloc(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
-                                                 int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
-                                                 const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
-                                                 int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                                 int num_partitions, int waves, hipStream_t stream) {
-  noalloc_error[0] = 0;
-  if (total_q <= 0 || num_seqs <= 0) return 0;
-  if (!q || !k_pages || !v_pages || !out || !block_tables || !cu_seqlens_q || !seq_lens_k || num_heads <= 0 || num_kv_heads <= 0 ||
-      num_heads % num_kv_heads || max_q_len < 1) {
-    snprintf(noalloc_error, sizeof noalloc_error, "null operand, or %d heads that are no multiple of %d kv heads", num_heads, num_kv_heads);
-    return PLLM_NOALLOC_BAD_ARGUMENT;
-  }
-  if (partition_size <= 0 || (partition_size & 63) || num_partitions < 1 || (long)max_q_len * (num_heads / num_kv_heads) > 64) {
-    snprintf(noalloc_error, sizeof noalloc_error,
-             "this entry point is the partitioned form: partition_size must be a positive multiple of 64 (got %d), num_partitions >= 1 "
-             "(got %d) and queries x heads per kv head at most 64 (got %ld)", partition_size, num_partitions,
-             (long)max_q_len * (num_heads / num_kv_heads));
-    return PLLM_NOALLOC_BAD_ARGUMENT;
-  }
-  const unsigned long long need = (unsigned long long)total_q * num_heads * num_partitions * kPartialFloats * sizeof(float);
-  if (need > PLLM_NOALLOC_SCRATCH_BYTES) {
-    snprintf(noalloc_error, sizeof noalloc_error,
-             "%d query rows x %d heads x %d partitions x (%d + 2) floats = %llu bytes of partial results; the library's array holds %u",
-             total_q, num_heads, num_partitions, D, need, (unsigned)PLLM_NOALLOC_SCRATCH_BYTES);
-    return PLLM_NOALLOC_TOO_LARGE;
-  }
-  float* partials = nullptr;
-  const int err = scratch_address(&partials);
-  if (err) return err;
-  const int rc = pllm_paged_attention_mfma(q, q_stride, k_pages, v_pages, out, out_stride, block_tables, bt_stride, cu_seqlens_q,
-                                           seq_lens_k, num_seqs, total_q, max_q_len, num_heads, num_kv_heads, block_size, scale, window,
-                                           partition_size, num_partitions, partials, waves, 0, nullptr, 0, stream);
-  if (rc == -2) {
-    snprintf(noalloc_error, sizeof noalloc_error, "the attention kernels refuse this shape (pages of %d positions, %d wavefronts, %d/%d heads)",
-             block_size, waves, num_heads, num_kv_heads);
-    return PLLM_NOALLOC_BAD_ARGUMENT;
-  }
-  return rc;
+PLLM_API const pllm_attention_api* pllm_attention_mfma_api() {
+  static const pllm_attention_api api = {D, &pllm_paged_attention_mfma, &warm_up_device_queries};
+  return &api;
 }

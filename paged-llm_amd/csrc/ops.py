@@ -9,6 +9,7 @@ is no CPU fallback, and a missing or unbuildable library raises at the first cal
 from __future__ import annotations
 
 import ctypes
+import logging
 from ctypes import c_float, c_int, c_long, c_longlong, c_ulonglong, c_void_p
 
 import numpy as np
@@ -16,6 +17,8 @@ import torch
 
 from . import build
 
+log = logging.getLogger("paged_llm_amd")
+_warned_plain_attention: list = []       # (said once per process)
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 MAX_HEAD_DIM_GENERIC = 256
@@ -193,14 +196,17 @@ def rope_scatter(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, 
 
 
 def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
-    """pages[dst[i]] = pages[src[i]] (whole pages of one layer's K or V)."""
+    """pages[dst[i]] = pages[src[i]] (whole pages of one tensor of a layer's cache, of any element type: the
+    bytes are copied in units of two or four)."""
     _on_gpu(pages, src, dst)
     _need(pages.is_contiguous() and pages.dim() >= 2, "pages must be contiguous [pages, ...]")
     _need(src.dtype == torch.int32 and dst.dtype == torch.int32 and src.shape == dst.shape and src.dim() == 1,
           "src and dst must be int32 vectors of one length")
-    page_elems = pages[0].numel()
-    _check(_fn("elementwise.hip", "pllm_copy_pages")(dtype_code(pages.dtype), _ptr(pages), _ptr(src), _ptr(dst),
-                                                      src.numel(), page_elems, _stream()), "copy_pages")
+    page_bytes = pages[0].numel() * pages.element_size()
+    _need(page_bytes % 2 == 0 and pages.data_ptr() % 4 == 0, "a page must be an even number of bytes")
+    unit, code = (4, F32) if page_bytes % 4 == 0 else (2, BF16)
+    _check(_fn("elementwise.hip", "pllm_copy_pages")(code, _ptr(pages), _ptr(src), _ptr(dst),
+                                                      src.numel(), page_bytes // unit, _stream()), "copy_pages")
 
 
 # ------------------------------------------------------------------------------------------- products
@@ -704,5 +710,10 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
                                     head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0,
                                     work_list=prompt_work_list(ctx, 0, group) if prompt else None)
+    if q.dtype == torch.bfloat16 and not _warned_plain_attention:
+        _warned_plain_attention.append(True)
+        log.warning("bfloat16 attention with pages of %d positions, head size %d, %d/%d heads runs on the plain kernel (one "
+                    "wavefront per token and head): the matrix-core kernels take pages of at least 16 positions, head sizes "
+                    "16..256 in steps of 16 and groups of at most 64 heads", bs, head_dim, num_heads, num_kv_heads)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
                                    num_kv_heads, head_dim, scale, window)

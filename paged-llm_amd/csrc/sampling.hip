@@ -271,7 +271,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   __shared__ float fscratch[16];
   __shared__ int iscratch[80];
   __shared__ ArgMax ascratch[16];
-  __shared__ int chosen;
+  __shared__ int chosen, chooser;
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* z = logits + (size_t)row * vocab;
   const int units = VEC ? vocab >> 2 : vocab;                    // pieces of four, or single elements
@@ -393,21 +393,26 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   }
   float kept_total;
   const float before = block_exclusive_scan(ks.sum, fscratch, kept_total);
-  if (tid == 0) chosen = -1;
+  if (tid == 0) { chosen = -1; chooser = -1; }
   __syncthreads();
   const long long rkey = request_key[row];
   const uint32_t bits = philox_first_word((uint32_t)step[row], 0u, (uint32_t)rkey, (uint32_t)(rkey >> 32),
                                           (uint32_t)seed, (uint32_t)(seed >> 32));
   const float u01 = (float)(bits >> 8) * (1.0f / 16777216.0f);   // [0, 1)
   const float target = u01 * kept_total;
-  // the thread whose share of the line holds the target takes the token there (one thread at most: shares do not overlap)
-  if (ks.sum > 0.f && before <= target && target < before + ks.sum) {
+  // The token is taken by the last thread, in thread order, that has tokens that stay and whose share of the line starts at
+  // or before the target.  The starts come out of a prefix sum and may be an ulp off each other's ends; "the last one that
+  // starts at or before" names exactly one thread whatever the rounding (a test of each thread's own interval could name
+  // two, or none), so a row's token depends on the row, the seed, the request and the step alone.
+  if (ks.sum > 0.f && before <= target) atomicMax(&chooser, tid);
+  __syncthreads();
+  if (chooser == tid) {
     Pick pk; pk.w = weigh; pk.threshold = threshold; pk.run = before; pk.target = target; pk.pick = -1; pk.last = -1;
     pk = PLLM_WALK(pk);
-    chosen = pk.pick >= 0 ? pk.pick : pk.last;
+    chosen = pk.pick >= 0 ? pk.pick : pk.last;               // (the target at or past the end of this share: its last token)
   }
   __syncthreads();
-  // (rounding at the very end of the line, or a row without a finite weight: the maximum)
+  // (a row without a finite weight: the maximum)
   if (tid == 0) out[row] = chosen >= 0 ? chosen : best.i;
 #undef PLLM_WALK
 }

@@ -6,7 +6,7 @@ import torch
 
 from ..cache.block_manager import CacheManager, GroupSpec
 from ..cache.kv_cache import KVCacheStorage
-from ..config.model_config import resolve_dtype
+from ..config.dtypes import resolve_dtype
 from ..config.registry import lookup_architecture, read_config_json
 from ..models.decoder import DecoderModel
 from ..weights.loader import load_weights

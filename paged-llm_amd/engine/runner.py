@@ -9,6 +9,8 @@ of the new tokens.
 
 from __future__ import annotations
 
+from collections import OrderedDict
+
 import numpy as np
 import torch
 
@@ -19,6 +21,44 @@ from .batch import GroupView, StepContext, StepEntry
 
 class StepError(ValueError):
     pass
+
+
+class GraphCache:
+    """Captured graphs by key.  Steps of single tokens and steps with prompt portions have a budget each, and within a
+    kind the entry that was replayed longest ago goes first: a burst of prompt shapes that never come back cannot push
+    out the graphs of the decode steps that run all the time (a graph that has gone must be captured again, which waits
+    for the GPU, and until then the step is not launched ahead)."""
+
+    def __init__(self, per_kind: int = 64):
+        self.per_kind = per_kind
+        self._kinds = {"decode": OrderedDict(), "prompt": OrderedDict()}
+
+    def _of(self, key) -> OrderedDict:
+        return self._kinds["prompt" if key[0] == "prompt" else "decode"]
+
+    def get(self, key):
+        """The entry, marked as used just now; None when there is none."""
+        entries = self._of(key)
+        entry = entries.get(key)
+        if entry is not None:
+            entries.move_to_end(key)
+        return entry
+
+    def put(self, key, entry) -> None:
+        entries = self._of(key)
+        while len(entries) >= self.per_kind and key not in entries:
+            entries.popitem(last=False)
+        entries[key] = entry
+        entries.move_to_end(key)
+
+    def __iter__(self):
+        return (key for entries in self._kinds.values() for key in entries)
+
+    def __len__(self) -> int:
+        return sum(len(entries) for entries in self._kinds.values())
+
+    def __contains__(self, key) -> bool:
+        return key in self._of(key)
 
 
 class ModelRunner:
@@ -37,7 +77,7 @@ class ModelRunner:
         self.max_graph_tokens = max_graph_tokens
         self.graph_after_sightings = max(1, graph_after_sightings)
         self._sightings: dict = {}
-        self._graphs: dict = {}
+        self._graphs = GraphCache()
         self._graph_pool = None               # one memory pool for the activations of all prompt-step graphs
         self.kv = kv_storage
         self.device = model.device
@@ -256,9 +296,7 @@ class ModelRunner:
         with torch.cuda.graph(graph, stream=stream):
             logits = self.model.forward(ctx, self.kv, self.states)
         entry.update(graph=graph, logits=logits, ctx=ctx)
-        if len(self._graphs) >= 64:
-            self._graphs.pop(next(iter(self._graphs)))
-        self._graphs[entry["key"]] = entry
+        self._graphs.put(entry["key"], entry)
 
     def _restage_decode(self, entry: dict, entries: list) -> int:
         """Write a decode step's arrays into the pinned buffer of its graph, in the layout of
@@ -518,9 +556,7 @@ class ModelRunner:
         with torch.cuda.graph(graph, stream=stream, pool=self._graph_pool):
             logits = self.model.forward(ctx, self.kv, self.states)
         entry.update(graph=graph, logits=logits, ctx=ctx)
-        if len(self._graphs) >= 64:
-            self._graphs.pop(next(iter(self._graphs)))
-        self._graphs[entry["key"]] = entry
+        self._graphs.put(entry["key"], entry)
 
     def _prompt_graph_step(self, key, entries: list, borrow: bool) -> torch.Tensor | None:
         entry = self._graphs.get(key)

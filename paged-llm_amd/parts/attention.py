@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..csrc import ops
-from .base import CacheSpec, Mixer
+from .base import BLOCK, CacheSpec, Mixer, PageTensor
 from .linear import linear, qkv_rotary_cache
 from .registry import BuildEnv, register_mixer
 from .spec import PartSpec, WeightSpec
@@ -65,8 +65,11 @@ class PagedAttention(Mixer):
 
     # ---- what it keeps
     def cache_spec(self):
+        """Keys as rows [kv_heads, positions, d]; values transposed inside the page [kv_heads, d, positions], so that
+        8 successive positions of one channel are one 16-byte load, the operand shape of the P*V matrix instruction."""
         kind = "window" if self.window > 0 else "full"
-        return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
+        nkv, d = self.num_kv_heads, self.head_dim
+        return CacheSpec(kind, (PageTensor("k", (nkv, BLOCK, d)), PageTensor("v", (nkv, d, BLOCK))), self.window)
 
     def graph_step_arrays(self, layout):
         """The prompt kernel's work list (pairs of sequence and tile, most keys first) for a replayed step."""
@@ -83,9 +86,10 @@ class PagedAttention(Mixer):
         if write and not self.kv_proj:
             raise RuntimeError("this attention layer has no k/v projections and must read another layer's cache")
         w_in = self.w_qkv if write or not self.kv_proj else self.w_qkv[: nh * d]
+        k_pages, v_pages = cache["k"], cache["v"]
         qkv = qkv_rotary_cache(h, w_in, ctx.positions, self.position, nh, nkv, d, view.slot_mapping if write else None,
-                               cache.k_pages if write else None, cache.v_pages if write else None, cache.block_size)
-        o = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
+                               k_pages if write else None, v_pages if write else None, cache.block_size)
+        o = ops.paged_attention(qkv, k_pages, v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
                                 nh, nkv, d, self.scale, self.window, ctx)
         return linear(o, self.w_o)
 

@@ -8,7 +8,7 @@ batch was cut.
 * ``Norm``            rows -> rows; ``add_norm`` fuses the residual sum in front of it.
 * ``PositionEncoding``  owns its tables; a mixer asks it to encode q/k (rotary) in place.
 * ``Mixer``           mixes information between the tokens of a request.  It may keep a growing
-                      cache (it then names a ``CacheSpec``: pages of keys and values) and/or a
+                      cache (it then names a ``CacheSpec``: the tensors of a page, shaped as it likes) and/or a
                       state of fixed size per request (``StateSpec``: a slot in a state tensor).
 * ``FeedForward``     rows -> rows, no mixing between tokens.
 * ``Block``           the arrangement of a layer's parts around the residual stream; the kind
@@ -24,17 +24,59 @@ import torch
 from .spec import WeightSpec
 
 
+BLOCK = "block"       # in the shape of a page tensor: the dimension that holds the positions of a page
+
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One tensor of what a mixer keeps per token: the shape of ONE page, with ``BLOCK`` where the positions of the
+    page go (any dimension, so a mixer may keep its record transposed inside the page).  ``dtype`` None: the
+    model's compute type."""
+    name: str
+    shape: tuple
+    dtype: torch.dtype | None = None
+
+    def __post_init__(self):
+        if tuple(self.shape).count(BLOCK) != 1 or not all(d == BLOCK or (isinstance(d, int) and d > 0) for d in self.shape):
+            raise ValueError(f"page tensor {self.name!r}: a shape of positive sizes with BLOCK exactly once, got {self.shape}")
+
+    def page_shape(self, block_size: int) -> tuple:
+        return tuple(block_size if d == BLOCK else d for d in self.shape)
+
+    def bytes_per_page(self, block_size: int, compute_dtype: torch.dtype) -> int:
+        elems = 1
+        for d in self.page_shape(block_size):
+            elems *= d
+        return elems * torch.empty((), dtype=self.dtype or compute_dtype).element_size()
+
+
 @dataclass(frozen=True)
 class CacheSpec:
-    """What a mixer keeps per token.  Layers with equal specs share a group of pages."""
-    kind: str                 # "full": all keys;  "window": only the last `window` positions
-    num_kv_heads: int
-    head_dim: int
+    """What a mixer keeps per token, in pages: which positions stay (``kind``) and the tensors of a page, which the
+    mixer names and shapes itself (keys and values of equal width, one latent vector, two records of different
+    widths ...).  The cache storage allocates ``[pages, *page shape]`` per named tensor and hands them to the mixer
+    by name; the cache manager only counts pages.  Layers with equal specs share a group of pages (one block table
+    per request and group)."""
+    kind: str                 # "full": all positions;  "window": only the last `window` positions
+    tensors: tuple            # of PageTensor
     window: int = 0           # > 0 for kind "window"
+
+    def __post_init__(self):
+        if self.kind not in ("full", "window") or (self.kind == "window") != (self.window > 0):
+            raise ValueError(f"cache kind {self.kind!r} with window {self.window}: \"full\", or \"window\" with a window > 0")
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a cache spec names at least one page tensor, each once; got {names}")
 
     def group_name(self) -> str:
         base = f"{self.kind}{self.window if self.kind == 'window' else ''}"
-        return f"{base}_kv{self.num_kv_heads}x{self.head_dim}"
+        def one(t):
+            dims = "x".join("B" if d == BLOCK else str(d) for d in t.shape)
+            return f"{t.name}{dims}" + (f":{str(t.dtype).split('.')[-1]}" if t.dtype is not None else "")
+        return base + "_" + "_".join(one(t) for t in self.tensors)
+
+    def bytes_per_page(self, block_size: int, compute_dtype: torch.dtype) -> int:
+        return sum(t.bytes_per_page(block_size, compute_dtype) for t in self.tensors)
 
 
 @dataclass(frozen=True)
@@ -137,8 +179,8 @@ class Mixer(Part):
     def forward(self, h, ctx, cache, state) -> torch.Tensor:
         """h: normed rows [T, hidden], as a tensor or as a pending norm (``parts.linear.linear`` and
         its relatives take both; ``parts.norm.rows_of(h)`` gives the tensor).  ctx: the step's StepContext.  cache: LayerCache of the
-        layer this mixer reads (with ``writable`` False when it belongs to another layer), or
-        None.  state: [slots, *shape] tensor, or None."""
+        layer this mixer reads (``cache[name]`` is the page tensor the mixer's CacheSpec names, [pages, *page shape];
+        ``writable`` is False when the cache belongs to another layer), or None.  state: [slots, *shape] tensor, or None."""
         raise NotImplementedError
 
 

@@ -48,8 +48,7 @@ def write_random_model(folder: str, hf_config: dict, seed: int = 0, dtype: str |
                        norm_jitter: bool = False) -> str:
     """Write ``folder/config.json`` and ``folder/model.safetensors``; returns the folder."""
     from safetensors.torch import save_file
-    cfg = dict(hf_config)
-    cfg.setdefault("architectures", ["LlamaForCausalLM"])
+    cfg = dict(hf_config)                                       # ("architectures" in it names the model, as everywhere)
     dtype = dtype or cfg.get("torch_dtype") or "float32"
     if dtype not in _STORED:
         raise KeyError(f"random weights are stored as float32 or bfloat16, not {dtype!r}")

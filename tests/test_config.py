@@ -4,7 +4,8 @@ import pytest
 import torch
 
 from paged_llm_amd import EngineConfig, SamplingParams
-from paged_llm_amd.config import LlamaConfig, lookup_architecture, read_config_json, resolve_dtype
+from paged_llm_amd.config import lookup_architecture, read_config_json, resolve_dtype
+from paged_llm_amd.models.llama import LlamaConfig
 from tests.tiny_configs import TINY_A, TINY_B, TINY_C
 
 MINIMAL = {"architectures": ["LlamaForCausalLM"], "vocab_size": 10, "hidden_size": 32, "intermediate_size": 8,
@@ -100,9 +101,27 @@ def test_sampling_params():
     assert SamplingParams(temperature=0.0).greedy and not sp.greedy
 
 
-def test_attention_backend_names():
-    from paged_llm_amd import EngineConfig
-    assert EngineConfig().attention_backend == "auto" and EngineConfig(attention_backend="hip").attention_backend == "hip"
-    for other in ("triton", "flash", "torch"):
-        with pytest.raises(ValueError, match="one attention implementation"):
-            EngineConfig(attention_backend=other)
+def test_there_is_no_attention_backend_option():
+    """The reference's EngineConfig picks one of its attention backends (pagedllm/config.py:27); this engine has
+    one implementation and no such knob: naming one is an error like any unknown option."""
+    with pytest.raises(TypeError):
+        EngineConfig(attention_backend="triton")
+
+
+def test_page_specs_are_the_mixers_to_shape():
+    """A cache spec names the tensors of a page with the page's positions wherever the mixer wants them; equal specs
+    give one group name, and sizes follow the declared shapes and element types."""
+    from paged_llm_amd.parts import BLOCK, CacheSpec, PageTensor
+    kv = CacheSpec("full", (PageTensor("k", (2, BLOCK, 16)), PageTensor("v", (2, 16, BLOCK))))
+    assert kv.group_name() == "full_k2xBx16_v2x16xB"
+    assert kv == CacheSpec("full", (PageTensor("k", (2, BLOCK, 16)), PageTensor("v", (2, 16, BLOCK))))
+    assert kv.bytes_per_page(16, torch.bfloat16) == 2 * 2 * 16 * 16 * 2
+    one = CacheSpec("window", (PageTensor("c", (BLOCK, 24), torch.float32),), window=7)
+    assert one.group_name() == "window7_cBx24:float32" and one.tensors[0].page_shape(8) == (8, 24)
+    assert one.bytes_per_page(8, torch.bfloat16) == 8 * 24 * 4
+    for bad in (lambda: PageTensor("k", (2, 16)), lambda: PageTensor("k", (BLOCK, BLOCK)), lambda: PageTensor("k", (BLOCK, 0)),
+                lambda: CacheSpec("full", ()), lambda: CacheSpec("window", (PageTensor("k", (BLOCK,)),)),
+                lambda: CacheSpec("full", (PageTensor("k", (BLOCK,)), PageTensor("k", (BLOCK, 2)))),
+                lambda: CacheSpec("ring", (PageTensor("k", (BLOCK,)),))):
+        with pytest.raises(ValueError):
+            bad()

@@ -185,6 +185,62 @@ def test_sampling_is_reproducible_and_independent_of_the_batch(folder_a):
     assert greedy.token_ids != a[0]
 
 
+def test_rows_of_one_step_with_different_sampling_settings(folder_a):
+    """Requests with different SamplingParams share steps (the reference zips rows and params in the scheduler's
+    order, pagedllm/engine.py:93-102; here the step function reorders its entries by token count and the sampler packs
+    the rows' settings into one buffer).  Prompt lengths are chosen against the order of arrival and the token budget is
+    small, so portions of some prompts run beside decoded tokens of others.  Settings that leave one token (temperature
+    0; top_k 1; a top_p that only the first token passes) must give the plain implementation's greedy tokens; for the
+    truly random rows every token must lie in the kept set of the plain distribution of the very row the engine sampled
+    from, and be what the kernel draws for that row alone with (seed, request id, tokens generated so far)."""
+    from paged_llm_amd import SamplingParams
+    from paged_llm_amd.csrc import ops
+    prompts = [helpers.random_tokens(n, 256, seed=300 + n) for n in (30, 5, 41, 12, 26, 3)]
+    settings = [SamplingParams(temperature=0.0, max_tokens=14, ignore_eos=True),
+                SamplingParams(temperature=0.9, top_k=40, top_p=0.95, max_tokens=14, ignore_eos=True),
+                SamplingParams(temperature=0.9, top_k=1, max_tokens=14, ignore_eos=True),
+                SamplingParams(temperature=1.6, top_k=-1, top_p=0.8, max_tokens=14, ignore_eos=True),
+                SamplingParams(temperature=1.3, top_p=1e-6, max_tokens=14, ignore_eos=True),
+                SamplingParams(temperature=0.0, max_tokens=14, ignore_eos=True)]
+    engine = engine_for(folder_a, seed=11, max_num_batched_tokens=24)
+    observed = Observed(engine)
+    rows_per_step = []
+    inner = engine.on_logits
+    def hook(requests, logits):
+        rows_per_step.append([(r.id, r.params) for r in requests])
+        inner(requests, logits)
+    engine.on_logits = hook
+    outs = engine.generate(prompts, settings)
+    # rows of different settings did share steps, greedy rows beside random ones
+    assert any(len({id(p) for _, p in rows}) >= 4 for rows in rows_per_step)
+    assert any(len(rows) < len(prompts) for rows in rows_per_step), "prompts were not cut: every step held all requests"
+    for o, sp in zip(outs, settings):
+        assert len(o.token_ids) == 14
+        tokens = o.prompt_token_ids + o.token_ids
+        want = helpers.plain_logits(folder_a, tokens)
+        one_token_left = sp.temperature < 1e-5 or sp.top_k == 1 or sp.top_p < 1e-3
+        if one_token_left:
+            assert o.token_ids == plain_greedy(folder_a, o.prompt_token_ids, 14), sp
+        distinct = 0
+        for i, token in enumerate(o.token_ids):
+            pos = len(o.prompt_token_ids) + i - 1
+            row = observed.rows[(o.seq_id, pos)]
+            assert helpers.worst(row, want[pos]) <= TOL["float32"], (o.seq_id, pos)
+            if one_token_left:
+                continue
+            kept = llama_plain.filtered_probabilities(torch.from_numpy(row), sp.temperature, sp.top_k, sp.top_p).numpy()
+            assert kept[token] > 0, f"request {o.seq_id}, token {i}: {token} is outside the kept set of its own settings"
+            distinct += token != int(np.argmax(row))
+            dev = lambda values, dtype: torch.tensor(values, dtype=dtype, device="cuda")
+            alone = ops.sample(torch.from_numpy(row)[None].cuda().contiguous(), dev([sp.temperature], torch.float32),
+                               dev([sp.top_k], torch.int32), dev([sp.top_p], torch.float32), dev([o.seq_id], torch.int64),
+                               dev([i], torch.int32), 11)
+            assert int(alone[0]) == token, f"request {o.seq_id}, token {i}: the row alone draws {int(alone[0])}, the step drew {token}"
+        if not one_token_left:
+            assert distinct >= 2, "the random rows only ever took the largest logit"
+    assert engine.cache_manager.num_free_pages() == 64
+
+
 def test_step_api_and_abort(folder_a):
     from paged_llm_amd import SamplingParams
     engine = engine_for(folder_a)

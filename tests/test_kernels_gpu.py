@@ -344,8 +344,18 @@ def test_sampling_keeps_or_drops_equal_logits_together(vocab):
     top_k = 2 both stay (one token is larger than each), and the fourth goes."""
     z = torch.full((1, vocab), -20.0)
     z[0, 5], z[0, vocab // 2], z[0, vocab - 3], z[0, 70] = 3.0, 2.5, 2.5, 2.0
-    got = set(sample_rows(z, 1.0, 2, 1.0, 200)[:, 0].tolist())
-    assert got == {5, vocab // 2, vocab - 3}
+    draws = 4000
+    got = sample_rows(z, 1.0, 2, 1.0, draws)[:, 0]
+    assert set(got.tolist()) == {5, vocab // 2, vocab - 3}
+    # ... and the draw is renormalised over that larger set (the reference cuts by sorted rank, pagedllm/sampler.py:25-31,
+    # keeps exactly top_k tokens and so one of the two equal ones, whichever its sort puts first)
+    want = torch.softmax(torch.tensor([3.0, 2.5, 2.5]), 0).numpy() * draws
+    counts = np.array([(got == i).sum().item() for i in (5, vocab // 2, vocab - 3)])
+    assert float(((counts - want) ** 2 / want).sum()) < 2 + 5 * math.sqrt(4) + 5
+    # the same for the mass filter: the two equal tokens pass or fail the cumulative mass together
+    mass = torch.softmax(z[0].double(), 0)
+    p_between = float(mass[5] + 0.5 * mass[vocab // 2])            # reached inside the tie group
+    assert set(sample_rows(z, 1.0, -1, p_between, 300)[:, 0].tolist()) == {5, vocab // 2, vocab - 3}
 
 
 def test_sampling_rows_do_not_depend_on_their_neighbours():

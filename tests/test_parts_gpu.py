@@ -82,9 +82,9 @@ def layer_cache(mixer, dtype: str, pages: int):
     from paged_llm_amd.cache.kv_cache import LayerCache
     spec = mixer.cache_spec()
     dev = torch.device("cuda:0")
-    k = torch.zeros((pages, spec.num_kv_heads, BLOCK, spec.head_dim), dtype=getattr(torch, dtype), device=dev)
-    v = torch.zeros((pages, spec.num_kv_heads, spec.head_dim, BLOCK), dtype=getattr(torch, dtype), device=dev)
-    return LayerCache(k, v, spec.group_name(), BLOCK, pages)
+    tensors = {t.name: torch.zeros((pages, *t.page_shape(BLOCK)), dtype=t.dtype or getattr(torch, dtype), device=dev)
+               for t in spec.tensors}
+    return LayerCache(tensors, spec.group_name(), BLOCK, pages)
 
 
 # ------------------------------------------------------------------------------------------- norm

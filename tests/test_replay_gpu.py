@@ -263,9 +263,9 @@ def test_request_longer_than_the_configured_positions(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("block_size", [8, 32])
+@pytest.mark.parametrize("block_size", [4, 8, 32])
 def test_every_mode_at_other_page_sizes(folders, dtype, block_size):
-    """Configuration B with pages of 8 positions (the matrix-core attention kernel needs 16: bfloat16 then takes
+    """Configuration B with pages of 4 and 8 positions (the matrix-core attention kernel needs 16: bfloat16 then takes
     the plain attention kernel behind the fused rotary epilogue and cache write) and of 32: whole, the last 32
     tokens one by one, portions of changing size, and mixed with pages used again."""
     folder = folders["B", "float32" if dtype == "float32" else "bfloat16"]
@@ -297,5 +297,22 @@ def test_every_mode_at_other_page_sizes(folders, dtype, block_size):
     got = helpers.replay_in_process(session, trace)
     assert len(got) == sum(len(t) for t in twice.values())
     check(got, folder, twice, dtype)
+    session.manager.check_invariants()
+    assert session.manager.num_free_pages() == session.manager.num_pages()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("block_size", [1, 2])
+def test_pages_of_one_and_two_positions(folders, dtype, block_size):
+    """The smallest pages the configuration accepts: every position (or pair) is a page of its own, so every key is
+    found through its own table entry.  Mixed batches with pages used again, configuration A."""
+    folder = folders["A", "float32" if dtype == "float32" else "bfloat16"]
+    reqs = {f"p{i}": helpers.random_tokens(n, 256, seed=700 + i) for i, n in enumerate((5, 17, 33, 40, 70, 9))}
+    trace, peak = mixed_trace(reqs, max_live=4, seed=9)
+    session = session_for(folder, dtype, peak, block_size)
+    assert session.manager.block_size == block_size
+    got = helpers.replay_in_process(session, trace)
+    assert len(got) == sum(len(t) for t in reqs.values())
+    check(got, folder, reqs, dtype)
     session.manager.check_invariants()
     assert session.manager.num_free_pages() == session.manager.num_pages()

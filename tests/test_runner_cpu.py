@@ -242,3 +242,24 @@ def test_layout_of_a_step_with_portions_replayed_from_a_graph():
     assert runner._prompt_graph_key([make(f"p{i}", [1, 2], 0) for i in range(5)]) is None
     runner.max_graph_tokens = 16
     assert runner._prompt_graph_key(entries) is None
+
+
+def test_graphs_of_decode_steps_outlive_a_burst_of_prompt_shapes():
+    """Captured graphs are kept per kind, least recently used out first: a hundred prompt-step shapes that never
+    come back do not cost the decode graph that is replayed between them, nor the prompt shape that is."""
+    from paged_llm_amd.engine.runner import GraphCache
+    cache = GraphCache(per_kind=64)
+    decode_key, hot_prompt = (8, 8, 2048), ("prompt", 8, 1, 256, 9, 2560, 0)
+    cache.put(decode_key, "decode graph")
+    cache.put(hot_prompt, "hot prompt graph")
+    for i in range(100):
+        cache.put(("prompt", 0, 1, 32 * (i + 1), 1, 4096, 0), f"one-off {i}")
+        assert cache.get(decode_key) == "decode graph" and cache.get(hot_prompt) == "hot prompt graph"
+    assert len(cache) == 65 and decode_key in cache and hot_prompt in cache
+    assert ("prompt", 0, 1, 32, 1, 4096, 0) not in cache and ("prompt", 0, 1, 3200, 1, 4096, 0) in cache
+    # within a kind: the one used longest ago goes
+    for i in range(70):
+        cache.put((i + 100, 1, 512), i)
+        cache.get(decode_key)
+    assert decode_key in cache and (100, 1, 512) not in cache and (169, 1, 512) in cache
+    assert sorted(k[0] for k in cache if k[0] != "prompt")[:2] == [8, 107]

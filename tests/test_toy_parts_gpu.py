@@ -248,8 +248,9 @@ def test_toy_model_is_built_from_registered_parts(toy_folder):
     from paged_llm_amd.engine.replay import ReplaySession
     s = ReplaySession(toy_folder, "float32", 256, None)
     groups = s.model.cache_groups()
-    assert sorted(groups) == ["full_kv1x16", "window7_kv1x16"]
-    assert groups["full_kv1x16"].owners == [0, 5] and groups["window7_kv1x16"].owners == [3]   # step 2 owns no pages
+    full, windowed = "full_k1xBx16_v1x16xB", "window7_k1xBx16_v1x16xB"
+    assert sorted(groups) == [full, windowed]
+    assert groups[full].owners == [0, 5] and groups[windowed].owners == [3]   # step 2 owns no pages
     assert "layers.4.norm2.weight" not in s.model.weight_specs() and "layers.4.norm1.weight" in s.model.weight_specs()
     assert sorted(s.model.state_specs()) == [1, 4]                                             # one state per step, not per layer
     assert "layers.2.mixer.k_proj.weight" not in s.model.weight_specs()
@@ -337,3 +338,154 @@ def test_toy_model_generates_through_the_entry_point_with_default_settings(toy_f
         assert out.token_ids == toks[len(prompt):] and out.num_cached_tokens == 0
     assert all(engine.cache_manager.num_free_pages(g) == engine.cache_manager.num_pages(g) for g in engine.cache_manager.groups)
     engine.cache_manager.check_invariants()
+
+
+# ------------------------------------------------------------------------------------------- a page of another shape
+LATENT = {"architectures": ["ToyLatentForCausalLM"], "vocab_size": 90, "hidden_size": 40, "intermediate_size": 56,
+          "heads": 2, "kv_heads": 1, "head_dim": 16, "latent": 24, "eps": 1e-5, "theta": 50.0, "max_position_embeddings": 256}
+
+
+def register_latent_toy():
+    from paged_llm_amd.config.registry import ARCHITECTURES, Architecture, register_architecture
+    from paged_llm_amd.parts import (BLOCK, CacheSpec, LayerSpec, Mixer, ModelSpec, PageTensor, PartSpec, WeightSpec,
+                                     register_mixer)
+    from paged_llm_amd.parts.linear import linear
+    if "ToyLatentForCausalLM" in ARCHITECTURES:
+        return
+
+    class PrefixMeanMixer(Mixer):
+        """Keeps one vector c_t = W_in x_t of ``latent`` floats per token, in pages of ONE tensor [positions, latent]
+        that are float32 whatever the model computes in; its output at token t is W_out mean(c_0 .. c_t).  Every
+        key weighs the same, so a wrong page anywhere in the prefix shows.  Reads and writes go through the block
+        table and the slots of its own cache group."""
+
+        def __init__(self, params, env):
+            self.hidden, self.latent = env.hidden_size, int(params["latent"])
+            self.dtype, self.device, self._w = env.dtype, env.device, {}
+
+        def weight_specs(self):
+            return {"in_proj.weight": WeightSpec((self.latent, self.hidden)), "out_proj.weight": WeightSpec((self.hidden, self.latent))}
+
+        def assign(self, name, tensor):
+            self._w[name] = tensor.to(device=self.device, dtype=self.dtype).contiguous()
+
+        def cache_spec(self):
+            return CacheSpec("full", (PageTensor("c", (BLOCK, self.latent), torch.float32),))
+
+        def forward(self, h, ctx, cache, state):
+            view, pages = ctx.groups[cache.group], cache["c"]
+            assert pages.dtype == torch.float32 and tuple(pages.shape[1:]) == (cache.block_size, self.latent)
+            c = linear(h, self._w["in_proj.weight"]).float()
+            pages.view(-1, self.latent).index_copy_(0, view.slot_mapping.long(), c)
+            out, at, bs = torch.empty_like(c), 0, cache.block_size
+            for s, (n, k_len) in enumerate(zip(ctx.q_lens, ctx.k_lens)):
+                pos = torch.arange(k_len, device=c.device)
+                kept = pages[view.block_tables[s, pos // bs].long(), pos % bs]            # [k_len, latent] through the table
+                means = kept.cumsum(0) / (pos + 1).unsqueeze(1)
+                out[at:at + n] = means[k_len - n:]
+                at += n
+            return linear(out.to(self.dtype), self._w["out_proj.weight"])
+
+    register_mixer("toy_prefix_mean", PrefixMeanMixer)
+
+    def build_spec(c):
+        norm = PartSpec("rmsnorm", {"eps": c["eps"]})
+        rotary = {"kind": "rotary", "params": {"head_dim": c["head_dim"], "theta": c["theta"], "scaling": None}}
+        attention = PartSpec("paged_attention", {"num_heads": c["heads"], "num_kv_heads": c["kv_heads"], "head_dim": c["head_dim"],
+                                                 "position": rotary})
+        mean = PartSpec("toy_prefix_mean", {"latent": c["latent"]})
+        ffn = PartSpec("gated_mlp", {"intermediate_size": c["intermediate_size"]})
+        block = PartSpec("prenorm", {"mixer_norm": "norm1", "mixer": "mixer", "feed_forward_norm": "norm2", "feed_forward": "ffn"})
+        layers = [LayerSpec(f"layers.{i}", block, {"mixer_norm": norm, "mixer": m, "feed_forward_norm": norm, "feed_forward": ffn})
+                  for i, m in enumerate([mean, attention, mean])]
+        return ModelSpec(hidden_size=c["hidden_size"], vocab_size=c["vocab_size"],
+                         embedding=PartSpec("token_embedding", {"vocab_size": c["vocab_size"]}), layers=layers, final_norm=norm,
+                         head=PartSpec("lm_head", {"vocab_size": c["vocab_size"], "tied": True}), embedding_name="embed",
+                         final_norm_name="norm", head_name="head", max_positions=c["max_position_embeddings"], stored_dtype="float32")
+
+    register_architecture(Architecture("ToyLatentForCausalLM", lambda raw: dict(raw), build_spec))
+
+
+def plain_latent(folder, tokens):
+    c, w = LATENT, {k: v.float() for k, v in plain.load_weights(folder).items()}
+    T, nh, nkv, d = len(tokens), c["heads"], c["kv_heads"], c["head_dim"]
+    angles = plain.rotary_angles(torch.arange(T), plain.inverse_frequencies(d, c["theta"], None))
+    x = w["embed.weight"][torch.tensor(tokens)]
+    for layer in range(3):
+        p = f"layers.{layer}."
+        h = plain.rms_norm(x, w[p + "norm1.weight"], c["eps"])
+        if layer == 1:
+            q = plain.apply_rotary((h @ w[p + "mixer.q_proj.weight"].T).view(T, nh, d), angles)
+            k = plain.apply_rotary((h @ w[p + "mixer.k_proj.weight"].T).view(T, nkv, d), angles)
+            v = (h @ w[p + "mixer.v_proj.weight"].T).view(T, nkv, d)
+            a = plain.causal_attention(q, k, v, d ** -0.5, None).reshape(T, nh * d) @ w[p + "mixer.o_proj.weight"].T
+        else:
+            kept = h @ w[p + "mixer.in_proj.weight"].T
+            means = kept.cumsum(0) / torch.arange(1, T + 1).unsqueeze(1)
+            a = means @ w[p + "mixer.out_proj.weight"].T
+        x = x + a
+        h = plain.rms_norm(x, w[p + "norm2.weight"], c["eps"])
+        x = x + plain.swiglu(h, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+    return (plain.rms_norm(x, w["norm.weight"], c["eps"]) @ w["embed.weight"].T).numpy()
+
+
+@pytest.fixture(scope="module")
+def latent_folder(tmp_path_factory):
+    register_latent_toy()
+    return helpers.make_folder(tmp_path_factory.mktemp("latent"), LATENT, seed=37, stored="float32")
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 5e-2)])
+def test_mixer_with_a_page_of_its_own_shape(latent_folder, dtype, tol):
+    """A mixer registered from here keeps one float32 tensor [positions, 24] per page, beside an attention layer
+    with its two tensors in the model's type: the storage allocates what each names, the pool is sized from their
+    bytes, copies after a fork move every tensor, and the model replays whole, in portions and mixed (pages used
+    again) against its plain implementation.  No file of the package knows this page shape."""
+    from paged_llm_amd.cache.block_manager import PageCopy
+    from paged_llm_amd.engine.replay import ReplaySession
+    from tests.test_replay_gpu import mixed_trace
+    reqs = {f"m{i}": helpers.random_tokens(n, LATENT["vocab_size"], seed=600 + i) for i, n in enumerate([2, 35, 80, 64, 19])}
+    want = {rid: plain_latent(latent_folder, toks) for rid, toks in reqs.items()}
+
+    def compare(got):
+        assert len(got) == sum(len(t) for t in reqs.values())
+        for (rid, pos), row in got.items():
+            err = helpers.worst(row, want[rid][pos])
+            assert err <= tol, f"{rid} position {pos}: {err:.3g}"
+
+    session = ReplaySession(latent_folder, dtype, 128, None)
+    groups = session.model.cache_groups()
+    mean_group, attn_group = "full_cBx24:float32", "full_k1xBx16_v1x16xB"
+    assert sorted(groups) == sorted([mean_group, attn_group]) and groups[mean_group].owners == [0, 2]
+    elem = 4 if dtype == "float32" else 2
+    assert groups[mean_group].bytes_per_page(16, session.model.dtype) == 2 * 16 * 24 * 4
+    assert groups[attn_group].bytes_per_page(16, session.model.dtype) == 2 * 16 * 16 * elem
+    held = session.storage.for_step(0)
+    assert set(held.tensors) == {"c"} and held["c"].dtype == torch.float32 and tuple(held["c"].shape) == (8, 16, 24)
+    assert set(session.storage.for_step(1).tensors) == {"k", "v"}
+    assert not session.runner.use_graphs                   # the toy mixer reads host lists: its steps are not captured
+
+    whole = TraceBuilder()
+    for rid, toks in reqs.items():
+        whole.step([(rid, toks, "all")], end=[rid])
+    compare(helpers.replay_in_process(session, whole))
+    # a page copy moves the mixer's tensor like any other (pages 1 and 2 hold the last request's vectors)
+    before = held["c"][1].clone()
+    assert before.abs().sum() > 0
+    session.storage.apply_copies({mean_group: [PageCopy(1, 5)]})
+    assert torch.equal(held["c"][5], before) and torch.equal(session.storage.for_step(2)["c"][5], session.storage.for_step(2)["c"][1])
+
+    portions = TraceBuilder()
+    for rid, toks in reqs.items():
+        at, sizes = 0, iter([2, 5, 1, 9, 3] * 40)
+        while at < len(toks):
+            n = min(next(sizes), len(toks) - at)
+            portions.step([(rid, toks[at:at + n], "all")], end=[rid] if at + n == len(toks) else [])
+            at += n
+    compare(helpers.replay_in_process(ReplaySession(latent_folder, dtype, 128, None), portions))
+
+    trace, peak = mixed_trace(reqs, max_live=3, seed=4)
+    session = ReplaySession(latent_folder, dtype, peak, None)
+    compare(helpers.replay_in_process(session, trace))
+    session.manager.check_invariants()
+    assert all(session.manager.num_free_pages(g) == session.manager.num_pages(g) for g in session.manager.groups)
