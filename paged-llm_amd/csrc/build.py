@@ -144,7 +144,7 @@ def load_library(source: str, defines: dict | None = None) -> ctypes.CDLL:
 
 # Sources every model needs, and the specialised ones per head size.
 COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip", "decode_linear.hip",
-                  "attention_noalloc.hip"]
+                  "attention_noalloc.hip", "stream_linear.hip"]
 # Head sizes whose attention library a full build makes (others are compiled at first use).
 USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 

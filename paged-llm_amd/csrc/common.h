@@ -23,6 +23,15 @@ template <typename T> __device__ __forceinline__ T from_f32(float x);
 template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16 from_f32<bf16>(float x) { return __float2bfloat16(x); }  // round to nearest even
 
+// One rotary pair turned by the angle whose cosine and sine are c and s.  Products and sums are rounded one by one (no
+// fused multiply-add), in every kernel that rotates: what one kernel writes into the cache and what another computes
+// for the same position are then the same bits, and equal to what plain float arithmetic gives.
+__device__ __forceinline__ void rotate_pair(float lo, float hi, float c, float s, float& out_lo, float& out_hi) {
+#pragma clang fp contract(off)
+  out_lo = lo * c - hi * s;
+  out_hi = hi * c + lo * s;
+}
+
 // Raw 16-bit pattern <-> float, for vector loads of bf16 data.
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {

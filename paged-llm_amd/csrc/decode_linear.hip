@@ -97,7 +97,9 @@ __device__ __forceinline__ void rope_store(const DecodeLinearParams& p, int m, i
     // q and k are rounded to bfloat16 by the projection before they are rotated
     lo = __bfloat162float(__float2bfloat16(lo));
     hi = __bfloat162float(__float2bfloat16(hi));
-    const bf16 out_lo = __float2bfloat16(lo * cs - hi * sn), out_hi = __float2bfloat16(hi * cs + lo * sn);
+    float rl, rh;
+    rotate_pair(lo, hi, cs, sn, rl, rh);
+    const bf16 out_lo = __float2bfloat16(rl), out_hi = __float2bfloat16(rh);
     if (head < nh) {
       bf16* q = (bf16*)p.out + (size_t)m * p.ldo + (size_t)head * d;
       q[ri] = out_lo;

@@ -43,9 +43,13 @@ PLLM_API int pllm_embed_gather(int dtype, const int* ids, const void* table, voi
 //   out[r] = T( (s * rsqrt(mean(s^2) + eps)) * w )
 // `row_index` (optional) picks the source rows, so the last norm runs only on rows whose logits
 // are wanted.  `x_out` (optional) receives the new residual rows (may alias x).
+// The sum may also come as float partial sums of `splits` ranges of a product's inner dimension (`parts`:
+// [splits][rows of x][hidden], `part_stride` floats from one range to the next): they are added in order, in float,
+// and take delta's place.
 template <typename T>
 __global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const int* __restrict__ row_index,
-                               const float* __restrict__ w, float eps, T* __restrict__ out, T* x_out, int hidden) {
+                               const float* __restrict__ w, float eps, T* __restrict__ out, T* x_out, int hidden,
+                               const float* __restrict__ parts, int splits, size_t part_stride) {
   extern __shared__ float lds[];
   float* row = lds;             // [hidden]
   float* scratch = lds + hidden;  // [16]
@@ -66,6 +70,17 @@ __global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const in
 #pragma unroll
         for (int j = 0; j < V; ++j) px.v[j] = from_f32<T>(to_f32(px.v[j]) + to_f32(pd.v[j]));
         if (x_out) reinterpret_cast<Piece*>(x_out + src * hidden)[c] = px;
+      } else if (parts) {
+        float d[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) d[j] = 0.f;
+        for (int sp = 0; sp < splits; ++sp) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) d[j] += parts[sp * part_stride + src * hidden + (size_t)c * V + j];
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) px.v[j] = from_f32<T>(to_f32(px.v[j]) + d[j]);
+        if (x_out) reinterpret_cast<Piece*>(x_out + src * hidden)[c] = px;
       }
 #pragma unroll
       for (int j = 0; j < V; ++j) {
@@ -77,8 +92,11 @@ __global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const in
   } else {
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
       float v = to_f32(xr[i]);
-      if (delta) {
-        v = to_f32(from_f32<T>(v + to_f32(delta[src * hidden + i])));
+      if (delta || parts) {
+        float d = 0.f;
+        if (delta) d = to_f32(delta[src * hidden + i]);
+        else for (int sp = 0; sp < splits; ++sp) d += parts[sp * part_stride + src * hidden + i];
+        v = to_f32(from_f32<T>(v + d));
         if (x_out) x_out[src * hidden + i] = from_f32<T>(v);
       }
       row[i] = v;
@@ -105,7 +123,8 @@ __global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const in
 template <typename T, int P>
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* __restrict__ delta, const int* __restrict__ row_index,
                                                            const float* __restrict__ w, float eps, T* __restrict__ out, T* x_out,
-                                                           int hidden, int rows) {
+                                                           int hidden, int rows, const float* __restrict__ parts, int splits,
+                                                           size_t part_stride) {
   constexpr int V = 16 / sizeof(T);
   struct alignas(16) Piece { T v[V]; };
   const int lane = threadIdx.x & 63;
@@ -139,6 +158,24 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
 #pragma unroll
       for (int j = 0; j < V; ++j) px[i].v[j] = from_f32<T>(to_f32(px[i].v[j]) + to_f32(pd[i].v[j]));
       if (x_out) reinterpret_cast<Piece*>(x_out + src * hidden)[c] = px[i];
+    } else if (parts) {
+      // the ranges' float sums of this piece, added in order (16-byte loads: hidden is a multiple of V, the buffer aligned)
+      struct alignas(16) Four { float v[4]; };
+      float d[V];
+#pragma unroll
+      for (int j = 0; j < V; ++j) d[j] = 0.f;
+      for (int sp = 0; sp < splits; ++sp) {
+        const Four* pp = reinterpret_cast<const Four*>(parts + sp * part_stride + src * hidden + (size_t)c * V);
+#pragma unroll
+        for (int q = 0; q < V / 4; ++q) {
+          const Four f = pp[q];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) d[q * 4 + j] += f.v[j];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) px[i].v[j] = from_f32<T>(to_f32(px[i].v[j]) + d[j]);
+      if (x_out) reinterpret_cast<Piece*>(x_out + src * hidden)[c] = px[i];
     }
 #pragma unroll
     for (int j = 0; j < V; ++j) acc += to_f32(px[i].v[j]) * to_f32(px[i].v[j]);
@@ -158,13 +195,14 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
 
 template <typename T>
 static int launch_rmsnorm(const T* x, const T* delta, const int* row_index, const float* w, float eps, T* out, T* x_out, int rows,
-                           int hidden, hipStream_t stream) {
+                           int hidden, const float* parts, int splits, size_t part_stride, hipStream_t stream) {
   constexpr int V = 16 / sizeof(T);
   const bool wide = hidden % V == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
-                    (!delta || ((uintptr_t)delta % 16) == 0) && (!x_out || ((uintptr_t)x_out % 16) == 0);
+                    (!delta || ((uintptr_t)delta % 16) == 0) && (!x_out || ((uintptr_t)x_out % 16) == 0) &&
+                    (!parts || (((uintptr_t)parts % 16) == 0 && part_stride % 4 == 0));
   const int per_lane = wide ? (hidden / V + 63) / 64 : 0;
   dim3 grid4((rows + 3) / 4), block(256);
-#define PLLM_ROWS(P_) hipLaunchKernelGGL((rmsnorm_rows_kernel<T, P_>), grid4, block, 0, stream, x, delta, row_index, w, eps, out, x_out, hidden, rows)
+#define PLLM_ROWS(P_) hipLaunchKernelGGL((rmsnorm_rows_kernel<T, P_>), grid4, block, 0, stream, x, delta, row_index, w, eps, out, x_out, hidden, rows, parts, splits, part_stride)
   if (wide && per_lane <= 2) PLLM_ROWS(2);
   else if (wide && per_lane <= 4) PLLM_ROWS(4);
   else if (wide && per_lane <= 8) PLLM_ROWS(8);
@@ -175,19 +213,23 @@ static int launch_rmsnorm(const T* x, const T* delta, const int* row_index, cons
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rmsnorm_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(rows), block, lds, stream, x, delta, row_index, w, eps, out, x_out, hidden);
+    hipLaunchKernelGGL(rmsnorm_kernel<T>, dim3(rows), block, lds, stream, x, delta, row_index, w, eps, out, x_out, hidden, parts, splits, part_stride);
   }
 #undef PLLM_ROWS
   return (int)hipGetLastError();
 }
 
 PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int* row_index, const float* w, float eps,
-                          void* out, void* x_out, int rows, int hidden, hipStream_t stream) {
+                          void* out, void* x_out, int rows, int hidden, const float* parts, int splits, long part_stride,
+                          hipStream_t stream) {
   if (rows <= 0) return 0;
+  if (parts && (delta || splits < 1 || part_stride < 0)) return -2;
   if (((size_t)hidden + 16) * sizeof(float) > 160 * 1024) return -2;  // a row must fit the LDS of the one-row-per-workgroup kernel
   if (dtype == PLLM_F32)
-    return launch_rmsnorm<float>((const float*)x, (const float*)delta, row_index, w, eps, (float*)out, (float*)x_out, rows, hidden, stream);
-  return launch_rmsnorm<bf16>((const bf16*)x, (const bf16*)delta, row_index, w, eps, (bf16*)out, (bf16*)x_out, rows, hidden, stream);
+    return launch_rmsnorm<float>((const float*)x, (const float*)delta, row_index, w, eps, (float*)out, (float*)x_out, rows, hidden, parts, splits,
+                                (size_t)part_stride, stream);
+  return launch_rmsnorm<bf16>((const bf16*)x, (const bf16*)delta, row_index, w, eps, (bf16*)out, (bf16*)x_out, rows, hidden, parts, splits,
+                              (size_t)part_stride, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -302,8 +344,10 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
       for (int j = 0; j < 8; ++j) {
         const float c = cs ? cs[i + j] : 1.f, s = sn ? sn[i + j] : 0.f;
         const float l = to_f32(lo.v[j]), u = to_f32(hi.v[j]);
-        out_lo.v[j] = from_f32<T>(l * c - u * s);
-        out_hi.v[j] = from_f32<T>(u * c + l * s);
+        float rl, ru;
+        rotate_pair(l, u, c, s, rl, ru);
+        out_lo.v[j] = from_f32<T>(rl);
+        out_hi.v[j] = from_f32<T>(ru);
       }
       T* dst = nullptr;
       if (head < num_heads) dst = h;
@@ -322,8 +366,9 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, int row_stride, const i
       T* h = row + (size_t)head * head_dim;
       const float lo = to_f32(h[a]), hi = to_f32(h[b]);
       const float c = cs ? cs[i] : 1.f, s = sn ? sn[i] : 0.f;
-      const T out_lo = from_f32<T>(lo * c - hi * s);
-      const T out_hi = from_f32<T>(hi * c + lo * s);
+      float rl, ru;
+      rotate_pair(lo, hi, c, s, rl, ru);
+      const T out_lo = from_f32<T>(rl), out_hi = from_f32<T>(ru);
       if (head < num_heads) {
         h[a] = out_lo;
         h[b] = out_hi;

@@ -68,7 +68,8 @@ def _on_gpu(*tensors: torch.Tensor | None) -> None:
 
 _SIGNATURES = {
     "pllm_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-    "pllm_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "pllm_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long,
+                     c_void_p],
     "pllm_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "pllm_rope_scatter": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -118,6 +119,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, delta: torch.Tens
     With ``delta`` the sum ``x + delta`` (float add, rounded to the element type) is the new
     residual; it is written back into ``x`` unless ``write_residual`` is False.  ``row_index``
     (int32) selects which rows are normed; the output then has one row per index.
+    ``delta`` may also be a float tensor [ranges, rows, hidden]: the partial sums of a product whose inner dimension
+    was cut into ranges (``stream_linear`` with SL_PARTIAL); they are added in order, in float, with x.
     """
     _on_gpu(x, weight, delta, row_index)
     _need(x.dim() == 2 and x.is_contiguous(), "x must be contiguous [rows, hidden]")
@@ -126,6 +129,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, delta: torch.Tens
           f"norm weight must be float32 [{H}], got {weight.dtype} {tuple(weight.shape)}")
     _need((H + 16) * 4 <= min(_max_lds_bytes(x.device), 160 * 1024),
           f"rmsnorm kernel stages one row in LDS as floats: hidden size {H} is above its limit")
+    parts = None
+    if delta is not None and delta.dim() == 3:
+        parts, delta = delta, None
+        _need(parts.dtype == torch.float32 and tuple(parts.shape[1:]) == tuple(x.shape) and parts.is_contiguous(),
+              f"partial sums must be contiguous float32 [ranges, {x.shape[0]}, {H}]")
     if delta is not None:
         _need(delta.shape == x.shape and delta.dtype == x.dtype and delta.is_contiguous(), "delta must match x")
     if row_index is not None:
@@ -135,9 +143,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, delta: torch.Tens
     else:
         rows = x.shape[0]
     out = torch.empty((rows, H), dtype=x.dtype, device=x.device)
-    x_out = x if (delta is not None and write_residual) else None
+    x_out = x if ((delta is not None or parts is not None) and write_residual) else None
     _check(_fn("elementwise.hip", "pllm_rmsnorm")(dtype_code(x.dtype), _ptr(x), _ptr(delta), _ptr(row_index), _ptr(weight),
-                                                   c_float(eps), _ptr(out), _ptr(x_out), rows, H, _stream()), "rmsnorm")
+                                                   c_float(eps), _ptr(out), _ptr(x_out), rows, H, _ptr(parts),
+                                                   0 if parts is None else parts.shape[0], 0 if parts is None else x.numel(),
+                                                   _stream()), "rmsnorm")
     return out
 
 
@@ -402,6 +412,123 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
              out.stride(0), M, N, K, _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")),
              _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)),
              int(r.get("head_dim", 0)), int(r.get("block_size", 0)), _stream()), "decode_linear")
+    return out
+
+
+# ------------------------------------------------------------------------------------------- products of 17 to a few hundred rows
+SL_BF16, SL_F32, SL_GATED, SL_PARTIAL, SL_ROPE_KV = 0, 1, 2, 3, 4
+STREAM_TILE_ROWS, STREAM_TILE_K = 16, 32
+_STREAM_SIG = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+
+
+class TiledWeight:
+    """A weight matrix [N, K] in the order the streaming product kernel reads it: blocks of 16 rows, each block's tiles of
+    16 rows x 32 columns one after the other along K, a tile being 1 KB in the order of the matrix instruction's operand
+    (lane g * 16 + r: row r, columns 8 g .. 8 g + 7); zero rows pad the blocks to a multiple of twelve.  ``pairing`` says
+    which rows share a block: "plain" (16 successive rows), "gated" (8 gate rows and the up rows of the same outputs), or
+    "rotary" (8 elements of the lower half of a head and their partners in the upper half, ``head_dim`` apart by half)."""
+
+    def __init__(self, tiles: torch.Tensor, out_features: int, in_features: int, pairing: str, head_dim: int = 0):
+        self.tiles, self.out_features, self.in_features, self.pairing, self.head_dim = tiles, out_features, in_features, pairing, head_dim
+
+    @property
+    def blocks(self) -> int:
+        return self.tiles.shape[0]
+
+
+def stream_linear_takes(w: torch.Tensor) -> bool:
+    return w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % STREAM_TILE_K == 0 and w.is_cuda
+
+
+def tile_weight(w: torch.Tensor, pairing: str = "plain", head_dim: int = 0) -> TiledWeight:
+    """The tiled copy of ``w`` [N, K] (bfloat16, K a multiple of 32).  "gated": w = [gate rows; up rows].  "rotary":
+    w = [q; k; v] rows of heads of ``head_dim`` (a multiple of 16) elements."""
+    _need(stream_linear_takes(w), "tiled weights: bfloat16 [N, K] on the GPU with K a multiple of 32")
+    N, K = w.shape
+    out_features = N
+    if pairing == "gated":
+        _need(N % 2 == 0, "a gated matrix holds gate rows and as many up rows")
+        half = N // 2
+        units = -(-half // 8)
+        j = torch.arange(units * 8, device=w.device).view(units, 8).clamp_(max=half - 1)
+        w = w.index_select(0, torch.cat([j, j + half], dim=1).reshape(-1))           # per block: 8 gate rows, their 8 up rows
+        out_features = half
+    elif pairing == "rotary":
+        _need(head_dim > 0 and head_dim % 16 == 0 and N % head_dim == 0, "rotary pairing: whole heads of a multiple of 16 elements")
+        heads, half = N // head_dim, head_dim // 2
+        lower = (torch.arange(heads, device=w.device).view(heads, 1, 1) * head_dim
+                 + torch.arange(half // 8, device=w.device).view(1, half // 8, 1) * 8 + torch.arange(8, device=w.device).view(1, 1, 8))
+        w = w.index_select(0, torch.cat([lower, lower + half], dim=2).reshape(-1))    # per block: 8 lower elements, their partners
+    else:
+        _need(pairing == "plain", f"unknown pairing {pairing!r}")
+    blocks = -(-w.shape[0] // 16)
+    blocks_padded = -(-blocks // 12) * 12                                 # (whole workgroups of 1, 2, 3 or 4 blocks)
+    if blocks_padded * 16 != w.shape[0]:
+        w = torch.cat([w, torch.zeros((blocks_padded * 16 - w.shape[0], K), dtype=w.dtype, device=w.device)])
+    tiles = w.view(blocks_padded, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()       # [block, k step, g, r, 8]
+    return TiledWeight(tiles, out_features, K, pairing, head_dim)
+
+
+def stream_linear_plan(M: int, N: int, K: int, compute_units: int) -> tuple[int, int]:
+    """(blocks of 16 weight rows per workgroup, ranges of K) for a product of M rows with N weight rows: by sizes only.
+    Four blocks per workgroup halve what the rows cost out of the caches and are taken where the matrix still gives
+    every compute unit a workgroup and the rows are at most 64 (the accumulators of 64 x 64 outputs are what a wavefront
+    has registers for); a matrix with fewer workgroups than compute units is cut along K."""
+    blocks = -(-N // 16)
+    nt = 2
+    row_blocks = -(-M // 128)
+    workgroups = -(-blocks // nt) * row_blocks
+    stages = -(-K // 256)
+    splits = 1
+    if workgroups < compute_units:
+        splits = max(1, min(compute_units // workgroups, stages // 2, 8))
+    return nt, splits
+
+
+def stream_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, nt: int | None = None, splits: int | None = None,
+                  rope: dict | None = None) -> torch.Tensor:
+    """x [M, K] bfloat16 times the tiled weights.  SL_BF16 / SL_F32: [M, N]; SL_GATED: silu(gate) * up [M, N / 2];
+    SL_PARTIAL: float [splits, M, N], the sums over ``splits`` ranges of K, to be added in that order; SL_ROPE_KV: q rotated
+    [M, heads * d], k (rotated) and v written to their pages (``rope`` as for ``decode_linear``)."""
+    _on_gpu(x, w.tiles)
+    M, K = x.shape
+    _need(x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0,
+          "stream_linear: bfloat16 rows that start on 16-byte boundaries")
+    _need(K == w.in_features and w.tiles.is_contiguous() and tuple(w.tiles.shape[1:]) == (K // 32, 4, 16, 8) and w.blocks % 12 == 0,
+          f"stream_linear: rows of {K} values against tiled weights of {w.in_features}")
+    _need({SL_GATED: "gated", SL_ROPE_KV: "rotary"}.get(epi, "plain") == w.pairing,
+          f"epilogue {epi} against weights tiled with the {w.pairing} pairing")
+    N = w.out_features
+    plan_nt, plan_splits = stream_linear_plan(M, N * (2 if epi == SL_GATED else 1), K, _num_compute_units(x.device))
+    nt = nt or plan_nt
+    splits = (plan_splits if epi == SL_PARTIAL else 1) if splits is None else splits
+    _need(splits == 1 or epi == SL_PARTIAL, "ranges of K give partial sums")
+    r = rope or {}
+    if epi == SL_PARTIAL:
+        out = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+    elif epi == SL_ROPE_KV:
+        nh, nkv, d, bs = r["num_heads"], r["num_kv_heads"], r["head_dim"], r["block_size"]
+        _need(d == w.head_dim and N == (nh + 2 * nkv) * d, "the weights were tiled for other heads")
+        kp, vp = r["k_pages"], r["v_pages"]
+        P = kp.shape[0]
+        _need(tuple(kp.shape) == (P, nkv, bs, d) and tuple(vp.shape) == (P, nkv, d, bs) and kp.is_contiguous() and vp.is_contiguous()
+              and kp.dtype == torch.bfloat16 and vp.dtype == torch.bfloat16, "bad cache pages")
+        for name in ("positions", "slots"):
+            t = r[name]
+            _need(t.dtype == torch.int32 and t.shape == (M,) and t.is_contiguous(), f"{name}: int32 [{M}]")
+        if r.get("cos") is not None:
+            for t in (r["cos"], r["sin"]):
+                _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == d // 2 and t.is_contiguous() and t.data_ptr() % 16 == 0,
+                      "rotary tables")
+        out = torch.empty((M, nh * d), dtype=torch.bfloat16, device=x.device)
+    else:
+        out = torch.empty((M, N), dtype=torch.float32 if epi == SL_F32 else torch.bfloat16, device=x.device)
+    f = _fn("stream_linear.hip", "pllm_stream_linear", signature=_STREAM_SIG)
+    _check(f(epi, _ptr(x), x.stride(0), _ptr(w.tiles), _ptr(out), out.stride(-2), M, N, K, w.blocks, nt, splits,
+             _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")), _ptr(r.get("k_pages")),
+             _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)), int(r.get("head_dim", 0)),
+             int(r.get("block_size", 0)), _stream()), "stream_linear")
     return out
 
 

@@ -64,6 +64,10 @@ class StepContext:
     # ``parts.base.Part.graph_step_arrays``) and ``graph_layout`` says how the batch is laid out.
     launch_cache: dict = field(default_factory=dict)
     graph_layout: object = None
+    # Set around a branch (mixer, feed-forward) by whoever will hand the branch's output to a norm as its delta, when
+    # that norm adds float partial sums itself: the branch's last product may then return [ranges, rows, hidden] float
+    # sums over ranges of its inner dimension instead of rows (``parts.linear.linear(..., partial_ok=...)``).
+    partial_sums_ok: bool = False
 
     @property
     def decode_only(self) -> bool:

@@ -108,13 +108,19 @@ class DecoderModel:
         assert self._ready, "weights not loaded"
         x = self.embedding.forward(ctx.input_ids)
         delta = None
-        for pos, step in enumerate(self.spec.schedule):
+        schedule = self.spec.schedule
+        last_takes_partial = bool(getattr(self.final_norm, "accepts_partial_sums", False))
+        for pos, step in enumerate(schedule):
             block = self.blocks[step.layer]
             cache = None
             if block.cache_spec() is not None:
                 owner = pos if step.cache_from is None else step.cache_from
                 cache = kv_storage.for_step(owner, writable=step.cache_from is None)
+            # whether the delta this block hands on may be float partial sums: what consumes it next says
+            ctx.partial_sums_ok = (self.blocks[schedule[pos + 1].layer].accepts_partial_delta() if pos + 1 < len(schedule)
+                                   else last_takes_partial)
             x, delta = block.forward(x, delta, ctx, cache, states.get(pos))
+        ctx.partial_sums_ok = False
         n = ctx.logits_index.numel()
         if n == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)

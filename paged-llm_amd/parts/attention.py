@@ -13,7 +13,7 @@ import torch
 
 from ..csrc import ops
 from .base import BLOCK, CacheSpec, Mixer, PageTensor
-from .linear import linear, qkv_rotary_cache
+from .linear import Weight, linear, qkv_rotary_cache
 from .registry import BuildEnv, register_mixer
 from .spec import PartSpec, WeightSpec
 
@@ -40,8 +40,8 @@ class PagedAttention(Mixer):
         self.position = env.position_encoding(PartSpec(**pos) if isinstance(pos, dict) else pos) if pos else None
         self.dtype, self.device = env.dtype, env.device
         self._w: dict[str, torch.Tensor] = {}
-        self.w_qkv: torch.Tensor | None = None
-        self.w_o: torch.Tensor | None = None
+        self.w_qkv: Weight | None = None
+        self.w_o: Weight | None = None
 
     # ---- weights
     def weight_specs(self):
@@ -59,8 +59,9 @@ class PagedAttention(Mixer):
 
     def finalize(self):
         names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.kv_proj else [])
-        self.w_qkv = torch.cat([self._w[n] for n in names], dim=0).contiguous()
-        self.w_o = self._w["o_proj.weight"].contiguous()
+        # (a layer without k/v projections only ever projects q: its matrix keeps the plain pairing)
+        self.w_qkv = Weight(torch.cat([self._w[n] for n in names], dim=0).contiguous(), "rotary" if self.kv_proj else "plain", self.head_dim)
+        self.w_o = Weight(self._w["o_proj.weight"].contiguous())
         self._w.clear()
 
     # ---- what it keeps
@@ -85,13 +86,13 @@ class PagedAttention(Mixer):
         write = cache.writable
         if write and not self.kv_proj:
             raise RuntimeError("this attention layer has no k/v projections and must read another layer's cache")
-        w_in = self.w_qkv if write or not self.kv_proj else self.w_qkv[: nh * d]
+        w_in = self.w_qkv if write or not self.kv_proj else self.w_qkv.rows(nh * d)
         k_pages, v_pages = cache["k"], cache["v"]
         qkv = qkv_rotary_cache(h, w_in, ctx.positions, self.position, nh, nkv, d, view.slot_mapping if write else None,
                                k_pages if write else None, v_pages if write else None, cache.block_size)
         o = ops.paged_attention(qkv, k_pages, v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
                                 nh, nkv, d, self.scale, self.window, ctx)
-        return linear(o, self.w_o)
+        return linear(o, self.w_o, partial_ok=bool(getattr(ctx, "partial_sums_ok", False)))
 
 
 register_mixer("paged_attention", PagedAttention)

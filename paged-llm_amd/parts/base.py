@@ -122,6 +122,10 @@ class Part:
 
 
 class Norm(Part):
+    # True when ``add_norm`` / ``pending`` also take, in delta's place, the float partial sums [ranges, rows, hidden]
+    # of a product whose inner dimension was cut into ranges (to be added in order, in float, with x).
+    accepts_partial_sums = False
+
     def forward(self, x: torch.Tensor, row_index: torch.Tensor | None = None) -> torch.Tensor:
         raise NotImplementedError
 
@@ -238,6 +242,11 @@ class Block(Part):
         for part in self.parts.values():
             out.update(part.graph_step_arrays(layout))
         return out
+
+    def accepts_partial_delta(self) -> bool:
+        """Whether the ``delta`` this block is handed may be float partial sums [ranges, rows, hidden] instead of rows
+        (it is, when the block's first act is to give it to a norm that takes them)."""
+        return False
 
     def weight_specs(self):
         return {f"{self.names[role]}.{name}": spec for role, part in self.parts.items()

@@ -8,7 +8,7 @@ import torch
 
 from ..csrc import ops
 from .base import FeedForward
-from .linear import gated_linear, linear
+from .linear import Weight, gated_linear, linear
 from .registry import BuildEnv, register_feed_forward
 from .spec import WeightSpec
 
@@ -25,8 +25,8 @@ class GatedMLP(FeedForward):
             raise NotImplementedError(f"gated feed-forward activation {act!r} (silu only)")
         self.dtype, self.device = env.dtype, env.device
         self._w: dict[str, torch.Tensor] = {}
-        self.w_gate_up: torch.Tensor | None = None
-        self.w_down: torch.Tensor | None = None
+        self.w_gate_up: Weight | None = None
+        self.w_down: Weight | None = None
 
     def weight_specs(self):
         return {"gate_proj.weight": WeightSpec((self.inter, self.hidden)),
@@ -39,13 +39,13 @@ class GatedMLP(FeedForward):
         self._w[name] = tensor.to(device=self.device, dtype=self.dtype)
 
     def finalize(self):
-        self.w_gate_up = torch.cat([self._w["gate_proj.weight"], self._w["up_proj.weight"]], dim=0).contiguous()
-        self.w_down = self._w["down_proj.weight"].contiguous()
+        self.w_gate_up = Weight(torch.cat([self._w["gate_proj.weight"], self._w["up_proj.weight"]], dim=0).contiguous(), "gated")
+        self.w_down = Weight(self._w["down_proj.weight"].contiguous())
         self._w.clear()
 
     def forward(self, h, ctx):
         act = gated_linear(h, self.w_gate_up)
-        return linear(act, self.w_down)
+        return linear(act, self.w_down, partial_ok=bool(getattr(ctx, "partial_sums_ok", False)))
 
 
 register_feed_forward("gated_mlp", GatedMLP)

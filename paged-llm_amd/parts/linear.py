@@ -3,12 +3,15 @@
 * float32: the plain kernel with float operands (the true 32-bit path), always.
 * bfloat16, at most 16 rows (decoding): the fused decode kernel, which also takes in a pending
   residual sum + norm in front and an activation or the rotary/cache write behind.
-* bfloat16, 17 to 64 rows and a small matrix: the same kernel's form for plain rows (the norm runs first).
+* bfloat16, 17 to 128 rows (decoding with many requests, short prompt portions): the streaming kernel over the
+  weights' tiled copy (``Weight``), with the same epilogues, or with float partial sums of ranges of K that the
+  consuming norm adds; where it was measured slower than the library (the gated product beyond 64 rows, the
+  output head) the library stays.
 * bfloat16, more rows (prompt portions): the vendor's matrix-product library, with bfloat16 or (logits)
   float results.
 
 The choice depends on the number of rows and the sizes only, never on the rows' content.  ``x`` may
-be a tensor or a ``PendingNorm``.
+be a tensor or a ``PendingNorm``; a weight may be a tensor [N, K] or a ``Weight``.
 """
 
 from __future__ import annotations
@@ -17,6 +20,71 @@ import torch
 
 from ..csrc import ops
 from .norm import PendingNorm, rows_of
+
+
+class Weight:
+    """A part's matrix [N, K] with, for bfloat16 matrices whose K is a multiple of 32, a second copy in the tiled
+    order that the streaming kernel reads (1 KB tiles in the matrix instruction's operand order; see
+    ``ops.tile_weight``).  ``pairing``: which rows share a tile, by what the epilogue behind the product needs:
+    "plain", "gated" ([gate; up] rows) or "rotary" ([q; k; v] rows of heads of ``head_dim``).  The plain copy serves
+    the other kernels and the library; a step reads one of the two."""
+
+    def __init__(self, plain: torch.Tensor, pairing: str = "plain", head_dim: int = 0):
+        self.plain = plain
+        self.pairing = pairing
+        ok = ops.stream_linear_takes(plain) and (pairing != "rotary" or (head_dim > 0 and head_dim % 16 == 0))
+        self.tiled = ops.tile_weight(plain, pairing, head_dim) if ok else None
+
+    @property
+    def shape(self):
+        return self.plain.shape
+
+    @property
+    def dtype(self):
+        return self.plain.dtype
+
+    def rows(self, count: int) -> torch.Tensor:
+        """The first ``count`` rows as a plain matrix (a view)."""
+        return self.plain[:count]
+
+
+STREAM_MIN_ROWS, STREAM_MAX_ROWS = 17, 128      # rows the streaming kernel is chosen for
+STREAM_GATED_MAX_ROWS = 64                      # the gated product: beyond, its rows' traffic costs more than the library's kernel
+STREAM_SMALL_MATRIX = 1 << 24                   # elements up to which a matrix is "small": cut along K, partial sums or one range
+
+
+def _plain(weight) -> torch.Tensor:
+    return weight.plain if isinstance(weight, Weight) else weight
+
+
+def _streams(x, weight, epi: int) -> bool:
+    """Whether this product goes to the streaming kernel: by sizes and row count only (measured on matrices of
+    2048 x 2048 to 11264 x 2048 and 2048 x 5632 against the library and the kernels for fewer rows)."""
+    if not (isinstance(weight, Weight) and weight.tiled is not None):
+        return False
+    rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
+    if not STREAM_MIN_ROWS <= rows <= STREAM_MAX_ROWS or x.dtype != torch.bfloat16:
+        return False
+    n, k = weight.shape
+    if epi == ops.SL_GATED:
+        return rows <= STREAM_GATED_MAX_ROWS
+    if epi == ops.SL_F32:
+        return False                                            # (the head: 32000 x 2048 was not faster than the library's kernel)
+    return n * k <= STREAM_SMALL_MATRIX
+
+
+def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: bool = False):
+    x = rows_of(x)
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    n, k = weight.shape
+    if epi == ops.SL_GATED:
+        return ops.stream_linear(x, weight.tiled, epi, nt=3)
+    nt, splits = ops.stream_linear_plan(x.shape[0], n, k, ops._num_compute_units(x.device))
+    if epi == ops.SL_BF16 and partial_ok and splits > 1:
+        return ops.stream_linear(x, weight.tiled, ops.SL_PARTIAL, nt=nt, splits=splits)
+    # one range of K: blocks of 16 weight rows of their own fill the GPU best for these matrices
+    return ops.stream_linear(x, weight.tiled, epi, nt=1 if -(-n // 16) <= 2 * ops._num_compute_units(x.device) else nt, rope=rope)
 
 
 def _fused(x, weight: torch.Tensor, epi: int, rope: dict | None = None):
@@ -34,8 +102,13 @@ def _fused(x, weight: torch.Tensor, epi: int, rope: dict | None = None):
     return None
 
 
-def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """x [T, K] (tensor or pending norm), weight [N, K] -> [T, N]."""
+def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = False) -> torch.Tensor:
+    """x [T, K] (tensor or pending norm), weight [N, K] -> [T, N].  ``partial_ok``: the caller hands the result to a
+    norm as its delta and that norm adds partial sums (``StepContext.partial_sums_ok``): the result may then be float
+    [ranges, T, N], the sums over ranges of K."""
+    if _streams(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16):
+        return _stream(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok=partial_ok)
+    weight = _plain(weight)
     if weight.dtype == torch.bfloat16:
         out = _fused(x, weight, ops.EPI_F32 if out_dtype == torch.float32 else ops.EPI_BF16)
         if out is not None:
@@ -46,8 +119,11 @@ def linear(x, weight: torch.Tensor, out_dtype: torch.dtype | None = None) -> tor
     return ops.gemm_generic(x, weight, out_dtype)
 
 
-def gated_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix."""
+def gated_linear(x, w_gate_up) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix (a tensor, or a ``Weight`` with the gated pairing)."""
+    if _streams(x, w_gate_up, ops.SL_GATED) and w_gate_up.pairing == "gated":
+        return _stream(x, w_gate_up, ops.SL_GATED)
+    w_gate_up = _plain(w_gate_up)
     if w_gate_up.dtype == torch.bfloat16:
         out = _fused(x, w_gate_up, ops.EPI_GATED)
         if out is not None:
@@ -55,7 +131,7 @@ def gated_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
     return ops.silu_mul(linear(x, w_gate_up))
 
 
-def qkv_rotary_cache(x, w_qkv: torch.Tensor, positions: torch.Tensor, position_encoding, num_heads: int, num_kv_heads: int,
+def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_heads: int, num_kv_heads: int,
                      head_dim: int, slot_mapping, k_pages, v_pages, block_size: int) -> torch.Tensor:
     """q, k, v projections, rotation of q and k, and the write of k and v into the cache pages.
     Returns q as rows of a matrix whose first num_heads * head_dim columns hold the rotated heads
@@ -74,9 +150,13 @@ def qkv_rotary_cache(x, w_qkv: torch.Tensor, positions: torch.Tensor, position_e
     if write and w_qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and whole_head_halves:
         rope = dict(positions=positions, cos=cos, sin=sin, slots=slot_mapping, k_pages=k_pages, v_pages=v_pages,
                     num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size)
-        q = _fused(x, w_qkv, ops.EPI_ROPE_KV, rope)
+        if (isinstance(w_qkv, Weight) and w_qkv.pairing == "rotary" and _streams(x, w_qkv, ops.SL_ROPE_KV)
+                and (cos is None or cos.data_ptr() % 16 == 0)):
+            return _stream(x, w_qkv, ops.SL_ROPE_KV, rope=rope)
+        q = _fused(x, _plain(w_qkv), ops.EPI_ROPE_KV, rope)
         if q is not None:
             return q
+    w_qkv = _plain(w_qkv)
     qkv = linear(x, w_qkv)
     ops.rope_scatter(qkv, positions, cos, sin, num_heads, num_kv_heads, head_dim, slot_mapping if write else None,
                      k_pages, v_pages, block_size, rotary_dim, interleaved)

@@ -18,7 +18,8 @@ from .spec import WeightSpec
 
 
 class PendingNorm:
-    """rows = norm(x[row_index] + delta[row_index]), not computed yet."""
+    """rows = norm(x[row_index] + delta[row_index]), not computed yet.  ``delta``: rows like x, or the float partial sums
+    [ranges, rows, hidden] of the product that made them, which the norm kernel adds in order."""
 
     def __init__(self, weight: torch.Tensor, eps: float, x: torch.Tensor, delta: torch.Tensor | None = None,
                  row_index: torch.Tensor | None = None, write_residual: bool = True):
@@ -55,7 +56,9 @@ class PendingNorm:
         return self._rows
 
     def fusable(self) -> bool:
-        return self._rows is None
+        """Whether a consumer's kernel may still take the sum and the norm in (not once the rows exist, and not when the
+        sum comes as float partial sums of a product, which only the norm kernel adds)."""
+        return self._rows is None and (self._summed or self.delta is None or self.delta.dim() == 2)
 
     def fused_arguments(self) -> dict:
         """Arguments for a kernel that takes the sum and the norm in; call ``fused_done`` after it."""
@@ -82,6 +85,9 @@ def rows_of(h) -> torch.Tensor:
 
 
 class RMSNorm(Norm):
+    # ``delta`` may be the float partial sums [ranges, rows, hidden] of a product cut along its inner dimension
+    accepts_partial_sums = True
+
     def __init__(self, params: dict, env: BuildEnv):
         self.eps = float(params["eps"])
         self.size = int(params.get("size", env.hidden_size))

@@ -72,6 +72,29 @@ def test_rmsnorm_with_residual_sum_and_row_choice(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [136, 2048, 8200, 99])
+def test_rmsnorm_adds_partial_sums_in_order(dtype, hidden):
+    """The residual's addend as float partial sums [ranges, rows, hidden] of a product cut along its inner dimension:
+    added in order in float, then with x, rounded once (every kernel form: rows in registers, a row per workgroup, and
+    widths that are no multiple of a 16-byte piece)."""
+    x = rnd(21, hidden, seed=7, dtype=dtype)
+    parts = rnd(3 * 21, hidden, seed=8).view(3, 21, hidden).contiguous()
+    w = 1 + 0.3 * rnd(hidden, seed=9)
+    summed = (x.float() + ((parts[0] + parts[1]) + parts[2])).to(dtype)
+    xg = x.cuda().clone()
+    out = ops().rmsnorm(xg, w.cuda(), 1e-5, delta=parts.cuda())
+    assert torch.equal(xg.cpu(), summed)
+    assert rel_err(out, plain.rms_norm(summed.float(), w, 1e-5)) <= TOL[dtype]
+    idx = torch.tensor([20, 0, 5, 5], dtype=torch.int32)
+    xg = x.cuda().clone()
+    out = ops().rmsnorm(xg, w.cuda(), 1e-5, delta=parts.cuda(), row_index=idx.cuda(), write_residual=False)
+    assert torch.equal(xg.cpu(), x)
+    assert rel_err(out, plain.rms_norm(summed.float()[idx.long()], w, 1e-5)) <= TOL[dtype]
+    with pytest.raises(ops().KernelError):
+        ops().rmsnorm(xg, w.cuda(), 1e-5, delta=parts[:, :20].contiguous().cuda())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_silu_mul(dtype):
     inter = 150
     gu = rnd(7, 2 * inter, seed=6, dtype=dtype, scale=2.0)
@@ -722,3 +745,92 @@ def test_decode_linear_rotary_and_cache_write(heads, kv_heads, d, bs, m):
         return qkv[:, :heads * d], kp, vp
     for a, b in zip(run_fused(), run_apart()):
         assert torch.equal(a.cpu(), b.cpu())
+
+
+# ----------------------------------------------------------------------------------- streaming products (17 rows and more)
+STREAM_SHAPES = [(48, 64), (100, 96), (517, 160), (2560, 2048), (2048, 5632), (96, 992), (33, 32)]
+
+
+@pytest.mark.parametrize("m", [1, 17, 33, 64, 100, 128, 200, 264])
+@pytest.mark.parametrize("n,k", STREAM_SHAPES)
+def test_stream_linear_plain_float_and_partial(m, n, k):
+    """Tiled weights, every number of rows (tiles of 32 rows, blocks of up to 128 along y), every blocking of the weight
+    rows that the rows' number allows, widths that are no multiple of the stage of 256 columns, and K cut into ranges."""
+    o = ops()
+    x, w = rnd(m, k, seed=50, dtype=torch.bfloat16), rnd(n, k, seed=51, dtype=torch.bfloat16)
+    tiled = o.tile_weight(w.cuda())
+    assert tiled.blocks % 12 == 0 and tiled.out_features == n
+    want = x.double() @ w.double().T
+    rows_per_block = -(-m // -(-m // 128))
+    for nt in (1, 2, 3, 4):
+        if nt >= 3 and rows_per_block > 64:
+            with pytest.raises(o.KernelError):
+                o.stream_linear(x.cuda(), tiled, o.SL_F32, nt=nt)
+            continue
+        assert rel_err(o.stream_linear(x.cuda(), tiled, o.SL_F32, nt=nt), want) <= 2e-5, nt
+    assert rel_err(o.stream_linear(x.cuda(), tiled, o.SL_BF16), want) <= 1e-2
+    stages = -(-k // 256)
+    for splits in {1, 2, stages} - {0}:
+        if splits > stages or -(-stages // splits) * (splits - 1) >= stages:
+            continue
+        parts = o.stream_linear(x.cuda(), tiled, o.SL_PARTIAL, splits=splits)
+        assert parts.shape == (splits, m, n) and parts.dtype == torch.float32
+        assert rel_err(parts.double().sum(0), want) <= 2e-5, splits
+
+
+def test_stream_linear_does_not_depend_on_the_other_rows():
+    """A row's sums are taken in an order that depends on its place in the matrix only: alone, among 40 or among 200 rows,
+    first or last, the same bits."""
+    o = ops()
+    x, w = rnd(200, 2048, seed=52, dtype=torch.bfloat16), rnd(300, 2048, seed=53, dtype=torch.bfloat16)
+    tiled = o.tile_weight(w.cuda())
+    whole = o.stream_linear(x.cuda(), tiled, o.SL_F32).cpu()
+    for lo, hi in ((0, 40), (150, 200), (77, 78), (0, 17)):
+        assert torch.equal(o.stream_linear(x[lo:hi].contiguous().cuda(), tiled, o.SL_F32).cpu(), whole[lo:hi]), (lo, hi)
+
+
+@pytest.mark.parametrize("m", [17, 41, 64, 128])
+@pytest.mark.parametrize("inter,k", [(176, 64), (250, 96), (5632, 2048)])
+def test_stream_linear_gated(m, inter, k):
+    o = ops()
+    x = rnd(m, k, seed=54, dtype=torch.bfloat16)
+    w = rnd(2 * inter, k, seed=55, dtype=torch.bfloat16, scale=k ** -0.5)
+    want = torch.nn.functional.silu(x.double() @ w[:inter].double().T) * (x.double() @ w[inter:].double().T)
+    tiled = o.tile_weight(w.cuda(), "gated")
+    for nt in (2, 3):
+        if nt == 3 and m > 64:
+            continue
+        assert rel_err(o.stream_linear(x.cuda(), tiled, o.SL_GATED, nt=nt), want) <= 1e-2
+    with pytest.raises(o.KernelError):
+        o.stream_linear(x.cuda(), tiled, o.SL_BF16)              # the rows are not in the plain order
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 32, 16), (32, 4, 64, 16), (3, 1, 96, 32), (8, 8, 128, 16), (5, 1, 48, 16), (2, 2, 16, 8)])
+@pytest.mark.parametrize("m", [17, 47, 64, 130])
+def test_stream_linear_rotary_and_cache_write(heads, kv_heads, d, bs, m):
+    """Against the product, then the rotary kernel: the same bits in q and in the pages (both round the projection to
+    bfloat16 before the rotation)."""
+    from paged_llm_amd.parts.registry import BuildEnv
+    from paged_llm_amd.parts.rope import RotaryEncoding
+    o = ops()
+    k_in, pages = 256, 24
+    rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, torch.bfloat16, torch.device("cuda"), 512, {}))
+    rope.prepare(512)
+    width = (heads + 2 * kv_heads) * d
+    x = rnd(m, k_in, seed=56, dtype=torch.bfloat16)
+    w = rnd(width, k_in, seed=57, dtype=torch.bfloat16, scale=k_in ** -0.5)
+    positions = torch.tensor([(37 * t + 11) % 500 for t in range(m)], dtype=torch.int32)
+    slots = torch.randperm(pages * bs, generator=torch.Generator().manual_seed(58))[:m].to(torch.int32)
+    slots[3] = -1                                                   # a row that writes nothing (padding of a replayed step)
+    tiled = o.tile_weight(w.cuda(), "rotary", head_dim=d)
+    kp = torch.zeros(pages, kv_heads, bs, d, dtype=torch.bfloat16).cuda()
+    vp = torch.zeros(pages, kv_heads, d, bs, dtype=torch.bfloat16).cuda()
+    q = o.stream_linear(x.cuda(), tiled, o.SL_ROPE_KV, rope=dict(
+        positions=positions.cuda(), cos=rope.cos, sin=rope.sin, slots=slots.cuda(), k_pages=kp, v_pages=vp, num_heads=heads,
+        num_kv_heads=kv_heads, head_dim=d, block_size=bs))
+    kp2, vp2 = torch.zeros_like(kp), torch.zeros_like(vp)
+    qkv = o.stream_linear(x.cuda(), o.tile_weight(w.cuda()), o.SL_BF16)
+    assert rel_err(qkv, x.double() @ w.double().T) <= 1e-2
+    o.rope_scatter(qkv, positions.cuda(), rope.cos, rope.sin, heads, kv_heads, d, slots.cuda(), kp2, vp2, bs)
+    assert torch.equal(q.cpu(), qkv[:, :heads * d].cpu()) and torch.equal(kp.cpu(), kp2.cpu()) and torch.equal(vp.cpu(), vp2.cpu())
+    assert kp.float().abs().sum() > 0 and vp.float().abs().sum() > 0

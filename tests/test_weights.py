@@ -45,15 +45,15 @@ def test_loader_fills_the_model_and_keeps_types(tmp_path):
         load_weights(model, d)
         want = torch.bfloat16 if dtype == "bfloat16" else torch.float32
         attn = model.blocks[0].mixer
-        assert attn.w_qkv.dtype == want and attn.w_qkv.shape == ((4 + 2 * 2) * 16, 64)
+        assert attn.w_qkv.dtype == want and tuple(attn.w_qkv.shape) == ((4 + 2 * 2) * 16, 64)
         q = stored["model.layers.0.self_attn.q_proj.weight"]
-        assert torch.equal(attn.w_qkv[:64].float(), q.float())                 # widening is exact
-        assert torch.equal(attn.w_qkv[64:96].float(), stored["model.layers.0.self_attn.k_proj.weight"].float())
+        assert torch.equal(attn.w_qkv.plain[:64].float(), q.float())                 # widening is exact
+        assert torch.equal(attn.w_qkv.plain[64:96].float(), stored["model.layers.0.self_attn.k_proj.weight"].float())
         norm = model.blocks[1].parts["mixer_norm"].weight
         assert norm.dtype == torch.float32                                     # norm weights are applied in float
         assert torch.equal(norm, stored["model.layers.1.input_layernorm.weight"].float())
         ffn = model.blocks[1].parts["feed_forward"]
-        assert torch.equal(ffn.w_gate_up[176:].float(), stored["model.layers.1.mlp.up_proj.weight"].float())
+        assert torch.equal(ffn.w_gate_up.plain[176:].float(), stored["model.layers.1.mlp.up_proj.weight"].float())
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
