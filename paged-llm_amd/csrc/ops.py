@@ -303,7 +303,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
 EPI_BF16, EPI_F32, EPI_GATED, EPI_ROPE_KV = 0, 1, 2, 3
 DECODE_MAX_ROWS = 16          # rows of the fused form with a sum or norm in front
 DECODE_WIDE_MAX_ROWS = 64     # rows of the form for plain rows
-_DECODE_SIG = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
+_DECODE_SIG = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                c_void_p]
 _lds_limit: dict = {}
@@ -359,8 +359,10 @@ def decode_linear_pays(rows: int, N: int, K: int, epi: int, staged: bool) -> boo
 
 def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: torch.Tensor | None = None,
                   norm_weight: torch.Tensor | None = None, eps: float = 0.0, x_out: torch.Tensor | None = None,
-                  row_index: torch.Tensor | None = None, rope: dict | None = None) -> torch.Tensor:
+                  row_index: torch.Tensor | None = None, rope: dict | None = None, tiled=None) -> torch.Tensor:
     """rows = x[row_index] (+ delta) -> optional RMS norm -> rows W^T -> epilogue, in one kernel.
+    ``tiled``: the matrix's ``TiledWeight`` with the pairing that goes with ``epi`` (at most 16 rows): the weights are then
+    streamed from that copy, in contiguous pieces, wherever the kernel works in units of 16 weight rows.
 
     epi EPI_BF16 / EPI_F32: [M, N] out.  EPI_GATED: w = [gate; up], out = silu(gate) * up [M, N/2].
     EPI_ROPE_KV: w = [q; k; v] rows; q is rotated and returned [M, heads * d]; k (rotated) and v go
@@ -386,6 +388,11 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
         _need(row_index.dtype == torch.int32 and row_index.dim() == 1 and row_index.is_contiguous(), "row_index: int32")
     N = w.shape[0]
     r = rope or {}
+    if tiled is not None:
+        _need(M <= DECODE_MAX_ROWS and tiled.in_features == K and tiled.pairing == {EPI_GATED: "gated", EPI_ROPE_KV: "rotary"}.get(epi, "plain")
+              and tiled.out_features * (2 if epi == EPI_GATED else 1) == N and tiled.tiles.is_contiguous()
+              and (epi != EPI_ROPE_KV or tiled.head_dim == r.get("head_dim")),
+              "the tiled copy does not belong to this matrix and epilogue")
     if epi == EPI_GATED:
         _need(N % 2 == 0, "gated product needs [gate; up] rows")
         N //= 2
@@ -408,7 +415,8 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
         out = torch.empty((M, N), dtype=torch.float32 if epi == EPI_F32 else torch.bfloat16, device=x.device)
     f = _fn("decode_linear.hip", "pllm_decode_linear", signature=_DECODE_SIG)
     _check(f(epi, _ptr(x), x.stride(0), _ptr(delta), delta.stride(0) if delta is not None else 0, _ptr(norm_weight), c_float(eps),
-             _ptr(x_out), x_out.stride(0) if x_out is not None else 0, _ptr(row_index), _ptr(w), w.stride(0), _ptr(out),
+             _ptr(x_out), x_out.stride(0) if x_out is not None else 0, _ptr(row_index), _ptr(w), w.stride(0),
+             None if tiled is None else _ptr(tiled.tiles), _ptr(out),
              out.stride(0), M, N, K, _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")),
              _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)),
              int(r.get("head_dim", 0)), int(r.get("block_size", 0)), _stream()), "decode_linear")

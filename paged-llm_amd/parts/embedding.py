@@ -7,7 +7,7 @@ import torch
 
 from ..csrc import ops
 from .base import Part
-from .linear import linear
+from .linear import Weight, linear
 from .registry import BuildEnv, register_embedding, register_head
 from .spec import WeightSpec
 
@@ -38,6 +38,7 @@ class LMHead(Part):
         self.tied = bool(params.get("tied", False))
         self.dtype, self.device = env.dtype, env.device
         self.weight: torch.Tensor | None = None
+        self._matrix = None
 
     def weight_specs(self):
         return {} if self.tied else {"weight": WeightSpec((self.vocab, self.hidden))}
@@ -49,9 +50,15 @@ class LMHead(Part):
 
     def tie(self, table: torch.Tensor) -> None:
         self.weight = table
+        self._matrix = None
+
+    def finalize(self) -> None:
+        self._matrix = None
 
     def forward(self, h) -> torch.Tensor:
-        return linear(h, self.weight, out_dtype=torch.float32)
+        if self._matrix is None:                      # (the tiled copy for decode steps, made once the matrix is there)
+            self._matrix = Weight(self.weight)
+        return linear(h, self._matrix, out_dtype=torch.float32)
 
 
 register_embedding("token_embedding", TokenEmbedding)

@@ -87,18 +87,27 @@ def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: b
     return ops.stream_linear(x, weight.tiled, epi, nt=1 if -(-n // 16) <= 2 * ops._num_compute_units(x.device) else nt, rope=rope)
 
 
-def _fused(x, weight: torch.Tensor, epi: int, rope: dict | None = None):
-    """The fused decode kernel if it takes the operands, else None."""
+_PAIRING_OF = {ops.EPI_GATED: "gated", ops.EPI_ROPE_KV: "rotary"}
+
+
+def _fused(x, weight, epi: int, rope: dict | None = None):
+    """The fused decode kernel if it takes the operands, else None.  With a ``Weight`` whose tiled copy has the pairing
+    of the epilogue, products of at most 16 rows stream the weights from that copy."""
+    tiled = None
+    if isinstance(weight, Weight):
+        if weight.tiled is not None and weight.pairing == _PAIRING_OF.get(epi, "plain"):
+            tiled = weight.tiled
+        weight = weight.plain
     if isinstance(x, PendingNorm):
         if x.fusable() and ops.decode_linear_takes(x.num_rows, x.x.shape[1], x.x, weight):
             args = x.fused_arguments()
-            out = ops.decode_linear(x.x, weight, epi, rope=rope, **args)
+            out = ops.decode_linear(x.x, weight, epi, rope=rope, tiled=tiled, **args)
             x.fused_done(args)
             return out
         x = x.rows()
     if (x.dtype == torch.bfloat16 and ops.decode_linear_takes(x.shape[0], x.shape[1], x, weight, staged=False)
             and ops.decode_linear_pays(x.shape[0], weight.shape[0], x.shape[1], epi, staged=False)):
-        return ops.decode_linear(x, weight, epi, rope=rope)
+        return ops.decode_linear(x, weight, epi, rope=rope, tiled=tiled if x.shape[0] <= ops.DECODE_MAX_ROWS else None)
     return None
 
 
@@ -108,11 +117,11 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
     [ranges, T, N], the sums over ranges of K."""
     if _streams(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16):
         return _stream(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok=partial_ok)
-    weight = _plain(weight)
     if weight.dtype == torch.bfloat16:
         out = _fused(x, weight, ops.EPI_F32 if out_dtype == torch.float32 else ops.EPI_BF16)
         if out is not None:
             return out
+    weight = _plain(weight)
     x = rows_of(x)
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         return ops.gemm_bf16(x, weight, out_dtype)
@@ -123,11 +132,11 @@ def gated_linear(x, w_gate_up) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix (a tensor, or a ``Weight`` with the gated pairing)."""
     if _streams(x, w_gate_up, ops.SL_GATED) and w_gate_up.pairing == "gated":
         return _stream(x, w_gate_up, ops.SL_GATED)
-    w_gate_up = _plain(w_gate_up)
     if w_gate_up.dtype == torch.bfloat16:
         out = _fused(x, w_gate_up, ops.EPI_GATED)
         if out is not None:
             return out
+    w_gate_up = _plain(w_gate_up)
     return ops.silu_mul(linear(x, w_gate_up))
 
 
@@ -153,7 +162,7 @@ def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_h
         if (isinstance(w_qkv, Weight) and w_qkv.pairing == "rotary" and _streams(x, w_qkv, ops.SL_ROPE_KV)
                 and (cos is None or cos.data_ptr() % 16 == 0)):
             return _stream(x, w_qkv, ops.SL_ROPE_KV, rope=rope)
-        q = _fused(x, _plain(w_qkv), ops.EPI_ROPE_KV, rope)
+        q = _fused(x, w_qkv, ops.EPI_ROPE_KV, rope)
         if q is not None:
             return q
     w_qkv = _plain(w_qkv)

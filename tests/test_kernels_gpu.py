@@ -834,3 +834,55 @@ def test_stream_linear_rotary_and_cache_write(heads, kv_heads, d, bs, m):
     o.rope_scatter(qkv, positions.cuda(), rope.cos, rope.sin, heads, kv_heads, d, slots.cuda(), kp2, vp2, bs)
     assert torch.equal(q.cpu(), qkv[:, :heads * d].cpu()) and torch.equal(kp.cpu(), kp2.cpu()) and torch.equal(vp.cpu(), vp2.cpu())
     assert kp.float().abs().sum() > 0 and vp.float().abs().sum() > 0
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 13, 16])
+@pytest.mark.parametrize("n,k", [(48, 64), (517, 160), (2560, 2048), (2048, 5632), (96, 992)])
+def test_decode_linear_streams_the_tiled_copy(m, n, k):
+    """At most 16 rows with the weights from their tiled copy: plain and float out, with the sum and norm in front, and
+    gated; the same sums in the same order as from the row-major matrix wherever that one is read in units of 16 rows too."""
+    o = ops()
+    x, w = rnd(m, k, seed=60, dtype=torch.bfloat16), rnd(n, k, seed=61, dtype=torch.bfloat16, scale=k ** -0.5)
+    tiled = o.tile_weight(w.cuda())
+    want = x.double() @ w.double().T
+    got = o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32, tiled=tiled)
+    assert rel_err(got, want) <= 2e-5
+    if m > 8:
+        assert torch.equal(got.cpu(), o.decode_linear(x.cuda(), w.cuda(), o.EPI_F32).cpu())
+    d, nw = rnd(m, k, seed=62, dtype=torch.bfloat16), 1 + 0.3 * rnd(k, seed=63)
+    h = plain.rms_norm((x.float() + d.float()).to(torch.bfloat16).float(), nw, 1e-4).to(torch.bfloat16)
+    if o.decode_linear_takes(m, k, x.cuda(), w.cuda()):                  # (the rows fit LDS)
+        x_out = torch.zeros(m, k, dtype=torch.bfloat16).cuda()
+        got = o.decode_linear(x.cuda(), w.cuda(), o.EPI_BF16, delta=d.cuda(), norm_weight=nw.cuda(), eps=1e-4, x_out=x_out, tiled=tiled)
+        assert rel_err(got, h.double() @ w.double().T) <= 1.5e-2
+    if n % 2 == 0:
+        half = n // 2
+        want = torch.nn.functional.silu(x.double() @ w[:half].double().T) * (x.double() @ w[half:].double().T)
+        assert rel_err(o.decode_linear(x.cuda(), w.cuda(), o.EPI_GATED, tiled=o.tile_weight(w.cuda(), "gated")), want) <= 1e-2
+        with pytest.raises(o.KernelError):
+            o.decode_linear(x.cuda(), w.cuda(), o.EPI_GATED, tiled=tiled)      # the plain pairing does not go with the gated epilogue
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(4, 2, 32, 16), (32, 4, 64, 16), (5, 1, 48, 16), (2, 2, 16, 8)])
+@pytest.mark.parametrize("m", [1, 8, 16])
+def test_decode_linear_rotary_from_the_tiled_copy(heads, kv_heads, d, bs, m):
+    from paged_llm_amd.parts.registry import BuildEnv
+    from paged_llm_amd.parts.rope import RotaryEncoding
+    o = ops()
+    k_in, pages = 256, 12
+    rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, torch.bfloat16, torch.device("cuda"), 512, {}))
+    rope.prepare(512)
+    width = (heads + 2 * kv_heads) * d
+    x = rnd(m, k_in, seed=64, dtype=torch.bfloat16)
+    w = rnd(width, k_in, seed=65, dtype=torch.bfloat16, scale=k_in ** -0.5)
+    positions = torch.tensor([(37 * t + 11) % 500 for t in range(m)], dtype=torch.int32)
+    slots = torch.randperm(pages * bs, generator=torch.Generator().manual_seed(66))[:m].to(torch.int32)
+    def run(tiled):
+        kp = torch.zeros(pages, kv_heads, bs, d, dtype=torch.bfloat16).cuda()
+        vp = torch.zeros(pages, kv_heads, d, bs, dtype=torch.bfloat16).cuda()
+        q = o.decode_linear(x.cuda(), w.cuda(), o.EPI_ROPE_KV, tiled=tiled, rope=dict(
+            positions=positions.cuda(), cos=rope.cos, sin=rope.sin, slots=slots.cuda(), k_pages=kp, v_pages=vp, num_heads=heads,
+            num_kv_heads=kv_heads, head_dim=d, block_size=bs))
+        return q.cpu().float(), kp.cpu().float(), vp.cpu().float()
+    for a, b in zip(run(o.tile_weight(w.cuda(), "rotary", head_dim=d)), run(None)):
+        assert (a - b).abs().max().item() <= 2e-2 * max(1.0, b.abs().max().item()) and b.abs().sum() > 0
