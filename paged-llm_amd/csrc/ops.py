@@ -433,7 +433,7 @@ _STREAM_SIG = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, 
 class TiledWeight:
     """A weight matrix [N, K] in the order the streaming product kernel reads it: blocks of 16 rows, each block's tiles of
     16 rows x 32 columns one after the other along K, a tile being 1 KB in the order of the matrix instruction's operand
-    (lane g * 16 + r: row r, columns 8 g .. 8 g + 7); zero rows pad the blocks to a multiple of twelve.  ``pairing`` says
+    (lane g * 16 + r: row r, columns 8 g .. 8 g + 7); zero rows pad the blocks to a multiple of 24.  ``pairing`` says
     which rows share a block: "plain" (16 successive rows), "gated" (8 gate rows and the up rows of the same outputs), or
     "rotary" (8 elements of the lower half of a head and their partners in the upper half, ``head_dim`` apart by half)."""
 
@@ -471,7 +471,7 @@ def tile_weight(w: torch.Tensor, pairing: str = "plain", head_dim: int = 0) -> T
     else:
         _need(pairing == "plain", f"unknown pairing {pairing!r}")
     blocks = -(-w.shape[0] // 16)
-    blocks_padded = -(-blocks // 12) * 12                                 # (whole workgroups of 1, 2, 3 or 4 blocks)
+    blocks_padded = -(-blocks // 24) * 24                                 # (whole workgroups of 1, 2, 3, 4 or 8 blocks)
     if blocks_padded * 16 != w.shape[0]:
         w = torch.cat([w, torch.zeros((blocks_padded * 16 - w.shape[0], K), dtype=w.dtype, device=w.device)])
     tiles = w.view(blocks_padded, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()       # [block, k step, g, r, 8]
@@ -503,7 +503,7 @@ def stream_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, nt: int |
     M, K = x.shape
     _need(x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0,
           "stream_linear: bfloat16 rows that start on 16-byte boundaries")
-    _need(K == w.in_features and w.tiles.is_contiguous() and tuple(w.tiles.shape[1:]) == (K // 32, 4, 16, 8) and w.blocks % 12 == 0,
+    _need(K == w.in_features and w.tiles.is_contiguous() and tuple(w.tiles.shape[1:]) == (K // 32, 4, 16, 8) and w.blocks % 24 == 0,
           f"stream_linear: rows of {K} values against tiled weights of {w.in_features}")
     _need({SL_GATED: "gated", SL_ROPE_KV: "rotary"}.get(epi, "plain") == w.pairing,
           f"epilogue {epi} against weights tiled with the {w.pairing} pairing")
@@ -537,6 +537,63 @@ def stream_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, nt: int |
              _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")), _ptr(r.get("k_pages")),
              _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)), int(r.get("head_dim", 0)),
              int(r.get("block_size", 0)), _stream()), "stream_linear")
+    return out
+
+
+_TILE_SIG = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+             c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+
+
+def tile_linear_plan(M: int, N: int, K: int, compute_units: int) -> int:
+    """Ranges of K for the tiled product of M rows with N weight rows: as many as give every compute unit a workgroup
+    (tiles of up to 128 rows x 128 weight rows), each at least four stages of 64 columns long."""
+    workgroups = -(-N // 128) * -(-M // 128)
+    stages = -(-K // 64)
+    if workgroups >= compute_units:
+        return 1
+    return max(1, min(compute_units // workgroups, stages // 4, 16))
+
+
+def tile_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, splits: int | None = None, rope: dict | None = None) -> torch.Tensor:
+    """As ``stream_linear``, for a few hundred rows: tiles of up to 128 rows x 128 weight rows per workgroup, both
+    operands through LDS."""
+    _on_gpu(x, w.tiles)
+    M, K = x.shape
+    _need(x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0,
+          "tile_linear: bfloat16 rows that start on 16-byte boundaries")
+    _need(K == w.in_features and w.tiles.is_contiguous() and tuple(w.tiles.shape[1:]) == (K // 32, 4, 16, 8) and w.blocks % 24 == 0,
+          f"tile_linear: rows of {K} values against tiled weights of {w.in_features}")
+    _need({SL_GATED: "gated", SL_ROPE_KV: "rotary"}.get(epi, "plain") == w.pairing,
+          f"epilogue {epi} against weights tiled with the {w.pairing} pairing")
+    N = w.out_features
+    if splits is None:
+        splits = tile_linear_plan(M, N * (2 if epi == SL_GATED else 1), K, _num_compute_units(x.device)) if epi == SL_PARTIAL else 1
+    _need(splits == 1 or epi == SL_PARTIAL, "ranges of K give partial sums")
+    r = rope or {}
+    if epi == SL_PARTIAL:
+        out = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+    elif epi == SL_ROPE_KV:
+        nh, nkv, d, bs = r["num_heads"], r["num_kv_heads"], r["head_dim"], r["block_size"]
+        _need(d == w.head_dim and N == (nh + 2 * nkv) * d, "the weights were tiled for other heads")
+        kp, vp = r["k_pages"], r["v_pages"]
+        P = kp.shape[0]
+        _need(tuple(kp.shape) == (P, nkv, bs, d) and tuple(vp.shape) == (P, nkv, d, bs) and kp.is_contiguous() and vp.is_contiguous()
+              and kp.dtype == torch.bfloat16 and vp.dtype == torch.bfloat16, "bad cache pages")
+        for name in ("positions", "slots"):
+            t = r[name]
+            _need(t.dtype == torch.int32 and t.shape == (M,) and t.is_contiguous(), f"{name}: int32 [{M}]")
+        if r.get("cos") is not None:
+            for t in (r["cos"], r["sin"]):
+                _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == d // 2 and t.is_contiguous() and t.data_ptr() % 16 == 0,
+                      "rotary tables")
+        out = torch.empty((M, nh * d), dtype=torch.bfloat16, device=x.device)
+    else:
+        out = torch.empty((M, N), dtype=torch.float32 if epi == SL_F32 else torch.bfloat16, device=x.device)
+    f = _fn("stream_linear.hip", "pllm_tile_linear", signature=_TILE_SIG)
+    _check(f(epi, _ptr(x), x.stride(0), _ptr(w.tiles), _ptr(out), out.stride(-2), M, N, K, w.blocks, splits,
+             _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")), _ptr(r.get("k_pages")),
+             _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)), int(r.get("head_dim", 0)),
+             int(r.get("block_size", 0)), _stream()), "tile_linear")
     return out
 
 

@@ -290,14 +290,14 @@ static int launch_stream(const StreamLinearParams& p, dim3 grid, hipStream_t str
 // Rows of a workgroup along y: as few blocks as 128 rows each allow, evenly filled, in tiles of 32 rows.
 PLLM_API int pllm_stream_linear_row_blocks(int M) { return (M + 127) / 128; }
 
-// nt: blocks of 16 weight rows per workgroup (1 to 4); the tiled weights hold a multiple of 12 blocks (zero rows at the end).
+// nt: blocks of 16 weight rows per workgroup (1 to 4); the tiled weights hold a multiple of 24 blocks (zero rows at the end).
 // splits > 1 with epi SL_PARTIAL only.
 PLLM_API int pllm_stream_linear(int epi, const void* x, int ldx, const void* wt, void* out, int ldo, int M, int N, int K,
                                 int weight_blocks, int nt, int splits, const int* positions, const float* cos_t, const float* sin_t,
                                 const int* slots, void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim,
                                 int block_size, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || (K % kChunkK) || (ldx & 7) || nt < 1 || nt > 4 || weight_blocks <= 0 || (weight_blocks % 12) || splits < 1) return -2;
+  if (K <= 0 || (K % kChunkK) || (ldx & 7) || nt < 1 || nt > 4 || weight_blocks <= 0 || (weight_blocks % 24) || splits < 1) return -2;
   if (splits > 1 && epi != SL_PARTIAL) return -2;
   if (epi == SL_ROPE_KV && (head_dim <= 0 || (head_dim % 16) || !slots || !k_pages || !v_pages || !positions ||
                             N != (num_heads + 2 * num_kv_heads) * head_dim || block_size <= 0 || (ldo & 3))) return -2;
@@ -355,5 +355,261 @@ PLLM_API int pllm_stream_linear(int epi, const void* x, int ldx, const void* wt,
   }
 #undef PLLM_SL_SHAPES
 #undef PLLM_SL
+  return -3;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same products for a few hundred rows (steps that hold a prompt portion, short prompts): tiles of up to 128 input
+// rows x 128 weight rows per workgroup, along x the blocks of weight rows, along y the blocks of input rows, along z
+// ranges of K.  With this many rows every workgroup of the kernel above would read all of them for its 32 weight rows;
+// here both operands of a stage (64 columns of K) come into LDS once per workgroup, brought by the four loader
+// wavefronts (the weights' tiles are 1 KB of contiguous memory each and land in operand order; the rows as above), and
+// the eight compute wavefronts, as 2 x 4 over the tile (MTW tiles of 16 input rows x 2 blocks of 16 weight rows each),
+// only read LDS and multiply.  No sums across wavefronts: each owns its outputs.  Epilogues as above.
+constexpr int kTileBlocksN = 8;                      // blocks of 16 weight rows per workgroup
+constexpr int kTileStageSteps = 2;                   // steps of 32 columns per stage
+
+template <int EPI, int MTW, int R>
+__global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const StreamLinearParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char sl_lds[];
+  constexpr int MT = 2 * MTW;                                    // tiles of 16 input rows per workgroup
+  constexpr int kWBlocks = kTileBlocksN * kTileStageSteps, kXBlocks = MT * kTileStageSteps;
+  constexpr int kSlotBytes = (kWBlocks + kXBlocks) * 1024;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nb = blockIdx.x, row0 = blockIdx.y * (MT * 16), split = blockIdx.z;
+  const int first_stage = split * p.stages_per_split;           // (stages of 64 columns here)
+  const int nstages = min(p.stages_per_split, p.num_stages - first_stage);
+  floatx4 acc[MTW][2];
+
+  if (wave >= kComputeWaves) {
+    const int l = wave - kComputeWaves;
+    const int xr = lane >> 2, xg = (lane & 3) ^ (xr >> 2);
+    constexpr int kBlocks = kWBlocks + kXBlocks, kPerLoader = (kBlocks + kLoaderWaves - 1) / kLoaderWaves;
+    auto issue = [&](int s) {
+      const int ks0 = (first_stage + s) * kTileStageSteps;
+      unsigned char* slot = sl_lds + (s % R) * kSlotBytes;
+#pragma unroll
+      for (int i = 0; i < kPerLoader; ++i) {
+        const int b = l + i * kLoaderWaves;
+        // Every loader issues the same number of loads per stage (the waits below count them): a loader whose share of
+        // the blocks is one short repeats its last block.
+        const int bb = min(b, kBlocks - 1);
+        const bf16* src;
+        if (bb < kWBlocks) {
+          const int u = bb / kTileStageSteps, st = bb - u * kTileStageSteps;
+          const int ks = min(ks0 + st, p.ksteps - 1);
+          src = p.wt + (((size_t)(nb * kTileBlocksN + u) * p.ksteps + ks) * 64 + lane) * 8;
+        } else {
+          const int bx = bb - kWBlocks, t = bx / kTileStageSteps, st = bx - t * kTileStageSteps;
+          const int row = min(row0 + t * 16 + xr, p.M - 1);
+          const int k = min((ks0 + st) * kChunkK + xg * 8, p.K - 8);
+          src = p.x + (size_t)row * p.ldx + k;
+        }
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)(slot + bb * 1024), 16, 0, 0);
+      }
+    };
+#pragma unroll
+    for (int s = 0; s < R - 1; ++s) {
+      if (s < nstages) issue(s);
+    }
+    for (int s = 0; s < nstages; ++s) {
+      // stage s has landed when at most the loads of the R - 2 stages behind it are under way (fewer near the end)
+      const int behind = min(R - 2, nstages - 1 - s);
+      if (behind >= 2) wait_loads_but<2 * kPerLoader>();
+      else if (behind == 1) wait_loads_but<kPerLoader>();
+      else wait_loads_but<0>();
+      stage_barrier();
+      if (s + R - 1 < nstages) issue(s + R - 1);
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < MTW; ++t) {
+      acc[t][0] = floatx4{0.f, 0.f, 0.f, 0.f};
+      acc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int wm = wave >> 2, wn = wave & 3;
+    const int r = lane & 15, g = lane >> 4;
+    const unsigned char* my_w = sl_lds + (wn * 2 * kTileStageSteps) * 1024 + lane * 16;
+    const unsigned char* my_x = sl_lds + (kWBlocks + wm * MTW * kTileStageSteps) * 1024 + (r * 4 + (g ^ (r >> 2))) * 16;
+    int slot = 0;
+    for (int s = 0; s < nstages; ++s) {
+      stage_barrier();
+      const int steps = min(kTileStageSteps, p.ksteps - (first_stage + s) * kTileStageSteps);
+      bf16x8 wf[kTileStageSteps][2], xf[kTileStageSteps][MTW];
+#pragma unroll
+      for (int st = 0; st < kTileStageSteps; ++st) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) wf[st][u] = *reinterpret_cast<const bf16x8*>(my_w + slot * kSlotBytes + (u * kTileStageSteps + st) * 1024);
+#pragma unroll
+        for (int t = 0; t < MTW; ++t) xf[st][t] = *reinterpret_cast<const bf16x8*>(my_x + slot * kSlotBytes + (t * kTileStageSteps + st) * 1024);
+      }
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int st = 0; st < kTileStageSteps; ++st) {
+        if (st < steps) {
+#pragma unroll
+          for (int t = 0; t < MTW; ++t) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[st][u], xf[st][t], acc[t][u], 0, 0, 0);
+          }
+        }
+      }
+      slot = slot + 1 == R ? 0 : slot + 1;
+    }
+
+    // ---- epilogue: a lane's four sums are four weight rows (4 g .. 4 g + 3 of the tile) of input row r
+    constexpr bool kPaired = EPI == SL_GATED || EPI == SL_ROPE_KV;
+#pragma unroll
+    for (int t = 0; t < MTW; ++t) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int m = row0 + (wm * MTW + t) * 16 + r;
+        const int unit = nb * kTileBlocksN + wn * 2 + u;
+        const floatx4 a = acc[t][u];
+        floatx4 partner = a;
+        if (kPaired) {                                           // tile rows 8-15 (the lanes 32 further on) hold the partners of rows 0-7
+#pragma unroll
+          for (int i = 0; i < 4; ++i) partner[i] = __shfl_down(a[i], 32, 64);
+        }
+        if (m >= p.M || (kPaired && g >= 2)) continue;
+        if (EPI == SL_GATED) {
+          const int n = unit * 8 + g * 4;
+          bf16 o[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[i] = __float2bfloat16((a[i] / (1.f + expf(-a[i]))) * partner[i]);
+          bf16* dst = (bf16*)p.out + (size_t)m * p.ldo + n;
+          if (n + 3 < p.N && (p.ldo & 3) == 0) *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(o);
+          else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) if (n + i < p.N) dst[i] = o[i];
+          }
+        } else if (EPI == SL_ROPE_KV) {
+          const int d = p.head_dim, half = d >> 1, per_head = half >> 3;
+          const int head = unit / per_head, ri = (unit - head * per_head) * 8 + g * 4;
+          const int nh = p.num_heads, nkv = p.num_kv_heads;
+          if (head >= nh + 2 * nkv) continue;
+          if (head < nh + nkv) {
+            floatx4 cs = {1.f, 1.f, 1.f, 1.f}, sn = {0.f, 0.f, 0.f, 0.f};
+            if (p.cos_t) {
+              const size_t at = (size_t)p.positions[m] * half + ri;
+              cs = *reinterpret_cast<const floatx4*>(p.cos_t + at);
+              sn = *reinterpret_cast<const floatx4*>(p.sin_t + at);
+            }
+            bf16 lo_out[4], hi_out[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float lo = __bfloat162float(__float2bfloat16(a[i])), up = __bfloat162float(__float2bfloat16(partner[i]));
+              float rl, ru;
+              rotate_pair(lo, up, cs[i], sn[i], rl, ru);
+              lo_out[i] = __float2bfloat16(rl);
+              hi_out[i] = __float2bfloat16(ru);
+            }
+            bf16* dst = nullptr;
+            if (head < nh) dst = (bf16*)p.out + (size_t)m * p.ldo + (size_t)head * d + ri;
+            else {
+              const int slot_kv = p.slots[m];
+              if (slot_kv >= 0) {
+                const int page = slot_kv / p.block_size, off = slot_kv - page * p.block_size;
+                dst = p.k_pages + (((size_t)page * nkv + (head - nh)) * p.block_size + off) * d + ri;
+              }
+            }
+            if (dst) {
+              *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(lo_out);
+              *reinterpret_cast<uint2*>(dst + half) = *reinterpret_cast<const uint2*>(hi_out);
+            }
+          } else {
+            const int slot_kv = p.slots[m];
+            if (slot_kv >= 0) {
+              const int page = slot_kv / p.block_size, off = slot_kv - page * p.block_size;
+              bf16* vdst = p.v_pages + ((size_t)page * nkv + (head - nh - nkv)) * d * p.block_size + off;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                vdst[(size_t)(ri + i) * p.block_size] = __float2bfloat16(a[i]);
+                vdst[(size_t)(ri + half + i) * p.block_size] = __float2bfloat16(partner[i]);
+              }
+            }
+          }
+        } else {
+          const int n = unit * 16 + g * 4;
+          if (EPI == SL_BF16) {
+            bf16 o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] = __float2bfloat16(a[i]);
+            bf16* dst = (bf16*)p.out + (size_t)m * p.ldo + n;
+            if (n + 3 < p.N && (p.ldo & 3) == 0) *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(o);
+            else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) if (n + i < p.N) dst[i] = o[i];
+            }
+          } else {
+            float* dst = (float*)p.out + ((size_t)(EPI == SL_PARTIAL ? split : 0) * p.M + m) * p.ldo + n;
+            if (n + 3 < p.N && (p.ldo & 3) == 0) *reinterpret_cast<floatx4*>(dst) = a;
+            else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) if (n + i < p.N) dst[i] = a[i];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int EPI, int MTW, int R>
+static int launch_tile(const StreamLinearParams& p, dim3 grid, hipStream_t stream) {
+  constexpr size_t lds = (size_t)R * (kTileBlocksN * kTileStageSteps + 2 * MTW * kTileStageSteps) * 1024;
+  static_assert(lds <= 160 * 1024, "LDS of one compute unit");
+  auto kernel = tile_linear_kernel<EPI, MTW, R>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(kStreamThreads), lds, stream, p);
+  return (int)hipGetLastError();
+}
+
+// The tiled weights hold a multiple of 8 blocks (of 24, in fact).  splits > 1 with epi SL_PARTIAL only.
+PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, void* out, int ldo, int M, int N, int K,
+                              int weight_blocks, int splits, const int* positions, const float* cos_t, const float* sin_t,
+                              const int* slots, void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim,
+                              int block_size, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || (K % kChunkK) || (ldx & 7) || weight_blocks <= 0 || (weight_blocks % kTileBlocksN) || splits < 1) return -2;
+  if (splits > 1 && epi != SL_PARTIAL) return -2;
+  if (epi == SL_ROPE_KV && (head_dim <= 0 || (head_dim % 16) || !slots || !k_pages || !v_pages || !positions ||
+                            N != (num_heads + 2 * num_kv_heads) * head_dim || block_size <= 0 || (ldo & 3))) return -2;
+  const int rows_of_w = epi == SL_GATED ? 2 * N : N;
+  if ((long)weight_blocks * 16 < rows_of_w) return -2;
+  StreamLinearParams p;
+  p.x = (const bf16*)x; p.ldx = ldx; p.wt = (const bf16*)wt; p.out = out; p.ldo = ldo; p.M = M; p.N = N; p.K = K;
+  p.positions = positions; p.cos_t = cos_t; p.sin_t = sin_t; p.slots = slots; p.k_pages = (bf16*)k_pages; p.v_pages = (bf16*)v_pages;
+  p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.head_dim = head_dim; p.block_size = block_size;
+  p.ksteps = K / kChunkK;
+  p.num_stages = (p.ksteps + kTileStageSteps - 1) / kTileStageSteps;
+  p.stages_per_split = (p.num_stages + splits - 1) / splits;
+  if ((long)p.stages_per_split * (splits - 1) >= p.num_stages) return -2;
+  const int m_blocks = pllm_stream_linear_row_blocks(M);
+  const int rows = (M + m_blocks - 1) / m_blocks, mtw = (rows + 31) / 32;       // tiles of 16 rows per wavefront: 1 to 4
+  const int n_blocks = ((rows_of_w + 15) / 16 + kTileBlocksN - 1) / kTileBlocksN;
+  if (m_blocks > 65535 || splits > 65535) return -2;
+  const dim3 grid(n_blocks, m_blocks, splits);
+#define PLLM_TL_SHAPES(EPI_)                                                  \
+  do {                                                                        \
+    switch (mtw) {                                                            \
+      case 1: return launch_tile<EPI_, 1, 4>(p, grid, stream);                \
+      case 2: return launch_tile<EPI_, 2, 4>(p, grid, stream);                \
+      case 3: return launch_tile<EPI_, 3, 4>(p, grid, stream);                \
+      case 4: return launch_tile<EPI_, 4, 4>(p, grid, stream);                \
+    }                                                                         \
+  } while (0)
+  switch (epi) {
+    case SL_BF16: PLLM_TL_SHAPES(SL_BF16); break;
+    case SL_F32: PLLM_TL_SHAPES(SL_F32); break;
+    case SL_GATED: PLLM_TL_SHAPES(SL_GATED); break;
+    case SL_PARTIAL: PLLM_TL_SHAPES(SL_PARTIAL); break;
+    case SL_ROPE_KV: PLLM_TL_SHAPES(SL_ROPE_KV); break;
+  }
+#undef PLLM_TL_SHAPES
   return -3;
 }

@@ -759,7 +759,7 @@ def test_stream_linear_plain_float_and_partial(m, n, k):
     o = ops()
     x, w = rnd(m, k, seed=50, dtype=torch.bfloat16), rnd(n, k, seed=51, dtype=torch.bfloat16)
     tiled = o.tile_weight(w.cuda())
-    assert tiled.blocks % 12 == 0 and tiled.out_features == n
+    assert tiled.blocks % 24 == 0 and tiled.out_features == n
     want = x.double() @ w.double().T
     rows_per_block = -(-m // -(-m // 128))
     for nt in (1, 2, 3, 4):
@@ -886,3 +886,53 @@ def test_decode_linear_rotary_from_the_tiled_copy(heads, kv_heads, d, bs, m):
         return q.cpu().float(), kp.cpu().float(), vp.cpu().float()
     for a, b in zip(run(o.tile_weight(w.cuda(), "rotary", head_dim=d)), run(None)):
         assert (a - b).abs().max().item() <= 2e-2 * max(1.0, b.abs().max().item()) and b.abs().sum() > 0
+
+
+@pytest.mark.parametrize("m", [17, 100, 129, 264, 300, 512, 640])
+@pytest.mark.parametrize("n,k", STREAM_SHAPES)
+def test_tile_linear_plain_float_and_partial(m, n, k):
+    """Tiles of up to 128 rows x 128 weight rows with both operands through LDS: every number of rows, widths that are no
+    multiple of a stage of 64 columns, fewer weight rows than a tile, and K cut into ranges."""
+    o = ops()
+    x, w = rnd(m, k, seed=70, dtype=torch.bfloat16), rnd(n, k, seed=71, dtype=torch.bfloat16)
+    tiled = o.tile_weight(w.cuda())
+    want = x.double() @ w.double().T
+    assert rel_err(o.tile_linear(x.cuda(), tiled, o.SL_F32), want) <= 2e-5
+    assert rel_err(o.tile_linear(x.cuda(), tiled, o.SL_BF16), want) <= 1e-2
+    stages = -(-k // 64)
+    for splits in {2, 3, stages}:
+        if splits > stages or -(-stages // splits) * (splits - 1) >= stages:
+            continue
+        parts = o.tile_linear(x.cuda(), tiled, o.SL_PARTIAL, splits=splits)
+        assert parts.shape == (splits, m, n) and rel_err(parts.double().sum(0), want) <= 2e-5, splits
+    alone = o.tile_linear(x[m // 2:m // 2 + 5].contiguous().cuda(), tiled, o.SL_F32)
+    assert torch.equal(alone.cpu(), o.tile_linear(x.cuda(), tiled, o.SL_F32)[m // 2:m // 2 + 5].cpu())     # a row's sums do not depend on the others
+
+
+@pytest.mark.parametrize("m", [130, 264])
+def test_tile_linear_gated_and_rotary(m):
+    from paged_llm_amd.parts.registry import BuildEnv
+    from paged_llm_amd.parts.rope import RotaryEncoding
+    o = ops()
+    inter, k = 250, 96
+    x = rnd(m, k, seed=72, dtype=torch.bfloat16)
+    w = rnd(2 * inter, k, seed=73, dtype=torch.bfloat16, scale=k ** -0.5)
+    want = torch.nn.functional.silu(x.double() @ w[:inter].double().T) * (x.double() @ w[inter:].double().T)
+    assert rel_err(o.tile_linear(x.cuda(), o.tile_weight(w.cuda(), "gated"), o.SL_GATED), want) <= 1e-2
+    heads, kv_heads, d, bs, pages, k_in = 5, 1, 48, 16, 24, 256
+    rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, torch.bfloat16, torch.device("cuda"), 512, {}))
+    rope.prepare(512)
+    x = rnd(m, k_in, seed=74, dtype=torch.bfloat16)
+    w = rnd((heads + 2 * kv_heads) * d, k_in, seed=75, dtype=torch.bfloat16, scale=k_in ** -0.5)
+    positions = torch.tensor([(37 * t + 11) % 500 for t in range(m)], dtype=torch.int32)
+    slots = torch.randperm(pages * bs, generator=torch.Generator().manual_seed(76))[:m].to(torch.int32)
+    kp = torch.zeros(pages, kv_heads, bs, d, dtype=torch.bfloat16).cuda()
+    vp = torch.zeros(pages, kv_heads, d, bs, dtype=torch.bfloat16).cuda()
+    q = o.tile_linear(x.cuda(), o.tile_weight(w.cuda(), "rotary", head_dim=d), o.SL_ROPE_KV, rope=dict(
+        positions=positions.cuda(), cos=rope.cos, sin=rope.sin, slots=slots.cuda(), k_pages=kp, v_pages=vp, num_heads=heads,
+        num_kv_heads=kv_heads, head_dim=d, block_size=bs))
+    kp2, vp2 = torch.zeros_like(kp), torch.zeros_like(vp)
+    qkv = o.tile_linear(x.cuda(), o.tile_weight(w.cuda()), o.SL_BF16)
+    o.rope_scatter(qkv, positions.cuda(), rope.cos, rope.sin, heads, kv_heads, d, slots.cuda(), kp2, vp2, bs)
+    assert torch.equal(q.cpu(), qkv[:, :heads * d].cpu()) and torch.equal(kp.cpu(), kp2.cpu()) and torch.equal(vp.cpu(), vp2.cpu())
+    assert kp.float().abs().sum() > 0
