@@ -527,8 +527,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (reported as such)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
-    ap.add_argument("--prefill-only", action="store_true", help="time only the 2048-token prefill (for profiling)")
-    ap.add_argument("--mixed-only", action="store_true", help="time only the step of --batch decoded tokens beside a 256-token portion (for profiling)")
+    ap.add_argument("--prefill-only", action="store_true", help="times one step that computes a prompt of 2048 tokens, and nothing else")
+    ap.add_argument("--mixed-only", action="store_true", help="times one step of --batch decoded tokens beside a prompt portion of 256 tokens, and nothing else")
     ap.add_argument("--attention", action="store_true", help="the reference's attention micro-benchmark cases instead")
     ap.add_argument("--e2e", action="store_true", help="the reference's end-to-end workload (64 requests, 256 in / 128 out) instead: "
                     "its published cases, or one case given by the options below (names as in the reference's benchmarks/bench.py)")
@@ -640,8 +640,27 @@ def main() -> int:
             flops = prefill_flops(cfg, PREFILL_TOKENS, 1)
             record["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3),
                                  "frac": round(flops / psec / PEAK_FLOPS[short], 4)}
+            # short prompts, one step each (replayed from graphs; what they cost is the products of a few hundred rows)
+            for n in (128, 512):
+                t = time_prefill(engine, n, seed=400 + n, repeats=5)
+                points[f"prefill_{n}_ms"] = round(t * 1e3, 3)
+                points[f"prefill_{n}_frac"] = round(prefill_flops(cfg, n, 1) / t / PEAK_FLOPS[short], 4)
             del engine
             torch.cuda.empty_cache()
+            # longer contexts at the headline batch, each with its own fraction of the memory roofline, and a long prompt
+            for context in (8192, 32768):
+                with tempfile.TemporaryDirectory() as long_folder:
+                    long_engine = make_engine(cfg, long_folder, args.dtype, max(args.batch, 4), context)
+                    s, mean_ctx = time_decode(long_engine, args.batch, context, 16, 4, seed=60)
+                    nbytes_step = numbers["weight_bytes"] + args.batch * mean_ctx * numbers["kv_bytes_per_token"]
+                    points[f"decode_b{args.batch}_ctx{context}"] = round(args.batch / s, 1)
+                    points[f"decode_b{args.batch}_ctx{context}_frac"] = round(nbytes_step / s / 1e9 / PEAK_HBM_GBS, 4)
+                    if context == 8192:
+                        t = time_prefill(long_engine, 8192, seed=500, repeats=2)
+                        points["prefill_8192"] = round(8192 / t, 1)
+                        points["prefill_8192_frac"] = round(prefill_flops(cfg, 8192, 1) / t / PEAK_FLOPS[short], 4)
+                    del long_engine
+                    torch.cuda.empty_cache()
             # the reference's end-to-end workload at 8 and 64 requests at a time (64 requests, 256 in / 128 out): output tokens/s
             e2e = run_e2e(cfg, args.dtype, [c for c in E2E_CASES if c["name"] in ("256in_128out_b8", "256in_128out_b64")])
             record["e2e"] = {name: row["output_tok_per_s"] for name, row in e2e.items()}

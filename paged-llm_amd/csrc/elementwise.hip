@@ -117,18 +117,22 @@ __global__ void rmsnorm_kernel(const T* x, const T* __restrict__ delta, const in
   }
 }
 
-// The same for rows of at most 64 * P pieces of 16 bytes: one wavefront per row keeps the row in registers
-// (P pieces per lane), so there is no LDS and no barrier, and a workgroup of four wavefronts does four rows.
-// The sum of squares is taken per lane over its pieces in order, then over the wavefront.
-template <typename T, int P>
+// The same for rows of at most 64 * WPR * P pieces of 16 bytes: WPR wavefronts per row keep the row in registers
+// (P pieces per lane).  WPR = 1: no LDS and no barrier, a workgroup of four wavefronts does four rows (many rows:
+// prompts).  WPR = 4: a workgroup per row, the wavefronts' sums of squares added through LDS in wavefront order (a
+// few dozen to a few hundred rows: with one wavefront per row such a step would keep a handful of compute units busy,
+// each walking a whole row and its addends: 4.9 us for 64 rows of 2048, 8.5 us for 128 rows with four ranges of
+// partial sums).  The sum of squares is taken per lane over its pieces in order, then over the wavefront.
+template <typename T, int P, int WPR>
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* __restrict__ delta, const int* __restrict__ row_index,
                                                            const float* __restrict__ w, float eps, T* __restrict__ out, T* x_out,
                                                            int hidden, int rows, const float* __restrict__ parts, int splits,
                                                            size_t part_stride) {
   constexpr int V = 16 / sizeof(T);
   struct alignas(16) Piece { T v[V]; };
-  const int lane = threadIdx.x & 63;
-  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  constexpr int kStride = 64 * WPR;                              // lanes that share a row
+  const int lane = WPR == 1 ? (threadIdx.x & 63) : threadIdx.x;
+  const int r = WPR == 1 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
   if (r >= rows) return;
   const size_t src = row_index ? (size_t)row_index[r] : (size_t)r;
   const int pieces = hidden / V;
@@ -141,18 +145,18 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
   Weights pw[kWeightsEarly ? P : 1];
 #pragma unroll
   for (int i = 0; i < P; ++i) {
-    const int c = min(lane + i * 64, pieces - 1);                // inside the row; what lies past it is not used
+    const int c = min(lane + i * kStride, pieces - 1);                // inside the row; what lies past it is not used
     px[i] = xr[c];
     if (delta) pd[i] = reinterpret_cast<const Piece*>(delta + src * hidden)[c];
   }
   if constexpr (kWeightsEarly) {
 #pragma unroll
-    for (int i = 0; i < P; ++i) pw[i] = reinterpret_cast<const Weights*>(w)[min(lane + i * 64, pieces - 1)];
+    for (int i = 0; i < P; ++i) pw[i] = reinterpret_cast<const Weights*>(w)[min(lane + i * kStride, pieces - 1)];
   }
   float acc = 0.f;
 #pragma unroll
   for (int i = 0; i < P; ++i) {
-    const int c = lane + i * 64;
+    const int c = lane + i * kStride;
     if (c >= pieces) continue;
     if (delta) {
 #pragma unroll
@@ -180,11 +184,20 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
 #pragma unroll
     for (int j = 0; j < V; ++j) acc += to_f32(px[i].v[j]) * to_f32(px[i].v[j]);
   }
-  const float inv = rsqrtf(wave_sum(acc) / (float)hidden + eps);
+  float total = wave_sum(acc);
+  if constexpr (WPR > 1) {
+    __shared__ float wave_totals[WPR];
+    if ((threadIdx.x & 63) == 0) wave_totals[threadIdx.x >> 6] = total;
+    __syncthreads();
+    total = wave_totals[0];
+#pragma unroll
+    for (int wv = 1; wv < WPR; ++wv) total += wave_totals[wv];
+  }
+  const float inv = rsqrtf(total / (float)hidden + eps);
   Piece* o = reinterpret_cast<Piece*>(out + (size_t)r * hidden);
 #pragma unroll
   for (int i = 0; i < P; ++i) {
-    const int c = lane + i * 64;
+    const int c = lane + i * kStride;
     if (c >= pieces) continue;
     Piece po;
 #pragma unroll
@@ -202,7 +215,15 @@ static int launch_rmsnorm(const T* x, const T* delta, const int* row_index, cons
                     (!parts || (((uintptr_t)parts % 16) == 0 && part_stride % 4 == 0));
   const int per_lane = wide ? (hidden / V + 63) / 64 : 0;
   dim3 grid4((rows + 3) / 4), block(256);
-#define PLLM_ROWS(P_) hipLaunchKernelGGL((rmsnorm_rows_kernel<T, P_>), grid4, block, 0, stream, x, delta, row_index, w, eps, out, x_out, hidden, rows, parts, splits, part_stride)
+  // few rows (decode steps of many requests, short prompt portions): a workgroup per row
+  if (wide && rows <= 1024 && per_lane >= 2 && per_lane <= 16) {
+    const int per_thread = (hidden / V + 255) / 256;
+#define PLLM_ROW_WG(P_) hipLaunchKernelGGL((rmsnorm_rows_kernel<T, P_, 4>), dim3(rows), block, 0, stream, x, delta, row_index, w, eps, out, x_out, hidden, rows, parts, splits, part_stride)
+    if (per_thread <= 1) PLLM_ROW_WG(1); else if (per_thread <= 2) PLLM_ROW_WG(2); else PLLM_ROW_WG(4);
+#undef PLLM_ROW_WG
+    return (int)hipGetLastError();
+  }
+#define PLLM_ROWS(P_) hipLaunchKernelGGL((rmsnorm_rows_kernel<T, P_, 1>), grid4, block, 0, stream, x, delta, row_index, w, eps, out, x_out, hidden, rows, parts, splits, part_stride)
   if (wide && per_lane <= 2) PLLM_ROWS(2);
   else if (wide && per_lane <= 4) PLLM_ROWS(4);
   else if (wide && per_lane <= 8) PLLM_ROWS(8);
