@@ -542,12 +542,13 @@ def stream_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, nt: int |
 
 _TILE_SIG = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+TILE_BLOCK_ROWS = 160           # input rows of one workgroup of the tiled kernel, at most
 
 
 def tile_linear_plan(M: int, N: int, K: int, compute_units: int) -> int:
     """Ranges of K for the tiled product of M rows with N weight rows: as many as give every compute unit a workgroup
-    (tiles of up to 128 rows x 128 weight rows), each at least four stages of 64 columns long."""
-    workgroups = -(-N // 128) * -(-M // 128)
+    (tiles of up to 160 rows x 128 weight rows), each at least four stages of 64 columns long."""
+    workgroups = -(-N // 128) * -(-M // TILE_BLOCK_ROWS)
     stages = -(-K // 64)
     if workgroups >= compute_units:
         return 1
@@ -555,7 +556,7 @@ def tile_linear_plan(M: int, N: int, K: int, compute_units: int) -> int:
 
 
 def tile_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, splits: int | None = None, rope: dict | None = None) -> torch.Tensor:
-    """As ``stream_linear``, for a few hundred rows: tiles of up to 128 rows x 128 weight rows per workgroup, both
+    """As ``stream_linear``, for a few hundred rows: tiles of up to 160 rows x 128 weight rows per workgroup, both
     operands through LDS."""
     _on_gpu(x, w.tiles)
     M, K = x.shape

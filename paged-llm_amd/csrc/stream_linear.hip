@@ -369,42 +369,70 @@ PLLM_API int pllm_stream_linear(int epi, const void* x, int ldx, const void* wt,
 constexpr int kTileBlocksN = 8;                      // blocks of 16 weight rows per workgroup
 constexpr int kTileStageSteps = 2;                   // steps of 32 columns per stage
 
-template <int EPI, int MTW, int R>
+// MT: tiles of 16 input rows per workgroup (the upper row of wavefronts takes the larger half).
+// What bounds a workgroup is what its compute unit can draw from the L2 (about 28 bytes a cycle when all compute units
+// draw: cycle stamps show the loaders' requests queueing, a stage of 34 KB taking 1,250 cycles, whatever the number of
+// stages in flight, with or without the products; four compute wavefronts as 2 x 2 with a third less LDS traffic took the
+// same time), so a tile is as large as registers and LDS allow, and matrices of many rows and few hundred input rows,
+// whose tiles cannot be large in both directions, stay with the library, which meets the same bound.
+template <int EPI, int MT, int R>
 __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const StreamLinearParams p) {
+  constexpr int CW = kComputeWaves;
   extern __shared__ __attribute__((aligned(16))) unsigned char sl_lds[];
-  constexpr int MT = 2 * MTW;                                    // tiles of 16 input rows per workgroup
+  constexpr int MTW = (MT + 1) / 2;                              // tiles of 16 input rows per wavefront (at most)
+  constexpr int WN = CW / 2, NTW = kTileBlocksN / WN;            // wavefronts along the weight rows, blocks of 16 weight rows each
   constexpr int kWBlocks = kTileBlocksN * kTileStageSteps, kXBlocks = MT * kTileStageSteps;
   constexpr int kSlotBytes = (kWBlocks + kXBlocks) * 1024;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nb = blockIdx.x, row0 = blockIdx.y * (MT * 16), split = blockIdx.z;
   const int first_stage = split * p.stages_per_split;           // (stages of 64 columns here)
   const int nstages = min(p.stages_per_split, p.num_stages - first_stage);
-  floatx4 acc[MTW][2];
+  floatx4 acc[MTW][NTW];
 
-  if (wave >= kComputeWaves) {
-    const int l = wave - kComputeWaves;
+  if (wave >= CW) {
+    const int l = wave - CW;
     const int xr = lane >> 2, xg = (lane & 3) ^ (xr >> 2);
     constexpr int kBlocks = kWBlocks + kXBlocks, kPerLoader = (kBlocks + kLoaderWaves - 1) / kLoaderWaves;
+    static_assert(kWBlocks % kLoaderWaves == 0, "a loader's i-th block is a weight tile for all loaders or for none");
+    // A loader's i-th block of a stage is the same block in every stage, kAdvance further along K: the addresses of the
+    // first stage are worked out once (a dozen vector instructions each, which issued before every load made the loaders
+    // the slowest part of a stage), a stage adds its offset.
+    const bf16* base[kPerLoader];
+#pragma unroll
+    for (int i = 0; i < kPerLoader; ++i) {
+      const int bb = min(l + i * kLoaderWaves, kBlocks - 1);     // (every loader issues the same number of loads per stage: the waits
+                                                                 //  below count them; a loader whose share is one short repeats its last block)
+      if (bb < kWBlocks) {
+        const int u = bb / kTileStageSteps, st = bb - u * kTileStageSteps;
+        base[i] = p.wt + (((size_t)(nb * kTileBlocksN + u) * p.ksteps + first_stage * kTileStageSteps + st) * 64 + lane) * 8;
+      } else {
+        const int bx = bb - kWBlocks, t = bx / kTileStageSteps, st = bx - t * kTileStageSteps;
+        const int row = min(row0 + t * 16 + xr, p.M - 1);        // rows past M repeat the last one: never stored
+        base[i] = p.x + (size_t)row * p.ldx + (first_stage * kTileStageSteps + st) * kChunkK + xg * 8;
+      }
+    }
+    const bool odd_steps = p.ksteps & 1;                         // K no multiple of 64: the last stage has one step only
     auto issue = [&](int s) {
-      const int ks0 = (first_stage + s) * kTileStageSteps;
       unsigned char* slot = sl_lds + (s % R) * kSlotBytes;
+      if (odd_steps && first_stage + s == p.num_stages - 1) {
+        // the stage that K cuts short: its second step repeats the first (and is not computed)
+        const int ks0 = (first_stage + s) * kTileStageSteps;
+#pragma unroll
+        for (int i = 0; i < kPerLoader; ++i) {
+          const int bb = min(l + i * kLoaderWaves, kBlocks - 1);
+          const bf16* src;
+          if (bb < kWBlocks) src = p.wt + (((size_t)(nb * kTileBlocksN + bb / kTileStageSteps) * p.ksteps + ks0) * 64 + lane) * 8;
+          else src = p.x + (size_t)min(row0 + ((bb - kWBlocks) / kTileStageSteps) * 16 + xr, p.M - 1) * p.ldx + ks0 * kChunkK + xg * 8;
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                           (__attribute__((address_space(3))) void*)(slot + bb * 1024), 16, 0, 0);
+        }
+        return;
+      }
 #pragma unroll
       for (int i = 0; i < kPerLoader; ++i) {
-        const int b = l + i * kLoaderWaves;
-        // Every loader issues the same number of loads per stage (the waits below count them): a loader whose share of
-        // the blocks is one short repeats its last block.
-        const int bb = min(b, kBlocks - 1);
-        const bf16* src;
-        if (bb < kWBlocks) {
-          const int u = bb / kTileStageSteps, st = bb - u * kTileStageSteps;
-          const int ks = min(ks0 + st, p.ksteps - 1);
-          src = p.wt + (((size_t)(nb * kTileBlocksN + u) * p.ksteps + ks) * 64 + lane) * 8;
-        } else {
-          const int bx = bb - kWBlocks, t = bx / kTileStageSteps, st = bx - t * kTileStageSteps;
-          const int row = min(row0 + t * 16 + xr, p.M - 1);
-          const int k = min((ks0 + st) * kChunkK + xg * 8, p.K - 8);
-          src = p.x + (size_t)row * p.ldx + k;
-        }
+        const int bb = min(l + i * kLoaderWaves, kBlocks - 1);
+        constexpr int kTileAdvance = kTileStageSteps * kTileElems, kRowAdvance = kTileStageSteps * kChunkK;
+        const bf16* src = base[i] + (size_t)s * (i * kLoaderWaves < kWBlocks ? kTileAdvance : kRowAdvance);
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)(slot + bb * 1024), 16, 0, 0);
       }
@@ -425,24 +453,29 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
   } else {
 #pragma unroll
     for (int t = 0; t < MTW; ++t) {
-      acc[t][0] = floatx4{0.f, 0.f, 0.f, 0.f};
-      acc[t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < NTW; ++u) acc[t][u] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    const int wm = wave >> 2, wn = wave & 3;
+    const int wm = wave / WN, wn = wave - wm * WN;
+    const int my_tiles = wm == 0 ? MTW : MT - MTW;               // (the same for the whole wavefront)
     const int r = lane & 15, g = lane >> 4;
-    const unsigned char* my_w = sl_lds + (wn * 2 * kTileStageSteps) * 1024 + lane * 16;
+    const unsigned char* my_w = sl_lds + (wn * NTW * kTileStageSteps) * 1024 + lane * 16;
     const unsigned char* my_x = sl_lds + (kWBlocks + wm * MTW * kTileStageSteps) * 1024 + (r * 4 + (g ^ (r >> 2))) * 16;
     int slot = 0;
     for (int s = 0; s < nstages; ++s) {
       stage_barrier();
       const int steps = min(kTileStageSteps, p.ksteps - (first_stage + s) * kTileStageSteps);
-      bf16x8 wf[kTileStageSteps][2], xf[kTileStageSteps][MTW];
+      // All operands of the stage are requested before the first product: the requests of the second step travel while
+      // the first step's products run (asked for step by step, a wavefront waited for LDS twice per stage, 200 cycles each,
+      // with its SIMD's other wavefront in the same place at the same time).
+      bf16x8 wf[kTileStageSteps][NTW], xf[kTileStageSteps][MTW];
 #pragma unroll
       for (int st = 0; st < kTileStageSteps; ++st) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) wf[st][u] = *reinterpret_cast<const bf16x8*>(my_w + slot * kSlotBytes + (u * kTileStageSteps + st) * 1024);
+        for (int u = 0; u < NTW; ++u) wf[st][u] = *reinterpret_cast<const bf16x8*>(my_w + slot * kSlotBytes + (u * kTileStageSteps + st) * 1024);
+        // (the lower row of wavefronts may have a tile less: it reads its last tile again and leaves the product out)
 #pragma unroll
-        for (int t = 0; t < MTW; ++t) xf[st][t] = *reinterpret_cast<const bf16x8*>(my_x + slot * kSlotBytes + (t * kTileStageSteps + st) * 1024);
+        for (int t = 0; t < MTW; ++t) xf[st][t] = *reinterpret_cast<const bf16x8*>(my_x + slot * kSlotBytes + (min(t, my_tiles - 1) * kTileStageSteps + st) * 1024);
       }
       asm volatile("" ::: "memory");
 #pragma unroll
@@ -450,8 +483,10 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
         if (st < steps) {
 #pragma unroll
           for (int t = 0; t < MTW; ++t) {
+            if (t < my_tiles) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[st][u], xf[st][t], acc[t][u], 0, 0, 0);
+              for (int u = 0; u < NTW; ++u) acc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[st][u], xf[st][t], acc[t][u], 0, 0, 0);
+            }
           }
         }
       }
@@ -463,9 +498,9 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
 #pragma unroll
     for (int t = 0; t < MTW; ++t) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int m = row0 + (wm * MTW + t) * 16 + r;
-        const int unit = nb * kTileBlocksN + wn * 2 + u;
+      for (int u = 0; u < NTW; ++u) {
+        const int m = t < my_tiles ? row0 + (wm * MTW + t) * 16 + r : p.M;
+        const int unit = nb * kTileBlocksN + wn * NTW + u;
         const floatx4 a = acc[t][u];
         floatx4 partner = a;
         if (kPaired) {                                           // tile rows 8-15 (the lanes 32 further on) hold the partners of rows 0-7
@@ -556,11 +591,11 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
   }
 }
 
-template <int EPI, int MTW, int R>
+template <int EPI, int MT, int R>
 static int launch_tile(const StreamLinearParams& p, dim3 grid, hipStream_t stream) {
-  constexpr size_t lds = (size_t)R * (kTileBlocksN * kTileStageSteps + 2 * MTW * kTileStageSteps) * 1024;
+  constexpr size_t lds = (size_t)R * (kTileBlocksN * kTileStageSteps + MT * kTileStageSteps) * 1024;
   static_assert(lds <= 160 * 1024, "LDS of one compute unit");
-  auto kernel = tile_linear_kernel<EPI, MTW, R>;
+  auto kernel = tile_linear_kernel<EPI, MT, R>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -569,11 +604,14 @@ static int launch_tile(const StreamLinearParams& p, dim3 grid, hipStream_t strea
   return (int)hipGetLastError();
 }
 
+// Blocks of input rows of the tiled kernel: of at most 160 rows (10 tiles of 16), evenly filled.
+PLLM_API int pllm_tile_linear_row_blocks(int M) { return (M + 159) / 160; }
+
 // The tiled weights hold a multiple of 8 blocks (of 24, in fact).  splits > 1 with epi SL_PARTIAL only.
 PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, void* out, int ldo, int M, int N, int K,
-                              int weight_blocks, int splits, const int* positions, const float* cos_t, const float* sin_t,
-                              const int* slots, void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim,
-                              int block_size, hipStream_t stream) {
+                              int weight_blocks, int splits, const int* positions, const float* cos_t,
+                              const float* sin_t, const int* slots, void* k_pages, void* v_pages, int num_heads, int num_kv_heads,
+                              int head_dim, int block_size, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K % kChunkK) || (ldx & 7) || weight_blocks <= 0 || (weight_blocks % kTileBlocksN) || splits < 1) return -2;
   if (splits > 1 && epi != SL_PARTIAL) return -2;
@@ -589,18 +627,22 @@ PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, v
   p.num_stages = (p.ksteps + kTileStageSteps - 1) / kTileStageSteps;
   p.stages_per_split = (p.num_stages + splits - 1) / splits;
   if ((long)p.stages_per_split * (splits - 1) >= p.num_stages) return -2;
-  const int m_blocks = pllm_stream_linear_row_blocks(M);
-  const int rows = (M + m_blocks - 1) / m_blocks, mtw = (rows + 31) / 32;       // tiles of 16 rows per wavefront: 1 to 4
+  const int m_blocks = pllm_tile_linear_row_blocks(M);
+  const int rows = (M + m_blocks - 1) / m_blocks, mt = (rows + 15) / 16;        // tiles of 16 rows per workgroup: 1 to 10
   const int n_blocks = ((rows_of_w + 15) / 16 + kTileBlocksN - 1) / kTileBlocksN;
   if (m_blocks > 65535 || splits > 65535) return -2;
   const dim3 grid(n_blocks, m_blocks, splits);
+  // (the kernel's row offset of a block along y is MT * 16: blocks are filled to whole tiles, the last one may be short)
+#define PLLM_TL(EPI_, MT_) return launch_tile<EPI_, MT_, (MT_ > 8 ? 3 : 4)>(p, grid, stream)
 #define PLLM_TL_SHAPES(EPI_)                                                  \
   do {                                                                        \
-    switch (mtw) {                                                            \
-      case 1: return launch_tile<EPI_, 1, 4>(p, grid, stream);                \
-      case 2: return launch_tile<EPI_, 2, 4>(p, grid, stream);                \
-      case 3: return launch_tile<EPI_, 3, 4>(p, grid, stream);                \
-      case 4: return launch_tile<EPI_, 4, 4>(p, grid, stream);                \
+    switch (mt) {                                                             \
+      case 1: case 2: PLLM_TL(EPI_, 2);                                       \
+      case 3: case 4: PLLM_TL(EPI_, 4);                                       \
+      case 5: case 6: PLLM_TL(EPI_, 6);                                       \
+      case 7: case 8: PLLM_TL(EPI_, 8);                                       \
+      case 9: PLLM_TL(EPI_, 9);                                               \
+      case 10: PLLM_TL(EPI_, 10);                                             \
     }                                                                         \
   } while (0)
   switch (epi) {
@@ -611,5 +653,6 @@ PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, v
     case SL_ROPE_KV: PLLM_TL_SHAPES(SL_ROPE_KV); break;
   }
 #undef PLLM_TL_SHAPES
+#undef PLLM_TL
   return -3;
 }
