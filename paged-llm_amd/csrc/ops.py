@@ -478,6 +478,13 @@ def tile_weight(w: torch.Tensor, pairing: str = "plain", head_dim: int = 0) -> T
     return TiledWeight(tiles, out_features, K, pairing, head_dim)
 
 
+def _whole_ranges(stages: int, splits: int) -> int:
+    """The largest number of ranges up to ``splits`` such that ranges of ceil(stages / ranges) stages leave none empty."""
+    while splits > 1 and -(-stages // splits) * (splits - 1) >= stages:
+        splits -= 1
+    return splits
+
+
 def stream_linear_plan(M: int, N: int, K: int, compute_units: int) -> tuple[int, int]:
     """(blocks of 16 weight rows per workgroup, ranges of K) for a product of M rows with N weight rows: by sizes only.
     Four blocks per workgroup halve what the rows cost out of the caches and are taken where the matrix still gives
@@ -490,7 +497,7 @@ def stream_linear_plan(M: int, N: int, K: int, compute_units: int) -> tuple[int,
     stages = -(-K // 256)
     splits = 1
     if workgroups < compute_units:
-        splits = max(1, min(compute_units // workgroups, stages // 2, 8))
+        splits = _whole_ranges(stages, max(1, min(compute_units // workgroups, stages // 2, 8)))
     return nt, splits
 
 
@@ -552,7 +559,7 @@ def tile_linear_plan(M: int, N: int, K: int, compute_units: int) -> int:
     stages = -(-K // 64)
     if workgroups >= compute_units:
         return 1
-    return max(1, min(compute_units // workgroups, stages // 4, 16))
+    return _whole_ranges(stages, max(1, min(compute_units // workgroups, stages // 4, 16)))
 
 
 def tile_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, splits: int | None = None, rope: dict | None = None) -> torch.Tensor:

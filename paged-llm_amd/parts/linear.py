@@ -146,10 +146,22 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
     return ops.gemm_generic(x, weight, out_dtype)
 
 
+TILE_GATED_ROWS = (161, 320)                    # rows for which the gated product takes the tiled kernel
+
+
 def gated_linear(x, w_gate_up) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix (a tensor, or a ``Weight`` with the gated pairing)."""
     if _streams(x, w_gate_up, ops.SL_GATED) and w_gate_up.pairing == "gated":
         return _stream(x, w_gate_up, ops.SL_GATED)
+    rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
+    if (isinstance(w_gate_up, Weight) and w_gate_up.tiled is not None and w_gate_up.pairing == "gated" and x.dtype == torch.bfloat16
+            and TILE_GATED_ROWS[0] <= rows <= TILE_GATED_ROWS[1]):
+        # Two blocks of input rows: the tiled kernel takes as long as the library's product there (11264 x 2048 at 264
+        # rows: 28 us both) and saves the activation kernel and its pass over the intermediate rows (5 us).
+        x = rows_of(x)
+        if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+            x = x.contiguous()
+        return ops.tile_linear(x, w_gate_up.tiled, ops.SL_GATED)
     if w_gate_up.dtype == torch.bfloat16:
         out = _fused(x, w_gate_up, ops.EPI_GATED)
         if out is not None:

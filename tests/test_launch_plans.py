@@ -43,3 +43,17 @@ def test_graph_batch_sizes_cover_every_batch_with_at_most_half_as_many_rows_agai
     assert sizes == sorted(sizes)
     assert len(set(sizes)) <= 24                                                       # few graphs for a batch that shrinks one by one
     assert [ModelRunner._bucket(n) for n in (1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 64, 65)] == [1, 2, 3, 4, 6, 6, 8, 8, 12, 16, 64, 96]
+
+
+def test_ranges_of_the_inner_dimension_are_never_empty():
+    """The products' plans cut K into ranges of equal numbers of stages; whatever the sizes, no range is left empty
+    (a matrix of 2048 x 5632 at 150 rows once asked for 16 ranges of 6 of its 88 stages)."""
+    from paged_llm_amd.csrc import ops
+    for rows in (17, 64, 100, 128, 129, 150, 160, 161, 264, 320, 400, 512, 640):
+        for n, k in ((2048, 2048), (2048, 5632), (2560, 2048), (4096, 4096), (96, 992), (2048, 14336), (32, 32)):
+            for cus in (256, 304, 64):
+                ranges, stages = ops.tile_linear_plan(rows, n, k, cus), -(-k // 64)
+                assert ranges == 1 or -(-stages // ranges) * (ranges - 1) < stages, (rows, n, k, ranges)
+                _, ranges = ops.stream_linear_plan(rows, n, k, cus)
+                stages = -(-k // 256)
+                assert ranges == 1 or -(-stages // ranges) * (ranges - 1) < stages, (rows, n, k, ranges)

@@ -316,3 +316,30 @@ def test_pages_of_one_and_two_positions(folders, dtype, block_size):
     check(got, folder, reqs, dtype)
     session.manager.check_invariants()
     assert session.manager.num_free_pages() == session.manager.num_pages()
+
+
+def test_steps_of_a_few_hundred_rows(tmp_path):
+    """Prompt portions of 129 to 640 tokens, alone and beside decoded tokens of other requests: the products of such steps
+    take the tiled kernel where a matrix is small (partial sums of ranges of K that the next norm adds) and, for the gated
+    product of 161 to 320 rows, its gated epilogue; widths are multiples of 32 so that the weights have their tiled copies.
+    Every row against the plain implementation."""
+    cfg = dict(ODD_BASE, num_hidden_layers=2, hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+               intermediate_size=704, vocab_size=300, max_position_embeddings=2048)
+    folder = helpers.make_folder(tmp_path, cfg, seed=8, stored="bfloat16")
+    reqs = {"long": helpers.random_tokens(150 + 264 + 129 + 330 + 640 + 200, 300, seed=2),
+            "a": helpers.random_tokens(40, 300, seed=3), "b": helpers.random_tokens(35, 300, seed=4)}
+    session = session_for(folder, "bfloat16", rounded(len(reqs["long"])) + 128)
+    from paged_llm_amd.parts.linear import Weight
+    mixer = session.model.blocks[0].mixer
+    assert isinstance(mixer.w_o, Weight) and mixer.w_o.tiled is not None and session.model.blocks[0].parts["feed_forward"].w_gate_up.tiled is not None
+    trace = TraceBuilder()
+    trace.step([("a", reqs["a"][:20], "last"), ("b", reqs["b"][:20], "last")])
+    at, side = 0, 20
+    for n in (150, 264, 129, 330, 640, 200):
+        entries = [("long", reqs["long"][at:at + n], [0, n // 2, n - 1])]
+        if side < 35:
+            entries += [("a", reqs["a"][side:side + 1], "all"), ("b", reqs["b"][side:side + 1], "all")]
+            side += 1
+        trace.step(entries)
+        at += n
+    check(helpers.replay_in_process(session, trace), folder, reqs, "bfloat16")
