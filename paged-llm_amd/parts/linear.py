@@ -51,11 +51,17 @@ class Weight:
 STREAM_MIN_ROWS, STREAM_MAX_ROWS = 17, 128      # rows the streaming kernel is chosen for
 TILE_MAX_ROWS = 640                             # rows up to which the tiled kernel is chosen for small matrices cut along K
 STREAM_GATED_MAX_ROWS = 64                      # the gated product: beyond, its rows' traffic costs more than the library's kernel
-STREAM_SMALL_MATRIX = 1 << 24                   # elements up to which a matrix is "small": cut along K, partial sums or one range
+STREAM_LONG_K, STREAM_LONG_K_MAX_ROWS = 8192, 64 # from this K on the rows' traffic limits the streaming kernel to so many rows
 
 
 def _plain(weight) -> torch.Tensor:
     return weight.plain if isinstance(weight, Weight) else weight
+
+
+def _few_weight_rows(weight) -> bool:
+    """Matrices with at most 32 weight rows per compute unit: their workgroups fit one round (with more rows, every
+    further workgroup reads all input rows again, and the library's larger tiles win: 11264 x 2048, 32000 x 2048)."""
+    return weight.shape[0] <= 32 * ops._num_compute_units(weight.plain.device)
 
 
 def _tiles(x, weight, partial_ok: bool) -> bool:
@@ -66,7 +72,7 @@ def _tiles(x, weight, partial_ok: bool) -> bool:
         return False
     rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
     n, k = weight.shape
-    return (STREAM_MAX_ROWS < rows <= TILE_MAX_ROWS and x.dtype == torch.bfloat16 and n * k <= STREAM_SMALL_MATRIX
+    return (STREAM_MAX_ROWS < rows <= TILE_MAX_ROWS and x.dtype == torch.bfloat16 and _few_weight_rows(weight)
             and ops.tile_linear_plan(rows, n, k, ops._num_compute_units(weight.plain.device)) > 1)
 
 
@@ -83,7 +89,7 @@ def _streams(x, weight, epi: int) -> bool:
         return rows <= STREAM_GATED_MAX_ROWS
     if epi == ops.SL_F32:
         return False                                            # (the head: 32000 x 2048 was not faster than the library's kernel)
-    return n * k <= STREAM_SMALL_MATRIX
+    return _few_weight_rows(weight) and (k < STREAM_LONG_K or rows <= STREAM_LONG_K_MAX_ROWS)
 
 
 def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: bool = False):
@@ -92,12 +98,12 @@ def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: b
         x = x.contiguous()
     n, k = weight.shape
     if epi == ops.SL_GATED:
-        return ops.stream_linear(x, weight.tiled, epi, nt=3)
-    nt, splits = ops.stream_linear_plan(x.shape[0], n, k, ops._num_compute_units(x.device))
-    if epi == ops.SL_BF16 and partial_ok and splits > 1:
-        return ops.stream_linear(x, weight.tiled, ops.SL_PARTIAL, nt=nt, splits=splits)
-    # one range of K: blocks of 16 weight rows of their own fill the GPU best for these matrices
-    return ops.stream_linear(x, weight.tiled, epi, nt=1 if -(-n // 16) <= 2 * ops._num_compute_units(x.device) else nt, rope=rope)
+        return ops.stream_linear(x, weight.tiled, epi)
+    if epi == ops.SL_BF16 and partial_ok:
+        nt, splits = ops.stream_linear_plan(x.shape[0], n, k, ops._num_compute_units(x.device), partial=True)
+        if splits > 1:
+            return ops.stream_linear(x, weight.tiled, ops.SL_PARTIAL, nt=nt, splits=splits)
+    return ops.stream_linear(x, weight.tiled, epi, rope=rope)
 
 
 _PAIRING_OF = {ops.EPI_GATED: "gated", ops.EPI_ROPE_KV: "rotary"}
@@ -105,7 +111,8 @@ _PAIRING_OF = {ops.EPI_GATED: "gated", ops.EPI_ROPE_KV: "rotary"}
 
 def _fused(x, weight, epi: int, rope: dict | None = None):
     """The fused decode kernel if it takes the operands, else None.  With a ``Weight`` whose tiled copy has the pairing
-    of the epilogue, products of at most 16 rows stream the weights from that copy."""
+    of the epilogue, products of at most 16 rows with the sum and norm in front stream the weights from that copy
+    (11264 x 2048: 12.3 against 13.4 us; 2560 x 2048 with the rotary epilogue: 7.4 against 7.9; 32000 x 2048: 29.0 against 30.4)."""
     tiled = None
     if isinstance(weight, Weight):
         if weight.tiled is not None and weight.pairing == _PAIRING_OF.get(epi, "plain"):
@@ -120,7 +127,9 @@ def _fused(x, weight, epi: int, rope: dict | None = None):
         x = x.rows()
     if (x.dtype == torch.bfloat16 and ops.decode_linear_takes(x.shape[0], x.shape[1], x, weight, staged=False)
             and ops.decode_linear_pays(x.shape[0], weight.shape[0], x.shape[1], epi, staged=False)):
-        return ops.decode_linear(x, weight, epi, rope=rope, tiled=tiled if x.shape[0] <= ops.DECODE_MAX_ROWS else None)
+        # (plain rows keep the row-major matrix: from the tiled copy 4096 x 4096 and 4096 x 14336 took 10.7 and 32.9 us at 8
+        #  rows against 9.3 and 27.7, and the smaller matrices the same time either way)
+        return ops.decode_linear(x, weight, epi, rope=rope)
     return None
 
 

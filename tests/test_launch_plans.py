@@ -57,3 +57,15 @@ def test_ranges_of_the_inner_dimension_are_never_empty():
                 _, ranges = ops.stream_linear_plan(rows, n, k, cus)
                 stages = -(-k // 256)
                 assert ranges == 1 or -(-stages // ranges) * (ranges - 1) < stages, (rows, n, k, ranges)
+
+
+def test_streaming_product_plans_by_sizes():
+    from paged_llm_amd.csrc import ops
+    plan, cus = ops.stream_linear_plan, 256
+    assert plan(64, 2048, 5632, cus) == (2, 4)                # 64 blocks of 32 weight rows x 4 ranges: a workgroup per compute unit
+    assert plan(64, 2048, 2048, cus) == (2, 4) and plan(64, 2560, 2048, cus) == (2, 3)
+    assert plan(64, 4096, 14336, cus) == (4, 4)               # long K, few rows: four blocks, fewer reads of the rows
+    assert plan(128, 4096, 14336, cus) == (2, 2)
+    assert plan(64, 2048, 2048, cus, partial=False) == (1, 1) and plan(64, 6144, 4096, cus, partial=False) == (2, 1)
+    assert ops.gated_blocks_per_workgroup(5632, cus) == 3 and ops.gated_blocks_per_workgroup(14336, cus) == 4
+    assert ops.gated_blocks_per_workgroup(8192, cus) == 4     # 1024 blocks: 342 workgroups of three would need a second round
