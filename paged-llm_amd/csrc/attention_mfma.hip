@@ -370,7 +370,9 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
         }
         dst[2 + db * 16 + g * 4 + i] = o;
       } else {
-        out[(size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D + db * 16 + g * 4 + i] = __float2bfloat16(o / l_tot);
+        // (times the reciprocal, as the one-wavefront form below and the merge kernel have it: with all keys in one
+        //  wavefront's block the three give the same bits)
+        out[(size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D + db * 16 + g * 4 + i] = __float2bfloat16(o * (1.f / l_tot));
       }
     }
     return;

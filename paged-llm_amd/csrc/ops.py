@@ -664,7 +664,7 @@ def _merge_lds_bytes(column_blocks: int, waves: int, head_dim: int) -> int:
 
 
 def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: int, group: int, head_dim: int,
-                   lds_limit: int) -> tuple[int, int, int]:
+                   lds_limit: int, compute_units: int = 256) -> tuple[int, int, int]:
     """(wavefronts per work item, partition_size, num_partitions) for a step.
 
     Prompt portions have many query tiles: one wavefront per tile walks all its keys (1, 0, 1).
@@ -680,10 +680,13 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
         max_waves //= 2
     if max_waves < 4:
         return 1, 0, 1
-    # Partitions only as far as they are needed to fill the GPU: fewer, longer work items are faster than
-    # many short ones plus a larger merge (measured for head sizes 64 and 128).
+    # Partitions only as far as they fill the GPU in one round: a workgroup of eight wavefronts has a compute unit to
+    # itself, so work items x partitions stay at or under the number of compute units (48 sequences x 4 kv heads x 2048
+    # keys at head size 64: 28.1 us in one piece on 192 compute units, 37.0 us in two partitions, which make 384
+    # workgroups and two rounds; 24 sequences: 18.8 us in two partitions against 21.9 in four and 24.5 in one), and
+    # fewer, longer work items are faster than many short ones plus a larger merge.
     items = num_seqs * num_kv_heads
-    want_parts = max(1, 384 // items)
+    want_parts = max(1, compute_units // items)
     size = 256                                        # at least four blocks of 64 keys per workgroup
     while (max_k_len + size - 1) // size > want_parts:
         size *= 2
@@ -691,11 +694,12 @@ def attention_plan(num_seqs: int, num_kv_heads: int, max_q_len: int, max_k_len: 
     waves = max_waves
     while waves > 4 and (waves // 2) * 64 >= min(size, max_k_len):
         waves //= 2
-    # Small heads (two blocks of keys under way per wavefront) and two or more work items per compute unit: two
-    # workgroups of four wavefronts on a compute unit stream faster than one of eight (64 sequences x 8 kv heads x
-    # 2048 keys at head size 64: a decode step of Llama-3.2-1B shapes 2.68 against 2.74 ms).  With one work item per
-    # compute unit, two partitions of four wavefronts each were slower in the step (2.81 against 2.75 ms at 4 kv heads).
-    if head_dim <= 64 and parts == 1 and items >= 512:
+    # Small heads (two blocks of keys under way per wavefront) and more work items than compute units: two
+    # workgroups of four wavefronts on a compute unit stream faster than eight-wavefront workgroups in two rounds
+    # (96 sequences x 4 kv heads x 2048 keys at head size 64: 48.7 against 57.5 us; 64 sequences x 8 kv heads: a decode
+    # step of Llama-3.2-1B shapes 2.68 against 2.74 ms).  At head size 128 eight wavefronts stay ahead (40 sequences x 8
+    # kv heads: 86.7 against 106.3 us).
+    if head_dim <= 64 and parts == 1 and items > compute_units:
         waves = 4
     return (waves, size, parts) if parts > 1 else (waves, 0, 1)
 
@@ -886,7 +890,7 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
             work = work.view(-1, 2)
             out = torch.empty((q.shape[0], num_heads * head_dim), dtype=q.dtype, device=q.device)
             if few:
-                waves, size, parts = attention_plan(few, num_kv_heads, 1, ctx.max_k_len, group, head_dim, lds)
+                waves, size, parts = attention_plan(few, num_kv_heads, 1, ctx.max_k_len, group, head_dim, lds, _num_compute_units(q.device))
                 paged_attention_mfma(q[:few], k_pages, v_pages, block_tables[:few], cu_seqlens_q[:few + 1], seq_lens_k[:few],
                                      num_heads, num_kv_heads, head_dim, scale, window, 1, size, parts, waves,
                                      2 if waves == 1 else 0, out=out[:few])
@@ -904,7 +908,7 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
             rows = sum(q_lens[:few])
             out = torch.empty((q.shape[0], num_heads * head_dim), dtype=q.dtype, device=q.device)
             max_q, max_k = max(q_lens[:few]), max(k_lens[:few])
-            waves, size, parts = attention_plan(few, num_kv_heads, max_q, max_k, group, head_dim, lds)
+            waves, size, parts = attention_plan(few, num_kv_heads, max_q, max_k, group, head_dim, lds, _num_compute_units(q.device))
             paged_attention_mfma(q[:rows], k_pages, v_pages, block_tables[:few], cu_seqlens_q[:few + 1], seq_lens_k[:few],
                                  num_heads, num_kv_heads, head_dim, scale, window, max_q, size, parts, waves,
                                  2 if waves == 1 else 0, out=out[:rows])
@@ -915,7 +919,8 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                                  num_kv_heads, head_dim, scale, window, max(q_lens[few:]), psize, pparts, 1, 2, out=out,
                                  work_list=prompt_work_list(ctx, few, group))
             return out
-        waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, group, head_dim, lds)
+        waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, group, head_dim, lds,
+                                            _num_compute_units(q.device))
         # Prompt portions: 32 columns per wavefront leave registers for two wavefronts per SIMD
         # (measured faster than 64 columns at one).
         prompt = waves == 1 and ctx.max_q_len * group > FEW_QUERY_COLUMNS and not ctx.capturing

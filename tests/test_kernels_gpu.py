@@ -665,6 +665,11 @@ def test_attention_plan():
     assert plan(2, 4, 1, 50, 8, 64, lds) == (1, 0, 1)
     assert plan(8, 8, 1, 2048, 4, 128, lds) == (8, 512, 4)
     assert plan(1, 8, 1, 100000, 4, 128, lds) == (8, 4096, 25)
+    assert plan(24, 4, 1, 2048, 8, 64, lds) == (8, 1024, 2)      # work items x partitions fill the compute units once, not twice
+    assert plan(48, 4, 1, 2048, 8, 64, lds) == (8, 0, 1)
+    assert plan(96, 4, 1, 2048, 8, 64, lds) == (4, 0, 1)         # more work items than compute units: two small workgroups each
+    assert plan(40, 8, 1, 2048, 4, 128, lds) == (8, 0, 1)
+    assert plan(48, 4, 1, 2048, 8, 64, lds, 304) == (8, 0, 1) and plan(24, 4, 1, 2048, 8, 64, lds, 64) == (4, 0, 1)
 
 
 # ----------------------------------------------------------------------------------- fused decode products
