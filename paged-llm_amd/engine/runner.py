@@ -63,7 +63,7 @@ class GraphCache:
 
 class ModelRunner:
     def __init__(self, model, kv_storage: KVCacheStorage, num_state_slots: int = 0, use_graphs: bool = False,
-                 max_graph_batch: int = 256, max_graph_tokens: int = 1024, graph_after_sightings: int = 2):
+                 max_graph_batch: int = 1024, max_graph_tokens: int = 1024, graph_after_sightings: int = 2):
         self.model = model
         # Graph replay needs every part of the model to do nothing but launch kernels on the
         # current stream; parts say so with ``graph_capturable`` (steps of single tokens) and

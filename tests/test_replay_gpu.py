@@ -343,3 +343,33 @@ def test_steps_of_a_few_hundred_rows(tmp_path):
         trace.step(entries)
         at += n
     check(helpers.replay_in_process(session, trace), folder, reqs, "bfloat16")
+
+
+@pytest.mark.parametrize("graph_rows", [256, 1024])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_hundreds_of_live_requests(folders, dtype, graph_rows, monkeypatch):
+    """300 requests decode together, once with more rows than the step function replays from a graph (the steps are then
+    launched kernel by kernel) and once as graphs of 384 rows; either way the products and the attention take their forms
+    for that many rows.  Every request's last rows against the plain implementation; some requests end on the way and
+    their pages go to late ones."""
+    import paged_llm_amd.engine.replay as replay
+    real = replay.build_runtime
+    monkeypatch.setattr(replay, "build_runtime", lambda *a, **kw: real(*a, **dict(kw, max_graph_batch=graph_rows)))
+    cfg = CONFIGS["B"]
+    folder = folders["B", "float32" if dtype == "float32" else "bfloat16"]
+    reqs = {f"q{i}": helpers.random_tokens(7 + i % 5, cfg["vocab_size"], seed=900 + i) for i in range(300)}
+    reqs.update({f"late{i}": helpers.random_tokens(6, cfg["vocab_size"], seed=1300 + i) for i in range(20)})
+    session = session_for(folder, dtype, 64 * 300)
+    assert session.runner.max_graph_batch == graph_rows
+    trace = TraceBuilder()
+    names = [f"q{i}" for i in range(300)]
+    for lo in range(0, 300, 100):                                    # the prompts but for their last three tokens, 100 requests a step
+        trace.step([(r, reqs[r][:-3], []) for r in names[lo:lo + 100]])
+    trace.step([(r, reqs[r][-3:-2], "all") for r in names])
+    trace.step([(r, reqs[r][-2:-1], "all") for r in names], end=names[:20])
+    late = [f"late{i}" for i in range(20)]
+    trace.step([(r, reqs[r][-1:], "all") for r in names[20:]] + [(r, reqs[r], "last") for r in late], end=names[20:] + late)
+    got = helpers.replay_in_process(session, trace)
+    assert len(got) == 300 * 2 + 280 + 20
+    assert any(k[0] != "prompt" and k[0] == 384 for k in session.runner._graphs) == (graph_rows >= 300 and session.runner.use_graphs)
+    check(got, folder, reqs, dtype)
