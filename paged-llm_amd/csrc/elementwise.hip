@@ -163,12 +163,27 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* x, const T* 
       for (int j = 0; j < V; ++j) px[i].v[j] = from_f32<T>(to_f32(px[i].v[j]) + to_f32(pd[i].v[j]));
       if (x_out) reinterpret_cast<Piece*>(x_out + src * hidden)[c] = px[i];
     } else if (parts) {
-      // the ranges' float sums of this piece, added in order (16-byte loads: hidden is a multiple of V, the buffer aligned)
+      // The ranges' float sums of this piece, added in order (16-byte loads: hidden is a multiple of V, the buffer
+      // aligned).  The first kEarly ranges (all there are, for most launches) are requested together before any is
+      // added: a loop over a number of ranges known only at run time asks for one, waits, adds, and asks for the
+      // next, a round trip to memory each.  A range past the last repeats it and is dropped by a select.
       struct alignas(16) Four { float v[4]; };
+      constexpr int kEarly = P == 1 ? 8 : (P == 2 ? 4 : 2);
+      Four early[kEarly][V / 4];
+#pragma unroll
+      for (int sp = 0; sp < kEarly; ++sp) {
+        const Four* pp = reinterpret_cast<const Four*>(parts + min(sp, splits - 1) * part_stride + src * hidden + (size_t)c * V);
+#pragma unroll
+        for (int q = 0; q < V / 4; ++q) early[sp][q] = pp[q];
+      }
       float d[V];
 #pragma unroll
       for (int j = 0; j < V; ++j) d[j] = 0.f;
-      for (int sp = 0; sp < splits; ++sp) {
+#pragma unroll
+      for (int sp = 0; sp < kEarly; ++sp)
+#pragma unroll
+        for (int j = 0; j < V; ++j) d[j] += sp < splits ? early[sp][j / 4].v[j % 4] : 0.f;
+      for (int sp = kEarly; sp < splits; ++sp) {
         const Four* pp = reinterpret_cast<const Four*>(parts + sp * part_stride + src * hidden + (size_t)c * V);
 #pragma unroll
         for (int q = 0; q < V / 4; ++q) {
