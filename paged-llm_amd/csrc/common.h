@@ -23,6 +23,15 @@ template <typename T> __device__ __forceinline__ T from_f32(float x);
 template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16 from_f32<bf16>(float x) { return __float2bfloat16(x); }  // round to nearest even
 
+// The gate's activation in a gated product, out = act(gate) * up, chosen by the feed-forward's configuration:
+// SiLU, z / (1 + exp(-z)), or GELU in its tanh form, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
+enum { PLLM_ACT_SILU = 0, PLLM_ACT_GELU_TANH = 1, PLLM_ACT_COUNT = 2 };
+
+__device__ __forceinline__ float gate_activation(float z, int act) {
+  if (act == PLLM_ACT_GELU_TANH) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z / (1.f + expf(-z));
+}
+
 // One rotary pair turned by the angle whose cosine and sine are c and s.  Products and sums are rounded one by one (no
 // fused multiply-add), in every kernel that rotates: what one kernel writes into the cache and what another computes
 // for the same position are then the same bits, and equal to what plain float arithmetic gives.

@@ -43,6 +43,7 @@ struct DecodeLinearParams {
   const int* positions; const float* cos_t; const float* sin_t; const int* slots;
   bf16* k_pages; bf16* v_pages;
   int num_heads, num_kv_heads, head_dim, block_size;
+  int activation;              // EPI_GATED: the gate's activation (PLLM_ACT_*)
 };
 
 __device__ __forceinline__ bf16x8 zero8() {
@@ -413,7 +414,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_linear_kernel(const DecodeL
           const int n = unit * 8 + row;
           if (row < 8 && n < N) {
             const float gate = total(lane) * row_scale, up = total(lane + 32) * row_scale;    // same outputs, 8 tile rows further
-            ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16((gate / (1.f + expf(-gate))) * up);
+            ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(gate_activation(gate, p.activation) * up);
           }
         } else if (row < 8) {  // EPI_ROPE_KV
           const int d = p.head_dim, half = d >> 1, per_head = half >> 3;
@@ -572,7 +573,7 @@ __global__ __launch_bounds__(512) void decode_linear_wide_kernel(const DecodeLin
           const int n = unit * 8 + row;
           if (row < 8 && n < N) {
             const float gate = total(lane), up = total(lane + 32);
-            ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16((gate / (1.f + expf(-gate))) * up);
+            ((bf16*)p.out)[(size_t)m * p.ldo + n] = __float2bfloat16(gate_activation(gate, p.activation) * up);
           }
         } else if (row < 8) {  // EPI_ROPE_KV
           const int half = p.head_dim >> 1, per_head = half >> 3;
@@ -674,8 +675,9 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
                                 void* x_out, int ldxo, const int* row_index, const void* W, int ldw, const void* Wt, void* out, int ldo, int M,
                                 int N, int K, const int* positions, const float* cos_t, const float* sin_t, const int* slots,
                                 void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim, int block_size,
-                                hipStream_t stream) {
+                                int activation, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
+  if (activation < 0 || activation >= PLLM_ACT_COUNT) return -2;
   if (M > 64 || (M > 16 && (delta || norm_w)) || K <= 0 || (K & 7) || (ldx & 7) || (W && (ldw & 7)) || (delta && (ldd & 7)) || (x_out && (ldxo & 7))) return -2;
   if ((!W && !Wt) || (Wt && (K & 31)) || (!W && M > 16)) return -2;
   DecodeLinearParams p;
@@ -683,7 +685,7 @@ PLLM_API int pllm_decode_linear(int epi, const void* x, int ldx, const void* del
   p.x_out = (bf16*)x_out; p.ldxo = ldxo; p.row_index = row_index; p.W = (const bf16*)W; p.ldw = ldw; p.Wt = (const bf16*)Wt; p.out = out; p.ldo = ldo;
   p.M = M; p.N = N; p.K = K; p.positions = positions; p.cos_t = cos_t; p.sin_t = sin_t; p.slots = slots;
   p.k_pages = (bf16*)k_pages; p.v_pages = (bf16*)v_pages; p.num_heads = num_heads; p.num_kv_heads = num_kv_heads;
-  p.head_dim = head_dim; p.block_size = block_size;
+  p.head_dim = head_dim; p.block_size = block_size; p.activation = activation;
   int units;
   switch (epi) {
     case EPI_BF16: case EPI_F32: units = (N + 15) / 16; break;

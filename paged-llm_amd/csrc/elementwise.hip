@@ -269,9 +269,9 @@ PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int
 }
 
 // ---------------------------------------------------------------------------------------------
-// Gated activation: out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(z) = z / (1 + exp(-z)).
+// Gated activation: out[t, i] = act(gu[t, i]) * gu[t, inter + i] (gate_activation in common.h).
 template <typename T, int V>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+__global__ void gate_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total, int act) {
   // Each thread handles V consecutive outputs of one row (V = 1, or a 16-byte piece).
   struct alignas(sizeof(T) * V) Piece { T v[V]; };
   const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
@@ -284,24 +284,25 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
 #pragma unroll
   for (int j = 0; j < V; ++j) {
     const float g = to_f32(pg.v[j]), u = to_f32(pu.v[j]);
-    po.v[j] = from_f32<T>((g / (1.f + expf(-g))) * u);
+    po.v[j] = from_f32<T>(gate_activation(g, act) * u);
   }
   *reinterpret_cast<Piece*>(out + idx) = po;
 }
 
-PLLM_API int pllm_silu_mul(int dtype, const void* gate_up, void* out, int num_tokens, int inter, hipStream_t stream) {
+PLLM_API int pllm_gate_mul(int dtype, int activation, const void* gate_up, void* out, int num_tokens, int inter, hipStream_t stream) {
   const size_t total = (size_t)num_tokens * inter;
   if (total == 0) return 0;
+  if (activation < 0 || activation >= PLLM_ACT_COUNT) return -2;
   const int elem = dtype == PLLM_F32 ? 4 : 2, wide = 16 / elem;
   const bool vec = inter % wide == 0 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0;
   const size_t items = vec ? total / wide : total;
   dim3 block(256), grid((unsigned)((items + 255) / 256));
   if (dtype == PLLM_F32) {
-    if (vec) hipLaunchKernelGGL((silu_mul_kernel<float, 4>), grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total);
-    else hipLaunchKernelGGL((silu_mul_kernel<float, 1>), grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total);
+    if (vec) hipLaunchKernelGGL((gate_mul_kernel<float, 4>), grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total, activation);
+    else hipLaunchKernelGGL((gate_mul_kernel<float, 1>), grid, block, 0, stream, (const float*)gate_up, (float*)out, inter, total, activation);
   } else {
-    if (vec) hipLaunchKernelGGL((silu_mul_kernel<bf16, 8>), grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total);
-    else hipLaunchKernelGGL((silu_mul_kernel<bf16, 1>), grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total);
+    if (vec) hipLaunchKernelGGL((gate_mul_kernel<bf16, 8>), grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total, activation);
+    else hipLaunchKernelGGL((gate_mul_kernel<bf16, 1>), grid, block, 0, stream, (const bf16*)gate_up, (bf16*)out, inter, total, activation);
   }
   PLLM_RETURN_LAST_ERROR();
 }

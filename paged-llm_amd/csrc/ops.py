@@ -70,7 +70,7 @@ _SIGNATURES = {
     "pllm_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "pllm_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long,
                      c_void_p],
-    "pllm_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "pllm_gate_mul": [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "pllm_rope_scatter": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "pllm_copy_pages": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p],
@@ -151,15 +151,27 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, delta: torch.Tens
     return out
 
 
-def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
-    """[T, 2I] -> silu(first half) * second half, [T, I]."""
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}      # the gate's activation in a gated product (PLLM_ACT_* in common.h)
+
+
+def activation_code(name: str) -> int:
+    _need(name in ACTIVATIONS, f"gate activation {name!r}: one of {sorted(ACTIVATIONS)}")
+    return ACTIVATIONS[name]
+
+
+def gate_mul(gate_up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """[T, 2I] -> act(first half) * second half, [T, I]."""
     _on_gpu(gate_up)
     _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gate_up must be contiguous [T, 2I]")
     T, I = gate_up.shape[0], gate_up.shape[1] // 2
     out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
-    _check(_fn("elementwise.hip", "pllm_silu_mul")(dtype_code(gate_up.dtype), _ptr(gate_up), _ptr(out), T, I, _stream()),
-           "silu_mul")
+    _check(_fn("elementwise.hip", "pllm_gate_mul")(dtype_code(gate_up.dtype), activation_code(activation), _ptr(gate_up), _ptr(out), T, I,
+                                                   _stream()), "gate_mul")
     return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    return gate_mul(gate_up, "silu")
 
 
 def rope_scatter(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
@@ -305,7 +317,7 @@ DECODE_MAX_ROWS = 16          # rows of the fused form with a sum or norm in fro
 DECODE_WIDE_MAX_ROWS = 64     # rows of the form for plain rows
 _DECODE_SIG = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-               c_void_p]
+               c_int, c_void_p]
 _lds_limit: dict = {}
 
 
@@ -359,12 +371,13 @@ def decode_linear_pays(rows: int, N: int, K: int, epi: int, staged: bool) -> boo
 
 def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: torch.Tensor | None = None,
                   norm_weight: torch.Tensor | None = None, eps: float = 0.0, x_out: torch.Tensor | None = None,
-                  row_index: torch.Tensor | None = None, rope: dict | None = None, tiled=None) -> torch.Tensor:
+                  row_index: torch.Tensor | None = None, rope: dict | None = None, tiled=None,
+                  activation: str = "silu") -> torch.Tensor:
     """rows = x[row_index] (+ delta) -> optional RMS norm -> rows W^T -> epilogue, in one kernel.
     ``tiled``: the matrix's ``TiledWeight`` with the pairing that goes with ``epi`` (at most 16 rows): the weights are then
     streamed from that copy, in contiguous pieces, wherever the kernel works in units of 16 weight rows.
 
-    epi EPI_BF16 / EPI_F32: [M, N] out.  EPI_GATED: w = [gate; up], out = silu(gate) * up [M, N/2].
+    epi EPI_BF16 / EPI_F32: [M, N] out.  EPI_GATED: w = [gate; up], out = act(gate) * up [M, N/2] (``activation``).
     EPI_ROPE_KV: w = [q; k; v] rows; q is rotated and returned [M, heads * d]; k (rotated) and v go
     into the cache pages; ``rope`` = dict(positions, cos, sin, slots, k_pages, v_pages, num_heads,
     num_kv_heads, head_dim, block_size).  ``x_out`` receives x + delta (the new residual).
@@ -419,7 +432,7 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
              None if tiled is None else _ptr(tiled.tiles), _ptr(out),
              out.stride(0), M, N, K, _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")),
              _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)),
-             int(r.get("head_dim", 0)), int(r.get("block_size", 0)), _stream()), "decode_linear")
+             int(r.get("head_dim", 0)), int(r.get("block_size", 0)), activation_code(activation), _stream()), "decode_linear")
     return out
 
 
@@ -427,7 +440,7 @@ def decode_linear(x: torch.Tensor, w: torch.Tensor, epi: int = EPI_BF16, delta: 
 SL_BF16, SL_F32, SL_GATED, SL_PARTIAL, SL_ROPE_KV = 0, 1, 2, 3, 4
 STREAM_TILE_ROWS, STREAM_TILE_K = 16, 32
 _STREAM_SIG = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
-               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
 
 
 class TiledWeight:
@@ -514,8 +527,8 @@ def gated_blocks_per_workgroup(out_features: int, compute_units: int) -> int:
 
 
 def stream_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, nt: int | None = None, splits: int | None = None,
-                  rope: dict | None = None) -> torch.Tensor:
-    """x [M, K] bfloat16 times the tiled weights.  SL_BF16 / SL_F32: [M, N]; SL_GATED: silu(gate) * up [M, N / 2];
+                  rope: dict | None = None, activation: str = "silu") -> torch.Tensor:
+    """x [M, K] bfloat16 times the tiled weights.  SL_BF16 / SL_F32: [M, N]; SL_GATED: act(gate) * up [M, N / 2];
     SL_PARTIAL: float [splits, M, N], the sums over ``splits`` ranges of K, to be added in that order; SL_ROPE_KV: q rotated
     [M, heads * d], k (rotated) and v written to their pages (``rope`` as for ``decode_linear``)."""
     _on_gpu(x, w.tiles)
@@ -558,12 +571,12 @@ def stream_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, nt: int |
     _check(f(epi, _ptr(x), x.stride(0), _ptr(w.tiles), _ptr(out), out.stride(-2), M, N, K, w.blocks, nt, splits,
              _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")), _ptr(r.get("k_pages")),
              _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)), int(r.get("head_dim", 0)),
-             int(r.get("block_size", 0)), _stream()), "stream_linear")
+             int(r.get("block_size", 0)), activation_code(activation), _stream()), "stream_linear")
     return out
 
 
 _TILE_SIG = [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
-             c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+             c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
 TILE_BLOCK_ROWS = 160           # input rows of one workgroup of the tiled kernel, at most
 
 
@@ -577,7 +590,8 @@ def tile_linear_plan(M: int, N: int, K: int, compute_units: int) -> int:
     return _whole_ranges(stages, max(1, min(compute_units // workgroups, stages // 4, 16)))
 
 
-def tile_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, splits: int | None = None, rope: dict | None = None) -> torch.Tensor:
+def tile_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, splits: int | None = None, rope: dict | None = None,
+                activation: str = "silu") -> torch.Tensor:
     """As ``stream_linear``, for a few hundred rows: tiles of up to 160 rows x 128 weight rows per workgroup, both
     operands through LDS."""
     _on_gpu(x, w.tiles)
@@ -616,7 +630,7 @@ def tile_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, splits: int
     _check(f(epi, _ptr(x), x.stride(0), _ptr(w.tiles), _ptr(out), out.stride(-2), M, N, K, w.blocks, splits,
              _ptr(r.get("positions")), _ptr(r.get("cos")), _ptr(r.get("sin")), _ptr(r.get("slots")), _ptr(r.get("k_pages")),
              _ptr(r.get("v_pages")), int(r.get("num_heads", 0)), int(r.get("num_kv_heads", 0)), int(r.get("head_dim", 0)),
-             int(r.get("block_size", 0)), _stream()), "tile_linear")
+             int(r.get("block_size", 0)), activation_code(activation), _stream()), "tile_linear")
     return out
 
 

@@ -57,6 +57,7 @@ struct StreamLinearParams {
   const int* positions; const float* cos_t; const float* sin_t; const int* slots;
   bf16* k_pages; bf16* v_pages;
   int num_heads, num_kv_heads, head_dim, block_size;
+  int activation;             // SL_GATED: the gate's activation (PLLM_ACT_*)
 };
 
 template <int N_>
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(kStreamThreads) void stream_linear_kernel(const Str
       const int n = unit * 8 + g * 4;
       bf16 o[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = __float2bfloat16((a[i] / (1.f + expf(-a[i]))) * up[i]);
+      for (int i = 0; i < 4; ++i) o[i] = __float2bfloat16(gate_activation(a[i], p.activation) * up[i]);
       bf16* dst = (bf16*)p.out + (size_t)m * p.ldo + n;
       if (n + 3 < p.N && (p.ldo & 3) == 0) *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(o);
       else {
@@ -295,7 +296,7 @@ PLLM_API int pllm_stream_linear_row_blocks(int M) { return (M + 127) / 128; }
 PLLM_API int pllm_stream_linear(int epi, const void* x, int ldx, const void* wt, void* out, int ldo, int M, int N, int K,
                                 int weight_blocks, int nt, int splits, const int* positions, const float* cos_t, const float* sin_t,
                                 const int* slots, void* k_pages, void* v_pages, int num_heads, int num_kv_heads, int head_dim,
-                                int block_size, hipStream_t stream) {
+                                int block_size, int activation, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K % kChunkK) || (ldx & 7) || nt < 1 || nt > 4 || weight_blocks <= 0 || (weight_blocks % 24) || splits < 1) return -2;
   if (splits > 1 && epi != SL_PARTIAL) return -2;
@@ -307,6 +308,8 @@ PLLM_API int pllm_stream_linear(int epi, const void* x, int ldx, const void* wt,
   p.x = (const bf16*)x; p.ldx = ldx; p.wt = (const bf16*)wt; p.out = out; p.ldo = ldo; p.M = M; p.N = N; p.K = K;
   p.positions = positions; p.cos_t = cos_t; p.sin_t = sin_t; p.slots = slots; p.k_pages = (bf16*)k_pages; p.v_pages = (bf16*)v_pages;
   p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.head_dim = head_dim; p.block_size = block_size;
+  if (activation < 0 || activation >= PLLM_ACT_COUNT) return -2;
+  p.activation = activation;
   p.ksteps = K / kChunkK;
   p.num_stages = (K + kStageK - 1) / kStageK;
   p.stages_per_split = (p.num_stages + splits - 1) / splits;
@@ -512,7 +515,7 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
           const int n = unit * 8 + g * 4;
           bf16 o[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o[i] = __float2bfloat16((a[i] / (1.f + expf(-a[i]))) * partner[i]);
+          for (int i = 0; i < 4; ++i) o[i] = __float2bfloat16(gate_activation(a[i], p.activation) * partner[i]);
           bf16* dst = (bf16*)p.out + (size_t)m * p.ldo + n;
           if (n + 3 < p.N && (p.ldo & 3) == 0) *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(o);
           else {
@@ -611,7 +614,7 @@ PLLM_API int pllm_tile_linear_row_blocks(int M) { return (M + 159) / 160; }
 PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, void* out, int ldo, int M, int N, int K,
                               int weight_blocks, int splits, const int* positions, const float* cos_t,
                               const float* sin_t, const int* slots, void* k_pages, void* v_pages, int num_heads, int num_kv_heads,
-                              int head_dim, int block_size, hipStream_t stream) {
+                              int head_dim, int block_size, int activation, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K % kChunkK) || (ldx & 7) || weight_blocks <= 0 || (weight_blocks % kTileBlocksN) || splits < 1) return -2;
   if (splits > 1 && epi != SL_PARTIAL) return -2;
@@ -623,6 +626,8 @@ PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, v
   p.x = (const bf16*)x; p.ldx = ldx; p.wt = (const bf16*)wt; p.out = out; p.ldo = ldo; p.M = M; p.N = N; p.K = K;
   p.positions = positions; p.cos_t = cos_t; p.sin_t = sin_t; p.slots = slots; p.k_pages = (bf16*)k_pages; p.v_pages = (bf16*)v_pages;
   p.num_heads = num_heads; p.num_kv_heads = num_kv_heads; p.head_dim = head_dim; p.block_size = block_size;
+  if (activation < 0 || activation >= PLLM_ACT_COUNT) return -2;
+  p.activation = activation;
   p.ksteps = K / kChunkK;
   p.num_stages = (p.ksteps + kTileStageSteps - 1) / kTileStageSteps;
   p.stages_per_split = (p.num_stages + splits - 1) / splits;

@@ -1,6 +1,6 @@
-"""Gated feed-forward: down(act(gate(x)) * up(x)) without bias, act = SiLU
-(pagedllm/model/llama.py:163-171).  gate and up are fused into one matrix [2I, H] when the
-weights arrive; the activation and the product run in float in one kernel."""
+"""Gated feed-forward: down(act(gate(x)) * up(x)) without bias; the reference's Llama has act = SiLU
+(pagedllm/model/llama.py:163-171), the part takes the activation as a parameter (``ops.ACTIVATIONS``).  gate and up
+are fused into one matrix [2I, H] when the weights arrive; the activation and the product run in float in one kernel."""
 
 from __future__ import annotations
 
@@ -20,9 +20,9 @@ class GatedMLP(FeedForward):
     def __init__(self, params: dict, env: BuildEnv):
         self.hidden = env.hidden_size
         self.inter = int(params["intermediate_size"])
-        act = params.get("activation", "silu")
-        if act != "silu":
-            raise NotImplementedError(f"gated feed-forward activation {act!r} (silu only)")
+        self.activation = params.get("activation", "silu")
+        if self.activation not in ops.ACTIVATIONS:
+            raise NotImplementedError(f"gated feed-forward activation {self.activation!r}: one of {sorted(ops.ACTIVATIONS)}")
         self.dtype, self.device = env.dtype, env.device
         self._w: dict[str, torch.Tensor] = {}
         self.w_gate_up: Weight | None = None
@@ -44,7 +44,7 @@ class GatedMLP(FeedForward):
         self._w.clear()
 
     def forward(self, h, ctx):
-        act = gated_linear(h, self.w_gate_up)
+        act = gated_linear(h, self.w_gate_up, self.activation)
         return linear(act, self.w_down, partial_ok=bool(getattr(ctx, "partial_sums_ok", False)))
 
 

@@ -92,13 +92,13 @@ def _streams(x, weight, epi: int) -> bool:
     return _few_weight_rows(weight) and (k < STREAM_LONG_K or rows <= STREAM_LONG_K_MAX_ROWS)
 
 
-def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: bool = False):
+def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: bool = False, activation: str = "silu"):
     x = rows_of(x)
     if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
         x = x.contiguous()
     n, k = weight.shape
     if epi == ops.SL_GATED:
-        return ops.stream_linear(x, weight.tiled, epi)
+        return ops.stream_linear(x, weight.tiled, epi, activation=activation)
     if epi == ops.SL_BF16 and partial_ok:
         nt, splits = ops.stream_linear_plan(x.shape[0], n, k, ops._num_compute_units(x.device), partial=True)
         if splits > 1:
@@ -109,7 +109,7 @@ def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: b
 _PAIRING_OF = {ops.EPI_GATED: "gated", ops.EPI_ROPE_KV: "rotary"}
 
 
-def _fused(x, weight, epi: int, rope: dict | None = None):
+def _fused(x, weight, epi: int, rope: dict | None = None, activation: str = "silu"):
     """The fused decode kernel if it takes the operands, else None.  With a ``Weight`` whose tiled copy has the pairing
     of the epilogue, products of at most 16 rows with the sum and norm in front stream the weights from that copy
     (11264 x 2048: 12.3 against 13.4 us; 2560 x 2048 with the rotary epilogue: 7.4 against 7.9; 32000 x 2048: 29.0 against 30.4)."""
@@ -121,7 +121,7 @@ def _fused(x, weight, epi: int, rope: dict | None = None):
     if isinstance(x, PendingNorm):
         if x.fusable() and ops.decode_linear_takes(x.num_rows, x.x.shape[1], x.x, weight):
             args = x.fused_arguments()
-            out = ops.decode_linear(x.x, weight, epi, rope=rope, tiled=tiled, **args)
+            out = ops.decode_linear(x.x, weight, epi, rope=rope, tiled=tiled, activation=activation, **args)
             x.fused_done(args)
             return out
         x = x.rows()
@@ -129,7 +129,7 @@ def _fused(x, weight, epi: int, rope: dict | None = None):
             and ops.decode_linear_pays(x.shape[0], weight.shape[0], x.shape[1], epi, staged=False)):
         # (plain rows keep the row-major matrix: from the tiled copy 4096 x 4096 and 4096 x 14336 took 10.7 and 32.9 us at 8
         #  rows against 9.3 and 27.7, and the smaller matrices the same time either way)
-        return ops.decode_linear(x, weight, epi, rope=rope)
+        return ops.decode_linear(x, weight, epi, rope=rope, activation=activation)
     return None
 
 
@@ -158,10 +158,11 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
 TILE_GATED_ROWS = (161, 320)                    # rows for which the gated product takes the tiled kernel
 
 
-def gated_linear(x, w_gate_up) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix (a tensor, or a ``Weight`` with the gated pairing)."""
+def gated_linear(x, w_gate_up, activation: str = "silu") -> torch.Tensor:
+    """act(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix (a tensor, or a ``Weight`` with the gated pairing);
+    ``activation``: one of ``ops.ACTIVATIONS``."""
     if _streams(x, w_gate_up, ops.SL_GATED) and w_gate_up.pairing == "gated":
-        return _stream(x, w_gate_up, ops.SL_GATED)
+        return _stream(x, w_gate_up, ops.SL_GATED, activation=activation)
     rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
     if (isinstance(w_gate_up, Weight) and w_gate_up.tiled is not None and w_gate_up.pairing == "gated" and x.dtype == torch.bfloat16
             and TILE_GATED_ROWS[0] <= rows <= TILE_GATED_ROWS[1]):
@@ -170,13 +171,13 @@ def gated_linear(x, w_gate_up) -> torch.Tensor:
         x = rows_of(x)
         if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
             x = x.contiguous()
-        return ops.tile_linear(x, w_gate_up.tiled, ops.SL_GATED)
+        return ops.tile_linear(x, w_gate_up.tiled, ops.SL_GATED, activation=activation)
     if w_gate_up.dtype == torch.bfloat16:
-        out = _fused(x, w_gate_up, ops.EPI_GATED)
+        out = _fused(x, w_gate_up, ops.EPI_GATED, activation=activation)
         if out is not None:
             return out
     w_gate_up = _plain(w_gate_up)
-    return ops.silu_mul(linear(x, w_gate_up))
+    return ops.gate_mul(linear(x, w_gate_up), activation)
 
 
 def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_heads: int, num_kv_heads: int,

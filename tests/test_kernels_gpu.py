@@ -101,6 +101,11 @@ def test_silu_mul(dtype):
     out = ops().silu_mul(gu.cuda())
     want = torch.nn.functional.silu(gu.float()[:, :inter]) * gu.float()[:, inter:]
     assert rel_err(out, want) <= TOL[dtype]
+    out = ops().gate_mul(gu.cuda(), "gelu_tanh")
+    want = torch.nn.functional.gelu(gu.float()[:, :inter], approximate="tanh") * gu.float()[:, inter:]
+    assert rel_err(out, want) <= TOL[dtype]
+    with pytest.raises(ops().KernelError):
+        ops().gate_mul(gu.cuda(), "gelu")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

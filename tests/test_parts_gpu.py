@@ -271,9 +271,34 @@ def test_feed_forward_part(dtype, tol, num_rows):
     assert rel(ff.forward(norm.pending(x.cuda()), None), want) <= tol
 
 
-def test_feed_forward_part_refuses_other_activations():
+def test_feed_forward_part_refuses_unknown_activations():
     with pytest.raises(NotImplementedError):
-        build("feed_forward", "gated_mlp", {"intermediate_size": 64, "activation": "gelu"}, env_for("bfloat16"))
+        build("feed_forward", "gated_mlp", {"intermediate_size": 64, "activation": "swish7"}, env_for("bfloat16"))
+
+
+@pytest.mark.parametrize("dtype,tol,num_rows", [("float32", 3e-5, 5), ("float32", 3e-5, 40)]
+                         + [("bfloat16", 3e-2, n) for n in (1, 8, 16, 40, 64, 130, 264, 700)])
+def test_feed_forward_part_with_another_activation(dtype, tol, num_rows):
+    """The gate's activation is a parameter of the part: GELU in its tanh form, through every kernel that holds the
+    activation (the fused decode product, the streaming and the tiled product's gated epilogues, the kernel of its own
+    behind the library's product; widths that give the weights their tiled copies), against the library's routine."""
+    hidden, inter = 256, 704
+    env = env_for(dtype, hidden=hidden)
+    ff = build("feed_forward", "gated_mlp", {"intermediate_size": inter, "activation": "gelu_tanh"}, env)
+    w = give_weights(ff, 18, dtype)
+    x = rows(num_rows, 19, dtype, hidden=hidden)
+
+    def want_of(h):
+        gate = torch.nn.functional.gelu(h @ w["gate_proj.weight"].T, approximate="tanh")
+        return (gate * (h @ w["up_proj.weight"].T)) @ w["down_proj.weight"].T
+    assert rel(ff.forward(x.cuda(), None), want_of(x.float())) <= tol
+    norm = build("norm", "rmsnorm", {"eps": EPS}, env)
+    nw = give_weights(norm, 20, dtype)["weight"]
+    h = plain.rms_norm(x.float(), nw, EPS).to(x.dtype).float()
+    assert rel(ff.forward(norm.pending(x.cuda()), None), want_of(h)) <= tol
+    # (the other activation would not pass: the two results are further apart than the bound)
+    silu = torch.nn.functional.silu(x.float() @ w["gate_proj.weight"].T) * (x.float() @ w["up_proj.weight"].T) @ w["down_proj.weight"].T
+    assert rel(silu, want_of(x.float())) > 2 * tol
 
 
 # ------------------------------------------------------------------------------------------ block
