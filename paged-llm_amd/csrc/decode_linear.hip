@@ -31,6 +31,7 @@ enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_GATED = 2, EPI_ROPE_KV = 3 };
 
 struct DecodeLinearParams {
   const bf16* x; int ldx;
+  int activation;              // EPI_GATED: the gate's activation (PLLM_ACT_*); here it fills a gap, and the arguments keep their places
   const bf16* delta; int ldd;
   const float* norm_w; float eps;
   bf16* x_out; int ldxo;
@@ -43,7 +44,6 @@ struct DecodeLinearParams {
   const int* positions; const float* cos_t; const float* sin_t; const int* slots;
   bf16* k_pages; bf16* v_pages;
   int num_heads, num_kv_heads, head_dim, block_size;
-  int activation;              // EPI_GATED: the gate's activation (PLLM_ACT_*)
 };
 
 __device__ __forceinline__ bf16x8 zero8() {

@@ -47,6 +47,7 @@ enum { SL_BF16 = 0, SL_F32 = 1, SL_GATED = 2, SL_PARTIAL = 3, SL_ROPE_KV = 4 };
 
 struct StreamLinearParams {
   const bf16* x; int ldx;
+  int activation;             // SL_GATED: the gate's activation (PLLM_ACT_*); here it fills a gap, and the arguments keep their places
   const bf16* wt;             // tiled weights [blocks of 16 rows][K / 32][64 lanes][8]
   void* out; int ldo;         // SL_PARTIAL: float [splits][M][ldo]
   int M, N, K;                // N: outputs (gated: half the weight rows)
@@ -57,7 +58,6 @@ struct StreamLinearParams {
   const int* positions; const float* cos_t; const float* sin_t; const int* slots;
   bf16* k_pages; bf16* v_pages;
   int num_heads, num_kv_heads, head_dim, block_size;
-  int activation;             // SL_GATED: the gate's activation (PLLM_ACT_*)
 };
 
 template <int N_>
