@@ -79,7 +79,8 @@ _SIGNATURES = {
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                      c_void_p],
     "pllm_sample": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_ulonglong, c_void_p,
-                    c_void_p],
+                    c_void_p, c_void_p],
+    "pllm_sample_workspace_bytes": [c_int, c_int],
     "pllm_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p],
 }
 _FUNCS: dict = {}
@@ -295,9 +296,29 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
+_sample_workspace: dict = {}
+
+
+def rows_sampled_by_candidates(rows: int, vocab: int, device) -> list:
+    """For the last ``sample`` call of this shape on the device: which rows went by their candidates (a look into the
+    call's workspace, for tests and measurements)."""
+    f = _fn("sampling.hip", "pllm_sample_workspace_bytes")
+    f.restype = c_long
+    need = int(f(rows, vocab))
+    workspace = _sample_workspace.get(str(torch.device(device)))
+    if not need or workspace is None:
+        return [False] * rows
+    chunks = need // 4 // (3 + 2 * 192) // rows
+    counts = workspace[: rows * chunks * 4].view(torch.int32).view(rows, chunks)
+    return (counts >= 0).all(dim=1).tolist()
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           request_key: torch.Tensor, step: torch.Tensor, seed: int) -> torch.Tensor:
-    """One token per row: greedy where temperature < 1e-5, else a draw under top-k / top-p."""
+           request_key: torch.Tensor, step: torch.Tensor, seed: int, candidates: bool = True) -> torch.Tensor:
+    """One token per row: greedy where temperature < 1e-5, else a draw under top-k / top-p.  ``candidates``: few rows
+    of a long vocabulary whose top_k is small are first cut into chunks that hand on their largest logits, and the
+    search and the draw run over those (a row's token depends on its own settings only either way; False walks every
+    row whole)."""
     _on_gpu(logits, temperature, top_k, top_p, request_key, step)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "logits: contiguous float32 [n, vocab]")
     n, V = logits.shape
@@ -305,9 +326,18 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
                       (request_key, torch.int64, "request_key"), (step, torch.int32, "step")):
         _need(t.dtype == dt and t.shape == (n,) and t.is_contiguous(), f"{nm}: {dt} [{n}]")
     out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    workspace = None
+    if candidates:
+        f = _fn("sampling.hip", "pllm_sample_workspace_bytes")
+        f.restype = c_long
+        need = int(f(n, V))
+        if need:
+            workspace = _sample_workspace.get(str(logits.device))
+            if workspace is None or workspace.numel() < need:
+                workspace = _sample_workspace[str(logits.device)] = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=logits.device)
     _check(_fn("sampling.hip", "pllm_sample")(_ptr(logits), n, V, _ptr(temperature), _ptr(top_k), _ptr(top_p),
                                                _ptr(request_key), _ptr(step), c_ulonglong(seed & (2**64 - 1)), _ptr(out),
-                                               _stream()), "sample")
+                                               _ptr(workspace), _stream()), "sample")
     return out
 
 

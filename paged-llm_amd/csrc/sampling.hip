@@ -12,6 +12,13 @@
 // The draw is the inverse CDF over the kept tokens in a fixed order (thread by thread) with one uniform
 // number per row from Philox4x32-10 keyed by (seed, request key, step), so a request's tokens do not
 // depend on its neighbours; every sum is taken in an order that depends on the row's length only.
+//
+// Few rows of a long vocabulary with a small top_k (the usual settings of a decode step) would leave the GPU to as
+// many workgroups as there are rows, each walking its whole row a dozen times.  For them the row is first cut into
+// chunks, one workgroup each (sample_candidates_kernel): a chunk hands on every logit that may be among the row's
+// top_k largest, a few more than top_k of its own, and its share of the sum of weights; the search and the draw then
+// run over those few hundred candidates (the same kernel, on the candidates instead of the row).  A row whose chunks
+// have too many candidates (many equal logits) goes the long way.
 #include "common.h"
 
 using namespace pllm;
@@ -38,6 +45,20 @@ __device__ __forceinline__ uint32_t float_key(float f) {
   const uint32_t u = __float_as_uint(f);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
+
+// Largest / smallest of one unsigned value per thread over the workgroup (scratch: 16 words of LDS).
+__device__ __forceinline__ uint32_t float_as_uint_max(uint32_t v, float* scratch) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, 64));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  __syncthreads();
+  if (lane == 0) reinterpret_cast<uint32_t*>(scratch)[wave] = v;
+  __syncthreads();
+  uint32_t t = reinterpret_cast<uint32_t*>(scratch)[0];
+  for (int w = 1; w < nwaves; ++w) t = max(t, reinterpret_cast<uint32_t*>(scratch)[w]);
+  return t;
+}
+__device__ __forceinline__ uint32_t float_as_uint_min(uint32_t v, float* scratch) { return ~float_as_uint_max(~v, scratch); }
 
 struct ArgMax { float v; int i; };
 __device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {
@@ -127,13 +148,13 @@ __device__ __forceinline__ float block_exclusive_scan(float v, float* fs, float&
 
 // f(value, index) for every element of the calling thread, in its fixed order; the visitor goes in and comes back by
 // value, so that what it gathers stays in registers.
-template <bool IN_REGS, bool VEC, class F>
-__device__ __forceinline__ F for_each_element(const float (&held)[IN_REGS ? kSlots : 1], const float* __restrict__ z, int units, int tid, F f) {
+template <bool IN_REGS, bool VEC, int HELD, class F>
+__device__ __forceinline__ F for_each_element(const float (&held)[HELD], const float* __restrict__ z, int units, int tid, F f) {
   constexpr int kPer = VEC ? 4 : 1;
   constexpr int kFlight = 8;                                     // requests under way per thread in a pass over memory
   if constexpr (IN_REGS) {
 #pragma unroll
-    for (int s = 0; s < kSlots; ++s) {
+    for (int s = 0; s < HELD; ++s) {
       const int u = (s / kPer) * kSampleThreads + tid, i = u * kPer + (s % kPer);
       if (u < units) f(held[s], i);
     }
@@ -263,24 +284,202 @@ struct Pick {                          // the first kept token at which the runn
   }
 };
 
-template <bool IN_REGS, bool VEC>
-__global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
-                                                                const int* __restrict__ top_k, const float* __restrict__ top_p,
-                                                                const long long* __restrict__ request_key, const int* __restrict__ step,
-                                                                unsigned long long seed, int* __restrict__ out) {
+// ---------------------------------------------------------------------------------------------
+// Candidates of a row: see the head of the file.  A row of `vocab` logits is cut into `chunks` chunks of `chunk` logits.
+constexpr int kCandThreads = 256;
+constexpr int kChunkPerThread = 16;          // logits of a chunk per thread (held in registers)
+constexpr int kChunkMost = kCandThreads * kChunkPerThread;
+constexpr int kMaxChunks = 64;               // (vocabularies of up to 262,144)
+constexpr int kChunkCap = 192;               // candidates a chunk may hand on (about 90 are expected at the largest top_k)
+constexpr int kCandTopK = 64;                // largest top_k that goes this way
+constexpr int kMaxCandidates = kMaxChunks * kChunkCap;
+static_assert(kMaxChunks <= 64, "a lane per chunk");
+static_assert(kCandThreads == 256 && kCandTopK <= kCandThreads, "four wavefronts, each with at least k / 4 threads");
+
+struct Candidates {                          // per row and chunk; null `count`: no candidates in this launch
+  int* count;                                // candidates of the chunk; -1: the row goes the long way
+  float* top;                                // the chunk's largest logit
+  float* sum;                                // sum over the chunk of 2^((v - top) * rate)
+  float* value;                              // [kChunkCap] per chunk
+  int* index;                                // their places in the row
+  int chunks, chunk;
+};
+
+__device__ __forceinline__ bool goes_by_candidates(float temp, int k, int vocab) { return temp >= 1e-5f && k > 0 && k <= kCandTopK && k < vocab; }
+
+__global__ __launch_bounds__(kCandThreads) void sample_candidates_kernel(const float* __restrict__ logits, int vocab,
+                                                                         const float* __restrict__ temperature,
+                                                                         const int* __restrict__ top_k, const Candidates cd) {
+  __shared__ float fscratch[16];
+  __shared__ float taus[kCandThreads / 64];
+  __shared__ int wave_counts[kCandThreads / 64];
+  const int row = blockIdx.y, c = blockIdx.x, tid = threadIdx.x;
+  const size_t slot = (size_t)row * cd.chunks + c;
+  const float temp = temperature[row];
+  const int k = top_k[row];
+  if (!goes_by_candidates(temp, k, vocab)) {
+    if (tid == 0) cd.count[slot] = -1;
+    return;
+  }
+  const float* z = logits + (size_t)row * vocab;
+  const int begin = c * cd.chunk, end = min(vocab, begin + cd.chunk);
+  // The chunk into registers (all loads under way at once), then this thread's largest and the chunk's largest.
+  float v[kChunkPerThread];
+#pragma unroll
+  for (int j = 0; j < kChunkPerThread; ++j) {
+    const int i = begin + j * kCandThreads + tid;
+    v[j] = i < end ? z[i] : -INFINITY;
+  }
+  float mine = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < kChunkPerThread; ++j) mine = fmaxf(mine, v[j]);
+  const float top = block_max(mine, fscratch);
+  // A bound from below on the chunk's k-th largest logit: each of the four wavefronts sorts its threads' largest (a
+  // bitonic network over the lanes) and takes the ceil(k / 4)-th; at least k logits of the chunk are as large as the
+  // smallest of those four, so the chunk's own k largest, and with them every logit of the chunk that may be among
+  // the row's k largest, are at or above it.
+  const int lane = tid & 63, wave = tid >> 6;
+  float sorted = mine;
+#pragma unroll
+  for (int size = 2; size <= 64; size <<= 1) {
+#pragma unroll
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      const float other = __shfl_xor(sorted, stride, 64);
+      const bool larger_here = ((lane & stride) == 0) == ((lane & size) == 0);     // (descending over the lanes in the end)
+      sorted = larger_here ? fmaxf(sorted, other) : fminf(sorted, other);
+    }
+  }
+  const float of_wave = __shfl(sorted, (k + 3) / 4 - 1, 64);
+  if (lane == 0) taus[wave] = of_wave;
+  __syncthreads();
+  const float tau = fminf(fminf(taus[0], taus[1]), fminf(taus[2], taus[3]));
+  // the chunk's share of the sum of weights, and how many of this thread's logits go on
+  const float rate = 1.4426950408889634f / fmaxf(temp, 1e-5f);
+  float sum = 0.f;
+  int n = 0;
+#pragma unroll
+  for (int j = 0; j < kChunkPerThread; ++j) {
+    const bool there = begin + j * kCandThreads + tid < end;
+    sum += there ? __builtin_amdgcn_exp2f((v[j] - top) * rate) : 0.f;
+    n += there && v[j] >= tau ? 1 : 0;
+  }
+  sum = block_sum(sum, fscratch);
+  // places in thread order: the wavefront's prefix, then the wavefronts before it
+  int incl = n;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  if (lane == 63) wave_counts[wave] = incl;
+  __syncthreads();
+  int before = incl - n, all = 0;
+  for (int w = 0; w < kCandThreads / 64; ++w) {
+    if (w < wave) before += wave_counts[w];
+    all += wave_counts[w];
+  }
+  if (tid == 0) {
+    cd.count[slot] = all <= kChunkCap ? all : -1;
+    cd.top[slot] = top;
+    cd.sum[slot] = sum;
+  }
+  if (all > kChunkCap) return;
+#pragma unroll
+  for (int j = 0; j < kChunkPerThread; ++j) {
+    const int i = begin + j * kCandThreads + tid;
+    if (i < end && v[j] >= tau) {
+      cd.value[slot * kChunkCap + before] = v[j];
+      cd.index[slot * kChunkCap + before] = i;
+      ++before;
+    }
+  }
+}
+
+// Whether a row's candidates are there (every chunk handed its own on); the same answer in both kernels below and in
+// every wavefront (a lane looks at one chunk: at most 64 of them).
+__device__ __forceinline__ bool has_candidates(const Candidates& cd, int row) {
+  const int lane = threadIdx.x & 63;
+  const int n = lane < cd.chunks ? cd.count[(size_t)row * cd.chunks + lane] : 0;
+  return __all(n >= 0);
+}
+
+// One row's token.  CAND: over the row's candidates; else over the whole row.
+template <bool IN_REGS, bool VEC, bool CAND>
+__device__ __forceinline__ void sample_row(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
+                                           const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                           const long long* __restrict__ request_key, const int* __restrict__ step,
+                                           unsigned long long seed, int* __restrict__ out, const Candidates& cd) {
+  static_assert(!CAND || (IN_REGS && !VEC), "candidates are few and of any number");
   __shared__ float fscratch[16];
   __shared__ int iscratch[80];
   __shared__ ArgMax ascratch[16];
   __shared__ int chosen, chooser;
+  __shared__ int starts[65];                                     // CAND: where each chunk's candidates begin (a lane per chunk), and their number
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* z = logits + (size_t)row * vocab;
-  const int units = VEC ? vocab >> 2 : vocab;                    // pieces of four, or single elements
+  int units = VEC ? vocab >> 2 : vocab;                          // pieces of four, or single elements
   constexpr int kPer = VEC ? 4 : 1;
+  float total_of_row = 0.f;                                      // CAND: the sum of the whole row's weights
+  if constexpr (CAND) {
+    // The chunks' candidates side by side in LDS, in the order of the chunks; the row's sum of weights from the
+    // chunks' shares (relative to the row's largest logit, in the order of the chunks).
+    __shared__ float gathered[kMaxCandidates];
+    __shared__ float total_s;
+    // (the first wavefront, a lane per chunk: where each chunk's candidates begin, the row's largest logit and its sum
+    //  of weights; sums over lanes in the fixed order of wave_sum)
+    if (tid < 64) {
+      const bool there = tid < cd.chunks;
+      const int n = there ? cd.count[(size_t)row * cd.chunks + tid] : 0;
+      const float chunk_top = there ? cd.top[(size_t)row * cd.chunks + tid] : -INFINITY;
+      const float chunk_sum = there ? cd.sum[(size_t)row * cd.chunks + tid] : 0.f;
+      int incl = n;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o, 64);
+        if (tid >= o) incl += up;
+      }
+      starts[tid] = incl - n;
+      if (tid == 63) starts[64] = incl;
+      const float top = wave_max(chunk_top);
+      const float rate = 1.4426950408889634f / fmaxf(temperature[row], 1e-5f);
+      const float sum = wave_sum(there ? chunk_sum * __builtin_amdgcn_exp2f((chunk_top - top) * rate) : 0.f);
+      if (tid == 0) total_s = sum;
+    }
+    __syncthreads();
+    // Wavefront w gathers chunks w, w + 8, ...: all of a wavefront's loads are requested before the first is stored.
+    {
+      const int lane = tid & 63, wave = tid >> 6;
+      constexpr int kTurns = kMaxChunks / (kSampleThreads / 64), kPieces = kChunkCap / 64;
+      float got[kTurns][kPieces];
+#pragma unroll
+      for (int turn = 0; turn < kTurns; ++turn) {
+        const int c = wave + turn * (kSampleThreads / 64);
+        const int n = c < cd.chunks ? starts[c + 1] - starts[c] : 0;
+#pragma unroll
+        for (int q = 0; q < kPieces; ++q)
+          got[turn][q] = lane + q * 64 < n ? cd.value[((size_t)row * cd.chunks + c) * kChunkCap + lane + q * 64] : 0.f;
+      }
+#pragma unroll
+      for (int turn = 0; turn < kTurns; ++turn) {
+        const int c = wave + turn * (kSampleThreads / 64);
+        const int n = c < cd.chunks ? starts[c + 1] - starts[c] : 0;
+#pragma unroll
+        for (int q = 0; q < kPieces; ++q)
+          if (lane + q * 64 < n) gathered[starts[c] + lane + q * 64] = got[turn][q];
+      }
+    }
+    __syncthreads();
+    units = starts[64];
+    total_of_row = total_s;
+    z = gathered;
+  }
+  const int num_elements = CAND ? units : vocab;
 
-  float held[IN_REGS ? kSlots : 1];
+  constexpr int kHeld = !IN_REGS ? 1 : (CAND ? kMaxCandidates / kSampleThreads : kSlots);      // elements of a thread in registers
+  float held[kHeld];
   if constexpr (IN_REGS) {
 #pragma unroll
-    for (int s = 0; s < kSlots; s += kPer) {
+    for (int s = 0; s < kHeld; s += kPer) {
       const int u = (s / kPer) * kSampleThreads + tid;
       if constexpr (VEC) {
         const float4 t = u < units ? reinterpret_cast<const float4*>(z)[u] : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -290,7 +489,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
       }
     }
   }
-#define PLLM_WALK(visitor) for_each_element<IN_REGS, VEC>(held, z, units, tid, visitor)
+#define PLLM_WALK(visitor) for_each_element<IN_REGS, VEC, kHeld>(held, z, units, tid, visitor)
 
   Extremes ex; ex.best.v = -INFINITY; ex.best.i = 0x7fffffff; ex.lowest = INFINITY;
   ex = PLLM_WALK(ex);
@@ -303,9 +502,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   Weigh weigh; weigh.zmax = best.v; weigh.rate = 1.4426950408889634f / fmaxf(temp, 1e-5f);
 
   int k = top_k[row];
-  if (k <= 0 || k > vocab) k = vocab;
+  if (k <= 0 || k > num_elements) k = num_elements;
   const float p = top_p[row];
-  const bool filtered = k < vocab || p < 1.f;
+  const bool filtered = k < num_elements || p < 1.f;
   // The sum of all weights: a pass of its own where nothing is filtered, else part of the search's first pass.
   SumOfWeights sw; sw.w = weigh; sw.sum = 0.f;
   float total = 0.f;
@@ -317,7 +516,107 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   constexpr int kSlotsHere = kWindowSlots<IN_REGS>;
   IntoWindow<kSlotsHere> win; win.n = 0; win.mass_up = 0.f;
   bool windowed = false;
-  if (filtered) {
+  if constexpr (CAND) {
+    if (filtered) {
+      // Few candidates, all in registers: first the k-th largest key, by histograms of 256 bins over the range of keys that
+      // still holds it (at first from the smallest to the largest candidate; the bin in which the k-th falls is the
+      // next range: three passes for keys a few million apart), then the fewer than k candidates above it, each with
+      // the weight of those above it, and the group at the k-th key as one.
+      __shared__ int hist[256];
+      __shared__ uint32_t lo_s, hi_s;
+      __shared__ int rank_s;
+      __shared__ uint32_t up_key[kCandTopK];
+      __shared__ float up_weight[kCandTopK];
+      __shared__ int up_counts[kSampleThreads / 64];
+      total = total_of_row;
+      const float lowest = -block_max(-ex.lowest, fscratch);
+      uint32_t lo = float_key(lowest), hi = float_key(best.v);
+      int rank = k;                                              // the key looked for is the rank-th largest of those in [lo, hi]
+      for (;;) {
+        const uint32_t span = hi - lo;
+        const int shift = span < 256u ? 0 : 24 - __clz(span);    // (span >> shift) < 256
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int s2 = 0; s2 < kHeld; ++s2) {
+          if (s2 * kSampleThreads + tid < units) {
+            const uint32_t key = float_key(held[s2]);
+            if (key - lo <= span) atomicAdd(&hist[(key - lo) >> shift], 1);
+          }
+        }
+        __syncthreads();
+        if (tid < 64) {                                          // lane l: bins 255 - 4 l down to 252 - 4 l
+          int mine[4], sum = 0;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) { mine[j] = hist[255 - 4 * tid - j]; sum += mine[j]; }
+          int incl = sum;
+#pragma unroll
+          for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(incl, o, 64);
+            if (tid >= o) incl += up;
+          }
+          const unsigned long long reached = __ballot(incl >= rank);
+          const int first = reached ? __ffsll((long long)reached) - 1 : 63;       // (the range holds at least rank candidates)
+          if (tid == first) {
+            int before = incl - sum, j = 0;
+            while (j < 3 && before + mine[j] < rank) { before += mine[j]; ++j; }
+            const uint32_t bin = 255 - 4 * tid - j;
+            const unsigned long long top_of_bin = (unsigned long long)lo + ((unsigned long long)bin << shift) + ((1ull << shift) - 1);
+            lo_s = lo + (bin << shift);
+            hi_s = top_of_bin < hi ? (uint32_t)top_of_bin : hi;
+            rank_s = rank - before;
+          }
+        }
+        __syncthreads();
+        lo = lo_s; hi = hi_s; rank = rank_s;
+        if (shift == 0) break;                                   // (a bin was one key)
+      }
+      const uint32_t found = lo;
+      const uint32_t kth = found;                                // k - rank candidates lie above it
+      // the candidates above the k-th key, in the order of the threads
+      int mine_up = 0;
+#pragma unroll
+      for (int s2 = 0; s2 < kHeld; ++s2) mine_up += (s2 * kSampleThreads + tid < units && float_key(held[s2]) > kth) ? 1 : 0;
+      const int lane = tid & 63, wave = tid >> 6;
+      int incl = mine_up;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+      }
+      if (lane == 63) up_counts[wave] = incl;
+      __syncthreads();
+      int at = incl - mine_up, num_up = 0;
+      for (int w = 0; w < kSampleThreads / 64; ++w) {
+        if (w < wave) at += up_counts[w];
+        num_up += up_counts[w];
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < kHeld; ++s2) {
+        if (s2 * kSampleThreads + tid < units && float_key(held[s2]) > kth) {
+          up_key[at] = float_key(held[s2]);
+          up_weight[at] = weigh(held[s2]);
+          ++at;
+        }
+      }
+      __syncthreads();
+      // Thread i < num_up: candidate i above the k-th key stays if what lies above it weighs at most p of the row;
+      // thread num_up: the group at the k-th key, above which all of them lie.  (Fewer than k lie above each.)
+      uint32_t dropped = 0, my_key = 0;
+      if (tid <= num_up) {
+        my_key = tid < num_up ? up_key[tid] : kth;
+        float above = 0.f;
+#pragma unroll 8
+        for (int j = 0; j < num_up; ++j) above += up_key[j] > my_key ? up_weight[j] : 0.f;
+        if (!(above <= p * total)) dropped = my_key;
+      }
+      // the largest key that goes; what stays is what lies above it
+      const uint32_t cut = float_as_uint_max(dropped, fscratch);
+      uint32_t lowest_kept = 0xffffffffu;
+      if (tid <= num_up && my_key > cut) lowest_kept = my_key;
+      threshold = float_as_uint_min(lowest_kept, fscratch);
+    }
+  } else if (filtered) {
     // kept(c)  <=>  count(key > c) < k  and  mass(key > c) <= p * total  is monotone in c; the threshold is the
     // smallest key of a token that stays.  [lo, hi]: kept(hi) holds, kept(lo - 1) does not, and both ends are keys of
     // tokens of the row (at the start its minimum, which cannot stay, and its maximum, which always does).  A pass takes
@@ -413,20 +712,68 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   }
   __syncthreads();
   // (a row without a finite weight: the maximum)
-  if (tid == 0) out[row] = chosen >= 0 ? chosen : best.i;
+  if (tid == 0) {
+    int token = chosen >= 0 ? chosen : best.i;
+    if constexpr (CAND) {                                          // the candidate's place in the row
+      int c = 0;
+      while (c + 1 < cd.chunks && token >= starts[c + 1]) ++c;
+      token = cd.index[((size_t)row * cd.chunks + c) * kChunkCap + (token - starts[c])];
+    }
+    out[row] = token;
+  }
 #undef PLLM_WALK
 }
 
+// A workgroup per row: by the row's candidates where every chunk handed its own on, else over the whole row.
+template <bool IN_REGS, bool VEC>
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
+                                                                const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                                const long long* __restrict__ request_key, const int* __restrict__ step,
+                                                                unsigned long long seed, int* __restrict__ out, const Candidates cd) {
+  if (cd.count && has_candidates(cd, blockIdx.x)) sample_row<true, false, true>(logits, vocab, temperature, top_k, top_p, request_key, step, seed, out, cd);
+  else sample_row<IN_REGS, VEC, false>(logits, vocab, temperature, top_k, top_p, request_key, step, seed, out, cd);
+}
+
+// Bytes of workspace with which pllm_sample sends rows with a small top_k by their candidates; 0: it would not (many
+// rows keep the GPU busy by themselves, a short row is walked quickly).
+static int candidate_chunks(int rows, int vocab, int* chunk) {
+  if (rows > 128 || vocab < 8192 || vocab > kMaxChunks * kChunkMost) return 0;
+  int chunks = (vocab + 2047) / 2048;
+  if (chunks > kMaxChunks) chunks = kMaxChunks;
+  *chunk = ((vocab + chunks - 1) / chunks + kCandThreads - 1) / kCandThreads * kCandThreads;      // at most kChunkMost
+  return (vocab + *chunk - 1) / *chunk;
+}
+PLLM_API long pllm_sample_workspace_bytes(int rows, int vocab) {
+  int chunk = 0;
+  const long slots = (long)rows * candidate_chunks(rows, vocab, &chunk);
+  return slots * (3 + 2 * kChunkCap) * 4;
+}
+
+// workspace: null, or pllm_sample_workspace_bytes(rows, vocab) bytes (16-byte aligned) that the call may use.
 PLLM_API int pllm_sample(const float* logits, int rows, int vocab, const float* temperature, const int* top_k,
                          const float* top_p, const long long* request_key, const int* step, unsigned long long seed,
-                         int* out, hipStream_t stream) {
+                         int* out, void* workspace, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) return -2;
   const bool vec = (vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0;
   const bool in_regs = vocab <= kSlots * kSampleThreads;
+  Candidates cd = {};
+  int chunk = 0;
+  const int chunks = workspace ? candidate_chunks(rows, vocab, &chunk) : 0;
+  if (chunks > 0) {
+    const size_t slots = (size_t)rows * chunks;
+    cd.count = (int*)workspace;
+    cd.top = (float*)workspace + slots;
+    cd.sum = (float*)workspace + 2 * slots;
+    cd.value = (float*)workspace + 3 * slots;
+    cd.index = (int*)workspace + (3 + kChunkCap) * slots;
+    cd.chunks = chunks;
+    cd.chunk = chunk;
+    hipLaunchKernelGGL(sample_candidates_kernel, dim3(chunks, rows), dim3(kCandThreads), 0, stream, logits, vocab, temperature, top_k, cd);
+  }
 #define PLLM_SAMPLE(IN_REGS_, VEC_)                                                                                          \
   hipLaunchKernelGGL((sample_kernel<IN_REGS_, VEC_>), dim3(rows), dim3(kSampleThreads), 0, stream, logits, vocab, temperature, top_k, \
-                     top_p, request_key, step, seed, out)
+                     top_p, request_key, step, seed, out, cd)
   if (in_regs && vec) PLLM_SAMPLE(true, true);
   else if (in_regs) PLLM_SAMPLE(true, false);
   else if (vec) PLLM_SAMPLE(false, true);

@@ -386,6 +386,66 @@ def test_sampling_keeps_or_drops_equal_logits_together(vocab):
     assert set(sample_rows(z, 1.0, -1, p_between, 300)[:, 0].tolist()) == {5, vocab // 2, vocab - 3}
 
 
+def kept_by_the_stated_rule(z_row, temperature, top_k, top_p):
+    """Probabilities under the rule the kernel states for itself: a token stays if fewer than top_k tokens have a larger
+    logit and the tokens with a larger logit weigh at most top_p; equal logits stay or go together (where no tie lies at
+    the cut this is the reference's distribution, pagedllm/sampler.py:21-35)."""
+    zz = z_row.double() / max(temperature, 1e-5)
+    n = zz.numel()
+    sz, idx = zz.sort(descending=True)
+    probs = torch.softmax(sz, 0)
+    exclusive = probs.cumsum(0) - probs
+    starts = torch.ones(n, dtype=torch.bool)
+    starts[1:] = sz[1:] != sz[:-1]
+    first = torch.cummax(torch.where(starts, torch.arange(n), torch.zeros(n, dtype=torch.long)), 0).values      # where each run of equal logits begins
+    keep = (first < (top_k if top_k > 0 else n)) & (exclusive[first] <= top_p)
+    out = torch.zeros(n, dtype=torch.double)
+    out[idx[keep]] = torch.softmax(sz[keep], 0)
+    return out
+
+
+@pytest.mark.parametrize("vocab", [32000, 50001, 128256, 262144])
+@pytest.mark.parametrize("top_k,top_p", [(50, 0.9), (64, 1.0), (1, 1.0), (20, 0.3)])
+def test_sampling_by_candidates_keeps_what_the_whole_row_keeps(vocab, top_k, top_p):
+    """Rows of a long vocabulary with a small top_k are cut into chunks that hand on their largest logits, and the search
+    and the draw run over those.  Three kinds of row: noise, a row in which few tokens carry the mass, and a row with
+    a group of equal logits across the cut at top_k (all of them stay).  Every drawn token belongs to the kept set, a
+    small kept set is drawn in full with frequencies that follow its probabilities, and the rows did go by their
+    candidates; a row of equal logits, whose chunks have too many candidates, goes the long way."""
+    z = rnd(4, vocab, seed=41, scale=1.0)
+    z[1] = z[1] * 0.1
+    z[1, (torch.arange(12) * 2503 + 7) % vocab] += torch.linspace(9.0, 6.0, 12)
+    tie = torch.topk(z[2], top_k + 3).indices[max(top_k - 2, 0):]        # ranks top_k - 1 .. top_k + 3 share one logit
+    z[2, tie] = z[2, tie].max()
+    z[3] = 1.5
+    draws = 400
+    got = sample_rows(z, 0.8, top_k, top_p, draws)
+    by_candidates = ops().rows_sampled_by_candidates(4, vocab, "cuda:0")
+    assert by_candidates == [True, True, True, False], by_candidates
+    for row in range(4):
+        probs = kept_by_the_stated_rule(z[row], 0.8, top_k, top_p)
+        if row < 2:                                                   # (no equal logits at the cut: the reference's own support)
+            assert torch.equal(probs > 0, plain.filtered_probabilities(z[row], 0.8, top_k, top_p) > 0)
+        drawn = got[:, row].long()
+        assert bool((probs[drawn] > 0).all()), f"row {row}: a filtered token was drawn"
+        kept = torch.nonzero(probs > 0).flatten()
+        if 0 < len(kept) <= 12:
+            assert set(drawn.tolist()) == set(kept.tolist()), f"row {row}"
+            counts = np.array([(drawn == i).sum().item() for i in kept])
+            want = probs[kept].numpy() * draws
+            chi2, dof = float(((counts - want) ** 2 / want).sum()), len(kept) - 1
+            assert chi2 < dof + 5 * math.sqrt(2 * max(dof, 1)) + 5, f"row {row}: chi-square {chi2:.1f} for {dof} degrees of freedom"
+    # the same rows walked whole: other draws (the tokens stand in another order), the same kept sets
+    zg = z.cuda()
+    t, k, p = torch.full((4,), 0.8).cuda(), torch.full((4,), top_k, dtype=torch.int32).cuda(), torch.full((4,), top_p).cuda()
+    keys = torch.arange(4, dtype=torch.int64).cuda()
+    kept_sets = [kept_by_the_stated_rule(z[row], 0.8, top_k, top_p) > 0 for row in range(4)]
+    for step in range(40):
+        whole = ops().sample(zg, t, k, p, keys, torch.full((4,), step, dtype=torch.int32).cuda(), 0, candidates=False).cpu()
+        for row in range(4):
+            assert bool(kept_sets[row][int(whole[row])]), (step, row)
+
+
 def test_sampling_rows_do_not_depend_on_their_neighbours():
     z = rnd(5, 50001, seed=23, scale=2.0)
     alone = torch.stack([sample_rows(z[r:r + 1], 0.9, 30, 0.9, 4)[:, 0] for r in range(5)], dim=1)
