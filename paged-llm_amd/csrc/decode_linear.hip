@@ -5,7 +5,7 @@
 //                         residual is written out by workgroup 0; RMS norm in float: the elements
 //                         take the norm's weights here, the row's 1 / rms goes onto the finished sums
 //   product               rows[M, K] * W[N, K]^T on the matrix cores, float accumulation
-//   epilogue              plain (bfloat16 or float out) | silu(gate) * up | rotary encoding of q and
+//   epilogue              plain (bfloat16 or float out) | act(gate) * up | rotary encoding of q and
 //                         k and the write of k, v into their cache pages
 //
 // One workgroup of 8 wavefronts owns units of 16 weight rows over all of K.  Its wavefronts deal the K

@@ -26,7 +26,7 @@
 //
 // One workgroup barrier per stage (an s_barrier alone: it does not wait for loads under way, so the weights keep
 // streaming across it).  At the end the eight wavefronts' sums are added through LDS in wavefront order and the epilogue
-// runs: bfloat16 or float out, silu(gate) * up, the rotary encoding of q and k with the write of k and v into their cache
+// runs: bfloat16 or float out, act(gate) * up, the rotary encoding of q and k with the write of k and v into their cache
 // pages, or float partial sums of a range of K ([splits, M, N]: matrices with few rows are cut along K so that every
 // compute unit streams; whoever consumes them adds the ranges in order).
 // Every output element is summed in one fixed order that does not depend on the number of rows.
