@@ -299,6 +299,19 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 _sample_workspace: dict = {}
 
 
+SAMPLE_CANDIDATES_TOP_K, SAMPLE_CANDIDATES_MASS_VOCAB = 64, 65536
+
+
+def sample_candidates_apply(temperature: float, top_k: int, top_p: float, vocab: int) -> bool:
+    """Whether a row with these settings may go by its candidates (the kernel's own rule, for callers that know the
+    settings on the host and can spare the launch that picks candidates when no row uses them)."""
+    if temperature < 1e-5:
+        return False
+    if 0 < top_k <= SAMPLE_CANDIDATES_TOP_K:
+        return top_k < vocab
+    return top_p < 1.0 and vocab >= SAMPLE_CANDIDATES_MASS_VOCAB
+
+
 def rows_sampled_by_candidates(rows: int, vocab: int, device) -> list:
     """For the last ``sample`` call of this shape on the device: which rows went by their candidates (a look into the
     call's workspace, for tests and measurements)."""

@@ -305,19 +305,31 @@ struct Candidates {                          // per row and chunk; null `count`:
   int chunks, chunk;
 };
 
-__device__ __forceinline__ bool goes_by_candidates(float temp, int k, int vocab) { return temp >= 1e-5f && k > 0 && k <= kCandTopK && k < vocab; }
+constexpr int kCandMassVocab = 65536;        // rows at least this long that are cut by their mass alone try the candidates too
+
+// The top_k with which a row's candidates are chosen; 0: the row is walked whole.  A row with a top_k of its own of at
+// most kCandTopK takes that.  A long row that is cut by its mass (top_p < 1) under no top_k, or a larger one, takes
+// kCandTopK: where few tokens carry the mass, the tokens that stay are among the kCandTopK largest, and the row's
+// workgroup sees that they are when fewer than kCandTopK stay (the next token then went by its mass, as it would
+// under any larger top_k); else it walks the row after all (a row of noise pays the detour, 20 us on 190).
+__device__ __forceinline__ int candidates_top_k(float temp, int k, float p, int vocab) {
+  if (temp < 1e-5f) return 0;
+  if (k > 0 && k <= kCandTopK) return k < vocab ? k : 0;
+  return (p < 1.f && vocab >= kCandMassVocab) ? kCandTopK : 0;
+}
 
 __global__ __launch_bounds__(kCandThreads) void sample_candidates_kernel(const float* __restrict__ logits, int vocab,
                                                                          const float* __restrict__ temperature,
-                                                                         const int* __restrict__ top_k, const Candidates cd) {
+                                                                         const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                                         const Candidates cd) {
   __shared__ float fscratch[16];
   __shared__ float taus[kCandThreads / 64];
   __shared__ int wave_counts[kCandThreads / 64];
   const int row = blockIdx.y, c = blockIdx.x, tid = threadIdx.x;
   const size_t slot = (size_t)row * cd.chunks + c;
   const float temp = temperature[row];
-  const int k = top_k[row];
-  if (!goes_by_candidates(temp, k, vocab)) {
+  const int k = candidates_top_k(temp, top_k[row], top_p[row], vocab);
+  if (k == 0) {
     if (tid == 0) cd.count[slot] = -1;
     return;
   }
@@ -403,9 +415,10 @@ __device__ __forceinline__ bool has_candidates(const Candidates& cd, int row) {
   return __all(n >= 0);
 }
 
-// One row's token.  CAND: over the row's candidates; else over the whole row.
+// One row's token.  CAND: over the row's candidates (false: they do not settle it, the row has to be walked); else over
+// the whole row.
 template <bool IN_REGS, bool VEC, bool CAND>
-__device__ __forceinline__ void sample_row(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
+__device__ __forceinline__ bool sample_row(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
                                            const int* __restrict__ top_k, const float* __restrict__ top_p,
                                            const long long* __restrict__ request_key, const int* __restrict__ step,
                                            unsigned long long seed, int* __restrict__ out, const Candidates& cd) {
@@ -497,13 +510,19 @@ __device__ __forceinline__ void sample_row(const float* __restrict__ logits, int
   const float temp = temperature[row];
   if (temp < 1e-5f) {
     if (tid == 0) out[row] = best.i;
-    return;
+    return true;
   }
   Weigh weigh; weigh.zmax = best.v; weigh.rate = 1.4426950408889634f / fmaxf(temp, 1e-5f);
 
   int k = top_k[row];
-  if (k <= 0 || k > num_elements) k = num_elements;
   const float p = top_p[row];
+  bool capped = false;                                           // CAND: the candidates were chosen under a smaller top_k than the row's own
+  if constexpr (CAND) {
+    const int own = k;
+    k = candidates_top_k(temp, own, p, vocab);
+    capped = k != own;
+  }
+  if (k <= 0 || k > num_elements) k = num_elements;
   const bool filtered = k < num_elements || p < 1.f;
   // The sum of all weights: a pass of its own where nothing is filtered, else part of the search's first pass.
   SumOfWeights sw; sw.w = weigh; sw.sum = 0.f;
@@ -615,6 +634,14 @@ __device__ __forceinline__ void sample_row(const float* __restrict__ logits, int
       uint32_t lowest_kept = 0xffffffffu;
       if (tid <= num_up && my_key > cut) lowest_kept = my_key;
       threshold = float_as_uint_min(lowest_kept, fscratch);
+      if (capped) {
+        // Fewer than k stay: the next token went by its mass, and would under the row's own top_k.  Else the row's
+        // own rule may keep more than these candidates hold.
+        int staying = 0;
+#pragma unroll
+        for (int s2 = 0; s2 < kHeld; ++s2) staying += (s2 * kSampleThreads + tid < units && float_key(held[s2]) >= threshold) ? 1 : 0;
+        if ((int)block_sum((float)staying, fscratch) >= k) return false;
+      }
     }
   } else if (filtered) {
     // kept(c)  <=>  count(key > c) < k  and  mass(key > c) <= p * total  is monotone in c; the threshold is the
@@ -721,6 +748,7 @@ __device__ __forceinline__ void sample_row(const float* __restrict__ logits, int
     }
     out[row] = token;
   }
+  return true;
 #undef PLLM_WALK
 }
 
@@ -730,8 +758,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
                                                                 const int* __restrict__ top_k, const float* __restrict__ top_p,
                                                                 const long long* __restrict__ request_key, const int* __restrict__ step,
                                                                 unsigned long long seed, int* __restrict__ out, const Candidates cd) {
-  if (cd.count && has_candidates(cd, blockIdx.x)) sample_row<true, false, true>(logits, vocab, temperature, top_k, top_p, request_key, step, seed, out, cd);
-  else sample_row<IN_REGS, VEC, false>(logits, vocab, temperature, top_k, top_p, request_key, step, seed, out, cd);
+  if (cd.count && has_candidates(cd, blockIdx.x) &&
+      sample_row<true, false, true>(logits, vocab, temperature, top_k, top_p, request_key, step, seed, out, cd))
+    return;
+  __syncthreads();                                               // (what the candidates' part left in LDS is done with)
+  sample_row<IN_REGS, VEC, false>(logits, vocab, temperature, top_k, top_p, request_key, step, seed, out, cd);
 }
 
 // Bytes of workspace with which pllm_sample sends rows with a small top_k by their candidates; 0: it would not (many
@@ -769,7 +800,7 @@ PLLM_API int pllm_sample(const float* logits, int rows, int vocab, const float* 
     cd.index = (int*)workspace + (3 + kChunkCap) * slots;
     cd.chunks = chunks;
     cd.chunk = chunk;
-    hipLaunchKernelGGL(sample_candidates_kernel, dim3(chunks, rows), dim3(kCandThreads), 0, stream, logits, vocab, temperature, top_k, cd);
+    hipLaunchKernelGGL(sample_candidates_kernel, dim3(chunks, rows), dim3(kCandThreads), 0, stream, logits, vocab, temperature, top_k, top_p, cd);
   }
 #define PLLM_SAMPLE(IN_REGS_, VEC_)                                                                                          \
   hipLaunchKernelGGL((sample_kernel<IN_REGS_, VEC_>), dim3(rows), dim3(kSampleThreads), 0, stream, logits, vocab, temperature, top_k, \

@@ -59,7 +59,9 @@ class Sampler:
         if all(p.temperature < 1e-5 for p in params):
             return self._to_host(ops.argmax(logits))
         temperature, top_k, top_p, keys, step = self._rows_to_device(params, request_keys, steps, logits.device)
-        return self._to_host(ops.sample(logits, temperature, top_k, top_p, keys, step, self.seed))
+        # (the kernel that picks a row's candidates is launched only when some row's settings can use them)
+        some = any(ops.sample_candidates_apply(p.temperature, p.top_k, p.top_p, logits.shape[1]) for p in params)
+        return self._to_host(ops.sample(logits, temperature, top_k, top_p, keys, step, self.seed, candidates=some))
 
     def _rows_to_device(self, params: list, request_keys: list, steps: list, device):
         """The rows' settings as device tensors.  They travel as one piece of pinned memory with one queued copy: five

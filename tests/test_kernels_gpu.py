@@ -446,6 +446,39 @@ def test_sampling_by_candidates_keeps_what_the_whole_row_keeps(vocab, top_k, top
             assert bool(kept_sets[row][int(whole[row])]), (step, row)
 
 
+@pytest.mark.parametrize("vocab", [70000, 128256])
+@pytest.mark.parametrize("top_k,top_p", [(-1, 0.9), (200, 0.8), (-1, 0.999)])
+def test_long_rows_cut_by_their_mass_try_the_candidates(vocab, top_k, top_p):
+    """A long row under top_p alone (or with a top_k beyond the candidates' reach) goes by the candidates of its 64 largest
+    logits when fewer than 64 tokens stay, and is walked whole when not; either way what is drawn is what the plain
+    implementation keeps.  Rows: a dozen tokens carry the mass; noise (thousands stay); a row where exactly the 64
+    largest carry it, equal among themselves (the candidates do not settle that one)."""
+    z = rnd(3, vocab, seed=43, scale=1.0)
+    z[0] = z[0] * 0.2
+    z[0, (torch.arange(12) * 3001 + 5) % vocab] += torch.linspace(14.0, 9.0, 12)
+    z[2] = z[2] * 0.01
+    z[2, (torch.arange(64) * 997 + 3) % vocab] = 20.0
+    draws = 300
+    got = sample_rows(z, 0.8, top_k, top_p, draws)
+    for row in range(3):
+        probs = kept_by_the_stated_rule(z[row], 0.8, top_k, top_p)
+        if row < 2:
+            assert torch.equal(probs > 0, plain.filtered_probabilities(z[row], 0.8, top_k, top_p) > 0)
+        drawn = got[:, row].long()
+        assert bool((probs[drawn] > 0).all()), f"row {row}: a filtered token was drawn"
+        kept = torch.nonzero(probs > 0).flatten()
+        if row == 2:
+            assert len(kept) == 64
+        if 0 < len(kept) <= 12:
+            counts = np.array([(drawn == i).sum().item() for i in kept])
+            want = probs[kept].numpy() * draws
+            likely = want >= 5                                      # (tokens that 300 draws can be expected to show)
+            assert bool((counts[likely] > 0).all()), f"row {row}: a token that stays was never drawn"
+            chi2, dof = float(((counts[likely] - want[likely]) ** 2 / want[likely]).sum()), int(likely.sum())
+            assert chi2 < dof + 5 * math.sqrt(2 * max(dof, 1)) + 5, f"row {row}: chi-square {chi2:.1f} for {dof} degrees of freedom"
+    assert len(set(got[:, 1].tolist())) > 100 and len(set(got[:, 2].tolist())) > 40      # (many of the tokens that stay were drawn)
+
+
 def test_sampling_rows_do_not_depend_on_their_neighbours():
     z = rnd(5, 50001, seed=23, scale=2.0)
     alone = torch.stack([sample_rows(z[r:r + 1], 0.9, 30, 0.9, 4)[:, 0] for r in range(5)], dim=1)
