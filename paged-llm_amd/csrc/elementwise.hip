@@ -269,6 +269,30 @@ PLLM_API int pllm_rmsnorm(int dtype, const void* x, const void* delta, const int
 }
 
 // ---------------------------------------------------------------------------------------------
+// A projection's bias: out[t, i] = in[t, i] + bias[i], the sums of the product and the bias both float, rounded once
+// to the output's type (projections with a bias take their product as float sums and come through here).
+template <typename T>
+__global__ void add_bias_kernel(const float* __restrict__ in, int ld_in, const float* __restrict__ bias, T* __restrict__ out, int ld_out,
+                                int cols, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / cols;
+  const int i = (int)(idx - t * cols);
+  out[t * ld_out + i] = from_f32<T>(in[t * ld_in + i] + bias[i]);
+}
+
+PLLM_API int pllm_add_bias(int dtype, const float* in, int ld_in, const float* bias, void* out, int ld_out, int rows, int cols,
+                           hipStream_t stream) {
+  const size_t total = (size_t)rows * cols;
+  if (total == 0) return 0;
+  if (cols > ld_in || cols > ld_out) return -2;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+  if (dtype == PLLM_F32) hipLaunchKernelGGL(add_bias_kernel<float>, grid, block, 0, stream, in, ld_in, bias, (float*)out, ld_out, cols, total);
+  else hipLaunchKernelGGL(add_bias_kernel<bf16>, grid, block, 0, stream, in, ld_in, bias, (bf16*)out, ld_out, cols, total);
+  PLLM_RETURN_LAST_ERROR();
+}
+
+// ---------------------------------------------------------------------------------------------
 // Gated activation: out[t, i] = act(gu[t, i]) * gu[t, inter + i] (gate_activation in common.h).
 template <typename T, int V>
 __global__ void gate_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total, int act) {

@@ -71,6 +71,7 @@ _SIGNATURES = {
     "pllm_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long,
                      c_void_p],
     "pllm_gate_mul": [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "pllm_add_bias": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "pllm_rope_scatter": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "pllm_copy_pages": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p],
@@ -173,6 +174,17 @@ def gate_mul(gate_up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
 
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return gate_mul(gate_up, "silu")
+
+
+def add_bias(sums: torch.Tensor, bias: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """float sums [T, N] + float bias [N], rounded once to ``dtype``."""
+    _on_gpu(sums, bias)
+    _need(sums.dtype == torch.float32 and sums.dim() == 2 and sums.stride(1) == 1, "add_bias: float rows with unit inner stride")
+    _need(bias.dtype == torch.float32 and bias.shape == (sums.shape[1],) and bias.is_contiguous(), f"bias: float32 [{sums.shape[1]}]")
+    out = torch.empty(sums.shape, dtype=dtype, device=sums.device)
+    _check(_fn("elementwise.hip", "pllm_add_bias")(dtype_code(dtype), _ptr(sums), sums.stride(0), _ptr(bias), _ptr(out), out.stride(0),
+                                                   sums.shape[0], sums.shape[1], _stream()), "add_bias")
+    return out
 
 
 def rope_scatter(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,

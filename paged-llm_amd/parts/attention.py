@@ -1,9 +1,10 @@
 """Causal attention over the paged cache with grouped heads.
 
-q/k/v projections without bias -> rotary encoding of q and k -> k and v written to their slots ->
+q/k/v projections -> rotary encoding of q and k -> k and v written to their slots ->
 attention over all keys of the request through the block table -> output projection
-(pagedllm/model/llama.py:131-160).  Sizes, the score scale, an optional window and the position
-encoding come in as parameters.  The three input projections are fused into one matrix when the
+(pagedllm/model/llama.py:131-160; the reference's Llama has no biases).  Sizes, the score scale, an optional window,
+the position encoding and whether the q/k/v projections have a bias (``qkv_bias``: tensors ``q_proj.bias`` ...; such
+a layer gives up the fused product-rotary-cache kernels) come in as parameters.  The three input projections are fused into one matrix when the
 weights arrive, so one product serves them.
 """
 
@@ -31,6 +32,7 @@ class PagedAttention(Mixer):
         self.window = int(params.get("window") or 0)
         # False for a layer that always reads another layer's cache: it then has no k/v weights.
         self.kv_proj = bool(params.get("kv_proj", True))
+        self.qkv_bias = bool(params.get("qkv_bias", False))
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"{self.num_heads} heads are no multiple of {self.num_kv_heads} kv heads")
         if not 1 <= self.head_dim <= ops.MAX_HEAD_DIM_GENERIC:
@@ -42,6 +44,7 @@ class PagedAttention(Mixer):
         self._w: dict[str, torch.Tensor] = {}
         self.w_qkv: Weight | None = None
         self.w_o: Weight | None = None
+        self.b_qkv: torch.Tensor | None = None
 
     # ---- weights
     def weight_specs(self):
@@ -50,18 +53,26 @@ class PagedAttention(Mixer):
         if self.kv_proj:
             specs["k_proj.weight"] = WeightSpec((kv, self.hidden))
             specs["v_proj.weight"] = WeightSpec((kv, self.hidden))
+        if self.qkv_bias:                                        # (kept in float: the bias is added to float sums)
+            specs["q_proj.bias"] = WeightSpec((q,), role="vector")
+            if self.kv_proj:
+                specs["k_proj.bias"] = WeightSpec((kv,), role="vector")
+                specs["v_proj.bias"] = WeightSpec((kv,), role="vector")
         return specs
 
     def assign(self, name, tensor):
-        if name not in self.weight_specs():
+        spec = self.weight_specs().get(name)
+        if spec is None:
             raise KeyError(name)
-        self._w[name] = tensor.to(device=self.device, dtype=self.dtype)
+        self._w[name] = tensor.to(device=self.device, dtype=torch.float32 if spec.role == "vector" else self.dtype)
 
     def finalize(self):
         names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.kv_proj else [])
         # (a layer without k/v projections only ever projects q: its matrix keeps the plain pairing)
         self.w_qkv = Weight(torch.cat([self._w[n] for n in names], dim=0).contiguous(), "rotary" if self.kv_proj else "plain", self.head_dim)
         self.w_o = Weight(self._w["o_proj.weight"].contiguous())
+        if self.qkv_bias:
+            self.b_qkv = torch.cat([self._w[n.replace(".weight", ".bias")] for n in names]).contiguous()
         self._w.clear()
 
     # ---- what it keeps
@@ -86,10 +97,12 @@ class PagedAttention(Mixer):
         write = cache.writable
         if write and not self.kv_proj:
             raise RuntimeError("this attention layer has no k/v projections and must read another layer's cache")
-        w_in = self.w_qkv if write or not self.kv_proj else self.w_qkv.rows(nh * d)
+        only_q = not write and self.kv_proj
+        w_in = self.w_qkv.rows(nh * d) if only_q else self.w_qkv
+        bias = self.b_qkv[: nh * d] if only_q and self.b_qkv is not None else self.b_qkv
         k_pages, v_pages = cache["k"], cache["v"]
         qkv = qkv_rotary_cache(h, w_in, ctx.positions, self.position, nh, nkv, d, view.slot_mapping if write else None,
-                               k_pages if write else None, v_pages if write else None, cache.block_size)
+                               k_pages if write else None, v_pages if write else None, cache.block_size, bias=bias)
         o = ops.paged_attention(qkv, k_pages, v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
                                 nh, nkv, d, self.scale, self.window, ctx)
         return linear(o, self.w_o, partial_ok=bool(getattr(ctx, "partial_sums_ok", False)))

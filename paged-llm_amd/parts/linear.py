@@ -133,10 +133,14 @@ def _fused(x, weight, epi: int, rope: dict | None = None, activation: str = "sil
     return None
 
 
-def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = False) -> torch.Tensor:
+def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = False, bias: torch.Tensor | None = None) -> torch.Tensor:
     """x [T, K] (tensor or pending norm), weight [N, K] -> [T, N].  ``partial_ok``: the caller hands the result to a
     norm as its delta and that norm adds partial sums (``StepContext.partial_sums_ok``): the result may then be float
-    [ranges, T, N], the sums over ranges of K."""
+    [ranges, T, N], the sums over ranges of K.  ``bias`` (float32 [N]): added to the product's float sums, the result
+    rounded once (a kernel of its own behind the product)."""
+    if bias is not None:
+        sums = linear(x, weight, torch.float32)
+        return ops.add_bias(sums, bias, out_dtype or _plain(weight).dtype)
     if _streams(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16):
         return _stream(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok=partial_ok)
     if out_dtype != torch.float32 and _tiles(x, weight, partial_ok):
@@ -181,13 +185,13 @@ def gated_linear(x, w_gate_up, activation: str = "silu") -> torch.Tensor:
 
 
 def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_heads: int, num_kv_heads: int,
-                     head_dim: int, slot_mapping, k_pages, v_pages, block_size: int) -> torch.Tensor:
+                     head_dim: int, slot_mapping, k_pages, v_pages, block_size: int, bias: torch.Tensor | None = None) -> torch.Tensor:
     """q, k, v projections, rotation of q and k, and the write of k and v into the cache pages.
     Returns q as rows of a matrix whose first num_heads * head_dim columns hold the rotated heads
     (the row stride may be larger).  With k_pages None only q is projected and rotated.
     ``position_encoding``: a part with ``cos``/``sin`` tables, ``rotary_dim`` and ``interleaved``, or None.
-    The fused kernel pairs element i with i + d/2 over the whole head; another rotated width or pairing
-    goes through the product and the rotary kernel apart."""
+    The fused kernel pairs element i with i + d/2 over the whole head; another rotated width or pairing, and
+    projections with a ``bias`` (float32, one value per row of ``w_qkv``), go through the product and the rotary kernel apart."""
     write = k_pages is not None
     cos = sin = None
     rotary_dim, interleaved = 0, False                      # no position encoding: nothing turns
@@ -196,7 +200,7 @@ def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_h
         rotary_dim = position_encoding.rotary_dim or head_dim
         interleaved = bool(position_encoding.interleaved)
     whole_head_halves = position_encoding is None or (rotary_dim == head_dim and not interleaved)
-    if write and w_qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and whole_head_halves:
+    if write and w_qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and whole_head_halves and bias is None:
         rope = dict(positions=positions, cos=cos, sin=sin, slots=slot_mapping, k_pages=k_pages, v_pages=v_pages,
                     num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size)
         if (isinstance(w_qkv, Weight) and w_qkv.pairing == "rotary" and _streams(x, w_qkv, ops.SL_ROPE_KV)
@@ -206,7 +210,7 @@ def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_h
         if q is not None:
             return q
     w_qkv = _plain(w_qkv)
-    qkv = linear(x, w_qkv)
+    qkv = linear(x, w_qkv, bias=bias)
     ops.rope_scatter(qkv, positions, cos, sin, num_heads, num_kv_heads, head_dim, slot_mapping if write else None,
                      k_pages, v_pages, block_size, rotary_dim, interleaved)
     return qkv

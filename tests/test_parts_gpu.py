@@ -196,6 +196,47 @@ def test_attention_part_whole_in_portions_and_token_by_token(dtype, tol, options
     assert rel(torch.cat(out_other), other_want) <= tol, "second sequence"
 
 
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+def test_attention_part_with_biased_projections(dtype, tol):
+    """q/k/v projections with a bias (a parameter of the part; the reference's Llama has none): the layer gives up the
+    fused product-rotary-cache kernels and adds the bias to the product's float sums.  Whole, then a portion and single
+    tokens, against the same steps written out with the library's routines."""
+    env = env_for(dtype)
+    params = {"num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "qkv_bias": True,
+              "position": {"kind": "rotary", "params": {"head_dim": HEAD_DIM, "theta": THETA, "scaling": None}}}
+    mixer = build("mixer", "paged_attention", params, env)
+    assert {"q_proj.bias", "k_proj.bias", "v_proj.bias"} <= set(mixer.weight_specs())
+    gen = torch.Generator().manual_seed(31)
+    w = {}
+    for name, spec in mixer.weight_specs().items():
+        t = (0.5 if name.endswith(".bias") else 0.08) * torch.randn(spec.shape, generator=gen)
+        w[name] = t if name.endswith(".bias") else t.to(getattr(torch, dtype)).float()
+        mixer.assign(name, w[name])
+    mixer.finalize()
+    L = 52
+    x = rows(L, 32, dtype)
+    xf = x.float()
+    inv = plain.inverse_frequencies(HEAD_DIM, THETA, None)
+    ang = plain.rotary_angles(torch.arange(L), inv)
+    rounded = lambda t: t.to(getattr(torch, dtype)).float()          # the projections' results in the compute type
+    q = rounded(xf @ w["q_proj.weight"].T + w["q_proj.bias"]).view(L, HEADS, HEAD_DIM)
+    k = rounded(xf @ w["k_proj.weight"].T + w["k_proj.bias"]).view(L, KV_HEADS, HEAD_DIM)
+    v = rounded(xf @ w["v_proj.weight"].T + w["v_proj.bias"]).view(L, KV_HEADS, HEAD_DIM)
+    o = plain.causal_attention(plain.apply_rotary(q, ang), plain.apply_rotary(k, ang), v, HEAD_DIM ** -0.5, None)
+    want = o.reshape(L, HEADS * HEAD_DIM) @ w["o_proj.weight"].T
+    without = plain.attention_block(xf, torch.arange(L), w, "", {"num_attention_heads": HEADS, "num_key_value_heads": KV_HEADS,
+                                                                 "head_dim": HEAD_DIM}, inv, None)
+    assert rel(without, want) > 10 * tol                           # (the bias matters: leaving it out would not pass)
+    group = mixer.cache_spec().group_name()
+    table = [4, 1, 6, 3]
+    got = mixer.forward(x.cuda(), step_context([(0, L)], [table], group, dtype), layer_cache(mixer, dtype, 8), None)
+    assert rel(got, want) <= tol, "whole"
+    cache, out = layer_cache(mixer, dtype, 8), []
+    for start, n in [(0, 33), (33, 2)] + [(p, 1) for p in range(35, L)]:
+        out.append(mixer.forward(x[start:start + n].cuda(), step_context([(start, n)], [table], group, dtype), cache, None))
+    assert rel(torch.cat(out), want) <= tol, "a portion and single tokens"
+
+
 def test_attention_part_refuses_sizes_its_kernels_do_not_take():
     env = env_for("bfloat16")
     with pytest.raises(ValueError, match="head sizes 1..256"):
