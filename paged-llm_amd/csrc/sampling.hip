@@ -155,6 +155,7 @@ __device__ __forceinline__ F for_each_element(const float (&held)[HELD], const f
   if constexpr (IN_REGS) {
 #pragma unroll
     for (int s = 0; s < HELD; ++s) {
+      if ((s / kPer) * kSampleThreads >= units) break;           // (the same for every thread: the slots from here on are empty)
       const int u = (s / kPer) * kSampleThreads + tid, i = u * kPer + (s % kPer);
       if (u < units) f(held[s], i);
     }
@@ -558,6 +559,7 @@ __device__ __forceinline__ bool sample_row(const float* __restrict__ logits, int
         __syncthreads();
 #pragma unroll
         for (int s2 = 0; s2 < kHeld; ++s2) {
+          if (s2 * kSampleThreads >= units) break;
           if (s2 * kSampleThreads + tid < units) {
             const uint32_t key = float_key(held[s2]);
             if (key - lo <= span) atomicAdd(&hist[(key - lo) >> shift], 1);
@@ -595,7 +597,10 @@ __device__ __forceinline__ bool sample_row(const float* __restrict__ logits, int
       // the candidates above the k-th key, in the order of the threads
       int mine_up = 0;
 #pragma unroll
-      for (int s2 = 0; s2 < kHeld; ++s2) mine_up += (s2 * kSampleThreads + tid < units && float_key(held[s2]) > kth) ? 1 : 0;
+      for (int s2 = 0; s2 < kHeld; ++s2) {
+        if (s2 * kSampleThreads >= units) break;
+        mine_up += (s2 * kSampleThreads + tid < units && float_key(held[s2]) > kth) ? 1 : 0;
+      }
       const int lane = tid & 63, wave = tid >> 6;
       int incl = mine_up;
 #pragma unroll
@@ -612,6 +617,7 @@ __device__ __forceinline__ bool sample_row(const float* __restrict__ logits, int
       }
 #pragma unroll
       for (int s2 = 0; s2 < kHeld; ++s2) {
+        if (s2 * kSampleThreads >= units) break;
         if (s2 * kSampleThreads + tid < units && float_key(held[s2]) > kth) {
           up_key[at] = float_key(held[s2]);
           up_weight[at] = weigh(held[s2]);
@@ -639,7 +645,10 @@ __device__ __forceinline__ bool sample_row(const float* __restrict__ logits, int
         // own rule may keep more than these candidates hold.
         int staying = 0;
 #pragma unroll
-        for (int s2 = 0; s2 < kHeld; ++s2) staying += (s2 * kSampleThreads + tid < units && float_key(held[s2]) >= threshold) ? 1 : 0;
+        for (int s2 = 0; s2 < kHeld; ++s2) {
+          if (s2 * kSampleThreads >= units) break;
+          staying += (s2 * kSampleThreads + tid < units && float_key(held[s2]) >= threshold) ? 1 : 0;
+        }
         if ((int)block_sum((float)staying, fscratch) >= k) return false;
       }
     }
