@@ -980,14 +980,17 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     // Two key groups (eight wavefronts, one workgroup per compute unit) for the head sizes that then still fit
     // into registers and LDS (up to 128): always where a wavefront of the four-wavefront kind needs more than half
     // of a SIMD's registers (head sizes above 96: two groups are then the only way to two wavefronts per SIMD,
-    // measured 1.4 times faster at 128), else when there are too few workgroups to keep two of the four-wavefront
-    // kind on every compute unit for most of the time (measured: faster up to about 2.5 workgroups per compute
-    // unit).
+    // measured 1.4 times faster at 128), else while the workgroups fit the compute units in one round, and for a
+    // single sequence in two (its tiles, handed out longest first, pair up a long one and a short one per compute
+    // unit: 2048 tokens 39.9 against 42.7 us; but two prompts of 1024 tokens 26.1 against 23.9 us, four of 512 19.4
+    // against 16.0, sixteen of 256 31.5 against 19.7, and one of 2560 62.0 against 52.4: there two workgroups of the
+    // four-wavefront kind per compute unit, each hiding the other's start and end, are faster).
     constexpr bool two_fits = D <= 128 && prefill_lds_bytes(2) <= 160 * 1024;
-    // (workgroups that find work: a sequence has as many tiles as its own queries need, the grid as many slots
-    // as the longest)
-    const long busy = (work_list ? (long)num_work * num_kv_heads : ((long)total_q * G / kCols + num_seqs) * num_kv_heads) * num_partitions;
-    const bool two = two_fits && (D > 96 || 2L * busy <= 5L * num_compute_units());
+    // (workgroups that find work: with a list exactly its entries; else a sequence has as many tiles as its own queries
+    // need, one more than its share at most)
+    const long busy = (work_list ? (long)num_work : ((long)total_q * G + kCols - 1) / kCols + (num_seqs - 1)) * num_kv_heads * num_partitions;
+    const long cus = num_compute_units();
+    const bool two = two_fits && (D > 96 || busy <= cus || (num_seqs == 1 && busy <= 2 * cus));
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
     if ((long)lds > pllm_max_lds()) return -2;
     auto kern = paged_attention_prefill_kernel<2, 1>;
