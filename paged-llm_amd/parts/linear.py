@@ -51,7 +51,7 @@ class Weight:
 STREAM_MIN_ROWS, STREAM_MAX_ROWS = 17, 128      # rows the streaming kernel is chosen for
 TILE_MAX_ROWS = 640                             # rows up to which the tiled kernel is chosen for small matrices cut along K
 STREAM_GATED_MAX_ROWS = 64                      # the gated product: beyond, its rows' traffic costs more than the library's kernel
-STREAM_LONG_K, STREAM_LONG_K_MAX_ROWS = 8192, 64 # from this K on the rows' traffic limits the streaming kernel to so many rows
+STREAM_LONG_K, STREAM_LONG_K_MAX_ROWS = 8192, 64 # from this K on a product in one range takes the streaming kernel up to so many rows
 
 
 def _plain(weight) -> torch.Tensor:
@@ -76,7 +76,7 @@ def _tiles(x, weight, partial_ok: bool) -> bool:
             and ops.tile_linear_plan(rows, n, k, ops._num_compute_units(weight.plain.device)) > 1)
 
 
-def _streams(x, weight, epi: int) -> bool:
+def _streams(x, weight, epi: int, partial_ok: bool = False) -> bool:
     """Whether this product goes to the streaming kernel: by sizes and row count only (measured on matrices of
     2048 x 2048 to 11264 x 2048 and 2048 x 5632 against the library and the kernels for fewer rows)."""
     if not (isinstance(weight, Weight) and weight.tiled is not None):
@@ -89,7 +89,9 @@ def _streams(x, weight, epi: int) -> bool:
         return rows <= STREAM_GATED_MAX_ROWS
     if epi == ops.SL_F32:
         return False                                            # (the head: 32000 x 2048 was not faster than the library's kernel)
-    return _few_weight_rows(weight) and (k < STREAM_LONG_K or rows <= STREAM_LONG_K_MAX_ROWS)
+    # (cut into ranges of K the long products stay ahead of the library up to 128 rows: 4096 x 14336 at 96 / 128 rows 45.7 / 55.4 us
+    #  against 62.6 / 74.8, 2048 x 8192 16.1 / 18.4 against 20.8)
+    return _few_weight_rows(weight) and (k < STREAM_LONG_K or rows <= STREAM_LONG_K_MAX_ROWS or (partial_ok and epi == ops.SL_BF16))
 
 
 def _stream(x, weight: Weight, epi: int, rope: dict | None = None, partial_ok: bool = False, activation: str = "silu"):
@@ -141,7 +143,7 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
     if bias is not None:
         sums = linear(x, weight, torch.float32)
         return ops.add_bias(sums, bias, out_dtype or _plain(weight).dtype)
-    if _streams(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16):
+    if _streams(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok):
         return _stream(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok=partial_ok)
     if out_dtype != torch.float32 and _tiles(x, weight, partial_ok):
         x = rows_of(x)
