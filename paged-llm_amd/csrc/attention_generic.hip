@@ -9,6 +9,7 @@
 //   cu_seqlens_q [num_seqs+1], seq_lens_k [num_seqs] (context length including the new tokens)
 // Query i of a sequence sits at position seq_len_k - num_q + i and sees keys n <= that position
 // (and n > position - window when window > 0).  Query head j reads kv head j / (heads / kv_heads).
+// A score may carry further terms (a cap, a slope times the distance, a sink per head: ScoreTerms).
 //
 // Keys are walked in tiles of 64 aligned to absolute positions 0, 64, 128, ..., so the order of
 // every sum for one (token, head) is the same however the tokens were cut into steps or batched.
@@ -24,7 +25,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     T* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_seqs, int num_heads,
-    int num_kv_heads, int head_dim, int block_size, float scale, int window) {
+    int num_kv_heads, int head_dim, int block_size, float scale, int window, ScoreTerms terms) {
   __shared__ float q_s[kMaxHeadDim];
   __shared__ float p_s[64];
   __shared__ int page_s[64];
@@ -51,6 +52,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
   const int dims_per_lane = (head_dim + 63) / 64;  // <= 4
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
+  if (terms.sinks) { m = terms.sinks[head]; l = 1.f; }          // as if one key with this score and no value had been seen
+  const float slope = terms.slopes ? terms.slopes[head] : 0.f;
 
   for (int n0 = (first_key / 64) * 64; n0 <= q_pos; n0 += 64) {
     const int n = n0 + lane;
@@ -62,10 +65,11 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
       const T* kr = k_pages + (((size_t)page * num_kv_heads + kvh) * block_size + (n % block_size)) * head_dim;
       float dot = 0.f;
       for (int i = 0; i < head_dim; ++i) dot = fmaf(q_s[i], to_f32(kr[i]), dot);
-      s = dot * scale;
+      s = capped_score(dot * scale, terms.cap);
+      if (terms.slopes) s += slope * (float)(n - q_pos);
     }
     const float m_new = fmaxf(m, wave_max(s));   // finite: the tile holds at least one visible key
-    const float alpha = expf(m - m_new);          // 0 on the first tile
+    const float alpha = expf(m - m_new);          // 0 on the first tile (without a sink)
     const float p = visible ? expf(s - m_new) : 0.f;
     l = l * alpha + wave_sum(p);
     m = m_new;
@@ -103,17 +107,20 @@ PLLM_API int pllm_paged_attention_generic(int dtype, const void* q, int q_stride
                                           void* out, int out_stride, const int* block_tables, int bt_stride,
                                           const int* cu_seqlens_q, const int* seq_lens_k, int num_seqs, int total_q,
                                           int num_heads, int num_kv_heads, int head_dim, int block_size, float scale,
-                                          int window, hipStream_t stream) {
+                                          int window, float score_cap, const float* slopes, const float* sinks,
+                                          hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (head_dim > kMaxHeadDim || head_dim <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
+  if (!(score_cap >= 0.f)) return -2;
+  const ScoreTerms terms{score_cap, slopes, sinks};
   dim3 grid(total_q, num_heads), block(64);
   if (dtype == PLLM_F32)
     hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_stride,
                        (const float*)k_pages, (const float*)v_pages, (float*)out, out_stride, block_tables, bt_stride,
-                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window);
+                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window, terms);
   else
     hipLaunchKernelGGL(paged_attention_generic_kernel<bf16>, grid, block, 0, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride,
-                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window);
+                       cu_seqlens_q, seq_lens_k, num_seqs, num_heads, num_kv_heads, head_dim, block_size, scale, window, terms);
   PLLM_RETURN_LAST_ERROR();
 }

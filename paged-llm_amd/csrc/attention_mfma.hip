@@ -30,6 +30,22 @@ using namespace pllm;
 #endif
 static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size must be 16..256 in steps of 16");
 
+// -DSCORE_TERMS=1 compiles the kernels with the further terms of a score (a cap, a slope times the distance, a sink
+// per head: ScoreTerms in common.h) as one more argument.  Without it there is no such argument: `terms` then names a
+// constant that says "none", and everything that reads it is compiled out.
+#ifndef SCORE_TERMS
+#define SCORE_TERMS 0
+#endif
+constexpr bool kTerms = SCORE_TERMS != 0;
+#if SCORE_TERMS
+#define PLLM_TERMS_PARAM , ScoreTerms terms
+#define PLLM_TERMS_ARG , terms
+#else
+#define PLLM_TERMS_PARAM
+#define PLLM_TERMS_ARG
+static constexpr ScoreTerms terms{0.f, nullptr, nullptr};
+#endif
+
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
@@ -55,6 +71,51 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 // v_exp_f32: 2^x, with 2^-inf = 0 and tiny results flushed to zero (harmless in a softmax).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Further terms of the scores (kernels compiled with them): the 16 raw products of one column in a block of 64 keys
+// (s[kt][i] belongs to key n0 + kt * 16 + g * 4 + i) are brought to their final form in log2 units,
+//   log2(e) * (cap(scale * s) + slope * (n - query position)),
+// with c tanh(x / c) = c (1 - 2 / (2^(2 log2(e) x / c) + 1)): right at both ends (2^inf = inf gives c, 2^-inf = 0
+// gives -c) and within c * 2^-23 everywhere, far below what rounding the probabilities to bfloat16 leaves.  Which
+// terms there are is the same for the whole launch, so each is a branch around sixteen scores, not inside them.
+struct ScoreForm {
+  float sl2;        // log2(e) * scale
+  float cap_l2;     // log2(e) * cap                  (cap > 0)
+  float cap_in;     // 2 log2(e) * scale / cap: what the raw product is multiplied by inside the power of two
+  bool capped, sloped;
+  __device__ __forceinline__ bool any() const { return capped || sloped; }
+};
+__device__ __forceinline__ ScoreForm score_form(const ScoreTerms& t, float scale) {
+  constexpr float l2e = 1.4426950408889634f;
+  ScoreForm f;
+  f.sl2 = scale * l2e;
+  f.capped = t.cap > 0.f;
+  f.sloped = t.slopes != nullptr;
+  f.cap_l2 = f.capped ? t.cap * l2e : 0.f;
+  f.cap_in = f.capped ? 2.f * l2e * scale / t.cap : 0.f;
+  return f;
+}
+__device__ __forceinline__ void final_scores(const ScoreForm& f, float slope_l2, float distance0, float (&s)[4][4]) {
+  if (f.capped) {
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        s[kt][i] = fmaf(-2.f * f.cap_l2, __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s[kt][i] * f.cap_in) + 1.f), f.cap_l2);
+  } else {
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[kt][i] *= f.sl2;
+  }
+  if (f.sloped) {                                               // slope_l2 = log2(e) * slope; distance0 = n0 + g * 4 - query position
+    const float base = slope_l2 * distance0;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[kt][i] += fmaf(slope_l2, (float)(kt * 16 + i), base);
+  }
+}
 
 // The four lanes that mirror a column are 16 lanes apart.  v_permlane16_swap exchanges the odd rows (of 16 lanes)
 // of one register with the even rows of another, v_permlane32_swap the upper half of one with the lower half of
@@ -93,7 +154,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
-    int block_size, float scale, int window, int partition_size, int num_partitions, float* __restrict__ partials) {
+    int block_size, float scale, int window, int partition_size, int num_partitions, float* __restrict__ partials PLLM_TERMS_PARAM) {
   // Fetch all arguments in one go (left alone, the compiler fetches each where it is first used, and every fetch is
   // a wait of its own in the chain lengths -> page table -> keys).
   constexpr bool kLookupsTogether = D <= 64;
@@ -132,6 +193,7 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
   bool my_valid[NCB];
   size_t my_out[NCB];
   bf16x8 qreg[NCB][KSTEPS];
+  float my_slope[NCB], my_sink[NCB];                            // (with further score terms only; both in log2 units)
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb) {
     const int c = col0 + cb * 16 + r;
@@ -141,6 +203,10 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     my_first[cb] = (window > 0 && my_qpos[cb] - window + 1 > 0) ? my_qpos[cb] - window + 1 : 0;
     const size_t row = (size_t)(q_begin + tok) * q_stride + (size_t)(kvh * G + hg) * D;
     my_out[cb] = (size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D;
+    if constexpr (kTerms) {
+      my_slope[cb] = (terms.slopes && my_valid[cb]) ? terms.slopes[kvh * G + hg] * kLog2e : 0.f;
+      my_sink[cb] = (terms.sinks && my_valid[cb]) ? terms.sinks[kvh * G + hg] * kLog2e : -INFINITY;
+    }
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
       const int dd = s * 32 + g * 8;
@@ -158,6 +224,22 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     for (int db = 0; db < DBLOCKS; ++db) acc[cb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
   const float sl2 = scale * kLog2e;
+  [[maybe_unused]] const ScoreForm form = score_form(terms, scale);
+  if constexpr (kTerms) {
+    // A head's sink enters as the state of a softmax that has seen one key with that score and no value.  Of the
+    // wavefronts that share a column, the first one of the partition that holds the column's first visible key
+    // has it (that partition has work for this column, and the merge counts it).
+    if (terms.sinks) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) {
+        const bool here = my_valid[cb] && wave == 0 && (partition_size == 0 || part == my_first[cb] / partition_size);
+        if (here) {
+          m_run[cb] = my_sink[cb];
+          l_run[cb] = g == 0 ? 1.f : 0.f;                         // (the four lanes of a column are added at the end)
+        }
+      }
+    }
+  }
   ConstantInts bt = as_constant(block_tables) + (size_t)seq * bt_stride;
   const size_t page_elems = (size_t)block_size * D;             // one kv head's part of a page
   const size_t page_stride = page_elems * num_kv_heads;
@@ -225,11 +307,27 @@ __global__ __launch_bounds__(WAVES * 64) void paged_attention_mfma_kernel(
     for (int cb = 0; cb < NCB; ++cb) {
       float sc[4][4];
       float mx = -INFINITY;
+      float mul = sl2;
+      if constexpr (kTerms) {
+        if (form.any()) {
+          float s[4][4];
+#pragma unroll
+          for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[kt][i] = s_t[kt][cb][i];
+          final_scores(form, my_slope[cb], (float)(n0 + g * 4 - my_qpos[cb]), s);
+#pragma unroll
+          for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_t[kt][cb][i] = s[kt][i];
+          mul = 1.f;
+        }
+      }
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float v = s_t[kt][cb][i] * sl2;
+          float v = s_t[kt][cb][i] * mul;
           if (!interior) {
             const int n = n0 + kt * 16 + g * 4 + i;
             const bool vis = blk.on[kt] && n <= my_qpos[cb] && n >= my_first[cb];
@@ -435,7 +533,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
     bf16* __restrict__ out, int out_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ seq_lens_k, int num_heads, int num_kv_heads,
     int block_size, float scale, int window, const int* __restrict__ work, int partition_size, int num_partitions,
-    float* __restrict__ partials) {
+    float* __restrict__ partials PLLM_TERMS_PARAM) {
   extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
   constexpr int kKTile = 64 * kKRow, kVTile = D * kVRow;         // elements of one group's keys / values of a step
   // keys [2 buffers][KG][64 rows][kKRow], then values [2 buffers][KG][D rows][kVRow].  Addresses are formed
@@ -500,6 +598,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
   bool my_valid[NCB];
   size_t my_out[NCB];
   bf16x8 qreg[NCB][KSTEPS];
+  float my_slope[NCB], my_sink[NCB];                            // (with further score terms only; both in log2 units)
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb) {
     const int c = col0 + cb * 16 + r;
@@ -509,6 +608,10 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
     my_first[cb] = (window > 0 && my_qpos[cb] - window + 1 > 0) ? my_qpos[cb] - window + 1 : 0;
     const size_t row = (size_t)(q_begin + tok) * q_stride + (size_t)(kvh * G + hg) * D;
     my_out[cb] = (size_t)(q_begin + tok) * out_stride + (size_t)(kvh * G + hg) * D;
+    if constexpr (kTerms) {
+      my_slope[cb] = (terms.slopes && my_valid[cb]) ? terms.slopes[kvh * G + hg] * kLog2e : 0.f;
+      my_sink[cb] = (terms.sinks && my_valid[cb]) ? terms.sinks[kvh * G + hg] * kLog2e : -INFINITY;
+    }
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
       const int dd = s * 32 + g * 8;
@@ -525,6 +628,22 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
     for (int db = 0; db < DBLOCKS; ++db) acc[cb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
   const float sl2 = scale * kLog2e;
+  [[maybe_unused]] const ScoreForm form = score_form(terms, scale);
+  if constexpr (kTerms) {
+    // A head's sink enters as the state of a softmax that has seen one key with that score and no value.  Of the
+    // key groups that share a column, the first one of the partition that holds the column's first visible key
+    // has it (that partition has work for this column, and the merge counts it).
+    if (terms.sinks) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) {
+        const bool here = my_valid[cb] && kg == 0 && (partition_size == 0 || part == my_first[cb] / partition_size);
+        if (here) {
+          m_run[cb] = my_sink[cb];
+          l_run[cb] = g == 0 ? 1.f : 0.f;                         // (the four lanes of a column are added at the end)
+        }
+      }
+    }
+  }
   const int* bt = block_tables + (size_t)seq * bt_stride;
   const size_t page_elems = (size_t)block_size * D;
   const size_t page_stride = page_elems * num_kv_heads;
@@ -585,7 +704,9 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
   // `masked` is a compile-time flag: blocks whose 64 keys every valid column of the wavefront may see take
   // the version without any comparison.  Columns past the end of the sequence (the last tile's surplus)
   // carry zero queries and are never stored; they go along with either version.
-  auto compute = [&](int buf, int n0, auto masked_tag) {
+  // (inlined at both of its places in every build: left to itself the compiler makes a call of the larger forms, with
+  //  the captured state passed through memory)
+  auto compute = [&](int buf, int n0, auto masked_tag) __attribute__((always_inline)) {
     constexpr bool kMasked = decltype(masked_tag)::value;
     const bf16* kb = PLLM_K_TILE(buf, kg);
     const bf16* vb = PLLM_V_TILE(buf, kg);
@@ -638,7 +759,24 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
       // The maximum is taken over the raw dot products (the scale is positive); the running
-      // maximum m_run is kept in scaled log2 units.
+      // maximum m_run is kept in scaled log2 units.  (With further terms the scores are brought to their final
+      // form in log2 units first, and the factor below is one.)
+      float mul = sl2;
+      if constexpr (kTerms) {
+        if (form.any()) {
+          float s[4][4];
+#pragma unroll
+          for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[kt][i] = s_t[kt][cb][i];
+          final_scores(form, my_slope[cb], (float)(n0 + g * 4 - my_qpos[cb]), s);
+#pragma unroll
+          for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_t[kt][cb][i] = s[kt][i];
+          mul = 1.f;
+        }
+      }
       float mx = -INFINITY;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
@@ -650,7 +788,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
           }
           mx = fmaxf(mx, s_t[kt][cb][i]);
         }
-      mx = group_max(mx) * sl2;
+      mx = group_max(mx) * mul;
       const float m_new = fmaxf(m_run[cb], mx);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = fast_exp2(m_run[cb] - m_safe);
@@ -660,7 +798,7 @@ __global__ __launch_bounds__(256 * KG, (D <= 96 || KG == 2) ? 2 : 1) void paged_
       for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = fast_exp2(fmaf(s_t[kt][cb][i], sl2, -m_safe));
+          const float p = fast_exp2(fmaf(s_t[kt][cb][i], mul, -m_safe));
           psum += p;
           p_op[kt >> 1][cb][(kt & 1) * 4 + i] = (__bf16)p;
         }
@@ -944,12 +1082,12 @@ static size_t merge_lds_bytes(int ncb, int waves) { return (size_t)(2 * waves * 
 // partition_size > 0 (a multiple of 64): num_partitions work items per tile each take one aligned
 //   partition of the keys and write partials into `partials` (total_q * heads * num_partitions *
 //   (D + 2) floats); a second kernel merges them.
-PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
-                                       int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
-                                       const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
-                                       int num_kv_heads, int block_size, float scale, int window, int partition_size,
-                                       int num_partitions, float* partials, int waves, int column_blocks, const int* work_list, int num_work,
-                                       hipStream_t stream) {
+static int launch_attention(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
+                            int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
+                            const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
+                            int num_kv_heads, int block_size, float scale, int window, int partition_size,
+                            int num_partitions, float* partials, int waves, int column_blocks, const int* work_list, int num_work,
+                            [[maybe_unused]] ScoreTerms terms, hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
   const int G = num_heads / num_kv_heads;
@@ -1003,7 +1141,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     }
     hipLaunchKernelGGL(kern, pgrid, dim3(two ? 512 : 256), lds, stream, (const bf16*)q, q_stride,
                        (const bf16*)k_pages, (const bf16*)v_pages, (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q,
-                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, work_list, partition_size, num_partitions, partials);
+                       seq_lens_k, num_heads, num_kv_heads, block_size, scale, window, work_list, partition_size, num_partitions, partials PLLM_TERMS_ARG);
     int perr = (int)hipGetLastError();
     if (perr || partition_size == 0) return perr;
     hipLaunchKernelGGL(attention_merge_kernel<false>, dim3((total_q * num_heads + 3) / 4), dim3(256), 0, stream, partials, (bf16*)out,
@@ -1021,7 +1159,7 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     }                                                                                                                                \
     hipLaunchKernelGGL(kern, grid, block, lds, stream, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages,         \
                        (bf16*)out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,           \
-                       block_size, scale, window, partition_size, num_partitions, partials);                                         \
+                       block_size, scale, window, partition_size, num_partitions, partials PLLM_TERMS_ARG);                          \
   } while (0)
 #define PLLM_BY_WAVES(NCB_)                                                                          \
   do {                                                                                               \
@@ -1044,6 +1182,35 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
     err = (int)hipGetLastError();
   }
   return err;
+}
+
+PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
+                                       int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
+                                       const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
+                                       int num_kv_heads, int block_size, float scale, int window, int partition_size,
+                                       int num_partitions, float* partials, int waves, int column_blocks, const int* work_list, int num_work,
+                                       hipStream_t stream) {
+  return launch_attention(q, q_stride, k_pages, v_pages, out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_seqs,
+                          total_q, max_q_len, num_heads, num_kv_heads, block_size, scale, window, partition_size, num_partitions,
+                          partials, waves, column_blocks, work_list, num_work, ScoreTerms{0.f, nullptr, nullptr}, stream);
+}
+
+// The same with further terms of the score: score_cap > 0 caps the scaled products (c tanh(x / c)), slopes [heads]
+// adds slope * (key position - query position), sinks [heads] gives every head a logit that takes part in the
+// softmax's sum only (null: none).  A library compiled without -DSCORE_TERMS=1 refuses any of them.
+PLLM_API int pllm_attention_mfma_score_terms() { return kTerms ? 1 : 0; }
+
+PLLM_API int pllm_paged_attention_mfma_terms(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
+                                             int out_stride, const int* block_tables, int bt_stride, const int* cu_seqlens_q,
+                                             const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
+                                             int num_kv_heads, int block_size, float scale, int window, int partition_size,
+                                             int num_partitions, float* partials, int waves, int column_blocks, const int* work_list,
+                                             int num_work, float score_cap, const float* slopes, const float* sinks, hipStream_t stream) {
+  const ScoreTerms given{score_cap, slopes, sinks};
+  if (!(score_cap >= 0.f) || (given.any() && !kTerms)) return -2;
+  return launch_attention(q, q_stride, k_pages, v_pages, out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_seqs,
+                          total_q, max_q_len, num_heads, num_kv_heads, block_size, scale, window, partition_size, num_partitions,
+                          partials, waves, column_blocks, work_list, num_work, given, stream);
 }
 
 // What the library that holds the no-allocation entry point needs from this one (see attention_noalloc.h): the head

@@ -147,12 +147,15 @@ COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip"
                   "attention_noalloc.hip", "stream_linear.hip"]
 # Head sizes whose attention library a full build makes (others are compiled at first use).
 USUAL_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
+# ... and those whose attention library with further score terms in its loops (-DSCORE_TERMS=1) it makes as well.
+SCORE_TERMS_HEAD_DIMS = (16, 32, 64, 128)
 
 
 def all_targets() -> list[tuple[str, dict]]:
     """Everything a full build compiles: the common sources plus the usual specialisations."""
     targets: list[tuple[str, dict]] = [(s, {}) for s in COMMON_SOURCES]
     targets += [("attention_mfma.hip", {"HEAD_DIM": d}) for d in USUAL_HEAD_DIMS]
+    targets += [("attention_mfma.hip", {"HEAD_DIM": d, "SCORE_TERMS": 1}) for d in SCORE_TERMS_HEAD_DIMS]
     return targets
 
 

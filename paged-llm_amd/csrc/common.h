@@ -32,6 +32,17 @@ __device__ __forceinline__ float gate_activation(float z, int act) {
   return z / (1.f + expf(-z));
 }
 
+// Terms of an attention score beside the scaled dot product x = scale * q.k, for mixers that have them:
+//   score(query position i, key position n, head h) = cap(x) + slopes[h] * (n - i),   cap(x) = c tanh(x / c) for c > 0,
+// and a logit sinks[h] that takes part in the softmax's sum and in nothing else (a key with no value).
+struct ScoreTerms {
+  float cap;            // 0: the product as it is
+  const float* slopes;  // [heads] floats or null
+  const float* sinks;   // [heads] floats or null
+  __host__ __device__ bool any() const { return cap > 0.f || slopes || sinks; }
+};
+__device__ __forceinline__ float capped_score(float x, float cap) { return cap > 0.f ? cap * tanhf(x / cap) : x; }
+
 // One rotary pair turned by the angle whose cosine and sine are c and s.  Products and sums are rounded one by one (no
 // fused multiply-add), in every kernel that rotates: what one kernel writes into the cache and what another computes
 // for the same position are then the same bits, and equal to what plain float arithmetic gives.

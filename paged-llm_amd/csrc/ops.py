@@ -78,7 +78,7 @@ _SIGNATURES = {
     "pllm_gemm_nt": [c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "pllm_paged_attention_generic": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                     c_void_p],
+                                     c_float, c_void_p, c_void_p, c_void_p],
     "pllm_sample": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_ulonglong, c_void_p,
                     c_void_p, c_void_p],
     "pllm_sample_workspace_bytes": [c_int, c_int],
@@ -276,9 +276,44 @@ def _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_l
     return S, bs
 
 
+class ScoreTerms:
+    """Further terms of an attention score, for mixers that have them (None everywhere else).  With x the scaled
+    product of a query at position i and a key at position n of head h:
+
+        score = cap(x) + slopes[h] * (n - i),     cap(x) = c * tanh(x / c) for ``cap`` = c > 0, x for 0,
+
+    and ``sinks[h]``: a logit that takes part in the softmax's sum and in nothing else.  ``slopes`` and ``sinks``
+    are float32 [heads] on the device or None."""
+
+    __slots__ = ("cap", "slopes", "sinks")
+
+    def __init__(self, cap: float = 0.0, slopes: torch.Tensor | None = None, sinks: torch.Tensor | None = None):
+        self.cap, self.slopes, self.sinks = float(cap), slopes, sinks
+
+    def any(self) -> bool:
+        return self.cap > 0.0 or self.slopes is not None or self.sinks is not None
+
+    def checked(self, num_heads: int, device) -> "ScoreTerms":
+        _need(self.cap >= 0.0 and self.cap == self.cap, f"a cap of the scores is positive, or 0 for none; got {self.cap}")
+        for name, t in (("slopes", self.slopes), ("sinks", self.sinks)):
+            if t is not None:
+                _on_gpu(t)
+                _need(t.dtype == torch.float32 and t.shape == (num_heads,) and t.is_contiguous() and t.device == device,
+                      f"{name}: float32 [{num_heads}] beside the queries, got {tuple(t.shape)} {t.dtype} on {t.device}")
+        return self
+
+
+def _terms_args(terms: "ScoreTerms | None", num_heads: int, device) -> tuple:
+    if terms is None:
+        return c_float(0.0), None, None
+    terms.checked(num_heads, device)
+    return c_float(terms.cap), _ptr(terms.slopes), _ptr(terms.sinks)
+
+
 def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_tables: torch.Tensor,
                             cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
-                            head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
+                            head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None,
+                            terms: ScoreTerms | None = None) -> torch.Tensor:
     """Causal attention over paged keys and values; one wavefront per (token, head), all in float.
 
     The caller guarantees (and the step function checks on the host) that every table entry
@@ -294,7 +329,8 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     _check(_fn("attention_generic.hip", "pllm_paged_attention_generic")(
         dtype_code(q.dtype), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0),
         _ptr(block_tables), block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, num_heads, num_kv_heads,
-        head_dim, bs, c_float(scale), int(window or 0), _stream()), "paged_attention_generic")
+        head_dim, bs, c_float(scale), int(window or 0), *_terms_args(terms, num_heads, q.device), _stream()),
+        "paged_attention_generic")
     return out
 
 
@@ -706,6 +742,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = 
 
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]
+_ATTN_TERMS_SIG = _ATTN_SIG[:-1] + [c_float, c_void_p, c_void_p, c_void_p]
 _attn_scratch: dict = {}
 _attn_scratch_retired: list = []      # outgrown buffers stay allocated: captured graphs still hold their addresses
 _attn_checked: set = set()
@@ -777,14 +814,16 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                          cu_seqlens_q: torch.Tensor, seq_lens_k: torch.Tensor, num_heads: int, num_kv_heads: int,
                          head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
                          num_partitions: int = 1, waves: int = 1, column_blocks: int = 0,
-                         out: torch.Tensor | None = None, work_list: torch.Tensor | None = None) -> torch.Tensor:
+                         out: torch.Tensor | None = None, work_list: torch.Tensor | None = None,
+                         terms: ScoreTerms | None = None) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
     work item into aligned partitions that a second kernel merges (best a multiple of 128 for prompt portions, whose
     workgroups walk the keys in steps of up to 128); ``waves`` > 1 shares the keys
     of a work item between the wavefronts of one workgroup (few queries per sequence only).  ``work_list``
     (prompt portions): int32 [n, 2] pairs of (sequence, tile of 128 query columns), the order in which the
-    kernel's workgroups take them (``prompt_work_list``)."""
+    kernel's workgroups take them (``prompt_work_list``).  ``terms``: further terms of the scores (``ScoreTerms``);
+    with any of them the kernels come from a library of their own, compiled with those terms in the score loop."""
     S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
     _need(mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs),
           f"MFMA attention takes bfloat16, head sizes 16..256 in steps of 16, pages of >= 16 positions and groups of <= 64 "
@@ -814,16 +853,24 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                 _attn_scratch_retired.append(ws)
             ws = torch.empty(max(floats, 1 << 22), dtype=torch.float32, device=q.device)
             _attn_scratch[key] = ws
-    if head_dim not in _attn_checked:                 # the library on disk is the one compiled for this head size
-        built = _fn("attention_mfma.hip", "pllm_attention_mfma_head_dim", {"HEAD_DIM": head_dim}, [])()
+    with_terms = terms is not None and terms.checked(num_heads, q.device).any()
+    defines = {"HEAD_DIM": head_dim, "SCORE_TERMS": 1} if with_terms else {"HEAD_DIM": head_dim}
+    if (head_dim, with_terms) not in _attn_checked:   # the library on disk is the one compiled for this head size
+        built = _fn("attention_mfma.hip", "pllm_attention_mfma_head_dim", defines, [])()
         _need(built == head_dim, f"attention library for head size {head_dim} reports head size {built}")
-        _attn_checked.add(head_dim)
-    f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", {"HEAD_DIM": head_dim}, _ATTN_SIG)
-    _check(f(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
-             block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
-             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks), _ptr(work_list),
-             0 if work_list is None else work_list.shape[0], _stream()),
-           "paged_attention_mfma")
+        has_terms = _fn("attention_mfma.hip", "pllm_attention_mfma_score_terms", defines, [])()
+        _need(bool(has_terms) == with_terms, f"attention library for head size {head_dim}: further score terms compiled in: {has_terms}")
+        _attn_checked.add((head_dim, with_terms))
+    args = (_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(block_tables),
+            block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
+            c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks),
+            _ptr(work_list), 0 if work_list is None else work_list.shape[0])
+    if with_terms:
+        f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma_terms", defines, _ATTN_TERMS_SIG)
+        _check(f(*args, *_terms_args(terms, num_heads, q.device), _stream()), "paged_attention_mfma")
+    else:
+        f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", defines, _ATTN_SIG)
+        _check(f(*args, _stream()), "paged_attention_mfma")
     return out
 
 
@@ -934,7 +981,7 @@ SPLIT_FROM_CONTEXT_TIMES_HEAD = 160_000   # context x head size of a few-query s
 
 
 def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim,
-                    scale, window, ctx) -> torch.Tensor:
+                    scale, window, ctx, terms: ScoreTerms | None = None) -> torch.Tensor:
     """Attention of one step's queries over the paged cache: the MFMA kernels for bfloat16 where they
     take the shape, else the plain kernel.  ``ctx`` gives host-side lengths for launch decisions.
 
@@ -962,11 +1009,11 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                 waves, size, parts = attention_plan(few, num_kv_heads, 1, ctx.max_k_len, group, head_dim, lds, _num_compute_units(q.device))
                 paged_attention_mfma(q[:few], k_pages, v_pages, block_tables[:few], cu_seqlens_q[:few + 1], seq_lens_k[:few],
                                      num_heads, num_kv_heads, head_dim, scale, window, 1, size, parts, waves,
-                                     2 if waves == 1 else 0, out=out[:few])
+                                     2 if waves == 1 else 0, out=out[:few], terms=terms)
             prompt_q = max(layout.portion_tokens, FEW_QUERY_COLUMNS // group + 1)     # enough columns for the prompt kernel's form
             psize, pparts = prompt_partitions(work.shape[0], num_kv_heads, layout.portion_context, _num_compute_units(q.device))
             paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
-                                 num_kv_heads, head_dim, scale, window, prompt_q, psize, pparts, 1, 2, out=out, work_list=work)
+                                 num_kv_heads, head_dim, scale, window, prompt_q, psize, pparts, 1, 2, out=out, work_list=work, terms=terms)
             return out
         q_lens, k_lens = ctx.q_lens, ctx.k_lens
         few = 0
@@ -980,13 +1027,13 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
             waves, size, parts = attention_plan(few, num_kv_heads, max_q, max_k, group, head_dim, lds, _num_compute_units(q.device))
             paged_attention_mfma(q[:rows], k_pages, v_pages, block_tables[:few], cu_seqlens_q[:few + 1], seq_lens_k[:few],
                                  num_heads, num_kv_heads, head_dim, scale, window, max_q, size, parts, waves,
-                                 2 if waves == 1 else 0, out=out[:rows])
+                                 2 if waves == 1 else 0, out=out[:rows], terms=terms)
             # the portions: rows, cu_seqlens_q and the output stay absolute, the per-sequence arrays start at `few`
             psize, pparts = prompt_partitions(sum(-(-n * group // PROMPT_TILE_COLUMNS) for n in q_lens[few:]), num_kv_heads,
                                               max(k_lens[few:]), _num_compute_units(q.device))
             paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
                                  num_kv_heads, head_dim, scale, window, max(q_lens[few:]), psize, pparts, 1, 2, out=out,
-                                 work_list=prompt_work_list(ctx, few, group))
+                                 work_list=prompt_work_list(ctx, few, group), terms=terms)
             return out
         waves, size, parts = attention_plan(ctx.num_seqs, num_kv_heads, ctx.max_q_len, ctx.max_k_len, group, head_dim, lds,
                                             _num_compute_units(q.device))
@@ -998,11 +1045,11 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
                                             _num_compute_units(q.device))
         return paged_attention_mfma(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads,
                                     head_dim, scale, window, ctx.max_q_len, size, parts, waves, 2 if waves == 1 else 0,
-                                    work_list=prompt_work_list(ctx, 0, group) if prompt else None)
+                                    work_list=prompt_work_list(ctx, 0, group) if prompt else None, terms=terms)
     if q.dtype == torch.bfloat16 and not _warned_plain_attention:
         _warned_plain_attention.append(True)
         log.warning("bfloat16 attention with pages of %d positions, head size %d, %d/%d heads runs on the plain kernel (one "
                     "wavefront per token and head): the matrix-core kernels take pages of at least 16 positions, head sizes "
                     "16..256 in steps of 16 and groups of at most 64 heads", bs, head_dim, num_heads, num_kv_heads)
     return paged_attention_generic(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads,
-                                   num_kv_heads, head_dim, scale, window)
+                                   num_kv_heads, head_dim, scale, window, terms=terms)

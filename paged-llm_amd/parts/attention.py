@@ -4,8 +4,11 @@ q/k/v projections -> rotary encoding of q and k -> k and v written to their slot
 attention over all keys of the request through the block table -> output projection
 (pagedllm/model/llama.py:131-160; the reference's Llama has no biases).  Sizes, the score scale, an optional window,
 the position encoding and whether the q/k/v projections have a bias (``qkv_bias``: tensors ``q_proj.bias`` ...; such
-a layer gives up the fused product-rotary-cache kernels) come in as parameters.  The three input projections are fused into one matrix when the
-weights arrive, so one product serves them.
+a layer gives up the fused product-rotary-cache kernels) come in as parameters, and so do further terms of the scores
+for layers that have them: ``score_cap`` c > 0 (the scaled product x becomes c tanh(x / c)), ``position_slopes`` (one
+number per head; slope * (key position - query position) is added after the cap) and ``sinks`` (True: a tensor
+``sinks`` [heads], one logit per head that takes part in the softmax's sum and in nothing else).  The three input
+projections are fused into one matrix when the weights arrive, so one product serves them.
 """
 
 from __future__ import annotations
@@ -33,6 +36,13 @@ class PagedAttention(Mixer):
         # False for a layer that always reads another layer's cache: it then has no k/v weights.
         self.kv_proj = bool(params.get("kv_proj", True))
         self.qkv_bias = bool(params.get("qkv_bias", False))
+        self.score_cap = float(params.get("score_cap") or 0.0)
+        slopes = params.get("position_slopes")
+        self.has_sinks = bool(params.get("sinks", False))
+        if self.score_cap < 0.0:
+            raise ValueError(f"a cap of the scores is positive (or 0 for none), got {self.score_cap}")
+        if slopes is not None and len(slopes) != self.num_heads:
+            raise ValueError(f"{len(slopes)} position slopes for {self.num_heads} heads")
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"{self.num_heads} heads are no multiple of {self.num_kv_heads} kv heads")
         if not 1 <= self.head_dim <= ops.MAX_HEAD_DIM_GENERIC:
@@ -41,6 +51,8 @@ class PagedAttention(Mixer):
         pos = params.get("position")
         self.position = env.position_encoding(PartSpec(**pos) if isinstance(pos, dict) else pos) if pos else None
         self.dtype, self.device = env.dtype, env.device
+        self.slopes = None if slopes is None else torch.tensor([float(x) for x in slopes], dtype=torch.float32, device=self.device)
+        self.terms: ops.ScoreTerms | None = None                 # put together in finalize(), once the sinks are there
         self._w: dict[str, torch.Tensor] = {}
         self.w_qkv: Weight | None = None
         self.w_o: Weight | None = None
@@ -58,6 +70,8 @@ class PagedAttention(Mixer):
             if self.kv_proj:
                 specs["k_proj.bias"] = WeightSpec((kv,), role="vector")
                 specs["v_proj.bias"] = WeightSpec((kv,), role="vector")
+        if self.has_sinks:
+            specs["sinks"] = WeightSpec((self.num_heads,), role="vector")
         return specs
 
     def assign(self, name, tensor):
@@ -73,6 +87,8 @@ class PagedAttention(Mixer):
         self.w_o = Weight(self._w["o_proj.weight"].contiguous())
         if self.qkv_bias:
             self.b_qkv = torch.cat([self._w[n.replace(".weight", ".bias")] for n in names]).contiguous()
+        terms = ops.ScoreTerms(self.score_cap, self.slopes, self._w["sinks"].contiguous() if self.has_sinks else None)
+        self.terms = terms if terms.any() else None
         self._w.clear()
 
     # ---- what it keeps
@@ -104,7 +120,7 @@ class PagedAttention(Mixer):
         qkv = qkv_rotary_cache(h, w_in, ctx.positions, self.position, nh, nkv, d, view.slot_mapping if write else None,
                                k_pages if write else None, v_pages if write else None, cache.block_size, bias=bias)
         o = ops.paged_attention(qkv, k_pages, v_pages, view.block_tables, ctx.cu_seqlens_q, ctx.seq_lens_k,
-                                nh, nkv, d, self.scale, self.window, ctx)
+                                nh, nkv, d, self.scale, self.window, ctx, terms=self.terms)
         return linear(o, self.w_o, partial_ok=bool(getattr(ctx, "partial_sums_ok", False)))
 
 

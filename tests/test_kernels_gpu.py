@@ -208,7 +208,7 @@ def paged_case(seq_lens_k, num_q, heads, kv_heads, d, bs, dtype, seed=0, spare=3
     return q, k_pages, v_pages, tables, cu, torch.tensor(seq_lens_k, dtype=torch.int32)
 
 
-def dense_attention(q, k_pages, v_pages, tables, cu, lens, heads, kv_heads, d, scale, window=None):
+def dense_attention(q, k_pages, v_pages, tables, cu, lens, heads, kv_heads, d, scale, window=None, **score_terms):
     bs = k_pages.shape[2]
     out = torch.empty(q.shape[0], heads * d)
     for s in range(len(lens)):
@@ -219,7 +219,11 @@ def dense_attention(q, k_pages, v_pages, tables, cu, lens, heads, kv_heads, d, s
         v = v_pages.float()[page, :, :, off]                       # [L, kv, d]
         q_full = torch.zeros(L, heads, d)
         q_full[L - (hi - lo):] = q[lo:hi].float().view(-1, heads, d)
-        o = plain.causal_attention(q_full, k, v, scale, window)
+        if score_terms:
+            from tests.toy_plain import attention_with_score_terms
+            o = attention_with_score_terms(q_full, k, v, scale, window, **score_terms)
+        else:
+            o = plain.causal_attention(q_full, k, v, scale, window)
         out[lo:hi] = o[L - (hi - lo):].reshape(hi - lo, heads * d)
     return out
 
@@ -280,6 +284,53 @@ def test_attention_one_far_key_stands_out():
     got = ops().paged_attention_generic(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
                                         d, 1.0).cpu()
     assert torch.allclose(got[0, :d], vp[page, 0, :, off], atol=1e-5)
+
+
+def score_terms_case(which, heads, seed=0):
+    """(keyword arguments of the plain attention, the kernels' ScoreTerms) for one of "cap", "slopes", "sinks", "all"."""
+    g = torch.Generator().manual_seed(seed)
+    cap = 0.8 if which in ("cap", "all") else 0.0
+    slopes = (0.002 * 4.0 ** torch.linspace(0, 2, heads)) if which in ("slopes", "all") else None      # 0.002 .. 0.032 a position
+    # (sinks as heavy as a few hundred keys together: leaving one out shows at long contexts too)
+    sinks = 7.0 + 1.5 * torch.randn(heads, generator=g) if which in ("sinks", "all") else None
+    on_gpu = lambda t: None if t is None else t.float().cuda().contiguous()
+    return dict(cap=cap, slopes=slopes, sinks=sinks), ops().ScoreTerms(cap, on_gpu(slopes), on_gpu(sinks))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["cap", "slopes", "sinks", "all"])
+@pytest.mark.parametrize("window", [0, 40])
+def test_paged_attention_generic_with_score_terms(dtype, which, window):
+    """Further terms of the scores (a cap, a slope times the distance, a sink per head), each alone and together, with
+    and without a window, against the plain attention with the same terms; each term must matter."""
+    heads, kv_heads, d, bs = 6, 2, 24, 8
+    lens, num_q = [150, 70, 9, 33], [30, 1, 9, 33]
+    q, kp, vp, tables, cu, sl = paged_case(lens, num_q, heads, kv_heads, d, bs, dtype, seed=21)
+    q = q * 2                                                   # scores of a few units: the cap has something to hold
+    scale = 1 / math.sqrt(d)
+    plain_terms, terms = score_terms_case(which, heads, seed=22)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, scale, window or None, **plain_terms)
+    without = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, scale, window or None)
+    tol = 2e-5 if dtype == torch.float32 else 1.6e-2
+    assert rel_err(without, want) > 5 * tol
+    got = ops().paged_attention_generic(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, scale,
+                                        window, terms=terms)
+    assert rel_err(got, want) <= tol
+
+
+def test_score_terms_are_checked():
+    heads, kv_heads, d, bs = 4, 2, 32, 16
+    q, kp, vp, tables, cu, sl = paged_case([20], [1], heads, kv_heads, d, bs, torch.bfloat16, seed=23)
+    args = (q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, 1.0, 0)
+    o = ops()
+    for bad in (o.ScoreTerms(-1.0), o.ScoreTerms(float("nan")), o.ScoreTerms(0.0, torch.zeros(heads + 1, device="cuda")),
+                o.ScoreTerms(0.0, None, torch.zeros(heads, device="cuda", dtype=torch.bfloat16)),
+                o.ScoreTerms(0.0, torch.zeros(heads))):
+        with pytest.raises(o.KernelError):
+            o.paged_attention_generic(*args, terms=bad)
+        with pytest.raises(o.KernelError):
+            o.paged_attention_mfma(*args, 1, terms=bad)
+    assert not o.ScoreTerms().any() and o.ScoreTerms(0.5).any()
 
 
 # ----------------------------------------------------------------------------------- sampling
@@ -595,6 +646,58 @@ def test_mfma_attention_one_far_key_stands_out(far):
         got = ops().paged_attention_mfma(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads,
                                          d, 1.0, 0, 1, *split).cpu().float()
         assert torch.allclose(got[0, 5 * d:6 * d], vp[page, 0, :, off].float(), atol=2e-2)
+
+
+@pytest.mark.parametrize("heads,kv_heads,d", [(8, 2, 64), (6, 2, 128), (4, 4, 32)])
+@pytest.mark.parametrize("which", ["cap", "slopes", "sinks", "all"])
+@pytest.mark.parametrize("window", [0, 200])
+def test_paged_attention_mfma_with_score_terms(heads, kv_heads, d, which, window):
+    """The matrix-core kernels with further score terms (compiled into a library of their own), in every form a step
+    may take: decoded tokens in one piece, in partitions (the sink then belongs to the partition that holds a query's
+    first visible key: with a window not the first one), with several wavefronts; prompt portions as workgroups that
+    share their keys, whole and in partitions."""
+    bs = 16
+    group = heads // kv_heads
+    plain_terms, terms = score_terms_case(which, heads, seed=24)
+    scale = 1 / math.sqrt(d)
+    # decoding and small portions
+    lens, num_q = [700, 33, 1030, 5, 64], [1, 1, 2, 1, 2]
+    q, kp, vp, tables, cu, sl = paged_case(lens, num_q, heads, kv_heads, d, bs, torch.bfloat16, seed=25)
+    q = q * 2
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, scale, window or None, **plain_terms)
+    assert rel_err(dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, scale, window or None), want) > 8e-2
+    args = (q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, scale, window, max(num_q))
+    cols = max(num_q) * group
+    ncb = 1 if cols <= 16 else (2 if cols <= 32 else 4)
+    for split in ((), (64, 17), (256, 5), (0, 1, 4), (0, 1, 8), (256, 5, 4), (128, 9, 8)):
+        if len(split) == 3 and ops()._merge_lds_bytes(ncb, split[2], d) > 160 * 1024:
+            continue
+        assert rel_err(ops().paged_attention_mfma(*args, *split, terms=terms), want) <= 1.6e-2, f"decode {split}"
+    # prompt portions: whole prompts and portions behind a context
+    lens, num_q = [300, 1100, 130], [300, 200, 64 // group + 3]
+    q, kp, vp, tables, cu, sl = paged_case(lens, num_q, heads, kv_heads, d, bs, torch.bfloat16, seed=26)
+    q = q * 2
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, scale, window or None, **plain_terms)
+    args = (q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, scale, window, max(num_q))
+    for split in ((0, 1, 1, 2), (128, 9, 1, 2), (512, 3, 1, 2), (0, 1, 1, 4)):
+        assert rel_err(ops().paged_attention_mfma(*args, *split, terms=terms), want) <= 1.6e-2, f"prompt {split}"
+
+
+def test_score_terms_through_the_planned_launch():
+    """Decoded tokens at long contexts beside prompt portions, launched as the engine launches a step (two launches,
+    partitions as planned), with all score terms at once."""
+    import types
+    heads, kv_heads, d, bs = 8, 2, 64, 16
+    plain_terms, terms = score_terms_case("all", heads, seed=27)
+    q_lens, k_lens = [1, 1, 2, 100, 300], [3000, 17, 4100, 2000, 300]
+    q, kp, vp, tables, cu, sl = paged_case(k_lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16, seed=28)
+    q = q * 2
+    ctx = types.SimpleNamespace(num_seqs=len(q_lens), max_q_len=max(q_lens), max_k_len=max(k_lens), q_lens=q_lens, k_lens=k_lens,
+                                capturing=False, device=torch.device("cuda"))
+    got = ops().paged_attention(q.cuda(), kp.cuda(), vp.cuda(), tables.cuda(), cu.cuda(), sl.cuda(), heads, kv_heads, d, 0.125, 0, ctx,
+                                terms=terms)
+    want = dense_attention(q, kp, vp, tables, cu, sl, heads, kv_heads, d, 0.125, None, **plain_terms)
+    assert rel_err(got, want) <= 1.6e-2
 
 
 @pytest.mark.parametrize("heads,kv_heads,d", [(32, 4, 64), (8, 2, 128), (6, 1, 96)])

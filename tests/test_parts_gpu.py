@@ -237,6 +237,55 @@ def test_attention_part_with_biased_projections(dtype, tol):
     assert rel(torch.cat(out), want) <= tol, "a portion and single tokens"
 
 
+@pytest.mark.parametrize("dtype,tol", DTYPES)
+@pytest.mark.parametrize("window", [0, 9])
+def test_attention_part_with_score_terms(dtype, tol, window):
+    """Scores with a cap, a slope per head times the distance and a sink per head (parameters of the part; the
+    reference's Llama has none of them): whole, then a portion and single tokens, against the plain attention with the
+    same terms; leaving any of them out would not pass."""
+    from tests.toy_plain import attention_with_score_terms
+    env = env_for(dtype)
+    slopes = [0.3 / (j + 1) for j in range(HEADS)]
+    params = {"num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM, "score_cap": 0.5, "position_slopes": slopes,
+              "sinks": True, "window": window,
+              "position": {"kind": "rotary", "params": {"head_dim": HEAD_DIM, "theta": THETA, "scaling": None}}}
+    mixer = build("mixer", "paged_attention", params, env)
+    assert mixer.weight_specs()["sinks"].shape == (HEADS,)
+    gen = torch.Generator().manual_seed(33)
+    w = {}
+    for name, spec in mixer.weight_specs().items():
+        t = (1.0 + torch.randn(spec.shape, generator=gen)) if name == "sinks" else 0.25 * torch.randn(spec.shape, generator=gen)
+        w[name] = t if name == "sinks" else t.to(getattr(torch, dtype)).float()
+        mixer.assign(name, w[name])
+    mixer.finalize()
+    L = 52
+    x = rows(L, 34, dtype)
+    xf = x.float()
+    ang = plain.rotary_angles(torch.arange(L), plain.inverse_frequencies(HEAD_DIM, THETA, None))
+    rounded = lambda t: t.to(getattr(torch, dtype)).float()
+    q = plain.apply_rotary(rounded(xf @ w["q_proj.weight"].T).view(L, HEADS, HEAD_DIM), ang)
+    k = plain.apply_rotary(rounded(xf @ w["k_proj.weight"].T).view(L, KV_HEADS, HEAD_DIM), ang)
+    v = rounded(xf @ w["v_proj.weight"].T).view(L, KV_HEADS, HEAD_DIM)
+    out_of = lambda o: o.reshape(L, HEADS * HEAD_DIM) @ w["o_proj.weight"].T
+    all_terms = dict(cap=0.5, slopes=torch.tensor(slopes), sinks=w["sinks"])
+    want = out_of(attention_with_score_terms(q, k, v, HEAD_DIM ** -0.5, window or None, **all_terms))
+    for left_out in all_terms:
+        fewer = {n: t for n, t in all_terms.items() if n != left_out}
+        assert rel(out_of(attention_with_score_terms(q, k, v, HEAD_DIM ** -0.5, window or None, **fewer)), want) > 4 * tol, left_out
+    group = mixer.cache_spec().group_name()
+    table = [4, 1, 6, 3]
+    got = mixer.forward(x.cuda(), step_context([(0, L)], [table], group, dtype), layer_cache(mixer, dtype, 8), None)
+    assert rel(got, want) <= tol, "whole"
+    cache, out = layer_cache(mixer, dtype, 8), []
+    for start, n in [(0, 33), (33, 2)] + [(p, 1) for p in range(35, L)]:
+        out.append(mixer.forward(x[start:start + n].cuda(), step_context([(start, n)], [table], group, dtype), cache, None))
+    assert rel(torch.cat(out), want) <= tol, "a portion and single tokens"
+    with pytest.raises(ValueError, match="slopes"):
+        build("mixer", "paged_attention", {**params, "position_slopes": slopes[:-1]}, env)
+    with pytest.raises(ValueError, match="cap"):
+        build("mixer", "paged_attention", {**params, "score_cap": -2.0}, env)
+
+
 def test_attention_part_refuses_sizes_its_kernels_do_not_take():
     env = env_for("bfloat16")
     with pytest.raises(ValueError, match="head sizes 1..256"):

@@ -139,6 +139,43 @@ def test_attention_special_cases():
     torch.testing.assert_close(plain.causal_attention(q, k, v, 0.3, window=99), plain.causal_attention(q, k, v, 0.3))
 
 
+def test_attention_with_score_terms_reduces_to_library_routines():
+    """The plain attention with further score terms (tests/toy_plain.py: the reference's model has none of them; the
+    attention part takes them as parameters): without terms it is the plain attention; slopes are an additive mask of
+    the library routine; a sink is one more key with that score and a value of zeros; a huge cap changes nothing and a
+    tiny one leaves the running mean of the values."""
+    from tests.toy_plain import attention_with_score_terms as awt
+    L, nh, nkv, d = 23, 4, 2, 16
+    q, k, v = rnd(L, nh, d, seed=15), rnd(L, nkv, d, seed=16), rnd(L, nkv, d, seed=17)
+    scale = d ** -0.5
+    torch.testing.assert_close(awt(q, k, v, scale, window=5), plain.causal_attention(q, k, v, scale, window=5))
+    kk, vv = k.repeat_interleave(2, 1).transpose(0, 1), v.repeat_interleave(2, 1).transpose(0, 1)
+    slopes = torch.tensor([0.5, 0.05, 0.0, 0.2])
+    dist = (torch.arange(L)[None, :] - torch.arange(L)[:, None]).float()
+    mask = slopes[:, None, None] * dist + torch.full((L, L), float("-inf")).triu(1)
+    want = F.scaled_dot_product_attention(q.transpose(0, 1), kk, vv, attn_mask=mask).transpose(0, 1)
+    torch.testing.assert_close(awt(q, k, v, scale, slopes=slopes), want, atol=1e-5, rtol=1e-5)
+    # (the sign: a positive slope turns a head towards the near keys; with a steep one the query sees itself only)
+    torch.testing.assert_close(awt(q, k, v, scale, slopes=torch.full((nh,), 200.0)), v.repeat_interleave(2, 1), atol=1e-5, rtol=1e-5)
+    # a sink = a key in front whose score is the sink whatever the query and whose value is zero; for one query:
+    sinks = torch.tensor([0.3, -1.0, 2.0, 0.0])
+    got = awt(q, k, v, scale, sinks=sinks)
+    i = 11
+    for j in range(nh):
+        x = torch.cat([sinks[j:j + 1], (q[i, j] @ k[:i + 1, j // 2].T) * scale])
+        want_row = torch.softmax(x, 0)[1:] @ v[:i + 1, j // 2]
+        torch.testing.assert_close(got[i, j], want_row, atol=1e-5, rtol=1e-5)
+    assert not torch.allclose(got, awt(q, k, v, scale), atol=1e-2)
+    torch.testing.assert_close(awt(q, k, v, scale, sinks=torch.full((nh,), -1e4)), awt(q, k, v, scale))
+    # the cap
+    torch.testing.assert_close(awt(q, k, v, scale, cap=1e4), awt(q, k, v, scale), atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(awt(q, k, v, scale, cap=1e-4)[7, 1], v[:8, 0].mean(0), atol=1e-3, rtol=1e-3)
+    capped = awt(q * 4, k * 4, v, scale, cap=2.0)                        # scores of +-10 and more, held to +-2
+    assert not torch.allclose(capped, awt(q * 4, k * 4, v, scale), atol=1e-2)
+    x = (q[5, 0] * 4) @ (k[:6, 0] * 4).T * scale
+    torch.testing.assert_close(capped[5, 0], torch.softmax(2.0 * torch.tanh(x / 2.0), 0) @ v[:6, 0], atol=1e-5, rtol=1e-5)
+
+
 def test_swiglu_is_silu_times_up():
     x, wg, wu, wd = rnd(3, 12, seed=15), rnd(20, 12, seed=16), rnd(20, 12, seed=17), rnd(12, 20, seed=18)
     want = F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)

@@ -3,8 +3,9 @@ change to the framework's files: a mixer with per-request state of fixed size (w
 replayed HIP graphs), a layer that runs twice, a layer that reads another layer's cache, a windowed
 attention layer with pages of its own whose rotary encoding turns only half of each head in interleaved
 pairs, a feed-forward with a router and experts, another position encoding (rotation angles on a
-linear grid of frequencies), and a block of another arrangement (one norm shared by a mixer and a
-feed-forward that run side by side).  The toy model is replayed whole, in portions and mixed, generated
+linear grid of frequencies), a block of another arrangement (one norm shared by a mixer and a
+feed-forward that run side by side), and an attention layer whose scores carry further terms (a cap, a
+slope per head times the distance, a sink per head).  The toy model is replayed whole, in portions and mixed, generated
 from through the entry point, and compared with a plain implementation written here."""
 
 import numpy as np
@@ -14,14 +15,16 @@ import torch
 from tests import helpers
 from tests.helpers import TraceBuilder
 from tests.plain import llama_plain as plain
+from tests.toy_plain import attention_with_score_terms
 
 pytestmark = pytest.mark.gpu
 
 TOY = {"architectures": ["ToyHybridForCausalLM"], "vocab_size": 120, "hidden_size": 48, "intermediate_size": 72,
        "heads": 3, "kv_heads": 1, "head_dim": 16, "decay": 0.8, "window": 7, "eps": 1e-5, "theta": 100.0,
-       "experts": 3, "expert_size": 24, "linear_base": 0.37, "max_position_embeddings": 256}
+       "experts": 3, "expert_size": 24, "linear_base": 0.37, "max_position_embeddings": 256,
+       "score_cap": 0.05, "slope_base": 0.25}
 # step -> (layer, cache_from): layer 1 (the stateful mixer) runs twice, step 2 reads the cache of step 0,
-# layer 4 is the block with one shared norm
+# layer 4 is the block with one shared norm, and its attention has the further score terms
 SCHEDULE = [(0, None), (1, None), (2, 0), (3, None), (1, None), (4, None)]
 PARTIAL_ROTARY = 8          # of 16 elements of a head, in interleaved pairs (layer 3)
 
@@ -160,7 +163,8 @@ def register_toy():
         # layers 0 and 2 share a cache, so they share the position encoding too (the linear grid); layer 3 has the
         # experts, a window and the partial interleaved rotation; layer 4 is the other arrangement
         mixers = [attention(linear_grid), PartSpec("toy_decay", {"decay": c["decay"]}), attention(linear_grid, kv_proj=False),
-                  attention(partial, window=c["window"]), attention()]
+                  attention(partial, window=c["window"]),
+                  attention(score_cap=c["score_cap"], position_slopes=toy_slopes(c), sinks=True)]
         layers = []
         for i, m in enumerate(mixers):
             if i == 4:
@@ -175,6 +179,10 @@ def register_toy():
                          head_name="head", max_positions=c["max_position_embeddings"], stored_dtype="float32")
 
     register_architecture(Architecture("ToyHybridForCausalLM", lambda raw: dict(raw), build_spec))
+
+
+def toy_slopes(c):
+    return [c["slope_base"] / 2 ** j for j in range(c["heads"])]
 
 
 def rotate_some(x, angles, width, interleaved):
@@ -222,7 +230,11 @@ def plain_toy(folder, tokens):
                 kept[step] = (k, v)
             else:
                 k, v = kept[cache_from]
-            o = plain.causal_attention(q, k, v, d ** -0.5, c["window"] if layer == 3 else None)
+            if layer == 4:
+                o = attention_with_score_terms(q, k, v, d ** -0.5, None, cap=c["score_cap"], slopes=torch.tensor(toy_slopes(c)),
+                                               sinks=w[p + "mixer.sinks"])
+            else:
+                o = plain.causal_attention(q, k, v, d ** -0.5, c["window"] if layer == 3 else None)
             a = o.reshape(T, nh * d) @ w[p + "mixer.o_proj.weight"].T
         if layer == 4:                                       # one norm, both branches from the same rows
             x = x + a + plain.swiglu(h, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
