@@ -181,7 +181,7 @@ class LLMEngine:
         taken where the sampling kernel leaves them on the GPU, so that the GPU goes from one step into the next
         without waiting for the host to see the tokens (see ``Scheduler.plan_ahead`` for when that is possible;
         the step's graph must exist already).  (the next plan, its logits), or None."""
-        if not self.run_ahead or self.cache_manager.uses_state or pending.on_device is None:
+        if not self.run_ahead or pending.on_device is None:
             return None
         ahead = self.scheduler.plan_ahead(plan)
         if ahead is None:
@@ -193,8 +193,11 @@ class LLMEngine:
             request = then.request
             row, count = row_of[request.id]
             rows.append(row)
+            # (a request's state of fixed size moves once per step, in the order of the steps on the stream, whoever
+            #  launched them; the state of a request that ends in ``plan`` is moved once more in its freed slot, which the
+            #  next owner's first step clears)
             entries.append(StepEntry(request.id, [0], request.computed + count, {g: cm.block_table(request.id, g) for g in self.groups},
-                                     None, [0], cm.table_version(request.id)))
+                                     cm.state_slot(request.id), [0], cm.table_version(request.id)))
         staged = self.runner.prepare(entries)
         if staged is None:
             return None                                      # (the pages taken for the next tokens stay with their requests)

@@ -352,6 +352,46 @@ def test_toy_model_generates_through_the_entry_point_with_default_settings(toy_f
     engine.cache_manager.check_invariants()
 
 
+def test_toy_model_steps_launched_ahead_with_state(toy_folder):
+    """Decode steps are launched one ahead of the tokens the host has seen, also for a model with per-request state of
+    fixed size: the state moves once per step in the order of the steps.  Requests stop on tokens of their own while the
+    step after already runs (it moves their state once more, in a slot that is freed then); the requests that take
+    those slots next must start from a fresh state."""
+    from paged_llm_amd import EngineConfig, SamplingParams
+    from paged_llm_amd.engine.llm_engine import LLMEngine
+    engine = LLMEngine(toy_folder, EngineConfig(dtype="float32", num_gpu_blocks=48, max_model_len=128, max_num_seqs=3))
+    assert engine.run_ahead and engine.cache_manager.uses_state
+
+    def greedy(prompt, n):
+        toks = list(prompt)
+        for _ in range(n):
+            toks.append(int(np.argmax(plain_toy(toy_folder, toks)[-1])))
+        return toks[len(prompt):]
+
+    seen_in_flight = 0
+    for round_, seeds in enumerate([(300, 301, 302), (303, 304, 305), (306, 307, 308)]):
+        prompts = [helpers.random_tokens(9 + 4 * i, TOY["vocab_size"], seed=sd) for i, sd in enumerate(seeds)]
+        want = [greedy(p, 14) for p in prompts]
+        stops = [w[k] for w, k in zip(want[:2], (5, 9))]             # (a request stops where that token comes first)
+        params = [SamplingParams(temperature=0.0, max_tokens=14, stop_token_ids=[t]) for t in stops] + \
+                 [SamplingParams(temperature=0.0, max_tokens=14, ignore_eos=True)]
+        ids = [engine.add_request(p, sp) for p, sp in zip(prompts, params)]
+        got = {i: [] for i in ids}
+        while engine.has_unfinished_requests:
+            for out in engine.step():
+                if out.new_token is not None:
+                    got[out.seq_id].append(out.new_token)
+            seen_in_flight += engine.step_in_flight
+        for rid, w, stop in zip(ids, want, stops + [None]):
+            upto = len(w) if stop is None else w.index(stop) + 1
+            assert got[rid] == w[:upto], f"round {round_}, request {rid}"
+        assert engine.cache_manager.slots.num_free == engine.cache_manager.slots.num_slots
+        if round_ == 1:
+            assert engine.stats.num_dropped_tokens >= 1                  # (a state was moved in a freed slot; a round follows)
+    assert seen_in_flight >= 10
+    engine.cache_manager.check_invariants()
+
+
 # ------------------------------------------------------------------------------------------- a page of another shape
 LATENT = {"architectures": ["ToyLatentForCausalLM"], "vocab_size": 90, "hidden_size": 40, "intermediate_size": 56,
           "heads": 2, "kv_heads": 1, "head_dim": 16, "latent": 24, "eps": 1e-5, "theta": 50.0, "max_position_embeddings": 256}
