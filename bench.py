@@ -35,6 +35,10 @@ MODELS = {
     "llama-3.2-1b": ("Llama-3.2-1B shapes", dict(
         TINYLLAMA, num_hidden_layers=16, num_key_value_heads=8, intermediate_size=8192, vocab_size=128256,
         rope_theta=500000.0, rope_scaling=_LLAMA3(32.0), tie_word_embeddings=True, max_position_embeddings=131072)),
+    "llama-3.2-3b": ("Llama-3.2-3B shapes", dict(
+        TINYLLAMA, num_hidden_layers=28, hidden_size=3072, num_attention_heads=24, num_key_value_heads=8, head_dim=128,
+        intermediate_size=8192, vocab_size=128256, rope_theta=500000.0, rope_scaling=_LLAMA3(32.0), tie_word_embeddings=True,
+        max_position_embeddings=131072)),
     "llama-3.1-8b": ("Llama-3.1-8B shapes", dict(
         TINYLLAMA, num_hidden_layers=32, hidden_size=4096, num_key_value_heads=8, head_dim=128, intermediate_size=14336,
         vocab_size=128256, rope_theta=500000.0, rope_scaling=_LLAMA3(8.0), max_position_embeddings=131072)),

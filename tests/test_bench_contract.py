@@ -25,4 +25,4 @@ def test_step_sizes_of_the_headline_configuration():
     # a 2048-token prompt: 3.969 TFLOP in the layers' products and the head row, 0.378 TFLOP of causal attention
     flops = bench.prefill_flops(bench.TINYLLAMA, 2048, 1)
     assert abs(flops - 4.347e12) < 0.01e12
-    assert set(bench.MODELS) == {"tinyllama-1.1b", "llama-3.2-1b", "llama-3.1-8b"}
+    assert set(bench.MODELS) == {"tinyllama-1.1b", "llama-3.2-1b", "llama-3.2-3b", "llama-3.1-8b"}
