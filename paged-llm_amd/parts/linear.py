@@ -50,6 +50,8 @@ class Weight:
 
 STREAM_MIN_ROWS, STREAM_MAX_ROWS = 17, 128      # rows the streaming kernel is chosen for
 TILE_MAX_ROWS = 640                             # rows up to which the tiled kernel is chosen for small matrices cut along K
+# ... and from so few rows on for matrices of so many elements that fill the GPU in so many ranges of K at most
+TILE_PARTIAL_FROM_ROWS, TILE_PARTIAL_MIN_ELEMENTS, TILE_PARTIAL_MOST_RANGES = 65, 1 << 24, 12
 STREAM_GATED_MAX_ROWS = 64                      # the gated product: beyond, its rows' traffic costs more than the library's kernel
 STREAM_LONG_K, STREAM_LONG_K_MAX_ROWS = 8192, 64 # from this K on a product in one range takes the streaming kernel up to so many rows
 
@@ -67,13 +69,24 @@ def _few_weight_rows(weight) -> bool:
 def _tiles(x, weight, partial_ok: bool) -> bool:
     """Whether this plain product goes to the tiled kernel (129 to 640 rows): only as partial sums of ranges of K, which
     give a small matrix enough workgroups, when whoever takes the result adds them (2048 x 5632 at 264 rows: 14 us against
-    the library's 23; 2048 x 2048: 8.5 against 12.5; in one range, or for 11264 x 2048, the library's kernels are faster)."""
+    the library's 23; 2048 x 2048: 8.5 against 12.5; in one range, or for 11264 x 2048, the library's kernels are faster).
+    Larger matrices take it from 65 rows on, where the streaming kernel is chosen otherwise: a workgroup's tile of 128
+    weight rows over a range of K draws the step's rows a quarter as often as the streaming kernel's 32 weight rows over
+    all of K (4096 x 14336 at 64 / 96 / 128 rows: 24.3 / 26.6 / 29.6 us against 28.3 / 45.5 / 55.2; 4096 x 4096: 10.7 / 12.0 /
+    13.7 against 13.0 / 16.6 / 19.0; 2048 x 5632 the same either way and 2048 x 2048 8.5 against 7.0 at 128 rows: those
+    stay).  Inside whole steps the gain shows from 65 rows on and where a dozen ranges fill the GPU (the norm kernel adds
+    them): Llama-3.1-8B shapes at 96 / 128 requests 9,361 -> 9,831 and 10,057 -> 10,633 tok/s, a prompt of 128 tokens 6.09 ->
+    5.52 ms; 2048 x 8192, which needs 16 ranges, lost 1 to 2 % there although it is faster on its own (12.5 against 15.9 us)."""
     if not (partial_ok and isinstance(weight, Weight) and weight.tiled is not None and weight.pairing == "plain"):
         return False
     rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
     n, k = weight.shape
-    return (STREAM_MAX_ROWS < rows <= TILE_MAX_ROWS and x.dtype == torch.bfloat16 and _few_weight_rows(weight)
-            and ops.tile_linear_plan(rows, n, k, ops._num_compute_units(weight.plain.device)) > 1)
+    if not (x.dtype == torch.bfloat16 and _few_weight_rows(weight)):
+        return False
+    ranges = ops.tile_linear_plan(rows, n, k, ops._num_compute_units(weight.plain.device))
+    if TILE_PARTIAL_FROM_ROWS <= rows <= STREAM_MAX_ROWS:
+        return n * k >= TILE_PARTIAL_MIN_ELEMENTS and 1 < ranges <= TILE_PARTIAL_MOST_RANGES
+    return STREAM_MAX_ROWS < rows <= TILE_MAX_ROWS and ranges > 1
 
 
 def _streams(x, weight, epi: int, partial_ok: bool = False) -> bool:
@@ -143,13 +156,13 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
     if bias is not None:
         sums = linear(x, weight, torch.float32)
         return ops.add_bias(sums, bias, out_dtype or _plain(weight).dtype)
-    if _streams(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok):
-        return _stream(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok=partial_ok)
     if out_dtype != torch.float32 and _tiles(x, weight, partial_ok):
         x = rows_of(x)
         if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
             x = x.contiguous()
         return ops.tile_linear(x, weight.tiled, ops.SL_PARTIAL)
+    if _streams(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok):
+        return _stream(x, weight, ops.SL_F32 if out_dtype == torch.float32 else ops.SL_BF16, partial_ok=partial_ok)
     if weight.dtype == torch.bfloat16:
         out = _fused(x, weight, ops.EPI_F32 if out_dtype == torch.float32 else ops.EPI_BF16)
         if out is not None:
@@ -162,18 +175,31 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
 
 
 TILE_GATED_ROWS = (161, 320)                    # rows for which the gated product takes the tiled kernel
+TILE_GATED_FROM_WHEN_FILLING = 24               # ... and from so few rows on when one block of rows already fills the GPU
+
+
+def _tiles_gated(x, weight, rows: int) -> bool:
+    """Whether the gated product goes to the tiled kernel.  With two blocks of input rows it takes as long as the library's
+    product (11264 x 2048 at 264 rows: 28 us both) and saves the activation kernel and its pass over the intermediate rows
+    (5 us).  A matrix whose tiles of 128 weight rows fill three quarters of the compute units by themselves takes it with
+    one block of rows as well, from a few rows on: there every workgroup draws its own weights and the step's few rows,
+    where the streaming kernel's workgroups of 32 to 64 weight rows draw the rows four times as often (28672 x 4096 at
+    32 / 64 / 128 rows: 46 / 46 / 52 us against 50 / 57 us streaming and 53 / 53 / 59 us in the library with the activation
+    kernel; 24576 x 2048 at 64 rows 27 against 33 and 30; a matrix of 16384 x 3072, 128 tiles, stays where it was)."""
+    if not (isinstance(weight, Weight) and weight.tiled is not None and weight.pairing == "gated" and x.dtype == torch.bfloat16):
+        return False
+    filling = weight.shape[0] // 128 >= 3 * ops._num_compute_units(weight.plain.device) // 4
+    return (TILE_GATED_FROM_WHEN_FILLING if filling else TILE_GATED_ROWS[0]) <= rows <= TILE_GATED_ROWS[1]
 
 
 def gated_linear(x, w_gate_up, activation: str = "silu") -> torch.Tensor:
     """act(x Wg^T) * (x Wu^T) with [Wg; Wu] stacked in one matrix (a tensor, or a ``Weight`` with the gated pairing);
     ``activation``: one of ``ops.ACTIVATIONS``."""
-    if _streams(x, w_gate_up, ops.SL_GATED) and w_gate_up.pairing == "gated":
-        return _stream(x, w_gate_up, ops.SL_GATED, activation=activation)
     rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
-    if (isinstance(w_gate_up, Weight) and w_gate_up.tiled is not None and w_gate_up.pairing == "gated" and x.dtype == torch.bfloat16
-            and TILE_GATED_ROWS[0] <= rows <= TILE_GATED_ROWS[1]):
-        # Two blocks of input rows: the tiled kernel takes as long as the library's product there (11264 x 2048 at 264
-        # rows: 28 us both) and saves the activation kernel and its pass over the intermediate rows (5 us).
+    tiles = _tiles_gated(x, w_gate_up, rows)
+    if not tiles and _streams(x, w_gate_up, ops.SL_GATED) and w_gate_up.pairing == "gated":
+        return _stream(x, w_gate_up, ops.SL_GATED, activation=activation)
+    if tiles:
         x = rows_of(x)
         if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
             x = x.contiguous()

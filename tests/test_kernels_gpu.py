@@ -1115,7 +1115,7 @@ def test_tile_linear_plain_float_and_partial(m, n, k):
     assert torch.equal(alone.cpu(), o.tile_linear(x.cuda(), tiled, o.SL_F32)[m // 2:m // 2 + 5].cpu())     # a row's sums do not depend on the others
 
 
-@pytest.mark.parametrize("m", [130, 264])
+@pytest.mark.parametrize("m", [17, 24, 49, 100, 130, 264])
 def test_tile_linear_gated_and_rotary(m):
     from paged_llm_amd.parts.registry import BuildEnv
     from paged_llm_amd.parts.rope import RotaryEncoding

@@ -361,6 +361,28 @@ def test_feed_forward_part(dtype, tol, num_rows):
     assert rel(ff.forward(norm.pending(x.cuda()), None), want) <= tol
 
 
+@pytest.mark.parametrize("num_rows", [16, 24, 40, 64, 100, 160, 200])
+def test_feed_forward_part_whose_gated_matrix_fills_the_gpu(num_rows):
+    """A gate/up matrix of so many rows that its tiles of 128 fill the compute units with one block of input rows takes
+    the tiled kernel from a few rows on (the rule is by sizes only); every row count on both sides of the rule's
+    limits, and fed by a norm that has not run yet."""
+    from paged_llm_amd.csrc import ops
+    from paged_llm_amd.parts import linear
+    hidden, inter = 64, 96 * ops._num_compute_units(torch.device("cuda:0")) // 2          # 2 x inter / 128 = 3/4 of the compute units
+    env = env_for("bfloat16", hidden=hidden)
+    ff = build("feed_forward", "gated_mlp", {"intermediate_size": inter}, env)
+    w = give_weights(ff, 41, "bfloat16")
+    x = rows(num_rows, 42, "bfloat16", hidden=hidden)
+    assert linear._tiles_gated(x.cuda(), ff.w_gate_up, num_rows) == (24 <= num_rows <= 320)
+    want = plain.swiglu(x.float(), w["gate_proj.weight"], w["up_proj.weight"], w["down_proj.weight"])
+    assert rel(ff.forward(x.cuda(), None), want) <= 3e-2
+    norm = build("norm", "rmsnorm", {"eps": EPS}, env)
+    nw = give_weights(norm, 43, "bfloat16")["weight"]
+    h = plain.rms_norm(x.float(), nw, EPS).to(x.dtype).float()
+    want = plain.swiglu(h, w["gate_proj.weight"], w["up_proj.weight"], w["down_proj.weight"])
+    assert rel(ff.forward(norm.pending(x.cuda()), None), want) <= 3e-2
+
+
 def test_feed_forward_part_refuses_unknown_activations():
     with pytest.raises(NotImplementedError):
         build("feed_forward", "gated_mlp", {"intermediate_size": 64, "activation": "swish7"}, env_for("bfloat16"))
@@ -389,6 +411,26 @@ def test_feed_forward_part_with_another_activation(dtype, tol, num_rows):
     # (the other activation would not pass: the two results are further apart than the bound)
     silu = torch.nn.functional.silu(x.float() @ w["gate_proj.weight"].T) * (x.float() @ w["up_proj.weight"].T) @ w["down_proj.weight"].T
     assert rel(silu, want_of(x.float())) > 2 * tol
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (2048, 8192), (2048, 2048)])
+@pytest.mark.parametrize("num_rows", [40, 65, 100, 128, 200])
+def test_products_that_may_leave_partial_sums(n, k, num_rows):
+    """A product whose result goes to a norm that adds partial sums may leave float sums over ranges of K: which kernel
+    takes it is decided by sizes and rows only (the tiled kernel from 65 rows on for matrices that a dozen ranges
+    spread over the GPU, the streaming kernel below and for smaller matrices, the tiled one beyond 128 rows), and
+    whatever comes back adds up to the product."""
+    from paged_llm_amd.parts import linear as L
+    gen = torch.Generator().manual_seed(n + k + num_rows)
+    w = (torch.randn(n, k, generator=gen) * k ** -0.5).to(torch.bfloat16)
+    x = torch.randn(num_rows, k, generator=gen).to(torch.bfloat16)
+    weight = L.Weight(w.cuda())
+    tiled = L._tiles(x.cuda(), weight, True)
+    assert tiled == (num_rows > 128 or (num_rows >= 65 and (n, k) == (4096, 4096)))
+    out = L.linear(x.cuda(), weight, partial_ok=True)
+    assert out.dtype == torch.float32 and out.dim() == 3 and out.shape[1:] == (num_rows, n)
+    assert rel(out.sum(0), x.float() @ w.float().T) <= 2e-3
+    assert L.linear(x.cuda(), weight).dtype == torch.bfloat16          # without the permission: rows, as ever
 
 
 # ------------------------------------------------------------------------------------------ block
