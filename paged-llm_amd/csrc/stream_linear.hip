@@ -369,7 +369,7 @@ PLLM_API int pllm_stream_linear(int epi, const void* x, int ldx, const void* wt,
 // wavefronts (the weights' tiles are 1 KB of contiguous memory each and land in operand order; the rows as above), and
 // the eight compute wavefronts, as 2 x 4 over the tile (MTW tiles of 16 input rows x 2 blocks of 16 weight rows each),
 // only read LDS and multiply.  No sums across wavefronts: each owns its outputs.  Epilogues as above.
-constexpr int kTileBlocksN = 8;                      // blocks of 16 weight rows per workgroup
+constexpr int kTileBlocksN = 8;                      // blocks of 16 weight rows per workgroup, at most (NB: 8 or 4)
 constexpr int kTileStageSteps = 2;                   // steps of 32 columns per stage
 
 // MT: tiles of 16 input rows per workgroup (the upper row of wavefronts takes the larger half).
@@ -378,13 +378,13 @@ constexpr int kTileStageSteps = 2;                   // steps of 32 columns per 
 // stages in flight, with or without the products; four compute wavefronts as 2 x 2 with a third less LDS traffic took the
 // same time), so a tile is as large as registers and LDS allow, and matrices of many rows and few hundred input rows,
 // whose tiles cannot be large in both directions, stay with the library, which meets the same bound.
-template <int EPI, int MT, int R>
+template <int EPI, int MT, int R, int NB>
 __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const StreamLinearParams p) {
   constexpr int CW = kComputeWaves;
   extern __shared__ __attribute__((aligned(16))) unsigned char sl_lds[];
   constexpr int MTW = (MT + 1) / 2;                              // tiles of 16 input rows per wavefront (at most)
-  constexpr int WN = CW / 2, NTW = kTileBlocksN / WN;            // wavefronts along the weight rows, blocks of 16 weight rows each
-  constexpr int kWBlocks = kTileBlocksN * kTileStageSteps, kXBlocks = MT * kTileStageSteps;
+  constexpr int WN = CW / 2, NTW = NB / WN;                      // wavefronts along the weight rows, blocks of 16 weight rows each
+  constexpr int kWBlocks = NB * kTileStageSteps, kXBlocks = MT * kTileStageSteps;
   constexpr int kSlotBytes = (kWBlocks + kXBlocks) * 1024;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nb = blockIdx.x, row0 = blockIdx.y * (MT * 16), split = blockIdx.z;
@@ -407,7 +407,7 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
                                                                  //  below count them; a loader whose share is one short repeats its last block)
       if (bb < kWBlocks) {
         const int u = bb / kTileStageSteps, st = bb - u * kTileStageSteps;
-        base[i] = p.wt + (((size_t)(nb * kTileBlocksN + u) * p.ksteps + first_stage * kTileStageSteps + st) * 64 + lane) * 8;
+        base[i] = p.wt + (((size_t)(nb * NB + u) * p.ksteps + first_stage * kTileStageSteps + st) * 64 + lane) * 8;
       } else {
         const int bx = bb - kWBlocks, t = bx / kTileStageSteps, st = bx - t * kTileStageSteps;
         const int row = min(row0 + t * 16 + xr, p.M - 1);        // rows past M repeat the last one: never stored
@@ -424,7 +424,7 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
         for (int i = 0; i < kPerLoader; ++i) {
           const int bb = min(l + i * kLoaderWaves, kBlocks - 1);
           const bf16* src;
-          if (bb < kWBlocks) src = p.wt + (((size_t)(nb * kTileBlocksN + bb / kTileStageSteps) * p.ksteps + ks0) * 64 + lane) * 8;
+          if (bb < kWBlocks) src = p.wt + (((size_t)(nb * NB + bb / kTileStageSteps) * p.ksteps + ks0) * 64 + lane) * 8;
           else src = p.x + (size_t)min(row0 + ((bb - kWBlocks) / kTileStageSteps) * 16 + xr, p.M - 1) * p.ldx + ks0 * kChunkK + xg * 8;
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                            (__attribute__((address_space(3))) void*)(slot + bb * 1024), 16, 0, 0);
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
 #pragma unroll
       for (int u = 0; u < NTW; ++u) {
         const int m = t < my_tiles ? row0 + (wm * MTW + t) * 16 + r : p.M;
-        const int unit = nb * kTileBlocksN + wn * NTW + u;
+        const int unit = nb * NB + wn * NTW + u;
         const floatx4 a = acc[t][u];
         floatx4 partner = a;
         if (kPaired) {                                           // tile rows 8-15 (the lanes 32 further on) hold the partners of rows 0-7
@@ -594,11 +594,22 @@ __global__ __launch_bounds__(kStreamThreads) void tile_linear_kernel(const Strea
   }
 }
 
-template <int EPI, int MT, int R>
+static int num_compute_units() {
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+template <int EPI, int MT, int R, int NB>
 static int launch_tile(const StreamLinearParams& p, dim3 grid, hipStream_t stream) {
-  constexpr size_t lds = (size_t)R * (kTileBlocksN * kTileStageSteps + MT * kTileStageSteps) * 1024;
+  constexpr size_t lds = (size_t)R * (NB * kTileStageSteps + MT * kTileStageSteps) * 1024;
   static_assert(lds <= 160 * 1024, "LDS of one compute unit");
-  auto kernel = tile_linear_kernel<EPI, MT, R>;
+  auto kernel = tile_linear_kernel<EPI, MT, R, NB>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -634,11 +645,21 @@ PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, v
   if ((long)p.stages_per_split * (splits - 1) >= p.num_stages) return -2;
   const int m_blocks = pllm_tile_linear_row_blocks(M);
   const int rows = (M + m_blocks - 1) / m_blocks, mt = (rows + 15) / 16;        // tiles of 16 rows per workgroup: 1 to 10
-  const int n_blocks = ((rows_of_w + 15) / 16 + kTileBlocksN - 1) / kTileBlocksN;
+  // Tiles of 128 weight rows, or of 64 where those would leave half of the compute units without a workgroup (products in
+  // one range of K over a matrix of few rows, one block of input rows: 11264 x 2048 at 128 rows 19.0 against 25.7 us; with
+  // two blocks of rows the wide tiles win, 26.1 against 37.3 us at 264 rows).
+  const int n_blocks8 = ((rows_of_w + 15) / 16 + kTileBlocksN - 1) / kTileBlocksN;
+  const bool narrow = epi != SL_PARTIAL && (long)n_blocks8 * m_blocks * 2 <= num_compute_units();
+  const int nb_per = narrow ? kTileBlocksN / 2 : kTileBlocksN;
+  const int n_blocks = ((rows_of_w + 15) / 16 + nb_per - 1) / nb_per;
   if (m_blocks > 65535 || splits > 65535) return -2;
   const dim3 grid(n_blocks, m_blocks, splits);
   // (the kernel's row offset of a block along y is MT * 16: blocks are filled to whole tiles, the last one may be short)
-#define PLLM_TL(EPI_, MT_) return launch_tile<EPI_, MT_, (MT_ > 8 ? 3 : 4)>(p, grid, stream)
+#define PLLM_TL(EPI_, MT_)                                                                       \
+  do {                                                                                           \
+    if (narrow) return launch_tile<EPI_, MT_, 4, kTileBlocksN / 2>(p, grid, stream);             \
+    return launch_tile<EPI_, MT_, (MT_ > 8 ? 3 : 4), kTileBlocksN>(p, grid, stream);             \
+  } while (0)
 #define PLLM_TL_SHAPES(EPI_)                                                  \
   do {                                                                        \
     switch (mt) {                                                             \

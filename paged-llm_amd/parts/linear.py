@@ -176,6 +176,7 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
 
 TILE_GATED_ROWS = (161, 320)                    # rows for which the gated product takes the tiled kernel
 TILE_GATED_FROM_WHEN_FILLING = 24               # ... and from so few rows on when one block of rows already fills the GPU
+TILE_GATED_FROM_WHEN_NARROW = 32                # ... or when the kernel takes tiles of 64 weight rows for it (one block of rows)
 
 
 def _tiles_gated(x, weight, rows: int) -> bool:
@@ -185,11 +186,20 @@ def _tiles_gated(x, weight, rows: int) -> bool:
     one block of rows as well, from a few rows on: there every workgroup draws its own weights and the step's few rows,
     where the streaming kernel's workgroups of 32 to 64 weight rows draw the rows four times as often (28672 x 4096 at
     32 / 64 / 128 rows: 46 / 46 / 52 us against 50 / 57 us streaming and 53 / 53 / 59 us in the library with the activation
-    kernel; 24576 x 2048 at 64 rows 27 against 33 and 30; a matrix of 16384 x 3072, 128 tiles, stays where it was)."""
+    kernel; 24576 x 2048 at 64 rows 27 against 33 and 30).  A matrix whose tiles of 128 fill at most half of the compute
+    units is cut into tiles of 64 weight rows by the kernel when there is one block of rows, twice the workgroups (11264 x
+    2048 at 64 / 96 / 128 / 160 rows: 14.0 / 16.1 / 19.0 / 21.7 us against 18.8 / 20.3 / 21.8 / 27.6 in the library with the
+    activation kernel and 14.8 streaming at 64; 16384 x 2048 at 32 / 64 rows: 15.7 / 16.8 against 19.0 / 21.0 streaming)."""
     if not (isinstance(weight, Weight) and weight.tiled is not None and weight.pairing == "gated" and x.dtype == torch.bfloat16):
         return False
-    filling = weight.shape[0] // 128 >= 3 * ops._num_compute_units(weight.plain.device) // 4
-    return (TILE_GATED_FROM_WHEN_FILLING if filling else TILE_GATED_ROWS[0]) <= rows <= TILE_GATED_ROWS[1]
+    tiles, cus = weight.shape[0] // 128, ops._num_compute_units(weight.plain.device)
+    if 4 * tiles >= 3 * cus:
+        first = TILE_GATED_FROM_WHEN_FILLING
+    elif 2 * tiles <= cus:
+        first = TILE_GATED_FROM_WHEN_NARROW
+    else:
+        first = TILE_GATED_ROWS[0]
+    return first <= rows <= TILE_GATED_ROWS[1]
 
 
 def gated_linear(x, w_gate_up, activation: str = "silu") -> torch.Tensor:

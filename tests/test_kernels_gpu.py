@@ -1116,16 +1116,19 @@ def test_tile_linear_plain_float_and_partial(m, n, k):
 
 
 @pytest.mark.parametrize("m", [17, 24, 49, 100, 130, 264])
-def test_tile_linear_gated_and_rotary(m):
+@pytest.mark.parametrize("wide", [False, True])
+def test_tile_linear_gated_and_rotary(m, wide):
+    """``wide``: matrices of so many rows that the kernel keeps its tiles of 128 weight rows (smaller ones, whose tiles of
+    128 would leave half of the compute units idle, are cut into tiles of 64)."""
     from paged_llm_amd.parts.registry import BuildEnv
     from paged_llm_amd.parts.rope import RotaryEncoding
     o = ops()
-    inter, k = 250, 96
+    inter, k = (16650, 64) if wide else (250, 96)
     x = rnd(m, k, seed=72, dtype=torch.bfloat16)
     w = rnd(2 * inter, k, seed=73, dtype=torch.bfloat16, scale=k ** -0.5)
     want = torch.nn.functional.silu(x.double() @ w[:inter].double().T) * (x.double() @ w[inter:].double().T)
     assert rel_err(o.tile_linear(x.cuda(), o.tile_weight(w.cuda(), "gated"), o.SL_GATED), want) <= 1e-2
-    heads, kv_heads, d, bs, pages, k_in = 5, 1, 48, 16, 24, 256
+    heads, kv_heads, d, bs, pages, k_in = (340, 3, 48, 16, 24, 64) if wide else (5, 1, 48, 16, 24, 256)
     rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, torch.bfloat16, torch.device("cuda"), 512, {}))
     rope.prepare(512)
     x = rnd(m, k_in, seed=74, dtype=torch.bfloat16)
