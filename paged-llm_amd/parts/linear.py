@@ -53,6 +53,7 @@ TILE_MAX_ROWS = 640                             # rows up to which the tiled ker
 # ... and from so few rows on for matrices of so many elements that fill the GPU in so many ranges of K at most
 TILE_PARTIAL_FROM_ROWS, TILE_PARTIAL_MIN_ELEMENTS, TILE_PARTIAL_MOST_RANGES = 65, 1 << 24, 12
 STREAM_GATED_MAX_ROWS = 64                      # the gated product: beyond, its rows' traffic costs more than the library's kernel
+                                                # (asked only where the tiled kernel does not take the product: _tiles_gated)
 STREAM_LONG_K, STREAM_LONG_K_MAX_ROWS = 8192, 64 # from this K on a product in one range takes the streaming kernel up to so many rows
 
 
