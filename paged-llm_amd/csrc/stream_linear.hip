@@ -618,8 +618,41 @@ static int launch_tile(const StreamLinearParams& p, dim3 grid, hipStream_t strea
   return (int)hipGetLastError();
 }
 
-// Blocks of input rows of the tiled kernel: of at most 160 rows (10 tiles of 16), evenly filled.
+// Blocks of input rows of the tiled kernel when the product is cut into ranges of K: of at most 160 rows (10 tiles of 16),
+// evenly filled.
 PLLM_API int pllm_tile_linear_row_blocks(int M) { return (M + 159) / 160; }
+
+// Tiles of 16 input rows per workgroup that the kernel is compiled for, for a block of `rows` input rows.
+static int tile_rows_compiled(int rows) {
+  const int mt = (rows + 15) / 16;
+  return mt <= 2 ? 2 : mt <= 4 ? 4 : mt <= 6 ? 6 : mt <= 8 ? 8 : mt;       // (9 and 10 as they are)
+}
+
+// Shape of the tiles of a product in one range of K: blocks of input rows (evenly filled, of 32 to 160 rows) x tiles of
+// 128 or 64 weight rows.  A workgroup has about 100 KB under way whatever its tile, so what counts first is how many
+// workgroups run at once: the shape with the most workgroups that still fit the compute units in one round (q/k/v of
+// 2560 x 2048 at 264 rows: 5 x 40 tiles of 64 x 64, 11.8 us, against 14.7 us as 3 x 40 and 16.9 us in the library with the
+// rotary kernel behind it; 11264 x 2048 with the gated epilogue at 128 rows: 176 tiles of 128 x 64, 19.0 us, against 25.7
+// as 88 tiles of 128 x 128), among equals the one that draws the fewest bytes, then the one with the fewest blocks of
+// rows; the largest tiles when even those need more than one round.
+static void tile_shape(int M, int weight_blocks16, int cus, int* m_blocks_out, int* nb_out) {
+  long best_wgs = -1, best_bytes = 0;
+  *m_blocks_out = pllm_tile_linear_row_blocks(M);
+  *nb_out = kTileBlocksN;
+  const int compiled[] = {10, 9, 8, 6, 4, 2};                   // tiles of 16 rows per block, the largest first
+  for (int mt : compiled) {
+    const int mb = (M + mt * 16 - 1) / (mt * 16);
+    if (tile_rows_compiled(((M + mb - 1) / mb)) != mt) continue;  // (the same blocks, evenly filled, fit a smaller shape)
+    for (int nb = kTileBlocksN; nb >= kTileBlocksN / 2; nb /= 2) {
+      const long n_blocks = (weight_blocks16 + nb - 1) / nb, wgs = n_blocks * mb;
+      if (wgs > cus) continue;
+      const long bytes = n_blocks * M + (long)mb * weight_blocks16 * 16;        // rows drawn, of K values each
+      if (wgs > best_wgs || (wgs == best_wgs && bytes < best_bytes)) {
+        best_wgs = wgs; best_bytes = bytes; *m_blocks_out = mb; *nb_out = nb;
+      }
+    }
+  }
+}
 
 // The tiled weights hold a multiple of 8 blocks (of 24, in fact).  splits > 1 with epi SL_PARTIAL only.
 PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, void* out, int ldo, int M, int N, int K,
@@ -643,14 +676,13 @@ PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, v
   p.num_stages = (p.ksteps + kTileStageSteps - 1) / kTileStageSteps;
   p.stages_per_split = (p.num_stages + splits - 1) / splits;
   if ((long)p.stages_per_split * (splits - 1) >= p.num_stages) return -2;
-  const int m_blocks = pllm_tile_linear_row_blocks(M);
-  const int rows = (M + m_blocks - 1) / m_blocks, mt = (rows + 15) / 16;        // tiles of 16 rows per workgroup: 1 to 10
-  // Tiles of 128 weight rows, or of 64 where those would leave half of the compute units without a workgroup (products in
-  // one range of K over a matrix of few rows, one block of input rows: 11264 x 2048 at 128 rows 19.0 against 25.7 us; with
-  // two blocks of rows the wide tiles win, 26.1 against 37.3 us at 264 rows).
-  const int n_blocks8 = ((rows_of_w + 15) / 16 + kTileBlocksN - 1) / kTileBlocksN;
-  const bool narrow = epi != SL_PARTIAL && (long)n_blocks8 * m_blocks * 2 <= num_compute_units();
-  const int nb_per = narrow ? kTileBlocksN / 2 : kTileBlocksN;
+  // Cut into ranges of K (the caller's plan, which fills the GPU with them): blocks of up to 160 rows x 128 weight rows.
+  // In one range: the shape that gives the most workgroups in one round.
+  int m_blocks = pllm_tile_linear_row_blocks(M), nb_per = kTileBlocksN;
+  if (epi != SL_PARTIAL) tile_shape(M, (rows_of_w + 15) / 16, num_compute_units(), &m_blocks, &nb_per);
+  const bool narrow = nb_per != kTileBlocksN;
+  const int rows = (M + m_blocks - 1) / m_blocks, mt = tile_rows_compiled(rows);     // tiles of 16 rows per workgroup: 2 to 10
+  m_blocks = (M + mt * 16 - 1) / (mt * 16);                                     // (blocks are filled to whole tiles, the last one may be short)
   const int n_blocks = ((rows_of_w + 15) / 16 + nb_per - 1) / nb_per;
   if (m_blocks > 65535 || splits > 65535) return -2;
   const dim3 grid(n_blocks, m_blocks, splits);

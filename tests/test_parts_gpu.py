@@ -196,6 +196,36 @@ def test_attention_part_whole_in_portions_and_token_by_token(dtype, tol, options
     assert rel(torch.cat(out_other), other_want) <= tol, "second sequence"
 
 
+@pytest.mark.parametrize("hidden,heads,kv_heads,head_dim", [(1024, 8, 2, 64), (2048, 24, 4, 128)])
+@pytest.mark.parametrize("num_rows", [40, 100, 128, 200, 300])
+def test_attention_part_at_the_row_counts_where_its_input_product_changes_kernels(hidden, heads, kv_heads, head_dim, num_rows):
+    """The q/k/v product with rotation and cache write goes to the fused, the streaming or the tiled kernel by sizes and
+    rows (a matrix of 2^23 elements and more takes the tiled kernel from 65 rows on, a smaller one beyond 128): a whole
+    prompt, then a portion with the rest behind it, against the plain block; the cache both ways must hold the same."""
+    env = env_for("bfloat16", hidden=hidden, max_positions=512)
+    params = {"num_heads": heads, "num_kv_heads": kv_heads, "head_dim": head_dim,
+              "position": {"kind": "rotary", "params": {"head_dim": head_dim, "theta": THETA, "scaling": None}}}
+    mixer = build("mixer", "paged_attention", params, env)
+    w = give_weights(mixer, 51, "bfloat16", std=hidden ** -0.5)
+    x = rows(num_rows, 52, "bfloat16", hidden=hidden)
+    cfg = {"num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": head_dim}
+    want = plain.attention_block(x.float(), torch.arange(num_rows), w, "", cfg, plain.inverse_frequencies(head_dim, THETA, None), None)
+    group = mixer.cache_spec().group_name()
+    pages = -(-num_rows // BLOCK)
+    table = [(11 * i + 3) % (pages + 2) for i in range(pages)]              # pages in no order (11 and pages + 2 share no factor here)
+    assert len(set(table)) == pages
+    whole_cache = layer_cache(mixer, "bfloat16", pages + 2)
+    got = mixer.forward(x.cuda(), step_context([(0, num_rows)], [table], group, "bfloat16"), whole_cache, None)
+    assert rel(got, want) <= 3e-2, "whole"
+    cut = num_rows - 30                                                       # the last 30 rows as a portion of their own
+    cache = layer_cache(mixer, "bfloat16", pages + 2)
+    first = mixer.forward(x[:cut].cuda(), step_context([(0, cut)], [table], group, "bfloat16"), cache, None)
+    rest = mixer.forward(x[cut:].cuda(), step_context([(cut, 30)], [table], group, "bfloat16"), cache, None)
+    assert rel(torch.cat([first, rest]), want) <= 3e-2, "two portions"
+    for name in ("k", "v"):                                                   # (rounded once from the same float sums, whichever kernel)
+        assert rel(cache[name], whole_cache[name].float().cpu()) <= 1e-2, name
+
+
 @pytest.mark.parametrize("dtype,tol", DTYPES)
 def test_attention_part_with_biased_projections(dtype, tol):
     """q/k/v projections with a bias (a parameter of the part; the reference's Llama has none): the layer gives up the
