@@ -681,6 +681,16 @@ def tile_linear_plan(M: int, N: int, K: int, compute_units: int) -> int:
     return _whole_ranges(stages, max(1, min(compute_units // workgroups, stages // 4, 16)))
 
 
+def tile_linear_shape(M: int, weight_rows: int, compute_units: int) -> tuple[int, int, int]:
+    """(rows per block of input rows, weight rows per tile, workgroups) that the tiled kernel takes for a product in one
+    range of K: the shape with the most workgroups in one round of the compute units (chosen in the library)."""
+    f = _fn("stream_linear.hip", "pllm_tile_linear_shape", signature=[c_int, c_int, c_int, c_void_p, c_void_p])
+    rows, tile = c_int(0), c_int(0)
+    wgs = f(int(M), int(weight_rows), int(compute_units), ctypes.byref(rows), ctypes.byref(tile))
+    _need(wgs > 0, f"tile_linear_shape({M}, {weight_rows}, {compute_units})")
+    return rows.value, tile.value, wgs
+
+
 def tile_linear(x: torch.Tensor, w: TiledWeight, epi: int = SL_BF16, splits: int | None = None, rope: dict | None = None,
                 activation: str = "silu") -> torch.Tensor:
     """As ``stream_linear``, for a few hundred rows: tiles of up to 160 rows x 128 weight rows per workgroup, both

@@ -654,6 +654,18 @@ static void tile_shape(int M, int weight_blocks16, int cus, int* m_blocks_out, i
   }
 }
 
+// What `tile_shape` chooses for M input rows and a matrix of `weight_rows` rows on `compute_units` compute units: rows per
+// block of input rows (a multiple of 16) and weight rows per tile (128 or 64); returns the number of workgroups.
+PLLM_API int pllm_tile_linear_shape(int M, int weight_rows, int compute_units, int* block_rows, int* tile_weight_rows) {
+  if (M <= 0 || weight_rows <= 0 || compute_units <= 0) return -2;
+  int m_blocks, nb;
+  tile_shape(M, (weight_rows + 15) / 16, compute_units, &m_blocks, &nb);
+  const int mt = tile_rows_compiled((M + m_blocks - 1) / m_blocks);
+  *block_rows = mt * 16;
+  *tile_weight_rows = nb * 16;
+  return ((M + mt * 16 - 1) / (mt * 16)) * (((weight_rows + 15) / 16 + nb - 1) / nb);
+}
+
 // The tiled weights hold a multiple of 8 blocks (of 24, in fact).  splits > 1 with epi SL_PARTIAL only.
 PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, void* out, int ldo, int M, int N, int K,
                               int weight_blocks, int splits, const int* positions, const float* cos_t,

@@ -1115,6 +1115,26 @@ def test_tile_linear_plain_float_and_partial(m, n, k):
     assert torch.equal(alone.cpu(), o.tile_linear(x.cuda(), tiled, o.SL_F32)[m // 2:m // 2 + 5].cpu())     # a row's sums do not depend on the others
 
 
+def test_tile_shapes_of_the_tiled_kernel():
+    """A product in one range of K takes the tile shape with the most workgroups in one round of the compute units; the
+    largest tiles when none fits; blocks of rows always cover the rows."""
+    shape = ops().tile_linear_shape
+    assert shape(264, 2560, 256) == (64, 64, 200)          # q/k/v of a 2048-wide model: 5 blocks of rows x 40 tiles
+    assert shape(264, 11264, 256) == (144, 128, 176)       # its gate/up product: two blocks x 88 tiles of 128
+    assert shape(128, 11264, 256) == (128, 64, 176)        # one block of rows: tiles of 64 weight rows
+    assert shape(64, 28672, 256) == (64, 128, 224)         # a large matrix fills the GPU with tiles of 128
+    assert shape(264, 28672, 256) == (144, 128, 448)       # nothing fits one round: the largest tiles
+    rng = np.random.default_rng(3)
+    for _ in range(500):
+        m, n, cus = int(rng.integers(1, 700)), int(rng.integers(1, 40000)), int(rng.choice([64, 104, 256, 304]))
+        rows, tile, wgs = shape(m, n, cus)
+        assert rows % 16 == 0 and 32 <= rows <= 160 and tile in (64, 128)
+        blocks, tiles = -(-m // rows), -(-n // tile)
+        assert wgs == blocks * tiles and (blocks - 1) * rows < m <= blocks * rows
+        if wgs > cus:                                      # then even the largest tiles do not fit one round
+            assert -(-m // 160) * -(-n // 128) > cus and tile == 128
+
+
 @pytest.mark.parametrize("m", [17, 24, 49, 100, 130, 264])
 @pytest.mark.parametrize("wide", [False, True])
 def test_tile_linear_gated_and_rotary(m, wide):
