@@ -175,11 +175,24 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
     return ops.gemm_generic(x, weight, out_dtype)
 
 
-TILE_ROTARY_ROWS = (129, 512)                   # rows for which the q/k/v product takes the tiled kernel with the rotary epilogue
+TILE_ROTARY_ROWS = (129, 1536)                  # rows for which the q/k/v product takes the tiled kernel with the rotary epilogue,
+                                                # as long as its tiles fit the compute units in one round
 TILE_ROTARY_FROM_WHEN_LARGE, TILE_ROTARY_LARGE_ELEMENTS = 65, 1 << 23   # ... and from so few rows on for matrices of so many elements
 TILE_GATED_ROWS = (161, 320)                    # rows for which the gated product takes the tiled kernel
 TILE_GATED_FROM_WHEN_FILLING = 24               # ... and from so few rows on when one block of rows already fills the GPU
 TILE_GATED_FROM_WHEN_NARROW = 32                # ... or when the kernel takes tiles of 64 weight rows for it (one block of rows)
+
+
+_one_round: dict = {}
+
+
+def _tiles_in_one_round(rows: int, weight) -> bool:
+    """Whether the tiled kernel's tiles for a product of ``rows`` rows in one range of K fit the compute units in one round."""
+    cus = ops._num_compute_units(weight.plain.device)
+    key = (rows, weight.shape[0], cus)
+    if key not in _one_round:
+        _one_round[key] = ops.tile_linear_shape(rows, weight.shape[0], cus)[2] <= cus
+    return _one_round[key]
 
 
 def _tiles_gated(x, weight, rows: int) -> bool:
@@ -248,10 +261,12 @@ def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_h
                     and _few_weight_rows(w_qkv) and (cos is None or cos.data_ptr() % 16 == 0))
         rows = x.num_rows if isinstance(x, PendingNorm) else x.shape[0]
         large = tiled_ok and w_qkv.shape[0] * w_qkv.shape[1] >= TILE_ROTARY_LARGE_ELEMENTS
-        if tiled_ok and (TILE_ROTARY_FROM_WHEN_LARGE if large else TILE_ROTARY_ROWS[0]) <= rows <= TILE_ROTARY_ROWS[1]:
+        if (tiled_ok and (TILE_ROTARY_FROM_WHEN_LARGE if large else TILE_ROTARY_ROWS[0]) <= rows <= TILE_ROTARY_ROWS[1]
+                and _tiles_in_one_round(rows, w_qkv)):
             # A few hundred rows: the tiled kernel in the shape that fills the GPU in one round, with the rotation and the
             # cache write in its epilogue (2560 x 2048 at 264 rows: 11.8 us against 16.9 in the library with the rotary kernel
-            # behind it; 6144 x 4096: 28 against 37; at 512 rows 14.9 against 19.0 and 42.5 against 43.5).  Larger matrices
+            # behind it; 6144 x 4096: 28 against 37; at 1024 rows 21.5 against 27.4, but 90.7 against 61.9 for 6144 x 4096,
+            # whose tiles need a second round there).  Larger matrices
             # from 65 rows on, ahead of the streaming kernel (6144 x 4096 at 96 / 128 rows: 20.6 / 22.1 us against 25.0 / 28.7;
             # 5120 x 3072: 14.3 / 17.1 against 17.7 / 20.2; 2560 x 2048: 10.0 either way).
             x = rows_of(x)
