@@ -1087,7 +1087,7 @@ static int launch_attention(const void* q, int q_stride, const void* k_pages, co
                             const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                             int num_kv_heads, int block_size, float scale, int window, int partition_size,
                             int num_partitions, float* partials, int waves, int column_blocks, const int* work_list, int num_work,
-                            [[maybe_unused]] ScoreTerms terms, hipStream_t stream) {
+                            int single_prompt, [[maybe_unused]] ScoreTerms terms, hipStream_t stream) {
   if (total_q <= 0 || num_seqs <= 0) return 0;
   if (num_kv_heads <= 0 || num_heads % num_kv_heads) return -2;
   const int G = num_heads / num_kv_heads;
@@ -1122,13 +1122,17 @@ static int launch_attention(const void* q, int q_stride, const void* k_pages, co
     // single sequence in two (its tiles, handed out longest first, pair up a long one and a short one per compute
     // unit: 2048 tokens 39.9 against 42.7 us; but two prompts of 1024 tokens 26.1 against 23.9 us, four of 512 19.4
     // against 16.0, sixteen of 256 31.5 against 19.7, and one of 2560 62.0 against 52.4: there two workgroups of the
-    // four-wavefront kind per compute unit, each hiding the other's start and end, are faster).
+    // four-wavefront kind per compute unit, each hiding the other's start and end, are faster).  `single_prompt`: the
+    // caller says that all queries but a few are one sequence's (a step replayed from a graph holds a padding sequence
+    // beside its portion, and its list of tiles has spare entries).
     constexpr bool two_fits = D <= 128 && prefill_lds_bytes(2) <= 160 * 1024;
     // (workgroups that find work: with a list exactly its entries; else a sequence has as many tiles as its own queries
     // need, one more than its share at most)
-    const long busy = (work_list ? (long)num_work : ((long)total_q * G + kCols - 1) / kCols + (num_seqs - 1)) * num_kv_heads * num_partitions;
+    const bool solo = num_seqs == 1 || single_prompt;
+    const long tiles_of_queries = ((long)total_q * G + kCols - 1) / kCols;
+    const long busy = (single_prompt ? tiles_of_queries : work_list ? (long)num_work : tiles_of_queries + (num_seqs - 1)) * num_kv_heads * num_partitions;
     const long cus = num_compute_units();
-    const bool two = two_fits && (D > 96 || busy <= cus || (num_seqs == 1 && busy <= 2 * cus));
+    const bool two = two_fits && (D > 96 || busy <= cus || (solo && busy <= 2 * cus));
     const size_t lds = prefill_lds_bytes(two ? 2 : 1);
     if ((long)lds > pllm_max_lds()) return -2;
     auto kern = paged_attention_prefill_kernel<2, 1>;
@@ -1192,10 +1196,11 @@ PLLM_API int pllm_paged_attention_mfma(const void* q, int q_stride, const void* 
                                        hipStream_t stream) {
   return launch_attention(q, q_stride, k_pages, v_pages, out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_seqs,
                           total_q, max_q_len, num_heads, num_kv_heads, block_size, scale, window, partition_size, num_partitions,
-                          partials, waves, column_blocks, work_list, num_work, ScoreTerms{0.f, nullptr, nullptr}, stream);
+                          partials, waves, column_blocks, work_list, num_work, 0, ScoreTerms{0.f, nullptr, nullptr}, stream);
 }
 
-// The same with further terms of the score: score_cap > 0 caps the scaled products (c tanh(x / c)), slopes [heads]
+// The same with a hint for the prompt kernel's form (single_prompt: all queries but a few belong to one sequence) and
+// with further terms of the score: score_cap > 0 caps the scaled products (c tanh(x / c)), slopes [heads]
 // adds slope * (key position - query position), sinks [heads] gives every head a logit that takes part in the
 // softmax's sum only (null: none).  A library compiled without -DSCORE_TERMS=1 refuses any of them.
 PLLM_API int pllm_attention_mfma_score_terms() { return kTerms ? 1 : 0; }
@@ -1205,12 +1210,13 @@ PLLM_API int pllm_paged_attention_mfma_terms(const void* q, int q_stride, const 
                                              const int* seq_lens_k, int num_seqs, int total_q, int max_q_len, int num_heads,
                                              int num_kv_heads, int block_size, float scale, int window, int partition_size,
                                              int num_partitions, float* partials, int waves, int column_blocks, const int* work_list,
-                                             int num_work, float score_cap, const float* slopes, const float* sinks, hipStream_t stream) {
+                                             int num_work, int single_prompt, float score_cap, const float* slopes, const float* sinks,
+                                             hipStream_t stream) {
   const ScoreTerms given{score_cap, slopes, sinks};
   if (!(score_cap >= 0.f) || (given.any() && !kTerms)) return -2;
   return launch_attention(q, q_stride, k_pages, v_pages, out, out_stride, block_tables, bt_stride, cu_seqlens_q, seq_lens_k, num_seqs,
                           total_q, max_q_len, num_heads, num_kv_heads, block_size, scale, window, partition_size, num_partitions,
-                          partials, waves, column_blocks, work_list, num_work, given, stream);
+                          partials, waves, column_blocks, work_list, num_work, single_prompt, given, stream);
 }
 
 // What the library that holds the no-allocation entry point needs from this one (see attention_noalloc.h): the head

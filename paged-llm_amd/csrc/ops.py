@@ -752,7 +752,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = 
 
 _ATTN_SIG = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
              c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]
-_ATTN_TERMS_SIG = _ATTN_SIG[:-1] + [c_float, c_void_p, c_void_p, c_void_p]
+_ATTN_TERMS_SIG = _ATTN_SIG[:-1] + [c_int, c_float, c_void_p, c_void_p, c_void_p]
 _attn_scratch: dict = {}
 _attn_scratch_retired: list = []      # outgrown buffers stay allocated: captured graphs still hold their addresses
 _attn_checked: set = set()
@@ -825,7 +825,7 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                          head_dim: int, scale: float, window: int, max_q_len: int, partition_size: int = 0,
                          num_partitions: int = 1, waves: int = 1, column_blocks: int = 0,
                          out: torch.Tensor | None = None, work_list: torch.Tensor | None = None,
-                         terms: ScoreTerms | None = None) -> torch.Tensor:
+                         terms: ScoreTerms | None = None, single_prompt: bool = False) -> torch.Tensor:
     """Causal attention over paged keys/values on the matrix cores (bfloat16).  ``max_q_len`` bounds
     the queries of any sequence of the batch; ``partition_size`` > 0 splits the keys of every
     work item into aligned partitions that a second kernel merges (best a multiple of 128 for prompt portions, whose
@@ -833,7 +833,8 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     of a work item between the wavefronts of one workgroup (few queries per sequence only).  ``work_list``
     (prompt portions): int32 [n, 2] pairs of (sequence, tile of 128 query columns), the order in which the
     kernel's workgroups take them (``prompt_work_list``).  ``terms``: further terms of the scores (``ScoreTerms``);
-    with any of them the kernels come from a library of their own, compiled with those terms in the score loop."""
+    with any of them the kernels come from a library of their own, compiled with those terms in the score loop.
+    ``single_prompt``: all queries but a few belong to one sequence (a hint for the prompt kernel's form)."""
     S, bs = _check_attention_args(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k, num_heads, num_kv_heads, head_dim)
     _need(mfma_attention_takes(q.dtype, num_heads, num_kv_heads, head_dim, bs),
           f"MFMA attention takes bfloat16, head sizes 16..256 in steps of 16, pages of >= 16 positions and groups of <= 64 "
@@ -875,9 +876,9 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
             block_tables.stride(0), _ptr(cu_seqlens_q), _ptr(seq_lens_k), S, T, int(max_q_len), num_heads, num_kv_heads, bs,
             c_float(scale), int(window or 0), int(partition_size), int(num_partitions), _ptr(ws), int(waves), int(column_blocks),
             _ptr(work_list), 0 if work_list is None else work_list.shape[0])
-    if with_terms:
+    if with_terms or single_prompt:
         f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma_terms", defines, _ATTN_TERMS_SIG)
-        _check(f(*args, *_terms_args(terms, num_heads, q.device), _stream()), "paged_attention_mfma")
+        _check(f(*args, int(bool(single_prompt)), *_terms_args(terms, num_heads, q.device), _stream()), "paged_attention_mfma")
     else:
         f = _fn("attention_mfma.hip", "pllm_paged_attention_mfma", defines, _ATTN_SIG)
         _check(f(*args, _stream()), "paged_attention_mfma")
@@ -1023,7 +1024,8 @@ def paged_attention(q, k_pages, v_pages, block_tables, cu_seqlens_q, seq_lens_k,
             prompt_q = max(layout.portion_tokens, FEW_QUERY_COLUMNS // group + 1)     # enough columns for the prompt kernel's form
             psize, pparts = prompt_partitions(work.shape[0], num_kv_heads, layout.portion_context, _num_compute_units(q.device))
             paged_attention_mfma(q, k_pages, v_pages, block_tables[few:], cu_seqlens_q[few:], seq_lens_k[few:], num_heads,
-                                 num_kv_heads, head_dim, scale, window, prompt_q, psize, pparts, 1, 2, out=out, work_list=work, terms=terms)
+                                 num_kv_heads, head_dim, scale, window, prompt_q, psize, pparts, 1, 2, out=out, work_list=work, terms=terms,
+                                 single_prompt=layout.num_portions == 2)      # (one portion and the padding sequence)
             return out
         q_lens, k_lens = ctx.q_lens, ctx.k_lens
         few = 0
