@@ -644,6 +644,9 @@ static void tile_shape(int M, int weight_blocks16, int cus, int* m_blocks_out, i
     const int mb = (M + mt * 16 - 1) / (mt * 16);
     if (tile_rows_compiled(((M + mb - 1) / mb)) != mt) continue;  // (the same blocks, evenly filled, fit a smaller shape)
     for (int nb = kTileBlocksN; nb >= kTileBlocksN / 2; nb /= 2) {
+      // (blocks of 144 and 160 rows only with tiles of 128 weight rows: twice the blocks of half the rows x tiles of 128
+      //  are as many workgroups and draw fewer bytes, so the other shape would never be chosen and is not compiled)
+      if (nb != kTileBlocksN && mt > 8) continue;
       const long n_blocks = (weight_blocks16 + nb - 1) / nb, wgs = n_blocks * mb;
       if (wgs > cus) continue;
       const long bytes = n_blocks * M + (long)mb * weight_blocks16 * 16;        // rows drawn, of K values each
@@ -701,7 +704,10 @@ PLLM_API int pllm_tile_linear(int epi, const void* x, int ldx, const void* wt, v
   // (the kernel's row offset of a block along y is MT * 16: blocks are filled to whole tiles, the last one may be short)
 #define PLLM_TL(EPI_, MT_)                                                                       \
   do {                                                                                           \
-    if (narrow) return launch_tile<EPI_, MT_, 4, kTileBlocksN / 2>(p, grid, stream);             \
+    if constexpr ((MT_) <= 8) {                                                                  \
+      if (narrow) return launch_tile<EPI_, MT_, 4, kTileBlocksN / 2>(p, grid, stream);           \
+    }                                                                                            \
+    if (narrow) return -3;                                                                       \
     return launch_tile<EPI_, MT_, (MT_ > 8 ? 3 : 4), kTileBlocksN>(p, grid, stream);             \
   } while (0)
 #define PLLM_TL_SHAPES(EPI_)                                                  \

@@ -1135,20 +1135,25 @@ def test_tile_shapes_of_the_tiled_kernel():
             assert -(-m // 160) * -(-n // 128) > cus and tile == 128
 
 
-@pytest.mark.parametrize("m", [17, 24, 49, 100, 130, 264])
-@pytest.mark.parametrize("wide", [False, True])
-def test_tile_linear_gated_and_rotary(m, wide):
-    """``wide``: matrices of so many rows that the kernel keeps its tiles of 128 weight rows (smaller ones, whose tiles of
-    128 would leave half of the compute units idle, are cut into tiles of 64)."""
+@pytest.mark.parametrize("m", [17, 24, 49, 64, 100, 130, 150, 264])
+@pytest.mark.parametrize("size", ["small", "middle", "large"])
+def test_tile_linear_gated_and_rotary(m, size):
+    """The kernel takes the tile shape that gives the most workgroups in one round: small matrices end up with blocks of 32
+    rows x tiles of 64 weight rows at every row count, matrices of a few thousand rows with tiles of 64 weight rows and
+    blocks that grow with the rows, and matrices whose tiles of 128 need more than one round keep the largest tiles."""
     from paged_llm_amd.parts.registry import BuildEnv
     from paged_llm_amd.parts.rope import RotaryEncoding
     o = ops()
-    inter, k = (16650, 64) if wide else (250, 96)
+    wide = size == "large"
+    inter, k = {"small": (250, 96), "middle": (5630, 64), "large": (16650, 64)}[size]
+    if size == "middle":
+        assert o.tile_linear_shape(m, 2 * inter, 256)[:2] == {17: (32, 64), 24: (32, 64), 49: (64, 64), 64: (64, 64), 100: (128, 64), 130: (96, 128),
+                                                               150: (96, 128), 264: (144, 128)}[m]
     x = rnd(m, k, seed=72, dtype=torch.bfloat16)
     w = rnd(2 * inter, k, seed=73, dtype=torch.bfloat16, scale=k ** -0.5)
     want = torch.nn.functional.silu(x.double() @ w[:inter].double().T) * (x.double() @ w[inter:].double().T)
     assert rel_err(o.tile_linear(x.cuda(), o.tile_weight(w.cuda(), "gated"), o.SL_GATED), want) <= 1e-2
-    heads, kv_heads, d, bs, pages, k_in = (340, 3, 48, 16, 24, 64) if wide else (5, 1, 48, 16, 24, 256)
+    heads, kv_heads, d, bs, pages, k_in = {"small": (5, 1, 48, 16, 24, 256), "middle": (100, 2, 48, 16, 24, 64), "large": (340, 3, 48, 16, 24, 64)}[size]
     rope = RotaryEncoding({"head_dim": d, "theta": 10000.0, "scaling": None}, BuildEnv(64, torch.bfloat16, torch.device("cuda"), 512, {}))
     rope.prepare(512)
     x = rnd(m, k_in, seed=74, dtype=torch.bfloat16)
