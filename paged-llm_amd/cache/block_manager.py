@@ -202,6 +202,12 @@ class CacheManager:
     def block_table(self, request, group: str) -> list[int]:
         return self._held[request].tables[group]
 
+    def step_fields(self, request) -> tuple:
+        """(block tables by group, state slot, table version) of ``request`` with one look-up, for whoever builds a
+        step's entries for hundreds of requests.  The tables are the manager's own lists: read them, do not keep them."""
+        h = self._held[request]
+        return h.tables, h.state_slot, h.version
+
     def table_version(self, request) -> int:
         """A number that changes whenever any block table of ``request`` does (a page appended, copied
         for a write, or given back by a window), and that no other state of any request shares: who
