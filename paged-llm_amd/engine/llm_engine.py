@@ -72,8 +72,25 @@ def _tokenizer_of(folder: str):
     return Tokenizer.from_file(path)
 
 
+_static_heap_frozen = False
+
+
+def _freeze_static_heap() -> None:
+    """What exists before the first engine of a process is built (the tensor library and everything else that was
+    imported: a million objects or so) lives as long as the process does.  Taken out of the garbage collector's
+    generations, it is no longer walked by every full collection; such a collection then costs what the engine's and the
+    live requests' objects cost (at 512 requests a pause of 50 ms every few dozen steps became one of 5 ms: 7.9 -> 6.6 ms a
+    step on average).  Once per process, and before the engine's own objects exist: an engine that is dropped later is
+    collected as ever."""
+    global _static_heap_frozen
+    if not _static_heap_frozen:
+        gc.collect()
+        gc.freeze()
+        _static_heap_frozen = True
+
+
 class LLMEngine:
-    freeze_static_heap = True          # False: the garbage collector keeps walking the objects that exist when an engine is built
+    freeze_static_heap = True          # False: the garbage collector keeps walking everything that was imported
     def __init__(self, model: str, config: EngineConfig | None = None, **overrides):
         """``model``: a folder with config.json and *.safetensors.  ``random_weights=SEED`` among
         the overrides fills the model of that folder's config.json with seeded random weights
@@ -81,6 +98,8 @@ class LLMEngine:
         seed_for_weights = overrides.pop("random_weights", None)
         self.config = cfg = config or EngineConfig(**overrides)
         self.device = require_gpu(cfg.device)
+        if self.freeze_static_heap:
+            _freeze_static_heap()
         if not os.path.isdir(model):
             raise FileNotFoundError(f"{model!r} is no folder (models are not downloaded)")
         self.tokenizer = _tokenizer_of(model)
@@ -113,13 +132,6 @@ class LLMEngine:
         self.run_ahead = True
         log.info("cache: %d pages of %d positions per group (%d positions, %.2f GiB)", pages, cfg.block_size,
                  pages * cfg.block_size, self.kv_cache.total_bytes() / 2**30)
-        # Everything that exists by now (the tensor library, the model, the kernels' tables: a million objects or so) will
-        # live as long as the process does.  Taken out of the garbage collector's generations, it is no longer walked by
-        # every full collection; such a collection then costs what the live requests' objects cost (at 512 requests a
-        # pause of 50 ms every few dozen steps became one of 5 ms: 7.9 -> 6.6 ms a step on average).
-        if self.freeze_static_heap:
-            gc.collect()
-            gc.freeze()
 
     # ------------------------------------------------------------------ requests
     def _token_ids(self, prompt) -> list:
