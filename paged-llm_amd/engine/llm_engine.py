@@ -170,11 +170,13 @@ class LLMEngine:
 
     # ------------------------------------------------------------------ one step
     def _entry(self, grant) -> StepEntry:
-        request, cm = grant.request, self.cache_manager
+        request = grant.request
         first = request.computed
-        return StepEntry(request.id, request.tokens[first:first + grant.count], first,
-                         {g: cm.block_table(request.id, g) for g in self.groups}, cm.state_slot(request.id),
-                         [grant.count - 1] if grant.samples else [], cm.table_version(request.id))
+        tables, slot, version = self.cache_manager.step_fields(request.id)
+        if len(tables) != len(self.groups):                      # (groups in the order the step function knows them)
+            tables = {g: tables[g] for g in self.groups}
+        return StepEntry(request.id, request.tokens[first:first + grant.count], first, tables, slot,
+                         [grant.count - 1] if grant.samples else [], version)
 
     def _sample(self, logits, grants: list):
         """Queues the sampling of the grants whose last row was asked for; (requests in the order of the rows, pending

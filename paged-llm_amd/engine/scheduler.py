@@ -186,14 +186,14 @@ class Scheduler:
             return None
         if not all(grant.samples for grant in plan.grants):
             return None
-        at_limit = lambda r: r.num_generated + 1 >= r.new_token_limit or len(r.tokens) + 1 >= self.max_positions
-        staying = sum(1 for grant in plan.grants if not at_limit(grant.request))
-        if self.queue and staying < self.max_active:
+        most = self.max_positions
+        ends = [r.num_generated + 1 >= r.new_token_limit or len(r.tokens) + 1 >= most for r in (grant.request for grant in plan.grants)]
+        if self.queue and len(ends) - sum(ends) < self.max_active:
             return None                       # a place comes free (or is free): the next plan may admit somebody
         ahead = StepPlan()
-        for grant in plan.grants:
+        for grant, at_limit in zip(plan.grants, ends):
             request = grant.request
-            if at_limit(request):
+            if at_limit:
                 continue                      # its last token comes from ``plan``
             if not self.cache.allocate(request.id, request.computed + grant.count, 1):
                 return None                   # (pages taken for the others so far are the ones their next step takes anyway)
