@@ -665,6 +665,16 @@ def main() -> int:
                         points["prefill_8192_frac"] = round(prefill_flops(cfg, 8192, 1) / t / PEAK_FLOPS[short], 4)
                     del long_engine
                     torch.cuda.empty_cache()
+            # many requests at once (the attention over the cache is most of such a step, and the host's part of it grows)
+            if numbers["kv_bytes_per_token"] * 512 * (args.context + 128) < 48e9:
+                with tempfile.TemporaryDirectory() as wide_folder:
+                    wide_engine = make_engine(cfg, wide_folder, args.dtype, 512, args.context)
+                    s, mean_ctx = time_decode(wide_engine, 512, args.context, 24, 6, seed=70)
+                    nbytes_step = numbers["weight_bytes"] + 512 * mean_ctx * numbers["kv_bytes_per_token"]
+                    points["decode_b512"] = round(512 / s, 1)
+                    points["decode_b512_frac"] = round(nbytes_step / s / 1e9 / PEAK_HBM_GBS, 4)
+                    del wide_engine
+                    torch.cuda.empty_cache()
             # the reference's end-to-end workload at 8 and 64 requests at a time (64 requests, 256 in / 128 out): output tokens/s
             e2e = run_e2e(cfg, args.dtype, [c for c in E2E_CASES if c["name"] in ("256in_128out_b8", "256in_128out_b64")])
             record["e2e"] = {name: row["output_tok_per_s"] for name, row in e2e.items()}
