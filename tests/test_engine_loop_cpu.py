@@ -201,3 +201,26 @@ def test_a_newcomer_is_admitted_at_once_although_steps_run_ahead():
     assert late not in [o.seq_id for o in first] and not engine.step_in_flight
     second = engine.step()                                       # the next one is planned afresh and takes it in
     assert late in [o.seq_id for o in second] and len(second) == 4
+
+
+def test_the_static_heap_is_frozen_once():
+    """What was imported before the first engine is taken out of the garbage collector's generations once per process;
+    objects made afterwards (an engine's own, the requests') are collected as ever."""
+    import gc
+    from paged_llm_amd.engine import llm_engine
+    llm_engine._freeze_static_heap()
+    frozen = gc.get_freeze_count()
+    assert llm_engine._static_heap_frozen and frozen > 0
+
+    class Node:
+        pass
+    a, b = Node(), Node()
+    a.other, b.other = b, a                                       # a cycle made after the freeze
+    import weakref
+    seen = weakref.ref(a)
+    del a, b
+    llm_engine._freeze_static_heap()                              # (a second call freezes nothing more)
+    assert gc.get_freeze_count() == frozen
+    gc.collect()
+    assert seen() is None
+
