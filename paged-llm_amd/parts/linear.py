@@ -175,7 +175,7 @@ def linear(x, weight, out_dtype: torch.dtype | None = None, partial_ok: bool = F
     return ops.gemm_generic(x, weight, out_dtype)
 
 
-TILE_ROTARY_ROWS = (129, 1536)                  # rows for which the q/k/v product takes the tiled kernel with the rotary epilogue,
+TILE_ROTARY_ROWS = (97, 1536)                   # rows for which the q/k/v product takes the tiled kernel with the rotary epilogue,
                                                 # as long as its tiles fit the compute units in one round
 TILE_ROTARY_FROM_WHEN_LARGE, TILE_ROTARY_LARGE_ELEMENTS = 65, 1 << 23   # ... and from so few rows on for matrices of so many elements
 TILE_GATED_ROWS = (161, 320)                    # rows for which the gated product takes the tiled kernel
@@ -268,7 +268,8 @@ def qkv_rotary_cache(x, w_qkv, positions: torch.Tensor, position_encoding, num_h
             # behind it; 6144 x 4096: 28 against 37; at 1024 rows 21.5 against 27.4, but 90.7 against 61.9 for 6144 x 4096,
             # whose tiles need a second round there).  Larger matrices
             # from 65 rows on, ahead of the streaming kernel (6144 x 4096 at 96 / 128 rows: 20.6 / 22.1 us against 25.0 / 28.7;
-            # 5120 x 3072: 14.3 / 17.1 against 17.7 / 20.2; 2560 x 2048: 10.0 either way).
+            # 5120 x 3072: 14.3 / 17.1 against 17.7 / 20.2); smaller ones from 97 rows (2560 x 2048 at 128 rows: 10.0 against 10.7
+            # on its own and 13.3 inside a step; decode at 128 requests 47.2 -> 48.5 k tok/s, a prompt of 128 tokens 1.77 -> 1.70 ms).
             x = rows_of(x)
             if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
                 x = x.contiguous()

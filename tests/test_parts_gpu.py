@@ -200,7 +200,7 @@ def test_attention_part_whole_in_portions_and_token_by_token(dtype, tol, options
 @pytest.mark.parametrize("num_rows", [40, 100, 128, 200, 300])
 def test_attention_part_at_the_row_counts_where_its_input_product_changes_kernels(hidden, heads, kv_heads, head_dim, num_rows):
     """The q/k/v product with rotation and cache write goes to the fused, the streaming or the tiled kernel by sizes and
-    rows (a matrix of 2^23 elements and more takes the tiled kernel from 65 rows on, a smaller one beyond 128): a whole
+    rows (a matrix of 2^23 elements and more takes the tiled kernel from 65 rows on, a smaller one from 97): a whole
     prompt, then a portion with the rest behind it, against the plain block; the cache both ways must hold the same."""
     env = env_for("bfloat16", hidden=hidden, max_positions=512)
     params = {"num_heads": heads, "num_kv_heads": kv_heads, "head_dim": head_dim,
