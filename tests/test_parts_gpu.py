@@ -414,16 +414,16 @@ def test_feed_forward_part_whose_gated_matrix_fills_the_gpu(num_rows):
 
 
 def test_which_gated_products_take_the_tiled_kernel():
-    """By sizes and rows only: matrices whose tiles of 128 weight rows fill at most half of the compute units from 32 rows on
+    """By sizes and rows only: matrices whose tiles of 128 weight rows fill at most half of the compute units from 17 rows on
     (the kernel cuts them into tiles of 64 then), those that fill three quarters from 24 on, those in between only with two
     blocks of input rows; nobody beyond 320 rows."""
     from paged_llm_amd.csrc import ops
     from paged_llm_amd.parts import linear as L
     cus = ops._num_compute_units(torch.device("cuda:0"))
     x = torch.zeros(1, 64, dtype=torch.bfloat16, device="cuda")
-    for tiles, first in ((3, 32), (cus // 2, 32), (cus // 2 + 8, 161), (3 * cus // 4, 24)):
+    for tiles, first in ((3, 17), (cus // 2, 17), (cus // 2 + 8, 161), (3 * cus // 4, 24)):
         w = L.Weight(torch.zeros(128 * tiles, 64, dtype=torch.bfloat16, device="cuda"), "gated")
-        for rows in (16, 23, 24, 31, 32, 100, 160, 161, 320, 321):
+        for rows in (16, 17, 23, 24, 31, 32, 100, 160, 161, 320, 321):
             assert L._tiles_gated(x, w, rows) == (first <= rows <= 320), (tiles, rows)
     assert not L._tiles_gated(x, L.Weight(torch.zeros(256, 64, dtype=torch.bfloat16, device="cuda")), 64)      # (not the gated pairing)
 
