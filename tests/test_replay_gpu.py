@@ -12,12 +12,18 @@ import torch
 
 from tests import helpers
 from tests.helpers import TraceBuilder
+from tests.plain import llama_plain
 from tests.tiny_configs import TINY_A, TINY_B, TINY_C
 
 pytestmark = pytest.mark.gpu
 
 # Largest difference allowed, relative to the largest logit of the request.
 TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+# Beside that bound, in bfloat16 the median error of a replay that compares this many rows or more is held against the
+# error that the plain implementation shows when it rounds wherever the reference's model hands a tensor on
+# (``forward(stored=bfloat16)``): the engine rounds in fewer places, so its median must stay below (measured
+# 0.0101 / 0.0104 / 0.0075 against 0.0107 / 0.0112 / 0.0080 for the three configurations).
+YARDSTICK_FROM_ROWS = 64
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 LENGTHS = {"A": [5, 17, 33, 40, 150], "B": [1, 9, 60, 100, 127], "C": [3, 64, 65, 200]}
 
@@ -41,16 +47,32 @@ def requests_for(name):
     return {f"r{i}": helpers.random_tokens(n, vocab, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
 
 
+_plain = {}
+
+
+def plain_rows(folder: str, tokens: list[int], stored=None) -> np.ndarray:
+    key = folder, tuple(tokens), stored
+    if key not in _plain:
+        if stored is None:
+            _plain[key] = helpers.plain_logits(folder, tokens)
+        else:
+            cfg, weights = llama_plain.read_config(folder), llama_plain.load_weights(folder)
+            _plain[key] = llama_plain.forward(cfg, weights, tokens, stored=stored).float().numpy()
+    return _plain[key]
+
+
 def check(got: dict, folder: str, reqs: dict, dtype: str):
     assert got, "nothing was compared"
-    by_req = {}
+    errs = {}
     for (rid, pos), row in got.items():
-        by_req.setdefault(rid, {})[pos] = row
-    for rid, rows in by_req.items():
-        want = helpers.plain_logits(folder, reqs[rid])
-        for pos, row in rows.items():
-            err = helpers.worst(row, want[pos])
-            assert err <= TOL[dtype], f"request {rid} position {pos}: relative error {err:.3g} > {TOL[dtype]}"
+        err = errs[rid, pos] = helpers.worst(row, plain_rows(folder, reqs[rid])[pos])
+        assert err <= TOL[dtype], f"request {rid} position {pos}: relative error {err:.3g} > {TOL[dtype]}"
+    if dtype == "bfloat16" and len(errs) >= YARDSTICK_FROM_ROWS:
+        median = sorted(errs.values())[len(errs) // 2]
+        ref = sorted(helpers.worst(plain_rows(folder, reqs[rid], torch.bfloat16)[pos], plain_rows(folder, reqs[rid])[pos])
+                     for rid, pos in errs)[len(errs) // 2]
+        assert median <= ref, (f"median relative error of {len(errs)} rows {median:.3g} against {ref:.3g} of the plain "
+                               "implementation rounding where the reference's model does")
 
 
 def rounded(n, m=64):
