@@ -93,6 +93,9 @@ class ModelRunner:
         self.states = {pos: torch.zeros((num_state_slots + 1, *ss.shape), dtype=ss.dtype, device=self.device)
                        for pos, ss in model.state_specs().items()}
         self.spare_state_slot = num_state_slots if self.states else -1
+        # Block tables already checked and converted for a step, by (request, cache group): a table keeps its version
+        # as long as nothing in it changes, so a request that decodes beside prompt portions is not converted again.
+        self._checked_rows: dict = {}
 
     # ------------------------------------------------------------------ batch -> device tensors
     def _stage(self, entries: list, fixed_blocks: int | None = None):
@@ -113,7 +116,7 @@ class ModelRunner:
         vocab, max_pos = self.model.spec.vocab_size, self.model.max_positions
         seen = set()
         q_lens, k_lens, starts = [], [], []
-        ids_parts, pos_parts = [], []
+        single_ids, ids_parts, pos_parts = [], [], []                 # single tokens as plain numbers: they come first
         wanted_of: dict = {}                                          # request id -> batch rows of its wanted tokens
         callers_order = [e.request_id for e in entries]
         entries = sorted(entries, key=lambda e: len(e.tokens))        # stable
@@ -125,8 +128,15 @@ class ModelRunner:
             if e.request_id in seen:
                 raise StepError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
-            toks = np.asarray(e.tokens, dtype=np.int64)
-            if toks.min() < 0 or toks.max() >= vocab:
+            if n == 1:
+                lowest = highest = int(e.tokens[0])
+                single_ids.append(lowest)
+            else:
+                toks = np.asarray(e.tokens, dtype=np.int64)
+                lowest, highest = toks.min(), toks.max()
+                ids_parts.append(toks)
+                pos_parts.append(np.arange(e.start, e.start + n, dtype=np.int64))
+            if lowest < 0 or highest >= vocab:
                 raise StepError(f"request {e.request_id!r}: token id outside [0, {vocab})")
             if e.start < 0 or e.start + n > max_pos:
                 raise StepError(f"request {e.request_id!r}: positions {e.start}..{e.start + n - 1} exceed the "
@@ -135,14 +145,13 @@ class ModelRunner:
                 if not 0 <= w < n:
                     raise StepError(f"request {e.request_id!r}: wanted row {w} outside its {n} tokens")
             wanted_of[e.request_id] = [offset + w for w in e.want]
-            ids_parts.append(toks)
-            pos_parts.append(np.arange(e.start, e.start + n, dtype=np.int64))
             q_lens.append(n)
             k_lens.append(e.start + n)
             starts.append(e.start)
             offset += n
-        T, S = offset, len(entries)
-        positions = np.concatenate(pos_parts)
+        T, S, singles = offset, len(entries), len(single_ids)
+        ids = np.concatenate([np.asarray(single_ids, dtype=np.int64)] + ids_parts)
+        positions = np.concatenate([np.asarray(starts[:singles], dtype=np.int64)] + pos_parts)
         logits_idx = [row for rid in callers_order for row in wanted_of[rid]]
 
         group_arrays = {}
@@ -153,7 +162,7 @@ class ModelRunner:
                 assert fixed_blocks >= max_blocks
                 max_blocks = fixed_blocks
             tables = np.zeros((S, max_blocks), dtype=np.int32)
-            slots = []
+            single_slots, slots = [], []
             for s, e in enumerate(entries):
                 table = e.block_tables.get(name)
                 if table is None:
@@ -162,22 +171,34 @@ class ModelRunner:
                 if len(table) < need:
                     raise StepError(f"request {e.request_id!r}: {len(table)} pages in group {name!r}, "
                                     f"{k_lens[s]} positions need {need}")
-                row = np.asarray(table[:need], dtype=np.int64)
                 # Pages a query of this step can see: from the first key inside the window on.
                 first_key = max(0, e.start - cs.window + 1) if cs.window > 0 else 0
-                live = row[first_key // bs:]
-                if live.size and (live.min() < 0 or live.max() >= num_pages):
-                    raise StepError(f"request {e.request_id!r}: page id outside [0, {num_pages}) in group {name!r}")
-                tables[s, :need] = np.where(row == NO_PAGE, 0, row)
-                p = pos_parts[s]
-                slots.append(row[p // bs] * bs + (p % bs))
-            group_arrays[name] = (tables, np.concatenate(slots).astype(np.int32))
+                known = self._checked_rows.get((e.request_id, name)) if e.table_version is not None else None
+                if known is not None and known[0] == (e.table_version, need, first_key // bs):
+                    shown = known[1]                                 # this table was checked and converted in an earlier step
+                else:
+                    row = np.asarray(table[:need], dtype=np.int64)
+                    live = row[first_key // bs:]
+                    if live.size and (live.min() < 0 or live.max() >= num_pages):
+                        raise StepError(f"request {e.request_id!r}: page id outside [0, {num_pages}) in group {name!r}")
+                    shown = np.where(row == NO_PAGE, 0, row).astype(np.int32)
+                    if e.table_version is not None:
+                        if len(self._checked_rows) >= 4096:
+                            self._checked_rows.clear()
+                        self._checked_rows[e.request_id, name] = ((e.table_version, need, first_key // bs), shown)
+                tables[s, :need] = shown
+                if s < singles:
+                    single_slots.append(table[e.start // bs] * bs + e.start % bs)
+                else:
+                    p = pos_parts[s - singles]
+                    slots.append(np.asarray(table[:need], dtype=np.int64)[p // bs] * bs + (p % bs))
+            group_arrays[name] = (tables, np.concatenate([np.asarray(single_slots, dtype=np.int64)] + slots).astype(np.int32))
 
         slots_state = np.asarray([-1 if e.state_slot is None else e.state_slot for e in entries], dtype=np.int32)
         if self.states and (slots_state < 0).any():
             raise StepError("this model keeps per-request state: every entry needs a state slot")
 
-        pieces = [np.concatenate(ids_parts).astype(np.int32), positions.astype(np.int32),
+        pieces = [ids.astype(np.int32), positions.astype(np.int32),
                   np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32), np.asarray(k_lens, dtype=np.int32),
                   slots_state, np.asarray(starts, dtype=np.int32), np.asarray(logits_idx, dtype=np.int32)]
         table_shapes = {}

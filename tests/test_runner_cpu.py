@@ -124,6 +124,43 @@ def test_decode_steps_restaged_in_place_equal_fresh_staging(runtime):
         manager.free(live[row][0])
 
 
+def test_tables_remembered_by_version_equal_tables_read_again(runtime):
+    """Staging remembers a checked block table under its version: over steps in which requests grow, end and are
+    replaced, single tokens beside portions, the staged arrays equal those of entries that carry no version (which
+    are read and checked every time), most tables are taken from memory, and a bad page under a new version is refused."""
+    manager, runner = runtime
+    g = next(iter(manager.groups))
+    rng = np.random.default_rng(5)
+    live, serial, remembered = {}, 0, 0
+    for step in range(50):
+        for row in range(3):
+            if row not in live or live[row][1] >= 36 or rng.random() < 0.08:
+                if row in live:
+                    manager.free(live[row][0])
+                serial += 1
+                live[row] = [f"m{serial}", 0]
+        versioned, plain = [], []
+        for row in range(3):
+            rid, start = live[row]
+            n = 1 if start and rng.random() < 0.7 else int(rng.integers(2, 6))
+            assert manager.allocate(rid, start, n)
+            toks = [int(t) for t in rng.integers(0, 256, n)]
+            known = runner._checked_rows.get((rid, g))
+            remembered += known is not None and known[0][0] == manager.table_version(rid)
+            versioned.append(StepEntry(rid, toks, start, {g: manager.block_table(rid, g)}, None, [n - 1], manager.table_version(rid)))
+            plain.append(StepEntry(rid, toks, start, {g: manager.block_table(rid, g)}, None, [n - 1]))
+            live[row][1] = start + n
+        got, want = runner._stage(versioned, 4), runner._stage(plain, 4)
+        assert np.array_equal(got[0], want[0]) and got[1:3] == want[1:3] and got[3]["k_lens"] == want[3]["k_lens"], f"step {step}"
+    assert remembered > 60
+    rid, start = live[0]
+    assert manager.allocate(rid, start, 1)
+    with pytest.raises(StepError, match="page id outside"):
+        runner._stage([StepEntry(rid, [1], start, {g: [999] * 4}, None, [0], -1)], 4)
+    for row in range(3):
+        manager.free(live[row][0])
+
+
 def test_table_version_changes_exactly_when_a_table_does(runtime):
     manager, _ = runtime
     assert manager.allocate("v", 0, 5)
