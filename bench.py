@@ -601,7 +601,7 @@ def main() -> int:
     with tempfile.TemporaryDirectory() as folder:
         engine = make_engine(cfg, folder, args.dtype, max(64, args.batch), args.context)
         if args.prefill_only:
-            psec = time_prefill(engine, PREFILL_TOKENS, seed=100)
+            psec = time_prefill(engine, PREFILL_TOKENS, seed=100, repeats=6)
             print(json.dumps({"prefill_ms": round(psec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / psec, 1),
                               "frac": round(prefill_flops(cfg, PREFILL_TOKENS, 1) / psec / PEAK_FLOPS[short], 4)}))
             return 0
@@ -640,7 +640,7 @@ def main() -> int:
             points[f"mixed_b{args.batch}_p256"] = mixed["tokens_per_s"]
             record["mixed_step"] = mixed
             record["points"] = points
-            psec = time_prefill(engine, PREFILL_TOKENS, seed=100)
+            psec = time_prefill(engine, PREFILL_TOKENS, seed=100, repeats=6)
             flops = prefill_flops(cfg, PREFILL_TOKENS, 1)
             record["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3),
                                  "frac": round(flops / psec / PEAK_FLOPS[short], 4)}

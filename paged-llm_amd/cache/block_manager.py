@@ -145,6 +145,7 @@ class _Holding:
     tables: dict[str, list[int]]
     state_slot: int | None = None
     version: int = 0          # a new number whenever any table changes (never reused by another holding)
+    digests: list = field(default_factory=list)   # chained digests of the request's first full pages, worked out ahead
 
 
 class CacheManager:
@@ -260,6 +261,7 @@ class CacheManager:
         if first == last:
             return
         hold = self._held[request]
+        ready = hold.digests
         for g, pool in self.pools.items():
             table = hold.tables[g]
             prev = pool.digest[table[first - 1]] if first > 0 else None
@@ -268,10 +270,26 @@ class CacheManager:
                 if pool.digest[page] is None:
                     if prev is None and i > 0:
                         break                      # predecessor not indexed: the chain cannot go on
-                    d = chain_digest(prev, tokens[i * bs:(i + 1) * bs])
+                    if i < len(ready) and (i == 0 or ready[i - 1] == prev):
+                        d = ready[i]               # worked out while the step ran, on the same chain
+                    else:
+                        d = chain_digest(prev, tokens[i * bs:(i + 1) * bs])
                     if not pool.remember(page, d):
                         break                      # same content already indexed under another page
                 prev = pool.digest[page]
+
+    def digests_ahead(self, request, tokens: list[int], after: int) -> None:
+        """The digests under which ``note_computed`` will index the full pages of ``tokens[:after]``, worked out
+        ahead of it: they depend on the tokens alone, so whoever launched a step that computes a long prompt portion
+        can have them made while the GPU runs, and the step's end only has to index them."""
+        hold = self._held.get(request) if self.prefix_caching else None
+        if hold is None:
+            return
+        bs, ready = self.block_size, hold.digests
+        prev = ready[-1] if ready else None
+        for i in range(len(ready), after // bs):
+            prev = chain_digest(prev, tokens[i * bs:(i + 1) * bs])
+            ready.append(prev)
 
     # ------------------------------------------------------------------ allocation
     def _first_needed_page(self, g: GroupSpec, num_computed: int) -> int:

@@ -130,6 +130,8 @@ class LLMEngine:
         self._flight = None
         # Launch the step after the one under way before waiting for its tokens (see ``_advance``); off: one step at a time.
         self.run_ahead = True
+        # Prompt portions of at least this many tokens have the digests of their pages made while the GPU computes them.
+        self.digests_ahead_from = 4 * cfg.block_size
         log.info("cache: %d pages of %d positions per group (%d positions, %.2f GiB)", pages, cfg.block_size,
                  pages * cfg.block_size, self.kv_cache.total_bytes() / 2**30)
 
@@ -257,6 +259,10 @@ class LLMEngine:
         else:
             plan, chosen, pending = flight
         ahead = self._launch_ahead(plan, pending)            # the GPU's next millisecond, queued before the host waits
+        if plan.prompt_tokens >= self.digests_ahead_from:    # (page digests of long portions: made while the GPU runs)
+            for g in plan.grants:
+                if g.count >= self.digests_ahead_from:
+                    self.cache_manager.digests_ahead(g.request.id, g.request.tokens, g.request.computed + g.count)
         sampled = {r.id: t for r, t in zip(chosen, pending.result())}
         committed = [g for g in plan.grants if not g.request.ended]      # (the others ended while this step already ran)
         ended = self.scheduler.commit(plan, sampled)

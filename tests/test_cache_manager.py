@@ -262,6 +262,67 @@ def test_random_orders_lose_nothing(seed, groups):
     assert all(m.num_free_pages(g) == 24 for g in m.groups) and m.slots.num_free == 5
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_digests_made_ahead_index_the_same_pages(seed):
+    """Two managers in lockstep under random orders of requests with shared prefixes, forks and decoded tokens; one
+    has the digests of a request's full pages made ahead (at random moments, for random lengths of what it holds):
+    after every action both index the same pages under the same digests."""
+    rng = random.Random(seed)
+    bs = 4
+    a, b = (CacheManager(FULL, 32, bs, enable_prefix_caching=True) for _ in range(2))
+    live: dict = {}
+    next_id = made = 0
+    for _ in range(500):
+        action = rng.random()
+        if action < 0.3 and len(live) < 8:
+            base = rng.choice([[1] * 8, [2] * 12, [3] * 17, []])
+            toks = base + [rng.randrange(50) for _ in range(rng.randrange(1, 30))]
+            (hits, n), (hits_b, n_b) = a.find_cached_prefix(toks), b.find_cached_prefix(toks)
+            assert (hits, n) == (hits_b, n_b)
+            first = min(len(toks) - n, rng.randrange(1, 24))
+            ok = a.allocate(next_id, n, first, hits)
+            assert ok == b.allocate(next_id, n, first, hits_b)
+            if ok:
+                if rng.random() < 0.7:
+                    a.digests_ahead(next_id, toks, rng.randrange(0, len(toks) + 1))
+                    made += 1
+                a.note_computed(next_id, toks, n, n + first)
+                b.note_computed(next_id, toks, n, n + first)
+                live[next_id] = [toks, n + first]
+            next_id += 1
+        elif action < 0.75 and live:
+            rid = rng.choice(list(live))
+            toks, done = live[rid]
+            if done == len(toks):
+                toks.append(rng.randrange(50))
+            n = min(len(toks) - done, rng.randrange(1, 9))
+            ok = a.allocate(rid, done, n)
+            assert ok == b.allocate(rid, done, n)
+            if ok:
+                if rng.random() < 0.5:
+                    a.digests_ahead(rid, toks, done + n)
+                    made += 1
+                a.note_computed(rid, toks, done, done + n)
+                b.note_computed(rid, toks, done, done + n)
+                live[rid][1] = done + n
+        elif action < 0.85 and live and len(live) < 8:
+            parent = rng.choice(list(live))
+            a.fork(parent, next_id)
+            b.fork(parent, next_id)
+            live[next_id] = [list(live[parent][0]), live[parent][1]]
+            next_id += 1
+        elif live:
+            rid = rng.choice(list(live))
+            a.free(rid)
+            b.free(rid)
+            del live[rid]
+        assert a.take_pending_copies() == b.take_pending_copies()
+        a.check_invariants()
+        for g in a.pools:
+            assert a.pools[g].digest == b.pools[g].digest and a.pools[g].by_digest == b.pools[g].by_digest
+    assert made > 50 and any(p.by_digest for p in a.pools.values())
+
+
 def test_no_prefix_reuse_for_models_with_state_slots():
     """A state of fixed size exists only as of the last token run: a request that entered behind a cached
     prefix would start from a state that never saw those tokens.  With state slots in use the prefix index

@@ -122,7 +122,7 @@ def stand_in_engine(num_pages, block_size, budget, max_seqs, prefix, run_ahead, 
     engine.stats = EngineStats()
     engine.tokenizer = None
     engine.on_logits = None
-    engine._live, engine._flight, engine.run_ahead = {}, None, run_ahead
+    engine._live, engine._flight, engine.run_ahead, engine.digests_ahead_from = {}, None, run_ahead, 2 * block_size
     engine._token_ids = lambda prompt: [int(t) for t in prompt]
     return engine
 
