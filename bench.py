@@ -67,16 +67,18 @@ def prefill_flops(cfg: dict, tokens: int, rows_with_logits: int) -> float:
     return 2.0 * tokens * m["matrix_params"] + 2.0 * rows_with_logits * m["head_params"] + m["attn_flops_per_pair"] * causal_pairs
 
 
-def make_engine(cfg: dict, folder: str, dtype: str, max_seqs: int, context: int):
+def make_engine(cfg: dict, folder: str, dtype: str, max_seqs: int, context: int, weights_of=None):
+    """An engine with random weights (seed 0), or on the weights that ``weights_of``, an engine of the same sizes, holds."""
     from paged_llm_amd import EngineConfig
     from paged_llm_amd.engine.llm_engine import LLMEngine
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg, f)
     block = 16
     pages = max_seqs * ((context + 128 + block - 1) // block) + 64
+    weights = {"random_weights": 0} if weights_of is None else {"weights_of": weights_of}
     return LLMEngine(folder, EngineConfig(
         block_size=block, num_gpu_blocks=pages, max_num_seqs=max_seqs, max_num_batched_tokens=8192,
-        max_model_len=context + 128, dtype=dtype, seed=0, enable_prefix_caching=True), random_weights=0)
+        max_model_len=context + 128, dtype=dtype, seed=0, enable_prefix_caching=True), **weights)
 
 
 def random_prompts(n: int, length: int, vocab: int, seed: int):
@@ -200,7 +202,7 @@ def e2e_prompts(num_prompts: int, input_len: int, output_len: int, shared_prefix
 
 
 def run_e2e(cfg: dict, dtype: str, cases: list, num_prompts: int = 64, input_len: int = 256, output_len: int = 128,
-            block_size: int = 16, max_num_batched_tokens: int = 4096, prefix_caching: bool = True) -> dict:
+            block_size: int = 16, max_num_batched_tokens: int = 4096, prefix_caching: bool = True, weights_of=None) -> dict:
     import torch
     from paged_llm_amd import EngineConfig, SamplingParams
     from paged_llm_amd.engine.llm_engine import LLMEngine
@@ -215,7 +217,8 @@ def run_e2e(cfg: dict, dtype: str, cases: list, num_prompts: int = 64, input_len
             engine = LLMEngine(folder, EngineConfig(
                 block_size=block_size, num_gpu_blocks=max(num_prompts, case["batch"]) * pages_per_request + 64,
                 max_num_seqs=case["batch"], max_num_batched_tokens=max_num_batched_tokens, max_model_len=input_len + output_len,
-                dtype=dtype, seed=0, enable_prefix_caching=prefix_caching), random_weights=0)
+                dtype=dtype, seed=0, enable_prefix_caching=prefix_caching),
+                **({"random_weights": 0} if weights_of is None else {"weights_of": weights_of}))
             # Other prompts first, twice: a step's graph is captured when its shape comes back (a shape that a pass
             # meets once, at the change from one batch of requests to the next, is captured in the second pass), and
             # the timed pass is to show the engine as it runs from then on.
@@ -649,8 +652,7 @@ def main() -> int:
                 t = time_prefill(engine, n, seed=400 + n, repeats=5)
                 points[f"prefill_{n}_ms"] = round(t * 1e3, 3)
                 points[f"prefill_{n}_frac"] = round(prefill_flops(cfg, n, 1) / t / PEAK_FLOPS[short], 4)
-            del engine
-            torch.cuda.empty_cache()
+            # (the first engine stays for its weights: the engines below whose positions its model covers run on them)
             # longer contexts at the headline batch, each with its own fraction of the memory roofline, and a long prompt
             for context in (8192, 32768):
                 with tempfile.TemporaryDirectory() as long_folder:
@@ -668,7 +670,7 @@ def main() -> int:
             # many requests at once (the attention over the cache is most of such a step, and the host's part of it grows)
             if numbers["kv_bytes_per_token"] * 512 * (args.context + 128) < 48e9:
                 with tempfile.TemporaryDirectory() as wide_folder:
-                    wide_engine = make_engine(cfg, wide_folder, args.dtype, 512, args.context)
+                    wide_engine = make_engine(cfg, wide_folder, args.dtype, 512, args.context, weights_of=engine)
                     s, mean_ctx = time_decode(wide_engine, 512, args.context, 24, 6, seed=70)
                     nbytes_step = numbers["weight_bytes"] + 512 * mean_ctx * numbers["kv_bytes_per_token"]
                     points["decode_b512"] = round(512 / s, 1)
@@ -676,8 +678,16 @@ def main() -> int:
                     del wide_engine
                     torch.cuda.empty_cache()
             # the reference's end-to-end workload at 8 and 64 requests at a time (64 requests, 256 in / 128 out): output tokens/s
-            e2e = run_e2e(cfg, args.dtype, [c for c in E2E_CASES if c["name"] in ("256in_128out_b8", "256in_128out_b64")])
+            e2e = run_e2e(cfg, args.dtype, [c for c in E2E_CASES if c["name"] in ("256in_128out_b8", "256in_128out_b64")],
+                          weights_of=engine)
             record["e2e"] = {name: row["output_tok_per_s"] for name, row in e2e.items()}
+            del engine
+            torch.cuda.empty_cache()
+            if args.model == "tinyllama-1.1b":
+                # prompts of 128 to 4096 tokens at Llama-3.2-1B shapes, one step each: milliseconds
+                other_name, other = MODELS["llama-3.2-1b"]
+                for n, row in run_prompt_sweep(other, args.dtype, [128, 512, 2048, 4096]).items():
+                    points[f"llama32_1b_prefill_{n}_ms"] = row["ms"]
             if short == "bf16":
                 # the same two fractions against what the GPU gives to a plain large copy and a plain large product
                 peaks = measured_peaks()

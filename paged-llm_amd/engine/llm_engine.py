@@ -89,13 +89,39 @@ def _freeze_static_heap() -> None:
         _static_heap_frozen = True
 
 
+def _shared_model(held, hf_config: dict, cfg: EngineConfig, device):
+    """``held`` (another engine's model) if it is the model that ``hf_config`` and ``cfg`` ask for; else one error
+    that says what differs."""
+    from ..config.dtypes import resolve_dtype
+    from ..config.registry import lookup_architecture
+    arch = lookup_architecture(hf_config)
+    spec = arch.build_spec(arch.read_config(hf_config))
+    problems = []
+    if spec != held.spec:
+        problems.append("the folder's config.json describes another model")
+    else:
+        wanted = resolve_dtype(cfg.dtype, spec.stored_dtype)
+        if wanted != held.dtype:
+            problems.append(f"it computes in {held.dtype}, this engine is to compute in {wanted}")
+        if max(spec.max_positions, cfg.max_model_len or 0) > held.max_positions:
+            problems.append(f"it covers {held.max_positions} positions, this engine needs {max(spec.max_positions, cfg.max_model_len or 0)}")
+    if held.device != device:
+        problems.append(f"it lives on {held.device}, this engine on {device}")
+    if problems:
+        raise ValueError("the other engine's weights cannot be shared: " + "; ".join(problems))
+    return held
+
+
 class LLMEngine:
     freeze_static_heap = True          # False: the garbage collector keeps walking everything that was imported
     def __init__(self, model: str, config: EngineConfig | None = None, **overrides):
         """``model``: a folder with config.json and *.safetensors.  ``random_weights=SEED`` among
         the overrides fills the model of that folder's config.json with seeded random weights
-        instead of reading tensors."""
+        instead of reading tensors.  ``weights_of=ENGINE`` runs on the weights that another engine of the same
+        config.json, compute type and device holds already (a second cache, scheduler and set of graphs over one
+        model in memory); that engine's model must cover this one's positions."""
         seed_for_weights = overrides.pop("random_weights", None)
+        weights_of = overrides.pop("weights_of", None)
         self.config = cfg = config or EngineConfig(**overrides)
         self.device = require_gpu(cfg.device)
         if self.freeze_static_heap:
@@ -104,7 +130,9 @@ class LLMEngine:
             raise FileNotFoundError(f"{model!r} is no folder (models are not downloaded)")
         self.tokenizer = _tokenizer_of(model)
         started = time.perf_counter()
-        if seed_for_weights is None:
+        if weights_of is not None:
+            self.model = _shared_model(weights_of.model, read_config_json(model), cfg, self.device)
+        elif seed_for_weights is None:
             self.model = load_model(model, cfg.dtype, self.device, cfg.max_model_len)
         else:
             from ..weights.random_init import fill_random

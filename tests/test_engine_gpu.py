@@ -34,7 +34,8 @@ def engine_for(folder, **kw):
     from paged_llm_amd.engine.llm_engine import LLMEngine
     base = dict(dtype="float32", num_gpu_blocks=64, block_size=16, max_num_batched_tokens=24, max_model_len=128)
     base.update(kw)
-    return LLMEngine(folder, EngineConfig(**base))
+    weights_of = base.pop("weights_of", None)
+    return LLMEngine(folder, EngineConfig(**base), **({} if weights_of is None else {"weights_of": weights_of}))
 
 
 def plain_greedy(folder, prompt, n):
@@ -256,6 +257,40 @@ def test_step_api_and_abort(folder_a):
         engine.add_request([999])
     with pytest.raises(ValueError, match="tokenizer"):
         engine.add_request("text")
+
+
+def test_two_engines_over_one_set_of_weights(folder_a, folder_b):
+    """``weights_of``: a second engine (its own cache, page size, scheduler and graphs) on the model that another one holds;
+    both give the plain implementation's tokens, taking turns step by step, and what does not fit is refused with the reason."""
+    from paged_llm_amd import SamplingParams
+    first = engine_for(folder_a, dtype="bfloat16", max_model_len=300)
+    second = engine_for(folder_a, dtype="bfloat16", weights_of=first, block_size=32, num_gpu_blocks=20, max_num_batched_tokens=64)
+    assert second.model is first.model and second.kv_cache is not first.kv_cache
+    prompts = [helpers.random_tokens(n, 256, seed=70 + n) for n in (5, 40, 70)]
+    params = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    seen = {}
+    for engine in (first, second):
+        seen[id(engine)] = Observed(engine)
+        for p in prompts:
+            engine.add_request(p, params)
+    done = {id(first): {}, id(second): {}}
+    while first.has_unfinished_requests or second.has_unfinished_requests:
+        for engine in (first, second):                       # the two take turns on the one stream
+            if engine.has_unfinished_requests:
+                for out in engine.step():
+                    if out.new_token is not None:
+                        done[id(engine)].setdefault(out.seq_id, []).append(out.new_token)
+    for engine in (first, second):
+        for (rid, pos), row in seen[id(engine)].rows.items():
+            prompt = prompts[[r for r in sorted(done[id(engine)])].index(rid)]
+            tokens = prompt + done[id(engine)][rid]
+            assert helpers.worst(row, helpers.plain_logits(folder_a, tokens[:pos + 1])[pos]) <= TOL["bfloat16"]
+    with pytest.raises(ValueError, match="another model"):
+        engine_for(folder_b, dtype="bfloat16", weights_of=first)
+    with pytest.raises(ValueError, match="computes in"):
+        engine_for(folder_a, dtype="float32", weights_of=first)
+    with pytest.raises(ValueError, match="positions"):
+        engine_for(folder_a, dtype="bfloat16", weights_of=first, max_model_len=400)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
